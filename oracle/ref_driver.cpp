@@ -1,0 +1,30 @@
+// TEST INFRASTRUCTURE ONLY.  C-callable shim around the *reference's own* CPU GEMM
+// (compiled from /root/reference by build_ref.sh into oracle/_ref/), so the tests can
+// check the oracle bit-for-bit against the real thing in the build container.
+// Calls only the reference's public API: de::CreateMatrixRef, de::Matrix::ptr,
+// de::cpu::DecxSetThreadingNum, de::blas::cpu::GEMM (srcs/includes/DECX/BLAS/BLAS.h:57,60).
+#include "DECX.h"
+#include <cstring>
+
+extern "C" int ref_cpu_gemm_f32(const float* A, const float* B, const float* C, float* D,
+                                uint32_t M, uint32_t N, uint32_t K, uint32_t threads)
+{
+    de::cpu::DecxSetThreadingNum(threads);
+    de::Matrix& mA = de::CreateMatrixRef(de::_FP32_, K, M);
+    de::Matrix& mB = de::CreateMatrixRef(de::_FP32_, N, K);
+    de::Matrix& mD = de::CreateMatrixRef(de::_FP32_, N, M);
+    for (uint32_t i = 0; i < M; ++i) std::memcpy(mA.ptr<float>(i, 0), A + (size_t)i * K, K * sizeof(float));
+    for (uint32_t i = 0; i < K; ++i) std::memcpy(mB.ptr<float>(i, 0), B + (size_t)i * N, N * sizeof(float));
+    if (C) {
+        de::Matrix& mC = de::CreateMatrixRef(de::_FP32_, N, M);
+        for (uint32_t i = 0; i < M; ++i) std::memcpy(mC.ptr<float>(i, 0), C + (size_t)i * N, N * sizeof(float));
+        de::blas::cpu::GEMM(mA, mB, mC, mD);
+        mC.release();
+    } else {
+        de::blas::cpu::GEMM(mA, mB, mD);
+    }
+    const int err = de::GetLastError()->error_type;
+    for (uint32_t i = 0; i < M; ++i) std::memcpy(D + (size_t)i * N, mD.ptr<float>(i, 0), N * sizeof(float));
+    mA.release(); mB.release(); mD.release();
+    return err;
+}

@@ -1,0 +1,319 @@
+"""Pins the CPU oracle before anything is compared against it.
+
+None of these checks re-types the oracle's formula: they use exact rational arithmetic,
+numpy float64, closed forms, a structurally different implementation, the committed
+outputs of the reference's own CPU GEMM, and (in the build container) the compiled
+reference itself.
+"""
+import glob
+import os
+import zlib
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+from decx_amd import synth
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+# ------------------------------------------------------------------ exact helpers (pure Python)
+
+def round_to_f32(x: Fraction) -> np.float32:
+    """Exact round-to-nearest-even of a rational to binary32 (normal range only)."""
+    if x == 0:
+        return np.float32(0.0)
+    sign = -1 if x < 0 else 1
+    x = abs(x)
+    e = 0
+    while x >= 2:
+        x /= 2; e += 1
+    while x < 1:
+        x *= 2; e -= 1
+    assert -126 <= e <= 127
+    scaled = x * (1 << 23)                  # in [2^23, 2^24)
+    q = scaled.numerator // scaled.denominator
+    rem = scaled - q
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and (q & 1)):
+        q += 1
+    return np.float32(sign * q * 2.0 ** (e - 23))
+
+
+def exact_chain(A, B, C=None):
+    M, K = A.shape
+    N = B.shape[1]
+    out = np.zeros((M, N), np.float32)
+    for i in range(M):
+        for j in range(N):
+            acc = Fraction(float(C[i, j])) if C is not None else Fraction(0)
+            for k in range(K):
+                acc = Fraction(float(round_to_f32(Fraction(float(A[i, k])) * Fraction(float(B[k, j])) + acc)))
+            out[i, j] = np.float32(float(acc))
+    return out
+
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.uint32 if a.dtype == np.float32 else np.uint16)
+
+
+def rel_err(got, ref, K):
+    return np.max(np.abs(got.astype(np.float64) - ref.astype(np.float64))) / (np.max(np.abs(ref)) * np.sqrt(K))
+
+
+# ------------------------------------------------------------------ half conversion
+
+def test_half_to_float_all_65536(oracle):
+    L = oracle.lib()
+    h = np.arange(65536, dtype=np.uint16)
+    want = h.view(np.float16).astype(np.float32)
+    got = np.array([L.oracle_half_to_float(int(v)) for v in h], np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(bits(got[~nan]), bits(want[~nan]))
+
+
+def test_float_to_half_rne(oracle):
+    L = oracle.lib()
+    rng = np.random.default_rng(7)
+    vals = np.concatenate([
+        rng.standard_normal(20000).astype(np.float32) * np.float32(3.0),
+        (rng.standard_normal(5000) * 1e-6).astype(np.float32),       # subnormal halves
+        (rng.standard_normal(2000) * 3e4).astype(np.float32),        # near overflow
+        np.array([0.0, -0.0, 65504.0, 65519.99, 65520.0, 1e9, -1e9, 2.0 ** -24, 2.0 ** -25,
+                  np.nextafter(np.float32(2.0 ** -25), np.float32(1)), 2.0 ** -14, 1.0 + 2.0 ** -11,
+                  1.0 + 3 * 2.0 ** -11, 2047.5, 2048.5, np.inf, -np.inf], np.float32)])
+    # every exact tie between two adjacent halves in one binade
+    h = np.arange(0x3c00, 0x4000, dtype=np.uint16).view(np.float16).astype(np.float32)
+    vals = np.concatenate([vals, (h[:-1] + h[1:]) / np.float32(2)])
+    with np.errstate(over="ignore"):
+        want = vals.astype(np.float16).view(np.uint16)
+    got = np.array([L.oracle_float_to_half(float(v)) for v in vals], np.uint16)
+    assert np.array_equal(got, want)
+
+
+# ------------------------------------------------------------------ seeded inputs
+
+def test_generator_c_and_numpy_agree(oracle):
+    for rows, cols, seed in [(7, 13, 0xA001), (64, 64, 0xB004), (1, 1, 5), (33, 1, 0xC002)]:
+        a = oracle.fill_uniform_f32(rows, cols, seed)
+        b = synth.uniform_f32(rows, cols, seed)
+        assert np.array_equal(bits(a), bits(b))
+        assert a.min() >= -1.0 and a.max() < 1.0
+
+
+def test_generator_statistics():
+    u = synth.uniform_f32(400, 500, 0xA004)
+    assert abs(u.mean()) < 0.01 and abs(u.std() - 1 / np.sqrt(3)) < 0.01
+    h = synth.normal_half(400, 500, 0xA003).astype(np.float32)
+    assert abs(h.mean()) < 0.01 and abs(h.std() - 0.5) < 0.01 and np.abs(h).max() <= 4.0
+
+
+# ------------------------------------------------------------------ fp32 chain
+
+@pytest.mark.parametrize("M,N,K,with_c", [(3, 4, 5, False), (5, 3, 9, True), (2, 7, 17, False)])
+def test_chain_matches_exact_rational_fma(oracle, M, N, K, with_c):
+    A = synth.uniform_f32(M, K, 11)
+    B = synth.uniform_f32(K, N, 12)
+    C = synth.uniform_f32(M, N, 13) if with_c else None
+    want = exact_chain(A, B, C)
+    assert np.array_equal(bits(oracle.gemm_f32(A, B, C)), bits(want))
+    assert np.array_equal(bits(oracle.gemm_f32_scalar(A, B, C)), bits(want))
+
+
+@pytest.mark.parametrize("M,N,K", [(37, 53, 29), (100, 150, 77), (64, 64, 64), (1, 1, 1), (129, 1, 257), (1, 200, 33)])
+@pytest.mark.parametrize("with_c", [False, True])
+def test_vectorised_chain_equals_scalar_chain(oracle, M, N, K, with_c):
+    A = synth.uniform_f32(M, K, 21)
+    B = synth.uniform_f32(K, N, 22)
+    C = synth.uniform_f32(M, N, 23) if with_c else None
+    assert np.array_equal(bits(oracle.gemm_f32(A, B, C)), bits(oracle.gemm_f32_scalar(A, B, C)))
+
+
+def test_chain_honours_pitch_and_row_subset(oracle):
+    M, N, K = 21, 35, 19
+    Ap = np.full((M, K + 5), np.nan, np.float32); Ap[:, :K] = synth.uniform_f32(M, K, 31)
+    Bp = np.full((K, N + 3), np.nan, np.float32); Bp[:, :N] = synth.uniform_f32(K, N, 32)
+    full = oracle.gemm_f32(Ap[:, :K], Bp[:, :N])
+    assert not np.isnan(full).any()
+    dense = oracle.gemm_f32(np.ascontiguousarray(Ap[:, :K]), np.ascontiguousarray(Bp[:, :N]))
+    assert np.array_equal(bits(full), bits(dense))
+    rows = [20, 0, 7]
+    sub = oracle.gemm_f32(Ap[:, :K], Bp[:, :N], rows=rows)
+    assert np.array_equal(bits(sub), bits(full[rows]))
+
+
+@pytest.mark.parametrize("M,N,K", [(37, 53, 29), (100, 150, 77), (256, 192, 300)])
+def test_chain_close_to_float64(oracle, M, N, K):
+    A = synth.uniform_f32(M, K, 41)
+    B = synth.uniform_f32(K, N, 42)
+    C = synth.uniform_f32(M, N, 43)
+    np64 = A.astype(np.float64) @ B.astype(np.float64)
+    brute = oracle.gemm_f64_brute(A, B)
+    assert np.max(np.abs(brute - np64)) < 1e-12 * K
+    assert rel_err(oracle.gemm_f32(A, B), np64, K) < 2e-7
+    assert rel_err(oracle.gemm_f32(A, B, C), np64 + C, K) < 2e-7
+    # a dropped C, a transposed operand or a sign flip is ~1e-1 on this scale
+    assert rel_err(oracle.gemm_f32(A, B), np64 + C, K) > 1e-3
+
+
+def test_closed_forms(oracle):
+    n = 67
+    B = synth.uniform_f32(n, 45, 51)
+    eye = np.eye(n, dtype=np.float32)
+    assert np.array_equal(bits(oracle.gemm_f32(eye, B)), bits(B))
+    A = synth.uniform_f32(45, n, 52)
+    assert np.array_equal(bits(oracle.gemm_f32(A, eye)), bits(A))
+    K = 1000
+    ones = oracle.gemm_f32(np.ones((9, K), np.float32), np.ones((K, 11), np.float32))
+    assert np.all(ones == K)
+    # asymmetric operands: D[i][j] = (i+1) * (j+1) * K, exact in fp32
+    a = np.repeat(np.arange(1, 6, dtype=np.float32)[:, None], 8, 1)
+    b = np.repeat(np.arange(1, 8, dtype=np.float32)[None, :], 8, 0)
+    assert np.array_equal(oracle.gemm_f32(a, b), 8 * np.outer(np.arange(1, 6), np.arange(1, 8)).astype(np.float32))
+
+
+def test_reference_sample_known_answer(oracle):
+    """samples/Matrix_Multiplication/MatMul.cpp:16-40: A[i][j] = j, B[i][j] = i, L = 1005, so every
+    element is sum l^2 = (L-1)L(2L-1)/6 = 337 853 530 (not exactly representable: fp32 tolerance);
+    with L = 100 the sum 328 350 stays below 2^24 and must be exact."""
+    for L, exact in [(1005, False), (100, True)]:
+        M, N = 13, 17
+        A = np.tile(np.arange(L, dtype=np.float32), (M, 1))
+        B = np.tile(np.arange(L, dtype=np.float32)[:, None], (1, N))
+        want = (L - 1) * L * (2 * L - 1) // 6
+        got = oracle.gemm_f32(A, B)
+        if exact:
+            assert np.all(got == np.float32(want))
+        else:
+            assert want == 337853530
+            assert np.max(np.abs(got.astype(np.float64) - want)) / want < 4e-6   # ~ sqrt(L) * 2^-24
+
+
+def test_alpha_beta_form(oracle):
+    M, N, K = 65, 130, 67
+    A = synth.uniform_f32(M, K, 61); B = synth.uniform_f32(K, N, 62); C = synth.uniform_f32(M, N, 63)
+    ref64 = A.astype(np.float64) @ B.astype(np.float64)
+    for alpha, beta in [(1.0, 1.0), (-0.75, 2.5), (0.0, 1.0), (2.0, 0.0)]:
+        got = oracle.gemm_f32(A, B, C, alpha, beta)
+        want = alpha * ref64 + beta * C
+        assert np.max(np.abs(got - want)) / (max(np.max(np.abs(want)), 1e-30) * np.sqrt(K)) < 2e-7
+    # alpha = beta = 1 differs from the seeded chain by rounding order only
+    assert rel_err(oracle.gemm_f32(A, B, C, 1.0, 1.0), oracle.gemm_f32(A, B, C), K) < 1e-7
+    assert np.array_equal(bits(oracle.gemm_f32(A, B, C, 1.0, 0.0)), bits(oracle.gemm_f32(A, B)))
+
+
+# ------------------------------------------------------------------ fp16
+
+def test_f16_oracle(oracle):
+    M, N, K = 45, 70, 83
+    A = synth.normal_half(M, K, 71); B = synth.normal_half(K, N, 72); C = synth.normal_half(M, N, 73)
+    ref64 = A.astype(np.float64) @ B.astype(np.float64)
+    got = oracle.gemm_f16(A, B)
+    assert rel_err(got, ref64, K) < 2e-4          # one half rounding of the output: <= 2^-11 relative
+    # the widened inputs through the fp32 chain, rounded once
+    want = oracle.gemm_f32(A.astype(np.float32), B.astype(np.float32)).astype(np.float16)
+    assert np.array_equal(bits(got), bits(want))
+    got = oracle.gemm_f16(A, B, C, 1.5, -0.5)
+    assert rel_err(got, 1.5 * ref64 - 0.5 * C.astype(np.float64), K) < 2e-4
+    rows = [3, 44]
+    assert np.array_equal(bits(oracle.gemm_f16(A, B, rows=rows)), bits(oracle.gemm_f16(A, B)[rows]))
+
+
+# ------------------------------------------------------------------ the multithreaded restatement
+
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (100, 150, 77), (1000, 1500, 777), (37, 53, 300), (8, 8, 1),
+                                   (129, 1, 257), (1, 200, 33), (300, 24, 129)])
+@pytest.mark.parametrize("threads", [1, 2, 7, 8, 16])
+def test_port_bit_equal_to_chain(oracle, M, N, K, threads):
+    if M * N * K > 1e8 and threads in (2, 7):
+        pytest.skip("large case covered at 1, 8 and 16 threads")
+    A = synth.uniform_f32(M, K, 81); B = synth.uniform_f32(K, N, 82); C = synth.uniform_f32(M, N, 83)
+    assert np.array_equal(bits(oracle.cpu_port_gemm_f32(A, B, None, threads)), bits(oracle.gemm_f32(A, B)))
+    assert np.array_equal(bits(oracle.cpu_port_gemm_f32(A, B, C, threads)), bits(oracle.gemm_f32(A, B, C)))
+
+
+def test_port_rejects_bad_layout(oracle):
+    import ctypes
+    L = oracle.lib()
+    a = np.zeros(64, np.float32)
+    p = a.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+    assert L.cpu_port_gemm_f32(p, p, None, p, 4, 4, 4, 7, 8, 0, 8, p, 1) == -1     # pitch not a multiple of 8
+    assert L.cpu_port_gemm_f32(p, p, None, p, 4, 12, 4, 8, 8, 0, 8, p, 1) == -1    # width exceeds pitch
+
+
+# ------------------------------------------------------------------ golden fixtures
+
+def load_inputs(g):
+    M, N, K = int(g["M"]), int(g["N"]), int(g["K"])
+    A = synth.uniform_f32(M, K, int(g["seed_a"]))
+    B = synth.uniform_f32(K, N, int(g["seed_b"]))
+    return M, N, K, A, B
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLD, "ref_f32_*.npz"))))
+def test_oracle_reproduces_reference_outputs(oracle, path):
+    """Outputs of the reference's own de::blas::cpu::GEMM, committed as data."""
+    g = np.load(path)
+    M, N, K, A, B = load_inputs(g)
+    assert zlib.crc32(g["D"].tobytes()) & 0xFFFFFFFF == int(g["crc"])
+    assert np.array_equal(bits(oracle.gemm_f32(A, B)), bits(g["D"]))
+    assert np.array_equal(bits(oracle.cpu_port_gemm_f32(A, B, None, int(g["threads"]))), bits(g["D"]))
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLD, "orc_f32_*.npz"))))
+def test_oracle_regression_fixtures_f32(oracle, path):
+    g = np.load(path)
+    M, N, K, A, B = load_inputs(g)
+    C = synth.uniform_f32(M, N, int(g["seed_c"])) if bool(g["with_c"]) else None
+    alpha = None if np.isnan(g["alpha"]) else float(g["alpha"])
+    beta = None if np.isnan(g["beta"]) else float(g["beta"])
+    assert np.array_equal(bits(oracle.gemm_f32(A, B, C, alpha, beta)), bits(g["D"]))
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLD, "orc_f16_*.npz"))))
+def test_oracle_regression_fixtures_f16(oracle, path):
+    g = np.load(path)
+    A = g["A"].view(np.float16); B = g["B"].view(np.float16)
+    C = g["C"].view(np.float16) if bool(g["with_c"]) else None
+    got = oracle.gemm_f16(A, B, C, float(g["alpha"]), float(g["beta"]))
+    assert np.array_equal(got.view(np.uint16), g["D"])
+
+
+def test_golden_set_is_complete():
+    assert len(glob.glob(os.path.join(GOLD, "ref_f32_*.npz"))) == 4
+    assert len(glob.glob(os.path.join(GOLD, "orc_f32_*.npz"))) == 5
+    assert len(glob.glob(os.path.join(GOLD, "orc_f16_*.npz"))) == 3
+
+
+# ------------------------------------------------------------------ the compiled reference (build container only)
+
+def _need_reference(oracle):
+    if not oracle.reference_available():
+        pytest.skip("compiled reference (oracle/_ref) not present on this host")
+
+
+@pytest.mark.parametrize("M,N,K,threads", [(64, 64, 64, 1), (256, 256, 256, 4), (1024, 1024, 1024, 8),
+                                           (1000, 1500, 777, 8), (1000, 1500, 777, 4), (512, 128, 1024, 2)])
+def test_chain_bit_equal_to_compiled_reference(oracle, M, N, K, threads):
+    _need_reference(oracle)
+    A = synth.uniform_f32(M, K, 91); B = synth.uniform_f32(K, N, 92)
+    D, err = oracle.reference_cpu_gemm_f32(A, B, None, threads)
+    assert err == 0
+    assert np.array_equal(bits(D), bits(oracle.gemm_f32(A, B)))
+    assert np.array_equal(bits(D), bits(oracle.cpu_port_gemm_f32(A, B, None, threads)))
+
+
+def test_reference_accumulate_form_agrees_on_the_rows_it_gets_right(oracle):
+    """The reference's fp32 D = A.B + C seeds every row of an 8-row block with the block's first
+    row of C (GEMM_fp32_kernels_x86_64.h:231-232), so only rows with row % 8 == 0 follow the
+    documented semantics; on those rows it must equal the oracle's seeded chain bit for bit."""
+    _need_reference(oracle)
+    M = N = K = 64
+    A = synth.uniform_f32(M, K, 93); B = synth.uniform_f32(K, N, 94); C = synth.uniform_f32(M, N, 95)
+    try:
+        D, err = oracle.reference_cpu_gemm_f32(A, B, C, 1)
+    except RuntimeError:
+        pytest.skip("the reference's accumulate form crashed in this process (it does so intermittently)")
+    want = oracle.gemm_f32(A, B, C)
+    assert np.array_equal(bits(D[::8]), bits(want[::8]))
