@@ -1,0 +1,70 @@
+"""Builds the native libraries in-tree (run on the build host; hipcc cross-compiles gfx950
+without a GPU):
+
+    decx_amd/lib/libdecx_hip.so        HIP kernels + the C ABI (include/decx_hip.h)
+    decx_amd/lib/libDECX_BLAS_HIP.so   C++ host layer: the de:: objects and entry points
+
+    python -m decx_amd.build
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+HOST = os.path.join(PKG, "host")
+LIB = os.path.join(PKG, "lib")
+OBJ = os.path.join(PKG, "lib", "obj")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
+             # packed-fp32 VALU forms are kept out of the generated code on purpose
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             "-Wno-unused-command-line-argument"]
+HIP_SOURCES = ["gemm_f32.hip", "gemm_f16.hip", "gemv_f32.hip", "capi.hip"]
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wextra",
+              "-I" + os.path.join(ROOT, "include")]
+
+
+def _run(cmd):
+    done = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if done.returncode != 0:
+        sys.stderr.write(" ".join(cmd) + "\n" + done.stdout)
+        raise RuntimeError("build step failed: " + cmd[-1])
+    return done.stdout
+
+
+def build_hip(verbose=False):
+    os.makedirs(OBJ, exist_ok=True)
+    objs = [os.path.join(OBJ, s.replace(".hip", ".o")) for s in HIP_SOURCES]
+    cmds = [[HIPCC] + HIP_FLAGS + ["-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(HIP_SOURCES, objs)]
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        list(pool.map(_run, cmds))
+    out = os.path.join(LIB, "libdecx_hip.so")
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs)
+    if verbose:
+        print("built", out)
+    return out
+
+
+def build_host(verbose=False):
+    srcs = sorted(f for f in os.listdir(HOST) if f.endswith(".cpp")) if os.path.isdir(HOST) else []
+    if not srcs:
+        return None
+    out = os.path.join(LIB, "libDECX_BLAS_HIP.so")
+    _run(["g++"] + HOST_FLAGS + ["-shared", "-o", out] + [os.path.join(HOST, s) for s in srcs] +
+         ["-L" + LIB, "-ldecx_hip", "-Wl,-rpath,$ORIGIN"])
+    if verbose:
+        print("built", out)
+    return out
+
+
+def build_all(verbose=False):
+    build_hip(verbose)
+    build_host(verbose)
+
+
+if __name__ == "__main__":
+    build_all(verbose=True)

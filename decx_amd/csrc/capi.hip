@@ -1,0 +1,299 @@
+// The C ABI declared in include/decx_hip.h: argument checking, the tile planner, and
+// thin wrappers over the HIP runtime.  No C++ type crosses this boundary.
+#include "../../include/decx_hip.h"
+#include "gemm_common.hpp"
+
+#include <cstring>
+
+using namespace decx_hip;
+
+namespace {
+
+struct DeviceState {
+    bool ready = false;
+    int device = -1;
+    int compute_units = 256;       // MI355X; used by the planner before init
+    hipDeviceProp_t prop;
+};
+DeviceState g_dev;
+
+inline int hip_rc(hipError_t e) { return (int)e; }
+inline hipStream_t as_stream(void* s) { return (hipStream_t)s; }
+
+inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+// Picks the block tile: cost = (tiles the busiest CU runs) x (tile area) / (relative speed
+// of that shape).  Big tiles win once they fill the chip; small tiles win while the grid
+// would otherwise leave CUs idle.  Ties go to the larger tile.
+int choose_tile(bool f16, uint32_t M, uint32_t N)
+{
+    int best = TILE_64x64;
+    double best_cost = 1e300;
+    for (int s = TILE_COUNT - 1; s >= 0; --s) {
+        const TileInfo ti = f16 ? tile_info_f16(s) : tile_info_f32(s);
+        const uint64_t tiles = (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
+        const uint64_t per_cu = (tiles + g_dev.compute_units - 1) / g_dev.compute_units;
+        const double cost = (double)per_cu * ti.bm * ti.bn / ti.rel_speed;
+        if (cost <= best_cost) { best_cost = cost; best = s; }
+    }
+    return best;
+}
+
+int check_gemm(const void* A, const void* B, const void* C, const void* D, uint32_t M, uint32_t N, uint32_t K,
+               uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd)
+{
+    if (M == 0 || N == 0) return DECX_HIP_OK;
+    if (!A || !B || !D) return DECX_HIP_E_INVALID_ARG;
+    if (lda < K || ldb < N || ldd < N || (C && ldc < N)) return DECX_HIP_E_INVALID_ARG;
+    return DECX_HIP_OK;
+}
+
+template <bool F16>
+int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, uint32_t N, uint32_t K,
+             uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha, float beta, void* stream,
+             int tile, int force_edge)
+{
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    const int rc = check_gemm(A, B, C, D, M, N, K, lda, ldb, ldc, ldd);
+    if (rc != DECX_HIP_OK || M == 0 || N == 0) return rc;
+    if (tile != DECX_HIP_TILE_AUTO && (tile < 0 || tile >= TILE_COUNT)) return DECX_HIP_E_INVALID_ARG;
+
+    if (!F16 && N == 1 && tile == DECX_HIP_TILE_AUTO && K > 0)
+        return launch_gemv_f32((const float*)A, (const float*)B, (const float*)C, (float*)D, M, K, lda,
+                               ldb, ldc, ldd, alpha, beta, as_stream(stream));
+
+    constexpr uint32_t per16 = F16 ? 8u : 4u;          // elements per 16 bytes
+    GemmArgs g;
+    std::memset(&g, 0, sizeof g);
+    g.A = A; g.B = B; g.C = C; g.D = D;
+    g.M = M; g.N = N; g.K = K;
+    g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldd = ldd;
+    g.alpha = alpha; g.beta = beta;
+    g.vec_ok = (aligned16(A) && aligned16(B) && aligned16(D) && (!C || aligned16(C)) &&
+                lda % per16 == 0 && ldb % per16 == 0 && ldd % per16 == 0 && (!C || ldc % per16 == 0)) ? 1u : 0u;
+    const int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile(F16, M, N) : tile;
+    const bool edge = force_edge != 0 || K == 0;
+    return F16 ? launch_gemm_f16(shape, edge, g, as_stream(stream))
+               : launch_gemm_f32(shape, edge, g, as_stream(stream));
+}
+
+}  // namespace
+
+extern "C" {
+
+int decx_hip_init(int device)
+{
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess) return hip_rc(e);
+    if (count <= 0 || device < 0 || device >= count) return DECX_HIP_E_NO_DEVICE;
+    if ((e = hipSetDevice(device)) != hipSuccess) return hip_rc(e);
+    if ((e = hipGetDeviceProperties(&g_dev.prop, device)) != hipSuccess) return hip_rc(e);
+    g_dev.device = device;
+    g_dev.compute_units = g_dev.prop.multiProcessorCount > 0 ? g_dev.prop.multiProcessorCount : 256;
+    g_dev.ready = true;
+    return DECX_HIP_OK;
+}
+
+int decx_hip_get_device_props(decx_hip_device_props* out)
+{
+    if (!out) return DECX_HIP_E_INVALID_ARG;
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    std::memset(out, 0, sizeof *out);
+    std::strncpy(out->name, g_dev.prop.name, sizeof out->name - 1);
+    std::strncpy(out->arch, g_dev.prop.gcnArchName, sizeof out->arch - 1);
+    out->compute_units = g_dev.prop.multiProcessorCount;
+    out->clock_khz = g_dev.prop.clockRate;
+    out->memory_clock_khz = g_dev.prop.memoryClockRate;
+    out->memory_bus_bits = g_dev.prop.memoryBusWidth;
+    out->lds_bytes_per_block = (int32_t)g_dev.prop.sharedMemPerBlock;
+    out->wavefront_size = g_dev.prop.warpSize;
+    out->global_mem_bytes = g_dev.prop.totalGlobalMem;
+    return DECX_HIP_OK;
+}
+
+const char* decx_hip_error_string(int code)
+{
+    switch (code) {
+    case DECX_HIP_OK:            return "success";
+    case DECX_HIP_E_INVALID_ARG: return "invalid argument (null pointer, pitch smaller than width, or unknown enum)";
+    case DECX_HIP_E_NOT_INIT:    return "decx_hip_init() has not been called";
+    case DECX_HIP_E_NO_DEVICE:   return "no usable GPU";
+    default:                     return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
+    }
+}
+
+int decx_hip_malloc(void** ptr, size_t bytes)
+{
+    if (!ptr) return DECX_HIP_E_INVALID_ARG;
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    return hip_rc(hipMalloc(ptr, bytes ? bytes : 1));
+}
+int decx_hip_free(void* ptr) { return ptr ? hip_rc(hipFree(ptr)) : DECX_HIP_OK; }
+
+int decx_hip_host_malloc(void** ptr, size_t bytes)
+{
+    if (!ptr) return DECX_HIP_E_INVALID_ARG;
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    return hip_rc(hipHostMalloc(ptr, bytes ? bytes : 1, hipHostMallocDefault));
+}
+int decx_hip_host_free(void* ptr) { return ptr ? hip_rc(hipHostFree(ptr)) : DECX_HIP_OK; }
+
+int decx_hip_memset_async(void* ptr, int value, size_t bytes, void* stream)
+{
+    if (!ptr && bytes) return DECX_HIP_E_INVALID_ARG;
+    if (!bytes) return DECX_HIP_OK;
+    return hip_rc(hipMemsetAsync(ptr, value, bytes, as_stream(stream)));
+}
+
+int decx_hip_memcpy2d_async(void* dst, size_t dst_pitch, const void* src, size_t src_pitch,
+                            size_t width_bytes, size_t height, int kind, void* stream)
+{
+    if (!width_bytes || !height) return DECX_HIP_OK;
+    if (!dst || !src || dst_pitch < width_bytes || src_pitch < width_bytes || kind < 0 || kind > 2)
+        return DECX_HIP_E_INVALID_ARG;
+    static const hipMemcpyKind kinds[3] = {hipMemcpyHostToDevice, hipMemcpyDeviceToHost, hipMemcpyDeviceToDevice};
+    return hip_rc(hipMemcpy2DAsync(dst, dst_pitch, src, src_pitch, width_bytes, height, kinds[kind], as_stream(stream)));
+}
+
+int decx_hip_stream_create(void** stream)
+{
+    if (!stream) return DECX_HIP_E_INVALID_ARG;
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    hipStream_t s;
+    const hipError_t e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);   // default priority
+    *stream = (e == hipSuccess) ? (void*)s : nullptr;
+    return hip_rc(e);
+}
+int decx_hip_stream_destroy(void* stream) { return stream ? hip_rc(hipStreamDestroy(as_stream(stream))) : DECX_HIP_OK; }
+int decx_hip_stream_sync(void* stream) { return hip_rc(hipStreamSynchronize(as_stream(stream))); }
+
+int decx_hip_event_create(void** event)
+{
+    if (!event) return DECX_HIP_E_INVALID_ARG;
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    hipEvent_t ev;
+    const hipError_t e = hipEventCreate(&ev);
+    *event = (e == hipSuccess) ? (void*)ev : nullptr;
+    return hip_rc(e);
+}
+int decx_hip_event_destroy(void* event) { return event ? hip_rc(hipEventDestroy((hipEvent_t)event)) : DECX_HIP_OK; }
+int decx_hip_event_record(void* event, void* stream)
+{
+    return event ? hip_rc(hipEventRecord((hipEvent_t)event, as_stream(stream))) : DECX_HIP_E_INVALID_ARG;
+}
+int decx_hip_event_sync(void* event)
+{
+    return event ? hip_rc(hipEventSynchronize((hipEvent_t)event)) : DECX_HIP_E_INVALID_ARG;
+}
+int decx_hip_event_elapsed_ms(void* start, void* stop, float* ms)
+{
+    if (!start || !stop || !ms) return DECX_HIP_E_INVALID_ARG;
+    return hip_rc(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+}
+
+int decx_hip_gemm_f32(const float* A, const float* B, const float* C, float* D, uint32_t M, uint32_t N, uint32_t K,
+                      uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha, float beta, void* stream)
+{
+    return run_gemm<false>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0);
+}
+
+int decx_hip_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, uint32_t M, uint32_t N,
+                      uint32_t K, uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha, float beta,
+                      void* stream)
+{
+    return run_gemm<true>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0);
+}
+
+int decx_hip_gemm_f32_tile(const float* A, const float* B, const float* C, float* D, uint32_t M, uint32_t N,
+                           uint32_t K, uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha,
+                           float beta, void* stream, int tile, int force_edge)
+{
+    return run_gemm<false>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, tile, force_edge);
+}
+
+int decx_hip_gemm_f16_tile(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, uint32_t M,
+                           uint32_t N, uint32_t K, uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                           float alpha, float beta, void* stream, int tile, int force_edge)
+{
+    return run_gemm<true>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, tile, force_edge);
+}
+
+int decx_hip_gemv_f32(const float* A, const float* x, const float* c, float* y, uint32_t M, uint32_t K, uint32_t lda,
+                      uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, void* stream)
+{
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    if (M == 0) return DECX_HIP_OK;
+    if (!A || !x || !y || lda < K || incx == 0 || incy == 0 || (c && incc == 0)) return DECX_HIP_E_INVALID_ARG;
+    return launch_gemv_f32(A, x, c, y, M, K, lda, incx, incc, incy, alpha, beta, as_stream(stream));
+}
+
+int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int aligned, decx_hip_plan* out)
+{
+    if (!out || (elem_bytes != 4 && elem_bytes != 2)) return DECX_HIP_E_INVALID_ARG;
+    std::memset(out, 0, sizeof *out);
+    if (M == 0 || N == 0) return DECX_HIP_OK;
+    const bool f16 = elem_bytes == 2;
+    if (!f16 && N == 1 && K > 0) {
+        out->path = DECX_HIP_PATH_GEMV;
+        out->tile_m = 8; out->tile_n = 1;
+        out->grid = (M + 7) / 8;
+        return DECX_HIP_OK;
+    }
+    const int shape = choose_tile(f16, M, N);
+    const TileInfo ti = f16 ? tile_info_f16(shape) : tile_info_f32(shape);
+    const uint32_t bk = f16 ? 64u : 16u;
+    out->path = shape;
+    out->tile_m = ti.bm; out->tile_n = ti.bn;
+    out->grid = ((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
+    out->edge = (M % ti.bm || N % ti.bn || K % bk || K == 0 || !aligned) ? 1 : 0;
+    return DECX_HIP_OK;
+}
+
+uint16_t decx_hip_float_to_half(float value)
+{
+    uint32_t f;
+    std::memcpy(&f, &value, 4);
+    const uint32_t sign = (f >> 16) & 0x8000u;
+    const uint32_t mag = f & 0x7fffffffu;
+    if (mag > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((mag >> 13) & 0x1ffu));    // NaN
+    if (mag >= 0x47800000u) return (uint16_t)(sign | 0x7c00u);                            // >= 2^16: inf
+    uint32_t bits;
+    if (mag >= 0x38800000u) {                 // normal half: drop 13 mantissa bits, rebias by 112
+        const uint32_t base = mag - 0x38000000u;
+        bits = base >> 13;
+        const uint32_t rest = base & 0x1fffu;
+        if (rest > 0x1000u || (rest == 0x1000u && (bits & 1u))) ++bits;   // carry may reach 0x7c00 = inf
+    } else if (mag >= 0x33000000u) {          // subnormal half
+        const uint32_t exp = mag >> 23;       // 102 .. 112
+        const uint32_t sig = (mag & 0x7fffffu) | 0x800000u;
+        const uint32_t shift = 126u - exp;    // 14 .. 24
+        bits = sig >> shift;
+        const uint32_t rest = sig & ((1u << shift) - 1u), half = 1u << (shift - 1);
+        if (rest > half || (rest == half && (bits & 1u))) ++bits;
+    } else {
+        bits = 0;
+    }
+    return (uint16_t)(sign | bits);
+}
+
+float decx_hip_half_to_float(uint16_t h)
+{
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    const uint32_t e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+    uint32_t f;
+    if (e == 0x1fu)      f = sign | 0x7f800000u | (m << 13);
+    else if (e)          f = sign | ((e + 112u) << 23) | (m << 13);
+    else if (!m)         f = sign;
+    else {
+        // subnormal: value = m * 2^-24; let the FPU normalise it
+        float v = (float)m * 5.9604644775390625e-08f;
+        std::memcpy(&f, &v, 4);
+        f |= sign;
+    }
+    float out;
+    std::memcpy(&out, &f, 4);
+    return out;
+}
+
+}  // extern "C"

@@ -1,0 +1,90 @@
+// Shared declarations of the gfx950 GEMM kernels: argument block, tile-shape table,
+// block -> tile mapping.  Device code here is written for CDNA4 only (wave64, MFMA,
+// 160 KB LDS per CU, 8 XCDs with one L2 each).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace decx_hip {
+
+typedef float    floatx4  __attribute__((ext_vector_type(4)));
+typedef float    floatx2  __attribute__((ext_vector_type(2)));
+typedef float    floatx16 __attribute__((ext_vector_type(16)));
+typedef _Float16 halfx8   __attribute__((ext_vector_type(8)));
+typedef _Float16 halfx4   __attribute__((ext_vector_type(4)));
+typedef uint32_t uintx4   __attribute__((ext_vector_type(4)));
+typedef uint32_t uintx2   __attribute__((ext_vector_type(2)));
+
+// One GEMM problem: D = A.B  (C == nullptr)  or  D = fma(C, beta, alpha * (A.B)).
+// All matrices row-major; ld* are row pitches in elements.
+struct GemmArgs {
+    const void* A;
+    const void* B;
+    const void* C;
+    void*       D;
+    uint32_t M, N, K;
+    uint32_t lda, ldb, ldc, ldd;
+    float alpha, beta;
+    uint32_t tiles_m, tiles_n;   // number of block tiles along M and N
+    uint32_t xcd_remap;          // 1: grid size is a multiple of 8, use the per-XCD ordering
+    uint32_t vec_ok;             // 1: every base pointer is 16-byte aligned and every pitch a multiple of 16 bytes
+};
+
+constexpr int kXcds = 8;        // MI355X: 8 accelerator complex dies, blocks are dealt to them round-robin
+constexpr int kGroupM = 4;      // tile-rows per L2 patch (4 x 8 tiles run together on one XCD's 32 CUs)
+
+// Maps the hardware block index to a tile.  Hardware deals consecutive block ids to
+// consecutive XCDs; each XCD has a private L2.  Step 1 gives every XCD a contiguous
+// range of logical ids, step 2 walks logical ids in groups of kGroupM tile-rows so the
+// 32 tiles resident on one XCD form a compact patch that shares A rows and B columns.
+__device__ __forceinline__ void block_to_tile(const GemmArgs& g, uint32_t& tile_m, uint32_t& tile_n)
+{
+    const uint32_t nb = g.tiles_m * g.tiles_n;
+    uint32_t id = blockIdx.x;
+    if (g.xcd_remap) id = (id % kXcds) * (nb / kXcds) + id / kXcds;
+    const uint32_t per_group = kGroupM * g.tiles_n;
+    const uint32_t group = id / per_group;
+    const uint32_t first_m = group * kGroupM;
+    const uint32_t rows = (g.tiles_m - first_m) < (uint32_t)kGroupM ? (g.tiles_m - first_m) : (uint32_t)kGroupM;
+    const uint32_t in_group = id % per_group;
+    tile_m = first_m + in_group % rows;
+    tile_n = in_group / rows;
+}
+
+// ---- tile-shape table shared by the planner and the launchers -----------------
+
+enum TileShape : int {
+    TILE_256x256 = 0,
+    TILE_128x128 = 1,
+    TILE_64x64   = 2,
+    TILE_COUNT   = 3,
+};
+
+struct TileInfo { int bm, bn, threads; float rel_speed; int blocks_per_cu; };
+
+// rel_speed: per-CU throughput of the shape relative to the largest one once the chip is
+// full (smaller tiles re-read more operand data per flop and keep fewer MFMAs in flight).
+__host__ inline TileInfo tile_info_f32(int shape)
+{
+    switch (shape) {
+    case TILE_256x256: return {256, 256, 512, 1.00f, 1};
+    case TILE_128x128: return {128, 128, 256, 0.80f, 2};
+    default:           return { 64,  64, 256, 0.45f, 4};
+    }
+}
+__host__ inline TileInfo tile_info_f16(int shape)
+{
+    switch (shape) {
+    case TILE_256x256: return {256, 256, 256, 1.00f, 1};
+    case TILE_128x128: return {128, 128, 128, 0.60f, 2};
+    default:           return { 64,  64,  64, 0.25f, 4};
+    }
+}
+
+int launch_gemm_f32(int shape, bool edge, const GemmArgs& args, hipStream_t stream);
+int launch_gemm_f16(int shape, bool edge, const GemmArgs& args, hipStream_t stream);
+int launch_gemv_f32(const float* A, const float* x, const float* c, float* y, uint32_t M, uint32_t K,
+                    uint32_t lda, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta,
+                    hipStream_t stream);
+
+}  // namespace decx_hip

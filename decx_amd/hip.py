@@ -1,0 +1,205 @@
+"""ctypes view of the C ABI (include/decx_hip.h) plus small numpy conveniences used by the
+tests, the smoke check and the benchmark.  There is no fallback: if the native library is
+missing or no GPU answers, this raises."""
+import ctypes
+import os
+
+import numpy as np
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "lib", "libdecx_hip.so")
+
+TILE_AUTO, TILE_256, TILE_128, TILE_64, PATH_GEMV = -1, 0, 1, 2, 16
+
+_vp = ctypes.c_void_p
+_u32 = ctypes.c_uint32
+_f = ctypes.c_float
+_sz = ctypes.c_size_t
+_int = ctypes.c_int
+
+
+class DeviceProps(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char * 64), ("arch", ctypes.c_char * 32), ("compute_units", ctypes.c_int32),
+                ("clock_khz", ctypes.c_int32), ("memory_clock_khz", ctypes.c_int32),
+                ("memory_bus_bits", ctypes.c_int32), ("lds_bytes_per_block", ctypes.c_int32),
+                ("wavefront_size", ctypes.c_int32), ("global_mem_bytes", ctypes.c_uint64)]
+
+
+class Plan(ctypes.Structure):
+    _fields_ = [("path", ctypes.c_int32), ("edge", ctypes.c_int32), ("tile_m", _u32), ("tile_n", _u32),
+                ("grid", _u32)]
+
+
+# name -> (restype, argtypes): every symbol include/decx_hip.h declares
+SYMBOLS = {
+    "decx_hip_init": (_int, [_int]),
+    "decx_hip_get_device_props": (_int, [ctypes.POINTER(DeviceProps)]),
+    "decx_hip_error_string": (ctypes.c_char_p, [_int]),
+    "decx_hip_malloc": (_int, [ctypes.POINTER(_vp), _sz]),
+    "decx_hip_free": (_int, [_vp]),
+    "decx_hip_host_malloc": (_int, [ctypes.POINTER(_vp), _sz]),
+    "decx_hip_host_free": (_int, [_vp]),
+    "decx_hip_memset_async": (_int, [_vp, _int, _sz, _vp]),
+    "decx_hip_memcpy2d_async": (_int, [_vp, _sz, _vp, _sz, _sz, _sz, _int, _vp]),
+    "decx_hip_stream_create": (_int, [ctypes.POINTER(_vp)]),
+    "decx_hip_stream_destroy": (_int, [_vp]),
+    "decx_hip_stream_sync": (_int, [_vp]),
+    "decx_hip_event_create": (_int, [ctypes.POINTER(_vp)]),
+    "decx_hip_event_destroy": (_int, [_vp]),
+    "decx_hip_event_record": (_int, [_vp, _vp]),
+    "decx_hip_event_sync": (_int, [_vp]),
+    "decx_hip_event_elapsed_ms": (_int, [_vp, _vp, ctypes.POINTER(_f)]),
+    "decx_hip_gemm_f32": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp]),
+    "decx_hip_gemm_f16": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp]),
+    "decx_hip_gemv_f32": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _vp]),
+    "decx_hip_gemm_f32_tile": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, _int, _int]),
+    "decx_hip_gemm_f16_tile": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, _int, _int]),
+    "decx_hip_gemm_plan": (_int, [_int, _u32, _u32, _u32, _int, ctypes.POINTER(Plan)]),
+    "decx_hip_float_to_half": (ctypes.c_uint16, [_f]),
+    "decx_hip_half_to_float": (_f, [ctypes.c_uint16]),
+}
+
+_lib = None
+
+
+class HipError(RuntimeError):
+    pass
+
+
+def lib():
+    """Loads libdecx_hip.so (built in-tree by decx_amd.build) and types its symbols."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise HipError("native library missing: %s (run `python -m decx_amd.build`)" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(L, name)       # AttributeError if the library does not export it
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+def check(rc, what=""):
+    if rc != 0:
+        raise HipError("%s failed: %d (%s)" % (what or "decx_hip call", rc, lib().decx_hip_error_string(rc).decode()))
+
+
+_inited = False
+
+
+def init(device=0):
+    global _inited
+    if not _inited:
+        check(lib().decx_hip_init(device), "decx_hip_init")
+        _inited = True
+
+
+def device_props():
+    init()
+    p = DeviceProps()
+    check(lib().decx_hip_get_device_props(ctypes.byref(p)))
+    return p
+
+
+def plan(elem_bytes, M, N, K, aligned=True):
+    p = Plan()
+    check(lib().decx_hip_gemm_plan(elem_bytes, M, N, K, 1 if aligned else 0, ctypes.byref(p)))
+    return p
+
+
+class DeviceMatrix:
+    """A pitched row-major matrix in HBM.  `pitch` in elements; padding columns are filled
+    with `pad_value` (NaN by default in tests) so that any kernel that touches them shows."""
+
+    def __init__(self, rows, cols, dtype, pitch=None, data=None, pad_value=None, offset_elems=0):
+        init()
+        self.rows, self.cols = rows, cols
+        self.dtype = np.dtype(dtype)
+        self.pitch = pitch if pitch is not None else cols
+        assert self.pitch >= cols
+        self.offset = offset_elems                  # deliberately misaligned bases for tests
+        self.nbytes = (max(rows, 1) * self.pitch + offset_elems) * self.dtype.itemsize
+        raw = _vp()
+        check(lib().decx_hip_malloc(ctypes.byref(raw), self.nbytes), "decx_hip_malloc")
+        self.raw = raw
+        self.ptr = _vp(raw.value + offset_elems * self.dtype.itemsize)
+        if data is not None or pad_value is not None:
+            host = np.empty((rows, self.pitch), self.dtype)
+            if pad_value is not None:
+                host[...] = pad_value
+            if data is not None:
+                host[:, :cols] = data
+            elif pad_value is None:
+                host[:, :cols] = 0
+            self.upload_raw(host)
+
+    def upload_raw(self, host):
+        host = np.ascontiguousarray(host, self.dtype)
+        assert host.shape == (self.rows, self.pitch)
+        if host.size:
+            check(lib().decx_hip_memcpy2d_async(self.ptr, host.nbytes, host.ctypes.data, host.nbytes,
+                                                host.nbytes, 1, 0, None), "upload")
+            check(lib().decx_hip_stream_sync(None))
+
+    def download_raw(self):
+        host = np.empty((self.rows, self.pitch), self.dtype)
+        if host.size:
+            check(lib().decx_hip_memcpy2d_async(host.ctypes.data, host.nbytes, self.ptr, host.nbytes,
+                                                host.nbytes, 1, 1, None), "download")
+            check(lib().decx_hip_stream_sync(None))
+        return host
+
+    def download(self):
+        return self.download_raw()[:, :self.cols].copy()
+
+    def free(self):
+        if self.raw is not None:
+            lib().decx_hip_free(self.raw)
+            self.raw = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def gemm(A, B, D, C=None, alpha=1.0, beta=1.0, stream=None, tile=TILE_AUTO, force_edge=False):
+    """D = A.B or fma(C, beta, alpha*A.B) on DeviceMatrix operands through the C ABI."""
+    assert A.dtype == B.dtype == D.dtype
+    M, K, N = A.rows, A.cols, B.cols
+    assert B.rows == K and D.rows == M and D.cols == N
+    L = lib()
+    f16 = A.dtype == np.float16
+    args = [A.ptr, B.ptr, C.ptr if C is not None else None, D.ptr, M, N, K, A.pitch, B.pitch,
+            C.pitch if C is not None else 0, D.pitch, alpha, beta, stream]
+    if tile == TILE_AUTO and not force_edge:
+        rc = (L.decx_hip_gemm_f16 if f16 else L.decx_hip_gemm_f32)(*args)
+    else:
+        rc = (L.decx_hip_gemm_f16_tile if f16 else L.decx_hip_gemm_f32_tile)(*args, tile, 1 if force_edge else 0)
+    check(rc, "gemm")
+
+
+def sync(stream=None):
+    check(lib().decx_hip_stream_sync(stream), "stream sync")
+
+
+class Timer:
+    """HIP events on the stream the kernels are launched on."""
+
+    def __init__(self):
+        init()
+        self.a, self.b = _vp(), _vp()
+        check(lib().decx_hip_event_create(ctypes.byref(self.a)))
+        check(lib().decx_hip_event_create(ctypes.byref(self.b)))
+
+    def start(self, stream=None):
+        check(lib().decx_hip_event_record(self.a, stream))
+
+    def stop(self, stream=None):
+        check(lib().decx_hip_event_record(self.b, stream))
+        check(lib().decx_hip_event_sync(self.b))
+        ms = _f()
+        check(lib().decx_hip_event_elapsed_ms(self.a, self.b, ctypes.byref(ms)))
+        return ms.value

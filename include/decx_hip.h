@@ -1,0 +1,152 @@
+/*
+ * decx_hip.h -- the C ABI of the MI355X (gfx950) dense-GEMM module.
+ *
+ * This is the whole surface through which host code reaches the GPU: plain pointers,
+ * sizes and scalars, no C++ types.  The C++ objects and entry points of the DECX API
+ * (include/DECX.h: de::GPU_Matrix, de::Memcpy, de::blas::cuda::GEMM) are implemented on
+ * top of these functions and nothing else.
+ *
+ * Conventions
+ *   - every function returns 0 on success; a positive value is a hipError_t, a negative
+ *     value one of the DECX_HIP_E_* codes below; decx_hip_error_string() names either;
+ *   - matrices are row-major; a pitch (lda, ldb, ...) is the distance between rows in
+ *     ELEMENTS and must be >= the row width; padding beyond the width is never read and
+ *     never written;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); launches are
+ *     asynchronous with respect to the host;
+ *   - fp16 payloads are IEEE binary16 bit patterns in uint16_t.
+ */
+#ifndef DECX_HIP_H_
+#define DECX_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DECX_HIP_API __attribute__((visibility("default")))
+
+enum {
+    DECX_HIP_OK            = 0,
+    DECX_HIP_E_INVALID_ARG = -1,   /* null pointer, pitch smaller than width, unknown enum */
+    DECX_HIP_E_NOT_INIT    = -2,   /* decx_hip_init() has not succeeded yet */
+    DECX_HIP_E_NO_DEVICE   = -3    /* no usable GPU */
+};
+
+typedef struct decx_hip_device_props {
+    char     name[64];
+    char     arch[32];             /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+    int32_t  compute_units;
+    int32_t  clock_khz;            /* peak engine clock */
+    int32_t  memory_clock_khz;
+    int32_t  memory_bus_bits;
+    int32_t  lds_bytes_per_block;
+    int32_t  wavefront_size;
+    uint64_t global_mem_bytes;
+} decx_hip_device_props;
+
+/* Tile shapes the planner chooses between (block tile BM x BN). */
+enum {
+    DECX_HIP_TILE_AUTO    = -1,
+    DECX_HIP_TILE_256x256 = 0,
+    DECX_HIP_TILE_128x128 = 1,
+    DECX_HIP_TILE_64x64   = 2,
+    DECX_HIP_PATH_GEMV    = 16     /* N == 1: bandwidth-bound row-dot kernel */
+};
+
+typedef struct decx_hip_plan {
+    int32_t  path;                 /* one of the enum above */
+    int32_t  edge;                 /* 1: the predicated (ragged-shape) kernel variant runs */
+    uint32_t tile_m, tile_n;       /* block tile */
+    uint32_t grid;                 /* workgroups launched */
+} decx_hip_plan;
+
+/* ---- device, memory, streams, events --------------------------------------------------
+ * Replaces de::InitCuda (srcs/modules/core/configs/config.cu:35-40), the device pool
+ * (srcs/modules/core/allocators, memory_management) and the stream / event pools
+ * (srcs/modules/core/cudaStream_management) as far as the GEMM path uses them. */
+DECX_HIP_API int decx_hip_init(int device);
+DECX_HIP_API int decx_hip_get_device_props(decx_hip_device_props* out);
+DECX_HIP_API const char* decx_hip_error_string(int code);
+
+DECX_HIP_API int decx_hip_malloc(void** ptr, size_t bytes);
+DECX_HIP_API int decx_hip_free(void* ptr);
+DECX_HIP_API int decx_hip_host_malloc(void** ptr, size_t bytes);     /* pinned host memory */
+DECX_HIP_API int decx_hip_host_free(void* ptr);
+DECX_HIP_API int decx_hip_memset_async(void* ptr, int value, size_t bytes, void* stream);
+
+/* kind: 0 host->device, 1 device->host, 2 device->device.  Pitches and width in BYTES.
+ * Replaces the cudaMemcpy2DAsync calls of de::Memcpy
+ * (srcs/modules/core/data transmission/data_transmission.cu:139-170). */
+DECX_HIP_API int decx_hip_memcpy2d_async(void* dst, size_t dst_pitch, const void* src, size_t src_pitch,
+                                         size_t width_bytes, size_t height, int kind, void* stream);
+
+DECX_HIP_API int decx_hip_stream_create(void** stream);
+DECX_HIP_API int decx_hip_stream_destroy(void* stream);
+DECX_HIP_API int decx_hip_stream_sync(void* stream);
+
+DECX_HIP_API int decx_hip_event_create(void** event);
+DECX_HIP_API int decx_hip_event_destroy(void* event);
+DECX_HIP_API int decx_hip_event_record(void* event, void* stream);
+DECX_HIP_API int decx_hip_event_sync(void* event);
+DECX_HIP_API int decx_hip_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* ---- the contraction -------------------------------------------------------------------
+ * D (M x N) = A (M x K) . B (K x N)                      when C == NULL
+ * D         = fma(C, beta, alpha * (A . B))              otherwise (C is M x N, may alias D)
+ *
+ * fp32: products and sums in fp32 on the matrix cores.  Replaces the kernels launched by
+ * cuda_GEMM_LS_planner<float>::run (srcs/modules/BLAS/GEMM/CUDA/large_squares/fp32/
+ * GEMM_fp32_callers.cu:56-122) behind de::blas::cuda::GEMM (GEMM_LS.cu:62-109,315-393).
+ * N == 1 is routed to the row-dot kernel that replaces cu_mat_m_vec_fp32
+ * (extreme_shapes/VMM_fp32.cu:104-146). */
+DECX_HIP_API int decx_hip_gemm_f32(const float* A, const float* B, const float* C, float* D,
+                                   uint32_t M, uint32_t N, uint32_t K,
+                                   uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                                   float alpha, float beta, void* stream);
+
+/* fp16 in, fp32 accumulate, one rounding to fp16 out.  Replaces the kernels launched by
+ * cuda_GEMM_LS_planner<de::Half>::run (large_squares/fp16/GEMM_fp16_callers.cu:57-124). */
+DECX_HIP_API int decx_hip_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
+                                   uint32_t M, uint32_t N, uint32_t K,
+                                   uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                                   float alpha, float beta, void* stream);
+
+/* y (M) = A (M x K) . x (K), optionally y = fma(c, beta, alpha * A.x).  incx / incc / incy
+ * are element strides (a K x 1 pitched matrix has incx = its pitch).  This is what
+ * decx_hip_gemm_f32 runs for N == 1; exported for callers that hold vectors. */
+DECX_HIP_API int decx_hip_gemv_f32(const float* A, const float* x, const float* c, float* y,
+                                   uint32_t M, uint32_t K, uint32_t lda,
+                                   uint32_t incx, uint32_t incc, uint32_t incy,
+                                   float alpha, float beta, void* stream);
+
+/* Same as decx_hip_gemm_f32 / _f16 with the planner's choice overridden (`tile` = one of
+ * DECX_HIP_TILE_*; AUTO = planner) and, with force_edge != 0, the predicated kernel
+ * variant forced even for shapes that are tile multiples.  For tests and tuning. */
+DECX_HIP_API int decx_hip_gemm_f32_tile(const float* A, const float* B, const float* C, float* D,
+                                        uint32_t M, uint32_t N, uint32_t K,
+                                        uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                                        float alpha, float beta, void* stream, int tile, int force_edge);
+DECX_HIP_API int decx_hip_gemm_f16_tile(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
+                                        uint32_t M, uint32_t N, uint32_t K,
+                                        uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                                        float alpha, float beta, void* stream, int tile, int force_edge);
+
+/* What the planner would run for this problem (no GPU work).  elem_bytes: 4 = fp32, 2 = fp16.
+ * `aligned` != 0 promises 16-byte aligned bases and pitches.  Replaces the scoring of
+ * cuda_GEMM_LS_planner<T>::plan (large_squares/common/cuda_GEMM_LS_planner.cu:108-224).
+ * Works without a GPU: before decx_hip_init() it assumes 256 compute units. */
+DECX_HIP_API int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int aligned,
+                                    decx_hip_plan* out);
+
+/* IEEE binary16 <-> binary32, round to nearest even; host-side helpers behind
+ * de::Float2Half / de::Half2Float (srcs/common/FP16/float_half_convert.cu:35-46). */
+DECX_HIP_API uint16_t decx_hip_float_to_half(float value);
+DECX_HIP_API float decx_hip_half_to_float(uint16_t bits);
+
+#ifdef __cplusplus
+}
+#endif
+#endif  /* DECX_HIP_H_ */

@@ -1,0 +1,97 @@
+"""CPU-only checks of the C ABI: the library loads, exports every symbol the header declares,
+and the parts that need no GPU (planner, half conversion, argument checks) behave."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from decx_amd import hip
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    names = set()
+    for fn in os.listdir(os.path.join(ROOT, "include")):
+        if fn.endswith(".h"):
+            text = open(os.path.join(ROOT, "include", fn)).read()
+            names.update(re.findall(r"DECX_HIP_API\s+[\w\s\*]+?\b(decx_hip_\w+)\s*\(", text))
+    return sorted(names)
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_symbols()
+    assert len(names) >= 25
+    raw = ctypes.CDLL(hip.LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), "libdecx_hip.so does not export " + n
+    assert set(names) == set(hip.SYMBOLS), "ctypes table and header disagree"
+    hip.lib()
+
+
+def test_half_conversion_matches_ieee_rne():
+    L = hip.lib()
+    h = np.arange(65536, dtype=np.uint16)
+    want = h.view(np.float16).astype(np.float32)
+    got = np.array([L.decx_hip_half_to_float(int(v)) for v in h], np.float32)
+    ok = ~np.isnan(want)
+    assert np.array_equal(np.isnan(got), ~ok)
+    assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32))
+    rng = np.random.default_rng(3)
+    vals = np.concatenate([rng.standard_normal(20000).astype(np.float32) * 5,
+                           (rng.standard_normal(4000) * 1e-6).astype(np.float32),
+                           (rng.standard_normal(2000) * 4e4).astype(np.float32),
+                           np.array([0.0, -0.0, 65504, 65519.99, 65520, 65536, 1e30, -1e30, 2.0 ** -24, 2.0 ** -25,
+                                     np.nextafter(np.float32(2.0 ** -25), np.float32(1)), 2.0 ** -14,
+                                     np.inf, -np.inf], np.float32)])
+    hh = np.arange(0x0001, 0x7bff, 37, dtype=np.uint16).view(np.float16).astype(np.float32)
+    vals = np.concatenate([vals, (hh[:-1] + hh[1:]) / np.float32(2)])           # ties and near-ties
+    with np.errstate(over="ignore"):
+        want = vals.astype(np.float16).view(np.uint16)
+    got = np.array([L.decx_hip_float_to_half(float(v)) for v in vals], np.uint16)
+    assert np.array_equal(got, want)
+
+
+def test_planner_choices():
+    # headline shapes take the big tile, the unpredicated variant
+    for eb, (M, N, K) in [(4, (8192, 8192, 8192)), (2, (4096, 4096, 4096)), (4, (65536, 256, 1024))]:
+        p = hip.plan(eb, M, N, K)
+        assert (p.path, p.edge, p.tile_m, p.tile_n) == (hip.TILE_256, 0, 256, 256)
+        assert p.grid == (M // 256) * (N // 256)
+    # small and ragged problems take smaller tiles so the chip fills, with the predicated variant
+    p = hip.plan(4, 1000, 1500, 777)
+    assert p.edge == 1 and p.tile_m < 256 and p.grid == -(-1000 // p.tile_m) * -(-1500 // p.tile_n)
+    assert hip.plan(4, 1024, 1024, 1024).tile_m < 256
+    assert hip.plan(4, 1024, 1024, 1024, aligned=False).edge == 1
+    # N == 1 goes to the row-dot kernel (fp32 only)
+    assert hip.plan(4, 8192, 1, 8192).path == hip.PATH_GEMV
+    assert hip.plan(2, 8192, 1, 8192).path != hip.PATH_GEMV
+    assert hip.plan(4, 0, 5, 5).grid == 0
+    bad = hip.Plan()
+    assert hip.lib().decx_hip_gemm_plan(3, 4, 4, 4, 1, ctypes.byref(bad)) == -1
+
+
+def test_compute_entry_points_refuse_to_run_uninitialised():
+    """Fresh process, no decx_hip_init: every GPU entry point reports NOT_INIT (-2) instead of
+    touching the device or falling back to anything."""
+    import subprocess
+    import sys
+    code = (
+        "import sys, ctypes; sys.path.insert(0, %r); from decx_amd import hip; L = hip.lib();"
+        "p = ctypes.c_void_p(16); q = ctypes.c_void_p();"
+        "assert L.decx_hip_gemm_f32(p, p, None, p, 4, 4, 4, 4, 4, 0, 4, 1.0, 1.0, None) == -2;"
+        "assert L.decx_hip_gemm_f16(p, p, None, p, 4, 4, 4, 4, 4, 0, 4, 1.0, 1.0, None) == -2;"
+        "assert L.decx_hip_gemv_f32(p, p, None, p, 4, 4, 4, 1, 1, 1, 1.0, 1.0, None) == -2;"
+        "assert L.decx_hip_malloc(ctypes.byref(q), 64) == -2;"
+        "assert L.decx_hip_stream_create(ctypes.byref(q)) == -2;"
+        "assert b'init' in L.decx_hip_error_string(-2)" % ROOT)
+    subprocess.run([sys.executable, "-c", code], check=True, timeout=120)
+
+
+def test_error_strings():
+    L = hip.lib()
+    assert L.decx_hip_error_string(0) == b"success"
+    assert b"invalid argument" in L.decx_hip_error_string(-1)
+    assert L.decx_hip_error_string(-99) == b"unknown error"

@@ -1,0 +1,304 @@
+"""Parity of the HIP GEMM path (through the C ABI) against the CPU oracle.
+
+Bar: max|d| / (max|ref| * sqrt(K)) <= 1e-5 for fp32 and <= 2e-3 for fp16; bit-exact where
+the mathematics makes the answer exactly representable (identity, small-integer products).
+"""
+import glob
+import os
+
+import numpy as np
+import pytest
+
+from decx_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+TOL_F32 = 1e-5
+TOL_F16 = 2e-3
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from decx_amd import hip as h
+    h.init()                    # raises if the library or the GPU is missing: no fallback
+    return h
+
+
+def rel_err(got, ref, K):
+    ref = ref.astype(np.float64)
+    scale = max(float(np.max(np.abs(ref))), 1e-30) * np.sqrt(max(K, 1))
+    return float(np.max(np.abs(got.astype(np.float64) - ref))) / scale
+
+
+def device_pitch(cols, dtype):
+    """The reference's device pitch rule: rows padded to 128 bytes
+    (srcs/modules/core/classes/GPU_Matrix.cu:35-61)."""
+    per = 128 // np.dtype(dtype).itemsize
+    return (cols + per - 1) // per * per
+
+
+def run(hip, A, B, C=None, alpha=1.0, beta=1.0, tile=-1, force_edge=False, pitches=None, offsets=(0, 0, 0, 0)):
+    """Uploads with NaN-poisoned padding, runs, checks the padding of D is untouched."""
+    dt = A.dtype
+    M, K = A.shape
+    N = B.shape[1]
+    pa, pb, pc, pd = pitches or (device_pitch(K, dt), device_pitch(N, dt), device_pitch(N, dt), device_pitch(N, dt))
+    dA = hip.DeviceMatrix(M, K, dt, pa, A, pad_value=np.nan, offset_elems=offsets[0])
+    dB = hip.DeviceMatrix(K, N, dt, pb, B, pad_value=np.nan, offset_elems=offsets[1])
+    dC = hip.DeviceMatrix(M, N, dt, pc, C, pad_value=np.nan, offset_elems=offsets[2]) if C is not None else None
+    sentinel = np.full((M, pd), -12345.0, dt)
+    dD = hip.DeviceMatrix(M, N, dt, pd, offset_elems=offsets[3])
+    dD.upload_raw(sentinel)
+    hip.gemm(dA, dB, dD, dC, alpha, beta, tile=tile, force_edge=force_edge)
+    hip.sync()
+    raw = dD.download_raw()
+    assert np.all(raw[:, N:] == dt.type(-12345.0)), "padding columns of D were written"
+    out = raw[:, :N].copy()
+    assert not np.isnan(out).any(), "NaN leaked from pitch padding into the result"
+    for d in (dA, dB, dC, dD):
+        if d is not None:
+            d.free()
+    return out
+
+
+# ------------------------------------------------------------------ golden fixtures
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLD, "*_f32_*.npz"))))
+def test_golden_f32(hip, path):
+    g = np.load(path)
+    M, N, K = int(g["M"]), int(g["N"]), int(g["K"])
+    A = synth.uniform_f32(M, K, int(g["seed_a"])); B = synth.uniform_f32(K, N, int(g["seed_b"]))
+    C = None; alpha = beta = 1.0
+    if "with_c" in g.files and bool(g["with_c"]):
+        C = synth.uniform_f32(M, N, int(g["seed_c"]))
+        if not np.isnan(g["alpha"]):
+            alpha, beta = float(g["alpha"]), float(g["beta"])
+    for tile in (-1, 0, 1, 2):
+        got = run(hip, A, B, C, alpha, beta, tile=tile)
+        assert rel_err(got, g["D"], K) <= TOL_F32, (path, tile)
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLD, "orc_f16_*.npz"))))
+def test_golden_f16(hip, path):
+    g = np.load(path)
+    K = int(g["K"])
+    A = g["A"].view(np.float16); B = g["B"].view(np.float16)
+    C = g["C"].view(np.float16) if bool(g["with_c"]) else None
+    for tile in (-1, 0, 1, 2):
+        got = run(hip, A, B, C, float(g["alpha"]), float(g["beta"]), tile=tile)
+        assert rel_err(got, g["D"].view(np.float16), K) <= TOL_F16, (path, tile)
+
+
+# ------------------------------------------------------------------ BASELINE configs, full or sampled
+
+def sample_rows(M, count, seed):
+    rng = np.random.default_rng(seed)
+    rows = set(rng.choice(M, size=min(count, M), replace=False).tolist())
+    rows.update([0, M - 1])                       # first and last row always
+    return np.array(sorted(rows), np.uint32)
+
+
+def test_config1_f32_1024_cubed(hip, oracle):
+    M = N = K = 1024
+    sa, sb, _ = synth.seeds(1)
+    A = synth.uniform_f32(M, K, sa); B = synth.uniform_f32(K, N, sb)
+    ref = oracle.gemm_f32(A, B)
+    for tile in (-1, 0, 1, 2):
+        assert rel_err(run(hip, A, B, tile=tile), ref, K) <= TOL_F32, tile
+
+
+def test_config2_f32_ragged_with_and_without_c(hip, oracle):
+    M, N, K = 1000, 1500, 777
+    sa, sb, sc = synth.seeds(2)
+    A = synth.uniform_f32(M, K, sa); B = synth.uniform_f32(K, N, sb); C = synth.uniform_f32(M, N, sc)
+    ref_ab = oracle.gemm_f32(A, B)
+    ref_abc = oracle.gemm_f32(A, B, C)                 # the CPU entry point's D = A.B + C
+    ref_axpby = oracle.gemm_f32(A, B, C, 1.0, 1.0)     # the GPU entry point with alpha = beta = 1
+    for tile in (-1, 0, 1, 2):
+        assert rel_err(run(hip, A, B, tile=tile), ref_ab, K) <= TOL_F32
+        got = run(hip, A, B, C, 1.0, 1.0, tile=tile)
+        assert rel_err(got, ref_abc, K) <= TOL_F32
+        assert rel_err(got, ref_axpby, K) <= TOL_F32
+    got = run(hip, A, B, C, -0.75, 2.5)
+    assert rel_err(got, oracle.gemm_f32(A, B, C, -0.75, 2.5), K) <= TOL_F32
+
+
+def test_config3_f16_4096_cubed_sampled(hip, oracle):
+    M = N = K = 4096
+    sa, sb, _ = synth.seeds(3)
+    A = synth.normal_half(M, K, sa); B = synth.normal_half(K, N, sb)
+    rows = sample_rows(M, 96, 3)
+    ref = oracle.gemm_f16(A, B, rows=rows)
+    got = run(hip, A, B)
+    assert rel_err(got[rows], ref, K) <= TOL_F16
+    # size-independent property: scaling A by 2 (exact in binary16) scales D by exactly 2
+    got2 = run(hip, (A * np.float16(2)).astype(np.float16), B)
+    assert np.array_equal(got2[rows], (got[rows] * np.float16(2)).astype(np.float16))
+
+
+def test_config4_f32_8192_cubed_sampled(hip, oracle):
+    M = N = K = 8192
+    sa, sb, _ = synth.seeds(4)
+    A = synth.uniform_f32(M, K, sa); B = synth.uniform_f32(K, N, sb)
+    rows = sample_rows(M, 64, 4)
+    ref = oracle.gemm_f32(A, B, rows=rows)
+    got = run(hip, A, B)
+    assert rel_err(got[rows], ref, K) <= TOL_F32
+    # column checksum: (1^T A) B == 1^T (A B), in float64 on the host
+    colsum = A.astype(np.float64).sum(axis=0) @ B.astype(np.float64)
+    assert np.max(np.abs(got.astype(np.float64).sum(axis=0) - colsum)) / np.max(np.abs(colsum)) < 1e-5
+
+
+def test_config5a_f32_tall_skinny_sampled(hip, oracle):
+    M, N, K = 65536, 256, 1024
+    sa, sb, _ = synth.seeds(5)
+    A = synth.uniform_f32(M, K, sa); B = synth.uniform_f32(K, N, sb)
+    rows = sample_rows(M, 512, 5)
+    ref = oracle.gemm_f32(A, B, rows=rows)
+    got = run(hip, A, B)
+    assert rel_err(got[rows], ref, K) <= TOL_F32
+
+
+def test_config5b_f32_gemv(hip, oracle):
+    M, N, K = 8192, 1, 8192
+    sa, sb, sc = synth.seeds(6)
+    A = synth.uniform_f32(M, K, sa); B = synth.uniform_f32(K, N, sb); C = synth.uniform_f32(M, N, sc)
+    assert hip.plan(4, M, N, K).path == hip.PATH_GEMV
+    assert rel_err(run(hip, A, B), oracle.gemm_f32(A, B), K) <= TOL_F32
+    assert rel_err(run(hip, A, B, C, 0.5, -2.0), oracle.gemm_f32(A, B, C, 0.5, -2.0), K) <= TOL_F32
+    # and the same column through the tiled kernel
+    assert rel_err(run(hip, A, B, tile=2), oracle.gemm_f32(A, B), K) <= TOL_F32
+
+
+# ------------------------------------------------------------------ edge cases
+
+SHAPES = [(1, 1, 1), (1, 7, 3), (7, 1, 3), (3, 5, 1), (31, 33, 17), (64, 64, 16), (65, 63, 15), (129, 257, 100),
+          (255, 256, 257), (300, 20, 40), (20, 300, 1025), (2, 2, 4097)]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+@pytest.mark.parametrize("tile", [0, 1, 2])
+def test_f32_ragged_shapes_every_tile(hip, oracle, M, N, K, tile):
+    A = synth.uniform_f32(M, K, 101); B = synth.uniform_f32(K, N, 102); C = synth.uniform_f32(M, N, 103)
+    assert rel_err(run(hip, A, B, tile=tile), oracle.gemm_f32(A, B), K) <= TOL_F32
+    assert rel_err(run(hip, A, B, C, 1.5, -0.5, tile=tile), oracle.gemm_f32(A, B, C, 1.5, -0.5), K) <= TOL_F32
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+@pytest.mark.parametrize("tile", [0, 1, 2])
+def test_f16_ragged_shapes_every_tile(hip, oracle, M, N, K, tile):
+    A = synth.normal_half(M, K, 111); B = synth.normal_half(K, N, 112); C = synth.normal_half(M, N, 113)
+    assert rel_err(run(hip, A, B, tile=tile), oracle.gemm_f16(A, B), K) <= TOL_F16
+    assert rel_err(run(hip, A, B, C, 1.5, -0.5, tile=tile), oracle.gemm_f16(A, B, C, 1.5, -0.5), K) <= TOL_F16
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_unaligned_pitches_and_bases(hip, oracle, dtype):
+    """Pitches that are not multiples of 16 bytes and bases off by one element: the kernels
+    must fall back to element loads, never to misaligned vector loads."""
+    M, N, K = 70, 90, 50
+    if dtype == np.float32:
+        A = synth.uniform_f32(M, K, 121); B = synth.uniform_f32(K, N, 122); C = synth.uniform_f32(M, N, 123)
+        ref = oracle.gemm_f32(A, B, C, 2.0, 1.0); tol = TOL_F32
+    else:
+        A = synth.normal_half(M, K, 121); B = synth.normal_half(K, N, 122); C = synth.normal_half(M, N, 123)
+        ref = oracle.gemm_f16(A, B, C, 2.0, 1.0); tol = TOL_F16
+    for tile in (0, 1, 2):
+        got = run(hip, A, B, C, 2.0, 1.0, tile=tile, pitches=(K + 1, N + 3, N + 5, N + 1), offsets=(1, 3, 1, 1))
+        assert rel_err(got, ref, K) <= tol
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2])
+def test_forced_edge_variant_equals_fast_variant(hip, tile):
+    """On tile-multiple shapes the predicated kernel and the unpredicated one run the same
+    arithmetic in the same order: bit-identical."""
+    M, N, K = 512, 512, 256
+    A = synth.uniform_f32(M, K, 131); B = synth.uniform_f32(K, N, 132)
+    assert np.array_equal(run(hip, A, B, tile=tile), run(hip, A, B, tile=tile, force_edge=True))
+    Ah = synth.normal_half(M, K, 133); Bh = synth.normal_half(K, N, 134)
+    assert np.array_equal(run(hip, Ah, Bh, tile=tile).view(np.uint16),
+                          run(hip, Ah, Bh, tile=tile, force_edge=True).view(np.uint16))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_exact_closed_forms(hip, dtype):
+    n = 200
+    rng = np.random.default_rng(5)
+    X = rng.integers(-8, 9, (n, 150)).astype(dtype)
+    eye = np.eye(n, dtype=dtype)
+    assert np.array_equal(run(hip, eye, X), X)                       # I . X == X, bit for bit
+    Y = rng.integers(-8, 9, (150, n)).astype(dtype)
+    assert np.array_equal(run(hip, Y, eye), Y)
+    K = 1000                                                         # ones . ones == K (K < 2^11 for half)
+    assert np.all(run(hip, np.ones((9, K), dtype), np.ones((K, 11), dtype)) == dtype(K))
+    a = rng.integers(-3, 4, (130, 96)).astype(dtype); b = rng.integers(-3, 4, (96, 140)).astype(dtype)
+    assert np.array_equal(run(hip, a, b), (a.astype(np.int64) @ b.astype(np.int64)).astype(dtype))
+
+
+def test_reference_sample_known_answer(hip):
+    """samples/Matrix_Multiplication/MatMul.cpp:16-40 with W=1013, H=1077, L=1005."""
+    W, H, L = 1013, 1077, 1005
+    A = np.tile(np.arange(L, dtype=np.float32), (H, 1))
+    B = np.tile(np.arange(L, dtype=np.float32)[:, None], (1, W))
+    got = run(hip, A, B)
+    assert np.max(np.abs(got.astype(np.float64) - 337853530.0)) / 337853530.0 < 4e-6
+
+
+def test_linearity_at_full_size(hip):
+    """(A1 + A2) . B == A1 . B + A2 . B up to rounding, at the fp32 headline size's tile shape."""
+    M = N = 2048; K = 1024
+    A1 = synth.uniform_f32(M, K, 141); A2 = synth.uniform_f32(M, K, 142); B = synth.uniform_f32(K, N, 143)
+    lhs = run(hip, A1 + A2, B)
+    rhs = run(hip, A1, B).astype(np.float64) + run(hip, A2, B).astype(np.float64)
+    assert np.max(np.abs(lhs - rhs)) / (np.max(np.abs(rhs)) * np.sqrt(K)) <= TOL_F32
+
+
+def test_c_may_alias_d(hip, oracle):
+    M, N, K = 100, 150, 77
+    A = synth.uniform_f32(M, K, 151); B = synth.uniform_f32(K, N, 152); C = synth.uniform_f32(M, N, 153)
+    dA = hip.DeviceMatrix(M, K, np.float32, data=A); dB = hip.DeviceMatrix(K, N, np.float32, data=B)
+    dD = hip.DeviceMatrix(M, N, np.float32, data=C)
+    hip.gemm(dA, dB, dD, dD, 1.0, 1.0)
+    hip.sync()
+    assert rel_err(dD.download(), oracle.gemm_f32(A, B, C, 1.0, 1.0), K) <= TOL_F32
+
+
+def test_empty_and_invalid_arguments(hip):
+    L = hip.lib()
+    d = hip.DeviceMatrix(4, 4, np.float32, data=np.ones((4, 4), np.float32))
+    p = d.ptr
+    assert L.decx_hip_gemm_f32(p, p, None, p, 0, 4, 4, 4, 4, 0, 4, 1.0, 1.0, None) == 0      # empty: nothing to do
+    assert L.decx_hip_gemm_f32(p, p, None, p, 4, 0, 4, 4, 4, 0, 4, 1.0, 1.0, None) == 0
+    assert L.decx_hip_gemm_f32(None, p, None, p, 4, 4, 4, 4, 4, 0, 4, 1.0, 1.0, None) == -1   # null operand
+    assert L.decx_hip_gemm_f32(p, p, None, p, 4, 4, 4, 3, 4, 0, 4, 1.0, 1.0, None) == -1      # lda < K
+    assert L.decx_hip_gemm_f32(p, p, p, p, 4, 4, 4, 4, 4, 3, 4, 1.0, 1.0, None) == -1         # ldc < N
+    assert L.decx_hip_gemm_f32_tile(p, p, None, p, 4, 4, 4, 4, 4, 0, 4, 1.0, 1.0, None, 9, 0) == -1
+    hip.sync()
+    assert np.all(d.download() == 1.0)
+    # K == 0: the product is empty, D = 0 (or beta * C)
+    out = hip.DeviceMatrix(4, 4, np.float32, data=np.full((4, 4), 7, np.float32))
+    assert L.decx_hip_gemm_f32(p, p, None, out.ptr, 4, 4, 0, 4, 4, 0, 4, 1.0, 1.0, None) == 0
+    hip.sync()
+    assert np.all(out.download() == 0.0)
+    assert L.decx_hip_gemm_f32(p, p, d.ptr, out.ptr, 4, 4, 0, 4, 4, 4, 4, 1.0, 3.0, None) == 0
+    hip.sync()
+    assert np.all(out.download() == 3.0)
+
+
+def test_stream_and_events(hip):
+    import ctypes
+    L = hip.lib()
+    s = ctypes.c_void_p()
+    assert L.decx_hip_stream_create(ctypes.byref(s)) == 0
+    A = synth.uniform_f32(256, 256, 161)
+    dA = hip.DeviceMatrix(256, 256, np.float32, data=A)
+    dI = hip.DeviceMatrix(256, 256, np.float32, data=np.eye(256, dtype=np.float32))
+    dD = hip.DeviceMatrix(256, 256, np.float32)
+    t = hip.Timer()
+    t.start(s)
+    hip.gemm(dA, dI, dD, stream=s)
+    ms = t.stop(s)
+    hip.sync(s)
+    assert ms > 0 and np.array_equal(dD.download(), A)
+    assert L.decx_hip_stream_destroy(s) == 0
