@@ -1,0 +1,188 @@
+#!/usr/bin/env python3
+"""Benchmark of the GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-extra]
+
+One step = one GEMM launch on operands already resident in HBM.  The headline line is the
+fp32 M=N=K=8192 product (dense fp32 MFMA roof); the same JSON line carries the fp16 4096^3
+product (dense fp16 MFMA roof) and the bandwidth-bound shapes under "other_workloads".
+The kernel time is measured with HIP events recorded on the launch stream.  The CPU
+baseline is the in-repo AVX2 restatement of the reference's multithreaded CPU GEMM, timed
+once on the host cores on the same workload and checked bit-for-bit against the scalar
+fma chain on sampled rows.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_F32_TFLOPS = 157.3      # MI355X dense fp32 matrix
+PEAK_F16_TFLOPS = 2500.0     # MI355X dense fp16 matrix
+PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
+
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by a
+# copy kernel of known size; None until measured for that workload.
+MEASURED_TRAFFIC = {}
+
+WORKLOADS = {
+    # name: (dtype, M, N, K, bound, config number for seeds, description)
+    "fp32_8192": ("f32", 8192, 8192, 8192, "mfma", 4, "fp32 GEMM C=A.B M=N=K=8192, uniform[-1,1]"),
+    "fp16_4096": ("f16", 4096, 4096, 4096, "mfma", 3, "fp16 GEMM (fp32 accumulate, fp16 out) M=N=K=4096, normal(0,0.5) clipped to [-4,4]"),
+    "fp32_1024": ("f32", 1024, 1024, 1024, "mfma", 1, "fp32 GEMM M=N=K=1024, uniform[-1,1]"),
+    "fp32_ragged": ("f32", 1000, 1500, 777, "mfma", 2, "fp32 GEMM M=1000 N=1500 K=777, uniform[-1,1]"),
+    "fp32_tall_skinny": ("f32", 65536, 256, 1024, "mfma", 5, "fp32 GEMM M=65536 N=256 K=1024, uniform[-1,1]"),
+    "fp32_gemv": ("f32", 8192, 1, 8192, "hbm", 6, "fp32 GEMM M=8192 N=1 K=8192 (GEMV-like), uniform[-1,1]"),
+}
+
+
+def make_inputs(name):
+    from decx_amd import synth
+    dt, M, N, K, _, cfg, _ = WORKLOADS[name]
+    sa, sb, _ = synth.seeds(cfg)
+    if dt == "f32":
+        return synth.uniform_f32(M, K, sa), synth.uniform_f32(K, N, sb)
+    return synth.normal_half(M, K, sa), synth.normal_half(K, N, sb)
+
+
+def device_pitch(cols, itemsize):
+    per = 128 // itemsize
+    return (cols + per - 1) // per * per
+
+
+def run_workload(name, steps, warmup, keep_inputs=False):
+    from decx_amd import hip
+    dt, M, N, K, bound, _, desc = WORKLOADS[name]
+    npdt = np.float32 if dt == "f32" else np.float16
+    A, B = make_inputs(name)
+    isz = np.dtype(npdt).itemsize
+    dA = hip.DeviceMatrix(M, K, npdt, device_pitch(K, isz), A)
+    dB = hip.DeviceMatrix(K, N, npdt, device_pitch(N, isz), B)
+    dD = hip.DeviceMatrix(M, N, npdt, device_pitch(N, isz))
+    for _ in range(warmup):
+        hip.gemm(dA, dB, dD)
+    hip.sync()
+    timer = hip.Timer()
+    t0 = time.perf_counter()
+    timer.start()
+    for _ in range(steps):
+        hip.gemm(dA, dB, dD)
+    kernel_ms = timer.stop() / steps            # HIP events on the launch stream
+    hip.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    flops = 2.0 * M * N * K
+    abytes = float(isz) * (M * K + K * N + M * N)
+    tflops = flops / (kernel_ms * 1e-3) / 1e12
+    gbs = abytes / (kernel_ms * 1e-3) / 1e9
+    if bound == "mfma":
+        peak = PEAK_F32_TFLOPS if dt == "f32" else PEAK_F16_TFLOPS
+        roof = {"bound": "mfma", "achieved": round(tflops, 3), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(tflops / peak, 4), "traffic": MEASURED_TRAFFIC.get(name)}
+    else:
+        roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC.get(name)}
+    p = hip.plan(isz, M, N, K)
+    out = {"workload": desc, "dtype": dt, "value": round(tflops, 3), "unit": "TFLOP/s",
+           "hbm_gbs_algorithmic": round(gbs, 1), "kernel_ms": round(kernel_ms, 5), "wall_ms_per_step": round(wall_ms, 5),
+           "plan": {"path": int(p.path), "tile": [int(p.tile_m), int(p.tile_n)], "grid": int(p.grid), "edge": int(p.edge)},
+           "roofline": roof}
+    result = (out, (A, B) if keep_inputs else None)
+    for d in (dA, dB, dD):
+        d.free()
+    return result
+
+
+def cpu_baseline(name, A, B):
+    """Times the AVX2 restatement of the reference CPU GEMM once on this host and checks it
+    bit-for-bit against the scalar fma chain on sampled rows."""
+    from oracle import binding as oracle
+    import ctypes
+    _, M, N, K, _, _, desc = WORKLOADS[name]
+    L = oracle.lib()
+    threads = min(int(L.cpu_port_max_threads()), os.cpu_count() or 1)
+    a, lda = oracle.aligned_f32(M, K); a[:, :K] = A
+    b, ldb = oracle.aligned_f32(K, N); b[:, :N] = B
+    d, ldd = oracle.aligned_f32(M, N)
+    scratch, _ = oracle.aligned_f32(1, int(L.cpu_port_scratch_floats(K, N)))
+    fp = ctypes.POINTER(ctypes.c_float)
+    args = [x.ctypes.data_as(fp) for x in (a, b)] + [None, d.ctypes.data_as(fp), M, N, K, lda, ldb, 0, ldd,
+                                                     scratch.ctypes.data_as(fp), threads]
+    t0 = time.perf_counter()
+    rc = L.cpu_port_gemm_f32(*args)
+    secs = time.perf_counter() - t0
+    assert rc == 0
+    rows = np.unique(np.random.default_rng(0).integers(0, M, 16)).astype(np.uint32)
+    chain = oracle.gemm_f32(A, B, rows=rows)
+    same = bool(np.array_equal(d[rows, :N].view(np.uint32), chain.view(np.uint32)))
+    return {"value": round(2.0 * M * N * K / secs / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": "one full call of the same workload (%s), %.2f s wall" % (desc.split(",")[0], secs),
+            "bit_equal_to_fma_chain": same}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="fp32_8192", choices=sorted(WORKLOADS) + ["copy_1GiB"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this GEMM path runs on one GPU; --gpus %d is not supported (use --gpus 1)" % args.gpus)
+
+    from decx_amd import hip
+    hip.init(0)
+    props = hip.device_props()
+
+    if args.workload == "copy_1GiB":
+        # counter calibration: a copy whose HBM traffic is known (1 GiB read + 1 GiB written per launch)
+        n = 1 << 30
+        src = hip.DeviceMatrix(1, n // 4, np.float32); dst = hip.DeviceMatrix(1, n // 4, np.float32)
+        hip.check(hip.lib().decx_hip_memset_async(src.ptr, 1, n, None))
+        for _ in range(args.warmup):
+            hip.check(hip.lib().decx_hip_calibration_copy(dst.ptr, src.ptr, n, None))
+        hip.sync()
+        timer = hip.Timer(); timer.start()
+        for _ in range(args.steps):
+            hip.check(hip.lib().decx_hip_calibration_copy(dst.ptr, src.ptr, n, None))
+        ms = timer.stop() / args.steps
+        print(json.dumps({"workload": "calibration copy 1 GiB", "kernel_ms": ms, "GB/s_read_plus_write": 2 * n / ms / 1e6}))
+        return
+
+    main_out, inputs = run_workload(args.workload, args.steps, args.warmup, keep_inputs=not args.no_cpu)
+    line = {
+        "metric": "GEMM TFLOP/s (fp32 8192^3 headline; fp16 4096^3 under other_workloads) on 1 MI355X",
+        "value": main_out["value"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": main_out["kernel_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": main_out["dtype"], "data": "synthetic",
+        "config": {"workload": main_out["workload"], "plan": main_out["plan"],
+                   "device": props.name.decode(), "arch": props.arch.decode(), "compute_units": int(props.compute_units),
+                   "clock_mhz": props.clock_khz / 1000.0,
+                   "peak_recomputed_tflops": round(props.compute_units * (256 if main_out["dtype"] == "f32" else 4096)
+                                                   * props.clock_khz * 1e3 / 1e12, 1)},
+        "wall_ms_per_step": main_out["wall_ms_per_step"],
+        "roofline": main_out["roofline"],
+    }
+    if not args.no_extra:
+        others = []
+        for name in WORKLOADS:
+            if name != args.workload:
+                steps = args.steps if WORKLOADS[name][1] * WORKLOADS[name][2] * WORKLOADS[name][3] < 2 ** 38 else max(3, args.steps // 4)
+                others.append(run_workload(name, max(steps, 1), args.warmup)[0])
+        line["other_workloads"] = others
+    if not args.no_cpu:
+        if main_out["dtype"] == "f32":
+            line["cpu_baseline"] = cpu_baseline(args.workload, *inputs)
+        else:
+            line["cpu_baseline"] = None          # the reference has no fp16 CPU GEMM
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -77,9 +77,27 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
                : launch_gemm_f32(shape, edge, g, as_stream(stream));
 }
 
+__global__ void __launch_bounds__(256) calibration_copy_kernel(uintx4* __restrict__ dst,
+                                                              const uintx4* __restrict__ src, size_t n16)
+{
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+}
+
 }  // namespace
 
 extern "C" {
+
+int decx_hip_calibration_copy(void* dst, const void* src, size_t bytes, void* stream)
+{
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    if (!bytes) return DECX_HIP_OK;
+    if (!dst || !src || (bytes & 15u) || !aligned16(dst) || !aligned16(src)) return DECX_HIP_E_INVALID_ARG;
+    const size_t n16 = bytes / 16;
+    const size_t want = (n16 + 255) / 256;
+    const dim3 grid((unsigned)(want < 16384 ? want : 16384)), block(256);
+    hipLaunchKernelGGL(calibration_copy_kernel, grid, block, 0, as_stream(stream), (uintx4*)dst, (const uintx4*)src, n16);
+    return (int)hipGetLastError();
+}
 
 int decx_hip_init(int device)
 {

@@ -141,6 +141,12 @@ DECX_HIP_API int decx_hip_gemm_f16_tile(const uint16_t* A, const uint16_t* B, co
 DECX_HIP_API int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int aligned,
                                     decx_hip_plan* out);
 
+/* A plain device-to-device copy kernel (128-bit loads and stores, `bytes` a multiple of 16,
+ * both pointers 16-byte aligned).  It has no counterpart in the reference: it exists so that
+ * hardware traffic counters can be scaled against a launch whose HBM traffic is known
+ * (reads = writes = `bytes`). */
+DECX_HIP_API int decx_hip_calibration_copy(void* dst, const void* src, size_t bytes, void* stream);
+
 /* IEEE binary16 <-> binary32, round to nearest even; host-side helpers behind
  * de::Float2Half / de::Half2Float (srcs/common/FP16/float_half_convert.cu:35-46). */
 DECX_HIP_API uint16_t decx_hip_float_to_half(float value);
