@@ -61,9 +61,21 @@ def build_host(verbose=False):
     return out
 
 
+def build_api_test(verbose=False):
+    """The C++ program the tests drive the public de:: API with (tests/cpp/de_api_test)."""
+    src = os.path.join(ROOT, "tests", "cpp", "de_api_test.cpp")
+    out = os.path.join(ROOT, "tests", "cpp", "de_api_test")
+    _run(["g++", "-O1", "-std=c++17", "-Wall", "-I" + os.path.join(ROOT, "include"), src, "-o", out,
+          "-L" + LIB, "-lDECX_BLAS_HIP", "-ldecx_hip", "-Wl,-rpath," + LIB, "-Wl,-rpath,$ORIGIN/../../decx_amd/lib"])
+    if verbose:
+        print("built", out)
+    return out
+
+
 def build_all(verbose=False):
     build_hip(verbose)
     build_host(verbose)
+    build_api_test(verbose)
 
 
 if __name__ == "__main__":

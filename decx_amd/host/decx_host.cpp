@@ -1,0 +1,477 @@
+// Host side of the DECX matrix-product API on MI355X: the de:: objects, transfers, the
+// status handle and the GEMM entry points.  Everything that touches the GPU goes through
+// the C ABI in decx_hip.h.
+#include "decx_internal.hpp"
+
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <thread>
+
+namespace {
+
+de::DH g_last_error = {0, "success: No error"};
+bool g_gpu_ready = false;
+uint64_t g_threads = 1;
+void* g_stream = nullptr;
+std::mutex g_mutex;
+
+const char* const kSuccess         = "success: No error";
+const char* const kCudaNotInit     = "error: CUDA should be initialized first";
+const char* const kTypeNotMatch    = "error: The types of the two objects are not equal";
+const char* const kOverranged      = "error: Failed to transfer data since it is out of range";
+const char* const kDevAllocFail    = "error: Fail to allocate memory on device";
+const char* const kHostAllocFail   = "error: Fail to allocate memory on RAM";
+const char* const kClassNotInit    = "error: The class is not initialized";
+const char* const kUnsupportedType = "error: The data type of the input onject is not supported";
+const char* const kInvalidParam    = "error: The parameter(s) is(are) invalid";
+
+uint32_t round_up(uint32_t v, uint32_t to) { return (v + to - 1) / to * to; }
+
+}  // namespace
+
+// ---------------------------------------------------------------- status
+
+void decx::err::set(de::DH* h, int code, const char* text)
+{
+    h->error_type = code;
+    std::strncpy(h->error_string, text, sizeof h->error_string - 1);
+    h->error_string[sizeof h->error_string - 1] = '\0';
+}
+void decx::err::success(de::DH* h) { set(h, decx::DECX_SUCCESS, kSuccess); }
+
+bool decx::err::from_hip(de::DH* h, int rc, const char* what)
+{
+    if (rc == DECX_HIP_OK) return false;
+    char text[100];
+    std::snprintf(text, sizeof text, "error: %s: %s", what, decx_hip_error_string(rc));
+    int code = decx::DECX_FAIL_CUDA_STREAM;
+    if (rc == DECX_HIP_E_NOT_INIT || rc == DECX_HIP_E_NO_DEVICE) code = decx::DECX_FAIL_CUDA_not_init;
+    else if (rc == DECX_HIP_E_INVALID_ARG) code = decx::DECX_FAIL_INVALID_PARAM;
+    else if (rc == 2 /* hipErrorOutOfMemory */) code = decx::DECX_FAIL_CUDA_ALLOCATION;
+    set(h, code, text);
+    return true;
+}
+
+bool decx::gpu_ready() { return g_gpu_ready; }
+std::mutex& decx::module_mutex() { return g_mutex; }
+
+void* decx::module_stream()
+{
+    if (!g_stream && g_gpu_ready) {
+        if (decx_hip_stream_create(&g_stream) != DECX_HIP_OK) g_stream = nullptr;   // null stream still works
+    }
+    return g_stream;
+}
+
+uint32_t decx::element_size(de::_DATA_TYPES_FLAGS_ type)
+{
+    switch (type) {
+    case de::_FP32_: case de::_INT32_: case de::_UCHAR4_: return 4;
+    case de::_FP16_: return 2;
+    case de::_FP64_: case de::_COMPLEX_F32_: case de::_UINT64_: return 8;
+    case de::_COMPLEX_F64_: case de::_VECTOR3F_: case de::_VECTOR4F_: return 16;
+    case de::_UINT8_: return 1;
+    default: return 0;
+    }
+}
+
+decx::HostBlock::~HostBlock()
+{
+    if (!ptr) return;
+    if (pinned) decx_hip_host_free(ptr); else std::free(ptr);
+}
+decx::DeviceBlock::~DeviceBlock() { if (ptr) decx_hip_free(ptr); }
+
+_DECX_API_ void de::InitCuda()
+{
+    const int rc = decx_hip_init(0);
+    g_gpu_ready = (rc == DECX_HIP_OK);
+    if (!g_gpu_ready) decx::err::from_hip(&g_last_error, rc, "InitCuda");
+}
+_DECX_API_ void de::InitCPUInfo()
+{
+    const unsigned n = std::thread::hardware_concurrency();
+    g_threads = n ? n : 1;
+}
+_DECX_API_ void de::cuda::DECX_CUDA_exit()
+{
+    if (g_stream) { decx_hip_stream_destroy(g_stream); g_stream = nullptr; }
+}
+_DECX_API_ void de::cpu::DecxSetThreadingNum(const uint64_t n) { g_threads = n ? n : 1; }
+_DECX_API_ de::DH* de::GetLastError() { return &g_last_error; }
+_DECX_API_ void de::ResetLastError() { decx::err::success(&g_last_error); }
+
+_DECX_API_ de::Half de::Float2Half(const float& x) { de::Half h; h.val = decx_hip_float_to_half(x); return h; }
+_DECX_API_ float de::Half2Float(const de::Half& x) { return decx_hip_half_to_float(x.val); }
+
+// ---------------------------------------------------------------- host matrix
+
+void decx::_Matrix::assign(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height)
+{
+    _type = type;
+    _layout._single_element_size = (int32_t)element_size(type);
+    _layout.width = width;
+    _layout.height = height;
+    const uint32_t per32 = _layout._single_element_size ? 32u / (uint32_t)_layout._single_element_size : 1u;
+    _layout.pitch = round_up(width, per32 ? per32 : 1u);
+}
+
+bool decx::_Matrix::allocate()
+{
+    auto block = std::make_shared<HostBlock>();
+    const size_t bytes = total_bytes();
+    block->bytes = bytes ? (bytes + 63) / 64 * 64 : 64;
+    block->ptr = std::aligned_alloc(64, block->bytes);
+    if (!block->ptr) { err::set(de::GetLastError(), DECX_FAIL_ALLOCATION, kHostAllocFail); return false; }
+    std::memset(block->ptr, 0, block->bytes);
+    _block = block;
+    _data = block->ptr;
+    return true;
+}
+
+decx::_Matrix::_Matrix() : _format(de::_NA_), _data(nullptr)
+{
+    _exp_data_ptr = &_data;
+    _exp_matrix_dscr = &_layout;
+    assign(de::_VOID_, 0, 0);
+}
+decx::_Matrix::_Matrix(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height, de::_DATA_FORMATS_ format)
+    : _format(format), _data(nullptr)
+{
+    _exp_data_ptr = &_data;
+    _exp_matrix_dscr = &_layout;
+    assign(type, width, height);
+    allocate();
+}
+decx::_Matrix::~_Matrix() {}
+uint32_t decx::_Matrix::Width() const { return _layout.width; }
+uint32_t decx::_Matrix::Height() const { return _layout.height; }
+void decx::_Matrix::release() { _block.reset(); _data = nullptr; }
+de::_DATA_TYPES_FLAGS_ decx::_Matrix::Type() const { return _type; }
+void decx::_Matrix::Reinterpret(const de::_DATA_TYPES_FLAGS_ t) { _type = t; }   // tag only, as the original
+de::_DATA_FORMATS_ decx::_Matrix::Format() const { return _format; }
+
+de::Matrix& decx::_Matrix::SoftCopy(de::Matrix& src)
+{
+    const _Matrix& s = dynamic_cast<_Matrix&>(src);
+    assign(s._type, s._layout.width, s._layout.height);
+    _format = s._format;
+    _block = s._block;                 // shared, reference counted
+    _data = s._data;
+    return *this;
+}
+
+void decx::_Matrix::re_construct(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height)
+{
+    if (_type == type && _layout.width == width && _layout.height == height && _data) return;
+    const size_t before = _block ? _block->bytes : 0;
+    assign(type, width, height);
+    if (total_bytes() > before || !_data) allocate();
+}
+
+int decx::_Matrix::move_storage(bool pinned)
+{
+    if (!_block || !_block->ptr) return DECX_HIP_E_INVALID_ARG;
+    auto block = std::make_shared<HostBlock>();
+    block->bytes = _block->bytes;
+    block->pinned = pinned;
+    if (pinned) {
+        const int rc = decx_hip_host_malloc(&block->ptr, block->bytes);
+        if (rc != DECX_HIP_OK) { block->ptr = nullptr; return rc; }
+    } else {
+        block->ptr = std::aligned_alloc(64, block->bytes);
+        if (!block->ptr) return 2;
+    }
+    std::memcpy(block->ptr, _block->ptr, block->bytes);
+    _block = block;
+    _data = block->ptr;
+    return DECX_HIP_OK;
+}
+
+_DECX_API_ de::Matrix* de::CreateMatrixPtr() { return new decx::_Matrix(); }
+_DECX_API_ de::Matrix& de::CreateMatrixRef() { return *(new decx::_Matrix()); }
+_DECX_API_ de::Matrix* de::CreateMatrixPtr(const de::_DATA_TYPES_FLAGS_ type, const uint32_t w, const uint32_t h,
+                                           const de::_DATA_FORMATS_ format)
+{
+    return new decx::_Matrix(type, w, h, format);
+}
+_DECX_API_ de::Matrix& de::CreateMatrixRef(const de::_DATA_TYPES_FLAGS_ type, const uint32_t w, const uint32_t h,
+                                           const de::_DATA_FORMATS_ format)
+{
+    return *(new decx::_Matrix(type, w, h, format));
+}
+
+_DECX_API_ de::DH de::cuda::PinMemory(de::Matrix& src)
+{
+    de::DH handle; decx::err::success(&handle);
+    decx::_Matrix* m = dynamic_cast<decx::_Matrix*>(&src);
+    if (!decx::gpu_ready()) { decx::err::set(&handle, decx::DECX_FAIL_CUDA_not_init, kCudaNotInit); return handle; }
+    if (!m || !m->is_init()) { decx::err::set(&handle, decx::DECX_FAIL_CLASS_NOT_INIT, kClassNotInit); return handle; }
+    if (m->is_pinned()) {
+        decx::err::set(&handle, decx::DECX_FAIL_HOST_MEM_REGISTERED, "error: The host memory is already page-locked");
+        return handle;
+    }
+    decx::err::from_hip(&handle, m->move_storage(true), "PinMemory");
+    return handle;
+}
+_DECX_API_ de::DH de::cuda::UnpinMemory(de::Matrix& src)
+{
+    de::DH handle; decx::err::success(&handle);
+    decx::_Matrix* m = dynamic_cast<decx::_Matrix*>(&src);
+    if (!m || !m->is_init()) { decx::err::set(&handle, decx::DECX_FAIL_CLASS_NOT_INIT, kClassNotInit); return handle; }
+    if (!m->is_pinned()) {
+        decx::err::set(&handle, decx::DECX_FAIL_HOST_MEM_UNREGISTERED, "error: The host memory is not page-locked");
+        return handle;
+    }
+    decx::err::from_hip(&handle, m->move_storage(false), "UnpinMemory");
+    return handle;
+}
+
+// ---------------------------------------------------------------- device matrix
+
+void decx::_GPU_Matrix::assign(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height)
+{
+    _type = type;
+    _layout._single_element_size = (int32_t)element_size(type);
+    _layout.width = width;
+    _layout.height = height;
+    const uint32_t per128 = _layout._single_element_size ? 128u / (uint32_t)_layout._single_element_size : 1u;
+    _layout.pitch = round_up(width, per128 ? per128 : 1u);
+}
+
+bool decx::_GPU_Matrix::allocate()
+{
+    auto block = std::make_shared<DeviceBlock>();
+    block->bytes = total_bytes();
+    int rc = decx_hip_malloc(&block->ptr, block->bytes);
+    if (rc == DECX_HIP_OK && block->bytes) {
+        rc = decx_hip_memset_async(block->ptr, 0, block->bytes, module_stream());
+        if (rc == DECX_HIP_OK) rc = decx_hip_stream_sync(module_stream());
+    }
+    if (rc != DECX_HIP_OK) {
+        block->ptr = (rc == DECX_HIP_E_NOT_INIT) ? nullptr : block->ptr;
+        if (rc == DECX_HIP_E_NOT_INIT) err::set(de::GetLastError(), DECX_FAIL_CUDA_not_init, kCudaNotInit);
+        else err::set(de::GetLastError(), DECX_FAIL_CUDA_ALLOCATION, kDevAllocFail);
+        return false;
+    }
+    _block = block;
+    return true;
+}
+
+decx::_GPU_Matrix::_GPU_Matrix() : _format(de::_NA_) { assign(de::_VOID_, 0, 0); }
+decx::_GPU_Matrix::_GPU_Matrix(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height, de::_DATA_FORMATS_ format)
+    : _format(format)
+{
+    assign(type, width, height);
+    allocate();
+}
+decx::_GPU_Matrix::~_GPU_Matrix() {}
+uint decx::_GPU_Matrix::Width() const { return _layout.width; }
+uint decx::_GPU_Matrix::Height() const { return _layout.height; }
+void decx::_GPU_Matrix::release() { _block.reset(); }
+de::_DATA_TYPES_FLAGS_ decx::_GPU_Matrix::Type() const { return _type; }
+void decx::_GPU_Matrix::Reinterpret(const de::_DATA_TYPES_FLAGS_ t) { _type = t; }
+de::_DATA_FORMATS_ decx::_GPU_Matrix::Format() const { return _format; }
+
+de::GPU_Matrix& decx::_GPU_Matrix::SoftCopy(de::GPU_Matrix& src)
+{
+    const _GPU_Matrix& s = dynamic_cast<_GPU_Matrix&>(src);
+    assign(s._type, s._layout.width, s._layout.height);
+    _format = s._format;
+    _block = s._block;
+    return *this;
+}
+
+bool decx::_GPU_Matrix::re_construct(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height)
+{
+    if (_type == type && _layout.width == width && _layout.height == height && is_init()) return true;
+    const size_t before = _block ? _block->bytes : 0;
+    assign(type, width, height);
+    if (total_bytes() > before || !is_init()) return allocate();
+    return true;
+}
+
+_DECX_API_ de::GPU_Matrix& de::CreateGPUMatrixRef() { return *(new decx::_GPU_Matrix()); }
+_DECX_API_ de::GPU_Matrix* de::CreateGPUMatrixPtr() { return new decx::_GPU_Matrix(); }
+_DECX_API_ de::GPU_Matrix* de::CreateGPUMatrixPtr(const de::_DATA_TYPES_FLAGS_ type, const uint32_t w, const uint32_t h,
+                                                  const de::_DATA_FORMATS_ format)
+{
+    return new decx::_GPU_Matrix(type, w, h, format);
+}
+_DECX_API_ de::GPU_Matrix& de::CreateGPUMatrixRef(const de::_DATA_TYPES_FLAGS_ type, const uint32_t w, const uint32_t h,
+                                                  const de::_DATA_FORMATS_ format)
+{
+    return *(new decx::_GPU_Matrix(type, w, h, format));
+}
+
+// ---------------------------------------------------------------- transfers
+
+_DECX_API_ de::DH de::Memcpy(de::Matrix& host, de::GPU_Matrix& device, const de::Point2D start_src,
+                             de::Point2D start_dst, const de::Point2D size, const int flag)
+{
+    de::DH handle; decx::err::success(&handle);
+    if (!decx::gpu_ready()) { decx::err::set(&handle, decx::DECX_FAIL_CUDA_not_init, kCudaNotInit); return handle; }
+    decx::_Matrix* h = dynamic_cast<decx::_Matrix*>(&host);
+    decx::_GPU_Matrix* d = dynamic_cast<decx::_GPU_Matrix*>(&device);
+    if (!h || !d || !h->is_init() || !d->is_init()) {
+        decx::err::set(&handle, decx::DECX_FAIL_CLASS_NOT_INIT, kClassNotInit); return handle;
+    }
+    if (h->Type() != d->Type()) { decx::err::set(&handle, decx::DECX_FAIL_TYPE_MOT_MATCH, kTypeNotMatch); return handle; }
+    if (flag != de::DECX_MEMCPY_H2D && flag != de::DECX_MEMCPY_D2H) {
+        decx::err::set(&handle, decx::DECX_FAIL_INVALID_PARAM, kInvalidParam); return handle;
+    }
+    const bool h2d = flag == de::DECX_MEMCPY_H2D;
+    const int64_t src_w = h2d ? h->Width() : d->Width(), src_h = h2d ? h->Height() : d->Height();
+    const int64_t dst_w = h2d ? d->Width() : h->Width(), dst_h = h2d ? d->Height() : h->Height();
+    if (start_src.x < 0 || start_src.y < 0 || start_dst.x < 0 || start_dst.y < 0 || size.x < 0 || size.y < 0 ||
+        (int64_t)start_src.x + size.x > src_w || (int64_t)start_src.y + size.y > src_h ||
+        (int64_t)start_dst.x + size.x > dst_w || (int64_t)start_dst.y + size.y > dst_h) {
+        decx::err::set(&handle, decx::DECX_FAIL_MEMCPY_OVERRANGED, kOverranged); return handle;
+    }
+    const size_t es = (size_t)h->get_layout()._single_element_size;
+    const size_t hp = (size_t)h->Pitch() * es, dp = (size_t)d->Pitch() * es;
+    const de::Point2D hs = h2d ? start_src : start_dst, ds = h2d ? start_dst : start_src;
+    char* hptr = (char*)h->data() + (size_t)hs.y * hp + (size_t)hs.x * es;
+    char* dptr = (char*)d->data() + (size_t)ds.y * dp + (size_t)ds.x * es;
+    void* S = decx::module_stream();
+    int rc = h2d ? decx_hip_memcpy2d_async(dptr, dp, hptr, hp, (size_t)size.x * es, (size_t)size.y, 0, S)
+                 : decx_hip_memcpy2d_async(hptr, hp, dptr, dp, (size_t)size.x * es, (size_t)size.y, 1, S);
+    if (rc == DECX_HIP_OK) rc = decx_hip_stream_sync(S);
+    decx::err::from_hip(&handle, rc, "Memcpy");
+    return handle;
+}
+
+// ---------------------------------------------------------------- the product
+
+namespace {
+
+// Checks shared by both GPU entry points (cuda_GEMM_LS_planner::validate in the original,
+// srcs/modules/BLAS/GEMM/CUDA/large_squares/common/cuda_GEMM_LS_planner.cu:227-258, plus the
+// C-shape check its CPU twin makes, srcs/modules/BLAS/GEMM/CPU/cpu_GEMM_config.cxx:208-225).
+// Unlike the original, a failed check returns before anything is launched.
+bool validate(const decx::_GPU_Matrix* A, const decx::_GPU_Matrix* B, const decx::_GPU_Matrix* C,
+              const decx::_GPU_Matrix* dst, const de::Number* alpha, const de::Number* beta, de::DH* h)
+{
+    if (!decx::gpu_ready()) { decx::err::set(h, decx::DECX_FAIL_CUDA_not_init, kCudaNotInit); return false; }
+    if (!A || !B || !dst || !A->is_init() || !B->is_init() || (C && !C->is_init())) {
+        decx::err::set(h, decx::DECX_FAIL_CLASS_NOT_INIT, kClassNotInit); return false;
+    }
+    if (A->Width() != B->Height()) {
+        decx::err::set(h, decx::DECX_FAIL_DimsNotMatching,
+                       "The width of matrix A and height of matrix B must be identical");
+        return false;
+    }
+    if (A->Type() != B->Type() || (C && C->Type() != A->Type())) {
+        decx::err::set(h, decx::DECX_FAIL_TYPE_MOT_MATCH, "Types of the input matrices must be matched");
+        return false;
+    }
+    if (C && (C->Height() != A->Height() || C->Width() != B->Width())) {
+        decx::err::set(h, decx::DECX_FAIL_DimsNotMatching,
+                       "The height and width of the matrix C should be identical to that of matrix A and matrix B");
+        return false;
+    }
+    if (alpha && beta && (alpha->Type() != A->Type() || beta->Type() != A->Type())) {
+        decx::err::set(h, decx::DECX_FAIL_TYPE_MOT_MATCH,
+                       "The input scalar alpha and beta must match the type of input matrices");
+        return false;
+    }
+    if (A->Type() != de::_FP32_ && A->Type() != de::_FP16_) {
+        decx::err::set(h, decx::DECX_FAIL_UNSUPPORTED_TYPE, kUnsupportedType); return false;
+    }
+    return true;
+}
+
+bool gemm_device(decx::_GPU_Matrix* A, decx::_GPU_Matrix* B, decx::_GPU_Matrix* C, decx::_GPU_Matrix* dst,
+                 float alpha, float beta, de::DH* h)
+{
+    std::lock_guard<std::mutex> guard(decx::module_mutex());
+    // C may be the same object as dst: keep its storage alive and its pitch in hand across the reshape
+    const uint32_t ldc = C ? C->Pitch() : 0;
+    const void* c_ptr = C ? C->data() : nullptr;
+    if (!dst->re_construct(A->Type(), B->Width(), A->Height())) return false;   // status already set
+    void* S = decx::module_stream();
+    int rc;
+    if (A->Type() == de::_FP32_)
+        rc = decx_hip_gemm_f32((const float*)A->data(), (const float*)B->data(), (const float*)c_ptr,
+                               (float*)dst->data(), A->Height(), B->Width(), A->Width(),
+                               A->Pitch(), B->Pitch(), ldc, dst->Pitch(), alpha, beta, S);
+    else
+        rc = decx_hip_gemm_f16((const uint16_t*)A->data(), (const uint16_t*)B->data(), (const uint16_t*)c_ptr,
+                               (uint16_t*)dst->data(), A->Height(), B->Width(), A->Width(),
+                               A->Pitch(), B->Pitch(), ldc, dst->Pitch(), alpha, beta, S);
+    if (rc == DECX_HIP_OK) rc = decx_hip_stream_sync(S);                     // result complete on return
+    return !decx::err::from_hip(h, rc, "GEMM");
+}
+
+float scalar_of(const de::Number& n)
+{
+    return n.Type() == de::_FP16_ ? de::Half2Float(n.get_data_ref<de::Half>()) : n.get_data_ref<float>();
+}
+
+}  // namespace
+
+_DECX_API_ void de::blas::cuda::GEMM(de::GPU_Matrix& A, de::GPU_Matrix& B, de::GPU_Matrix& dst)
+{
+    decx::_GPU_Matrix* a = dynamic_cast<decx::_GPU_Matrix*>(&A);
+    decx::_GPU_Matrix* b = dynamic_cast<decx::_GPU_Matrix*>(&B);
+    decx::_GPU_Matrix* d = dynamic_cast<decx::_GPU_Matrix*>(&dst);
+    if (!validate(a, b, nullptr, d, nullptr, nullptr, de::GetLastError())) return;
+    gemm_device(a, b, nullptr, d, 1.f, 1.f, de::GetLastError());
+}
+
+_DECX_API_ void de::blas::cuda::GEMM(de::GPU_Matrix& A, de::GPU_Matrix& B, de::GPU_Matrix& C, de::GPU_Matrix& dst,
+                                     const de::Number alpha, const de::Number beta)
+{
+    decx::_GPU_Matrix* a = dynamic_cast<decx::_GPU_Matrix*>(&A);
+    decx::_GPU_Matrix* b = dynamic_cast<decx::_GPU_Matrix*>(&B);
+    decx::_GPU_Matrix* c = dynamic_cast<decx::_GPU_Matrix*>(&C);
+    decx::_GPU_Matrix* d = dynamic_cast<decx::_GPU_Matrix*>(&dst);
+    if (!c) { decx::err::set(de::GetLastError(), decx::DECX_FAIL_CLASS_NOT_INIT, kClassNotInit); return; }
+    if (!validate(a, b, c, d, &alpha, &beta, de::GetLastError())) return;
+    gemm_device(a, b, c, d, scalar_of(alpha), scalar_of(beta), de::GetLastError());
+}
+
+namespace {
+
+// Host-matrix form: stage through device memory.  The original declares these overloads
+// (srcs/includes/DECX/BLAS/BLAS.h:69-70) and defines them nowhere.
+void gemm_host(de::Matrix& A, de::Matrix& B, de::Matrix* C, de::Matrix& dst)
+{
+    de::DH* h = de::GetLastError();
+    decx::_Matrix* a = dynamic_cast<decx::_Matrix*>(&A);
+    decx::_Matrix* b = dynamic_cast<decx::_Matrix*>(&B);
+    decx::_Matrix* c = C ? dynamic_cast<decx::_Matrix*>(C) : nullptr;
+    decx::_Matrix* d = dynamic_cast<decx::_Matrix*>(&dst);
+    if (!decx::gpu_ready()) { decx::err::set(h, decx::DECX_FAIL_CUDA_not_init, kCudaNotInit); return; }
+    if (!a || !b || !d || !a->is_init() || !b->is_init() || (C && (!c || !c->is_init()))) {
+        decx::err::set(h, decx::DECX_FAIL_CLASS_NOT_INIT, kClassNotInit); return;
+    }
+    decx::_GPU_Matrix dA(a->Type(), a->Width(), a->Height(), de::_NA_);
+    decx::_GPU_Matrix dB(b->Type(), b->Width(), b->Height(), de::_NA_);
+    decx::_GPU_Matrix dC, dD;
+    if (!dA.is_init() || !dB.is_init()) return;
+    const de::Point2D zero(0, 0);
+    de::DH r = de::Memcpy(A, dA, zero, zero, de::Point2D(a->Width(), a->Height()), de::DECX_MEMCPY_H2D);
+    if (r.error_type == decx::DECX_SUCCESS)
+        r = de::Memcpy(B, dB, zero, zero, de::Point2D(b->Width(), b->Height()), de::DECX_MEMCPY_H2D);
+    if (r.error_type == decx::DECX_SUCCESS && c) {
+        dC.re_construct(c->Type(), c->Width(), c->Height());
+        if (!dC.is_init()) return;
+        r = de::Memcpy(*C, dC, zero, zero, de::Point2D(c->Width(), c->Height()), de::DECX_MEMCPY_H2D);
+    }
+    if (r.error_type != decx::DECX_SUCCESS) { *h = r; return; }
+    if (!validate(&dA, &dB, c ? &dC : nullptr, &dD, nullptr, nullptr, h)) return;
+    if (!gemm_device(&dA, &dB, c ? &dC : nullptr, &dD, 1.f, 1.f, h)) return;
+    d->re_construct(a->Type(), b->Width(), a->Height());
+    r = de::Memcpy(dst, dD, zero, zero, de::Point2D(dD.Width(), dD.Height()), de::DECX_MEMCPY_D2H);
+    if (r.error_type != decx::DECX_SUCCESS) *h = r;
+}
+
+}  // namespace
+
+_DECX_API_ void de::blas::cuda::GEMM(de::Matrix& A, de::Matrix& B, de::Matrix& dst) { gemm_host(A, B, nullptr, dst); }
+_DECX_API_ void de::blas::cuda::GEMM(de::Matrix& A, de::Matrix& B, de::Matrix& C, de::Matrix& dst)
+{
+    gemm_host(A, B, &C, dst);
+}

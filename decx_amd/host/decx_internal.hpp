@@ -1,0 +1,107 @@
+// Implementation classes behind the public de:: objects.  Host C++ only: the GPU is
+// reached exclusively through the C ABI of decx_hip.h.
+#pragma once
+#include "DECX.h"
+#include "decx_hip.h"
+
+#include <cstddef>
+#include <memory>
+#include <mutex>
+
+namespace decx {
+
+// Status helpers (the library-side view of de::DH).
+namespace err {
+void set(de::DH* h, int code, const char* text);
+void success(de::DH* h);
+// Translates a decx_hip return code into the handle; returns true when rc signals failure.
+bool from_hip(de::DH* h, int rc, const char* what);
+}  // namespace err
+
+bool gpu_ready();
+uint32_t element_size(de::_DATA_TYPES_FLAGS_ type);
+
+// Reference-counted storage shared by SoftCopy aliases.
+struct HostBlock {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    bool pinned = false;
+    ~HostBlock();
+};
+struct DeviceBlock {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    ~DeviceBlock();
+};
+
+// Host matrix.  Layout rule of the original (srcs/modules/core/classes/Matrix.cxx:35-64):
+// pitch = width rounded up to 32 bytes of elements, storage zero-filled.
+class _Matrix : public de::Matrix {
+    de::MatrixLayout _layout;
+    de::_DATA_TYPES_FLAGS_ _type;
+    de::_DATA_FORMATS_ _format;
+    std::shared_ptr<HostBlock> _block;
+    void* _data;                       // what _exp_data_ptr points at
+    void assign(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height);
+    bool allocate();
+
+public:
+    _Matrix();
+    _Matrix(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height, de::_DATA_FORMATS_ format);
+    virtual uint32_t Width() const;
+    virtual uint32_t Height() const;
+    virtual void release();
+    virtual de::Matrix& SoftCopy(de::Matrix& src);
+    virtual de::_DATA_TYPES_FLAGS_ Type() const;
+    virtual void Reinterpret(const de::_DATA_TYPES_FLAGS_ new_type);
+    virtual de::_DATA_FORMATS_ Format() const;
+    virtual ~_Matrix();
+
+    uint32_t Pitch() const { return _layout.pitch; }
+    const de::MatrixLayout& get_layout() const { return _layout; }
+    bool is_init() const { return _data != nullptr; }
+    void* data() const { return _data; }
+    size_t total_bytes() const { return (size_t)_layout.pitch * _layout.height * _layout._single_element_size; }
+    void re_construct(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height);
+    bool is_pinned() const { return _block && _block->pinned; }
+    int move_storage(bool pinned);     // 0 or a decx_hip error code
+};
+
+// Device matrix.  Layout rule of the original (srcs/modules/core/classes/GPU_Matrix.cu:35-61):
+// pitch = width rounded up to 128 bytes of elements, storage zero-filled.
+class _GPU_Matrix : public de::GPU_Matrix {
+    de::MatrixLayout _layout;
+    de::_DATA_TYPES_FLAGS_ _type;
+    de::_DATA_FORMATS_ _format;
+    std::shared_ptr<DeviceBlock> _block;
+    void assign(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height);
+    bool allocate();
+
+public:
+    _GPU_Matrix();
+    _GPU_Matrix(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height, de::_DATA_FORMATS_ format);
+    virtual uint Width() const;
+    virtual uint Height() const;
+    virtual void release();
+    virtual de::_DATA_TYPES_FLAGS_ Type() const;
+    virtual void Reinterpret(const de::_DATA_TYPES_FLAGS_ new_type);
+    virtual de::GPU_Matrix& SoftCopy(de::GPU_Matrix& src);
+    virtual de::_DATA_FORMATS_ Format() const;
+    virtual ~_GPU_Matrix();
+
+    uint32_t Pitch() const { return _layout.pitch; }
+    const de::MatrixLayout& get_layout() const { return _layout; }
+    bool is_init() const { return _block && _block->ptr; }
+    void* data() const { return _block ? _block->ptr : nullptr; }
+    size_t total_bytes() const { return (size_t)_layout.pitch * _layout.height * _layout._single_element_size; }
+    // Reshapes; storage is reallocated (and zero-filled) only when it has to grow
+    // (srcs/modules/core/classes/GPU_Matrix.cu:120-134).  Returns false on allocation failure.
+    bool re_construct(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height);
+};
+
+// One stream for the module, created on first use; one mutex around every GEMM call
+// (the original guards its cached planner with a plain flag).
+void* module_stream();
+std::mutex& module_mutex();
+
+}  // namespace decx

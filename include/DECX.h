@@ -1,0 +1,268 @@
+/*
+ * DECX.h -- public C++ interface of the MI355X-native dense-GEMM module.
+ *
+ * Source- and ABI-compatible with the part of the DECX user API that the matrix
+ * multiplication path touches, so code written against the original library
+ * (samples/Matrix_Multiplication/MatMul.cpp) builds and links unchanged:
+ *
+ *   de::DH, de::GetLastError            srcs/includes/DECX/basic.h:84-98,127-159
+ *   de::_DATA_TYPES_FLAGS_, formats     srcs/includes/DECX/classes/type_info.h:20-53
+ *   de::Half, de::Point2D               srcs/includes/DECX/classes/class_utils.h:19-60
+ *   de::Number, Float2Half, Half2Float  srcs/includes/DECX/classes/DecxNumber.h:17-188
+ *   de::Matrix, de::MatrixLayout        srcs/includes/DECX/classes/Matrix.h:34-105
+ *   de::GPU_Matrix, Pin/UnpinMemory     srcs/includes/DECX/classes/GPU_Matrix.h:19-65
+ *   de::Memcpy (matrix form)            srcs/includes/DECX/classes/decx_memcpy.h:29-48
+ *   de::blas::cuda::GEMM                srcs/includes/DECX/BLAS/BLAS.h:69-76
+ *
+ * Same class layouts (vtable order, the two shadow pointers of de::Matrix), same enum
+ * values, same width-before-height argument order.  The namespace stays `cuda` because
+ * it is part of the API's spelling; everything behind it is HIP on gfx950, reached
+ * through the C ABI in decx_hip.h.
+ *
+ * Not provided here: de::blas::cpu::GEMM (the CPU path is not part of this module), and
+ * the vector / tensor containers, which the matrix product does not use.
+ */
+#ifndef DECX_AMD_PUBLIC_H_
+#define DECX_AMD_PUBLIC_H_
+
+#ifndef __cplusplus
+#error "DECX.h is a C++ header; C callers use decx_hip.h"
+#endif
+
+#include <cstdint>
+#include <cstdio>
+
+typedef unsigned char uchar;
+typedef unsigned int uint;
+
+#define _DECX_API_ __attribute__((visibility("default")))
+#define _SHADOW_ATTRIBUTE_(__actual_type) __actual_type*
+
+/* ------------------------------------------------------------------ status handle */
+namespace de {
+
+typedef struct DECX_Handle {
+    int  error_type;           /* one of decx::DECX_error_types below */
+    char error_string[100];
+} DH;
+
+/* The user-facing enum of the original header, kept value for value. */
+enum DECX_error_types {
+    DECX_SUCCESS = 0x00, DECX_FAIL_not_init = 0x01, DECX_FAIL_FFT_error_length = 0x02,
+    DECX_FAIL_DimsNotMatching = 0x03, DECX_FAIL_Complex_comparing = 0x04, DECX_FAIL_ConvBadKernel = 0x05,
+    DECX_FAIL_StepError = 0x06, DECX_FAIL_ChannelError = 0x07, DECX_FAIL_CVNLM_BadArea = 0x08,
+    DECX_FAIL_FileNotExist = 0x09, DECX_GEMM_DimsError = 0x0a, DECX_FAIL_ErrorFlag = 0x0b,
+    DECX_FAIL_DimError = 0x0c, DECX_FAIL_ErrorParams = 0x0d, DECX_FAIL_StoreError = 0x0e,
+    DECX_FAIL_MNumNotMatching = 0x0f, DECX_FAIL_ALLOCATION = 0x10
+};
+
+_DECX_API_ void InitCuda();          /* selects GPU 0 and reads its properties; must precede Memcpy / GEMM */
+_DECX_API_ void InitCPUInfo();       /* records the host's hardware concurrency */
+_DECX_API_ DH*  GetLastError();      /* process-global status of the last failing call */
+_DECX_API_ void ResetLastError();
+
+namespace cuda { _DECX_API_ void DECX_CUDA_exit(); }
+namespace cpu  { _DECX_API_ void DecxSetThreadingNum(const uint64_t _thread_num); }
+
+}  // namespace de
+
+/* The codes the library actually writes into de::DH::error_type: the original library
+ * sets its *internal* numbering (srcs/common/Handle/decx_handle.h:47-179), which differs
+ * from the user-facing enum above; both are kept. */
+namespace decx {
+enum DECX_error_types {
+    DECX_SUCCESS = 0x00, DECX_FAIL_CPU_not_init = 0x01, DECX_FAIL_FFT_error_length = 0x02,
+    DECX_FAIL_DimsNotMatching = 0x03, DECX_FAIL_Complex_comparing = 0x04, DECX_FAIL_ConvBadKernel = 0x05,
+    DECX_FAIL_CVNLM_BadArea = 0x06, DECX_FAIL_ErrorFlag = 0x07, DECX_FAIL_ALLOCATION = 0x08,
+    DECX_FAIL_CUDA_STREAM = 0x09, DECX_FAIL_CLASS_NOT_INIT = 0x0a, DECX_FAIL_TYPE_MOT_MATCH = 0x0b,
+    DECX_FAIL_INVALID_PARAM = 0x0c, DECX_FAIL_IMAGE_LOAD_FAILED = 0x0d, DECX_FAIL_CUDA_EVENT = 0x0e,
+    MULTIPLE_REFERENCES = 0x0f, CPU_HYPER_THREADING = 0x10, MEMCPY_DIFFERENT_TYPES = 0x11,
+    DECX_FAIL_MEMCPY_OVERRANGED = 0x12, DECX_FAIL_UNSUPPORTED_TYPE = 0x13, DECX_FAIL_HOST_MEM_REGISTERED = 0x14,
+    DECX_FAIL_HOST_MEM_UNREGISTERED = 0x15, DECX_FAIL_CUDA_not_init = 0x16, DECX_FAIL_CUDA_ALLOCATION = 0x17
+};
+}  // namespace decx
+
+/* ------------------------------------------------------------------ element types */
+namespace de {
+
+enum _DATA_TYPES_FLAGS_ {
+    _VOID_ = 0, _FP32_ = 1, _FP64_ = 2, _FP16_ = 3, _INT32_ = 4, _COMPLEX_F32_ = 5, _COMPLEX_F64_ = 6,
+    _UINT64_ = 7, _UINT8_ = 8, _UCHAR4_ = 12, _VECTOR3F_ = 14, _VECTOR4F_ = 15
+};
+
+enum _DATA_FORMATS_ { _NA_ = 0, _RGB_ = 1, _YUV444_ = 2, _HSV_ = 3, _CPLX_CARTESIAN_ = 4, _CPLX_POLAR_ = 5 };
+
+enum GEMM_properties { HALF_GEMM_DIRECT = 0, HALF_GEMM_ACCURATE = 1 };
+
+struct Half { unsigned short val; };                 /* IEEE binary16 bit pattern */
+
+typedef struct __attribute__((aligned(8))) complex_f {
+    float real, image;
+    complex_f(const float r, const float i) : real(r), image(i) {}
+    complex_f() {}
+} CPf;
+
+typedef struct __attribute__((aligned(16))) complex_d {
+    double real, image;
+    complex_d(const double r, const double i) : real(r), image(i) {}
+    complex_d() : real(0), image(0) {}
+} CPd;
+
+struct __attribute__((aligned(8))) Point2D {         /* [x = along the width, y = along the height] */
+    int32_t x, y;
+    Point2D(const int32_t _x, const int32_t _y) : x(_x), y(_y) {}
+    Point2D(const uint32_t _x, const uint32_t _y) : x((int32_t)_x), y((int32_t)_y) {}
+    Point2D() {}
+};
+
+_DECX_API_ Half  Float2Half(const float& __x);       /* round to nearest even */
+_DECX_API_ float Half2Float(const Half& __x);
+
+/* A tagged scalar: carries alpha / beta of the four-matrix GEMM. */
+class _DECX_API_ Number {
+    union __attribute__((aligned(16))) _data {
+        float _fp32; double _fp64; CPf _cplxf32; CPd _cplxd64; uint8_t _u8; int32_t _i32; Half _fp16;
+        _data() { _cplxd64.real = 0.0; _cplxd64.image = 0.0; }
+    };
+    _data   _number;
+    int32_t _data_type_flag;
+
+public:
+    Number() : _data_type_flag(_VOID_) {}
+    Number(const int32_t v) : _data_type_flag(_INT32_)       { _number._i32 = v; }
+    Number(const uint8_t v) : _data_type_flag(_UINT8_)       { _number._u8 = v; }
+    Number(const float v)   : _data_type_flag(_FP32_)        { _number._fp32 = v; }
+    Number(const double v)  : _data_type_flag(_FP64_)        { _number._fp64 = v; }
+    Number(const Half v)    : _data_type_flag(_FP16_)        { _number._fp16 = v; }
+    Number(const CPf v)     : _data_type_flag(_COMPLEX_F32_) { _number._cplxf32 = v; }
+    Number(const CPd v)     : _data_type_flag(_COMPLEX_F64_) { _number._cplxd64 = v; }
+
+    int32_t Type() const { return _data_type_flag; }
+    template <typename _Ty> _Ty get_data() { return *((_Ty*)&_number); }
+    template <typename _Ty> const _Ty& get_data_ref() const { return *((const _Ty*)&_number); }
+
+    Number& operator=(const float v)   { _number._fp32 = v;    _data_type_flag = _FP32_;        return *this; }
+    Number& operator=(const double v)  { _number._fp64 = v;    _data_type_flag = _FP64_;        return *this; }
+    Number& operator=(const CPf v)     { _number._cplxf32 = v; _data_type_flag = _COMPLEX_F32_; return *this; }
+    Number& operator=(const CPd v)     { _number._cplxd64 = v; _data_type_flag = _COMPLEX_F64_; return *this; }
+    Number& operator=(const uint8_t v) { _number._u8 = v;      _data_type_flag = _UINT8_;       return *this; }
+    Number& operator=(const int32_t v) { _number._i32 = v;     _data_type_flag = _INT32_;       return *this; }
+    Number& operator=(const Half v)    { _number._fp16 = v;    _data_type_flag = _FP16_;        return *this; }
+
+    void Print() {
+        switch (_data_type_flag) {
+        case _FP32_:        printf("%f\n", get_data<float>()); break;
+        case _FP16_:        printf("%f\n", Half2Float(get_data<Half>())); break;
+        case _FP64_:        printf("%f\n", get_data<double>()); break;
+        case _INT32_:       printf("%d\n", get_data<int32_t>()); break;
+        case _UINT8_:       printf("%d\n", (int32_t)get_data<uint8_t>()); break;
+        case _COMPLEX_F32_: printf("(%f, %f)\n", get_data<CPf>().real, get_data<CPf>().image); break;
+        default: break;
+        }
+    }
+};
+typedef const Number& InputNumber;
+typedef Number& OutputNumber;
+typedef Number& InOutNumber;
+
+/* ------------------------------------------------------------------ host matrix */
+
+struct MatrixLayout {
+    uint32_t width, height;
+    uint32_t pitch;                    /* row stride in elements: width rounded up to 32 bytes */
+    int32_t  _single_element_size;
+};
+
+class _DECX_API_ Matrix {
+protected:
+    _SHADOW_ATTRIBUTE_(void*)        _exp_data_ptr;        /* -> the implementation's data pointer */
+    _SHADOW_ATTRIBUTE_(MatrixLayout) _exp_matrix_dscr;     /* -> the implementation's layout */
+
+public:
+    Matrix() {}
+    virtual uint32_t Width() const = 0;
+    virtual uint32_t Height() const = 0;
+
+    template <typename _ptr_type> _ptr_type* ptr(const int row, const int col) {
+        return ((_ptr_type*)*this->_exp_data_ptr) + this->_exp_matrix_dscr->pitch * row + col;
+    }
+
+    virtual void release() = 0;
+    virtual Matrix& SoftCopy(Matrix& src) = 0;
+    virtual _DATA_TYPES_FLAGS_ Type() const = 0;
+    virtual void Reinterpret(const _DATA_TYPES_FLAGS_ _new_type) = 0;
+    virtual _DATA_FORMATS_ Format() const = 0;
+    ~Matrix() {}
+};
+typedef const Matrix& InputMatrix;
+typedef Matrix& OutputMatrix;
+typedef Matrix& InOutMatrix;
+
+_DECX_API_ Matrix* CreateMatrixPtr();
+_DECX_API_ Matrix& CreateMatrixRef();
+_DECX_API_ Matrix* CreateMatrixPtr(const _DATA_TYPES_FLAGS_ type, const uint32_t _width, const uint32_t _height,
+                                   const _DATA_FORMATS_ format = _NA_);
+_DECX_API_ Matrix& CreateMatrixRef(const _DATA_TYPES_FLAGS_ type, const uint32_t _width, const uint32_t _height,
+                                   const _DATA_FORMATS_ format = _NA_);
+
+/* ------------------------------------------------------------------ device matrix */
+
+class _DECX_API_ GPU_Matrix {
+public:
+    GPU_Matrix() {}
+    virtual uint Width() const = 0;
+    virtual uint Height() const = 0;
+    virtual void release() = 0;
+    virtual _DATA_TYPES_FLAGS_ Type() const = 0;
+    virtual void Reinterpret(const _DATA_TYPES_FLAGS_ _new_type) = 0;
+    virtual GPU_Matrix& SoftCopy(GPU_Matrix& src) = 0;
+    virtual _DATA_FORMATS_ Format() const = 0;
+    ~GPU_Matrix() {}
+};
+typedef const GPU_Matrix& InputGPUMatrix;
+typedef GPU_Matrix& OutputGPUMatrix;
+typedef GPU_Matrix& InOutGPUMatrix;
+
+_DECX_API_ GPU_Matrix& CreateGPUMatrixRef();
+_DECX_API_ GPU_Matrix* CreateGPUMatrixPtr();
+_DECX_API_ GPU_Matrix* CreateGPUMatrixPtr(const _DATA_TYPES_FLAGS_ type, const uint32_t _width, const uint32_t _height,
+                                          const _DATA_FORMATS_ format = _NA_);
+_DECX_API_ GPU_Matrix& CreateGPUMatrixRef(const _DATA_TYPES_FLAGS_ type, const uint32_t _width, const uint32_t _height,
+                                          const _DATA_FORMATS_ format = _NA_);
+
+namespace cuda {
+/* Makes the host matrix's storage page-locked (faster, asynchronous-capable transfers) and
+ * back.  The storage is moved, not registered in place; pointers obtained from ptr<T>()
+ * before the call must be re-read. */
+_DECX_API_ DH PinMemory(Matrix& src);
+_DECX_API_ DH UnpinMemory(Matrix& src);
+}
+
+/* ------------------------------------------------------------------ transfers */
+
+enum DECX_Memcpy_Flags { DECX_MEMCPY_H2D = 0, DECX_MEMCPY_D2H = 1 };
+
+/* Copies the cpy_size = [W, H] region that starts at start_src in the source object to
+ * start_dst in the destination object; the source is the host matrix for H2D and the
+ * device matrix for D2H.  Blocks until the copy has finished. */
+_DECX_API_ DH Memcpy(Matrix& __host, GPU_Matrix& __device, const Point2D start_src, Point2D start_dst,
+                     const Point2D cpy_size, const int _memcpy_flag);
+
+/* ------------------------------------------------------------------ the product */
+namespace blas {
+namespace cuda {
+/* dst <- A . B.  dst is reshaped to B.Width() x A.Height() of A's type (its storage is
+ * reallocated only when it has to grow).  Returns when the result is complete. */
+_DECX_API_ void GEMM(GPU_Matrix& A, GPU_Matrix& B, GPU_Matrix& dst);
+/* dst <- alpha . (A . B) + beta . C; alpha and beta must carry A's element type. */
+_DECX_API_ void GEMM(GPU_Matrix& A, GPU_Matrix& B, GPU_Matrix& C, GPU_Matrix& dst,
+                     const Number alpha, const Number beta);
+/* Host-matrix forms: operands are staged through device memory around the same kernels. */
+_DECX_API_ void GEMM(Matrix& A, Matrix& B, Matrix& dst);
+_DECX_API_ void GEMM(Matrix& A, Matrix& B, Matrix& C, Matrix& dst);
+}  // namespace cuda
+}  // namespace blas
+
+}  // namespace de
+
+#endif  /* DECX_AMD_PUBLIC_H_ */

@@ -1,0 +1,259 @@
+// Exercises the public C++ API (include/DECX.h) the way a user of the original library
+// would (cf. samples/Matrix_Multiplication/MatMul.cpp:74-113): factories, ptr<T>(),
+// de::Memcpy, de::blas::cuda::GEMM, de::GetLastError.
+//
+//   de_api_test host                      checks that need no GPU; exit code 0 = all passed
+//   de_api_test gpu                       self-contained GPU checks (closed forms, error paths)
+//   de_api_test gemm <dir> <f32|f16> M N K <withC 0|1> <alpha> <beta>
+//                                         reads dense A.bin B.bin [C.bin] from <dir>, writes D.bin
+#include "DECX.h"
+
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+#include <string>
+#include <vector>
+
+static int g_failures = 0;
+#define CHECK(cond) do { if (!(cond)) { ++g_failures; std::cerr << "FAILED line " << __LINE__ << ": " #cond "\n"; } } while (0)
+
+static int host_checks()
+{
+    // pitch rule of host matrices: rows padded to 32 bytes; storage zero-filled
+    de::Matrix& a = de::CreateMatrixRef(de::_FP32_, 777, 5);
+    CHECK(a.Width() == 777 && a.Height() == 5 && a.Type() == de::_FP32_ && a.Format() == de::_NA_);
+    CHECK(a.ptr<float>(1, 0) - a.ptr<float>(0, 0) == 784);
+    CHECK(((uintptr_t)a.ptr<float>(0, 0) & 31u) == 0);
+    bool zero = true;
+    for (int r = 0; r < 5; ++r) for (int c = 0; c < 784; ++c) zero &= (*a.ptr<float>(r, c) == 0.f);
+    CHECK(zero);
+    de::Matrix& h = de::CreateMatrixRef(de::_FP16_, 1, 3);
+    CHECK(h.ptr<de::Half>(1, 0) - h.ptr<de::Half>(0, 0) == 16);
+    de::Matrix* e = de::CreateMatrixPtr();
+    CHECK(e->Width() == 0 && e->Height() == 0 && e->Type() == de::_VOID_);
+
+    // SoftCopy aliases the storage
+    de::Matrix& alias = de::CreateMatrixRef();
+    alias.SoftCopy(a);
+    *a.ptr<float>(2, 3) = 42.f;
+    CHECK(alias.Width() == 777 && *alias.ptr<float>(2, 3) == 42.f);
+    a.release();
+    CHECK(*alias.ptr<float>(2, 3) == 42.f);            // still alive through the alias
+    alias.Reinterpret(de::_INT32_);
+    CHECK(alias.Type() == de::_INT32_ && alias.Width() == 777);
+
+    // Number and Half
+    de::Number n(1.5f);
+    CHECK(n.Type() == de::_FP32_ && n.get_data<float>() == 1.5f);
+    n = de::Float2Half(0.333251953125f);
+    CHECK(n.Type() == de::_FP16_ && n.get_data<de::Half>().val == 0x3555);
+    CHECK(sizeof(de::Number) == 32 && sizeof(de::DH) == 104 && sizeof(de::MatrixLayout) == 16);
+    CHECK(de::Float2Half(1.0f).val == 0x3c00 && de::Float2Half(-2.0f).val == 0xc000);
+    CHECK(de::Float2Half(65520.f).val == 0x7c00 && de::Float2Half(65519.f).val == 0x7bff);
+    CHECK(de::Float2Half(1.0f + 0x1p-11f).val == 0x3c00 && de::Float2Half(1.0f + 3 * 0x1p-11f).val == 0x3c02);
+    de::Half one; one.val = 0x3c00;
+    CHECK(de::Half2Float(one) == 1.0f);
+    de::Half sub; sub.val = 0x0001;
+    CHECK(de::Half2Float(sub) == 0x1p-24f);
+
+    // status handle; GPU entry points before InitCuda report "CUDA not initialised" (0x16)
+    de::ResetLastError();
+    CHECK(de::GetLastError()->error_type == 0 && std::string(de::GetLastError()->error_string) == "success: No error");
+    de::Matrix& src = de::CreateMatrixRef(de::_FP32_, 8, 8);
+    de::GPU_Matrix* none = de::CreateGPUMatrixPtr();
+    de::DH r = de::Memcpy(src, *none, de::Point2D(0, 0), de::Point2D(0, 0), de::Point2D(8, 8), de::DECX_MEMCPY_H2D);
+    CHECK(r.error_type == decx::DECX_FAIL_CUDA_not_init);
+    de::blas::cuda::GEMM(*none, *none, *none);
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_CUDA_not_init);
+    de::ResetLastError();
+    de::blas::cuda::GEMM(src, src, src);
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_CUDA_not_init);
+    CHECK(de::cuda::PinMemory(src).error_type == decx::DECX_FAIL_CUDA_not_init);
+    de::InitCPUInfo();
+    de::cpu::DecxSetThreadingNum(4);
+    return g_failures;
+}
+
+template <typename T> static void fill(de::Matrix& m, T (*f)(int, int))
+{
+    for (int i = 0; i < (int)m.Height(); ++i) for (int j = 0; j < (int)m.Width(); ++j) *m.ptr<T>(i, j) = f(i, j);
+}
+
+static int gpu_checks()
+{
+    de::InitCPUInfo();
+    de::InitCuda();
+    de::ResetLastError();
+    const de::Point2D O(0, 0);
+
+    // the original sample: A[i][j] = j, B[i][j] = i  =>  every element = sum l^2, l < L
+    const uint32_t W = 1013, H = 1077, L = 1005;
+    de::Matrix& A = de::CreateMatrixRef(de::_FP32_, L, H);
+    de::Matrix& B = de::CreateMatrixRef(de::_FP32_, W, L);
+    de::Matrix& D = de::CreateMatrixRef(de::_FP32_, W, H);
+    fill<float>(A, [](int, int j) { return (float)j; });
+    fill<float>(B, [](int i, int) { return (float)i; });
+    de::GPU_Matrix& dA = de::CreateGPUMatrixRef(de::_FP32_, L, H);
+    de::GPU_Matrix& dB = de::CreateGPUMatrixRef(de::_FP32_, W, L);
+    de::GPU_Matrix& dD = de::CreateGPUMatrixRef();                     // empty: GEMM shapes it
+    CHECK(de::Memcpy(A, dA, O, O, de::Point2D(L, H), de::DECX_MEMCPY_H2D).error_type == 0);
+    CHECK(de::Memcpy(B, dB, O, O, de::Point2D(W, L), de::DECX_MEMCPY_H2D).error_type == 0);
+    de::blas::cuda::GEMM(dA, dB, dD);
+    CHECK(de::GetLastError()->error_type == 0);
+    CHECK(dD.Width() == W && dD.Height() == H && dD.Type() == de::_FP32_);
+    CHECK(de::Memcpy(D, dD, O, O, de::Point2D(W, H), de::DECX_MEMCPY_D2H).error_type == 0);
+    double worst = 0;
+    for (uint32_t i = 0; i < H; ++i) for (uint32_t j = 0; j < W; ++j)
+        worst = std::fmax(worst, std::fabs((double)*D.ptr<float>(i, j) - 337853530.0) / 337853530.0);
+    CHECK(worst < 4e-6);
+
+    // four-matrix form, alpha = 2, beta = -1, C = ones: 2 * sum - 1; C aliasing dst
+    de::GPU_Matrix& dC = de::CreateGPUMatrixRef(de::_FP32_, W, H);
+    de::Matrix& C = de::CreateMatrixRef(de::_FP32_, W, H);
+    fill<float>(C, [](int, int) { return 1.f; });
+    CHECK(de::Memcpy(C, dC, O, O, de::Point2D(W, H), de::DECX_MEMCPY_H2D).error_type == 0);
+    de::blas::cuda::GEMM(dA, dB, dC, dC, de::Number(2.f), de::Number(-1.f));
+    CHECK(de::GetLastError()->error_type == 0);
+    CHECK(de::Memcpy(D, dC, O, O, de::Point2D(W, H), de::DECX_MEMCPY_D2H).error_type == 0);
+    worst = 0;
+    for (uint32_t i = 0; i < H; ++i) for (uint32_t j = 0; j < W; ++j)
+        worst = std::fmax(worst, std::fabs((double)*D.ptr<float>(i, j) - (2 * 337853530.0 - 1)) / 675707059.0);
+    CHECK(worst < 4e-6);
+
+    // dst shrinks without reallocation, grows with it; sub-region copies honour both pitches
+    de::GPU_Matrix& dS = de::CreateGPUMatrixRef(de::_FP32_, 40, 50);
+    de::Matrix& S = de::CreateMatrixRef(de::_FP32_, 40, 50);
+    fill<float>(S, [](int i, int j) { return (float)(i * 100 + j); });
+    CHECK(de::Memcpy(S, dS, de::Point2D(3, 2), de::Point2D(5, 7), de::Point2D(10, 20), de::DECX_MEMCPY_H2D).error_type == 0);
+    de::Matrix& back = de::CreateMatrixRef(de::_FP32_, 40, 50);
+    CHECK(de::Memcpy(back, dS, de::Point2D(5, 7), de::Point2D(1, 1), de::Point2D(10, 20), de::DECX_MEMCPY_D2H).error_type == 0);
+    bool same = true;
+    for (int i = 0; i < 20; ++i) for (int j = 0; j < 10; ++j) same &= (*back.ptr<float>(1 + i, 1 + j) == *S.ptr<float>(2 + i, 3 + j));
+    CHECK(same && *back.ptr<float>(0, 0) == 0.f && *back.ptr<float>(21, 11) == 0.f);
+    CHECK(de::Memcpy(S, dS, O, O, de::Point2D(41, 50), de::DECX_MEMCPY_H2D).error_type == decx::DECX_FAIL_MEMCPY_OVERRANGED);
+    CHECK(de::Memcpy(S, dS, de::Point2D(35, 0), O, de::Point2D(10, 1), de::DECX_MEMCPY_H2D).error_type == decx::DECX_FAIL_MEMCPY_OVERRANGED);
+
+    // error paths: shape, type, scalar type, unsupported type; nothing is launched
+    de::ResetLastError();
+    de::blas::cuda::GEMM(dA, dA, dD);                                   // 1005 != 1077
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_DimsNotMatching);
+    de::ResetLastError();
+    de::GPU_Matrix& dH = de::CreateGPUMatrixRef(de::_FP16_, W, L);
+    de::blas::cuda::GEMM(dA, dH, dD);
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_TYPE_MOT_MATCH);
+    de::ResetLastError();
+    de::blas::cuda::GEMM(dA, dB, dC, dD, de::Number(1.0), de::Number(1.f));    // alpha is fp64
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_TYPE_MOT_MATCH);
+    de::ResetLastError();
+    de::blas::cuda::GEMM(dA, dB, dS, dD, de::Number(1.f), de::Number(1.f));    // C has the wrong shape
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_DimsNotMatching);
+    de::ResetLastError();
+    de::GPU_Matrix& d64 = de::CreateGPUMatrixRef(de::_FP64_, 8, 8);
+    de::blas::cuda::GEMM(d64, d64, dD);
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_UNSUPPORTED_TYPE);
+    de::ResetLastError();
+    CHECK(de::Memcpy(A, dH, O, O, de::Point2D(1, 1), de::DECX_MEMCPY_H2D).error_type == decx::DECX_FAIL_TYPE_MOT_MATCH);
+    CHECK(dD.Width() == W && dD.Height() == H);                          // failed calls left dst alone
+
+    // fp16 through the objects: ones(64 x 96) . ones(96 x 32) = 96, alpha/beta as de::Half
+    de::Matrix& hA = de::CreateMatrixRef(de::_FP16_, 96, 64);
+    de::Matrix& hB = de::CreateMatrixRef(de::_FP16_, 32, 96);
+    de::Matrix& hD = de::CreateMatrixRef(de::_FP16_, 32, 64);
+    fill<de::Half>(hA, [](int, int) { de::Half h; h.val = 0x3c00; return h; });
+    fill<de::Half>(hB, [](int, int) { de::Half h; h.val = 0x3c00; return h; });
+    de::GPU_Matrix& gA = de::CreateGPUMatrixRef(de::_FP16_, 96, 64);
+    de::GPU_Matrix& gB = de::CreateGPUMatrixRef(de::_FP16_, 32, 96);
+    de::GPU_Matrix& gD = de::CreateGPUMatrixRef(de::_FP16_, 32, 64);
+    de::Memcpy(hA, gA, O, O, de::Point2D(96, 64), de::DECX_MEMCPY_H2D);
+    de::Memcpy(hB, gB, O, O, de::Point2D(32, 96), de::DECX_MEMCPY_H2D);
+    de::blas::cuda::GEMM(gA, gB, gD);
+    de::blas::cuda::GEMM(gA, gB, gD, gD, de::Number(de::Float2Half(0.5f)), de::Number(de::Float2Half(2.f)));   // 48 + 192
+    CHECK(de::GetLastError()->error_type == 0);
+    de::Memcpy(hD, gD, O, O, de::Point2D(32, 64), de::DECX_MEMCPY_D2H);
+    bool ok = true;
+    for (int i = 0; i < 64; ++i) for (int j = 0; j < 32; ++j) ok &= (de::Half2Float(*hD.ptr<de::Half>(i, j)) == 240.f);
+    CHECK(ok);
+
+    // host-matrix overload and pinned staging
+    de::Matrix& I = de::CreateMatrixRef(de::_FP32_, 50, 50);
+    fill<float>(I, [](int i, int j) { return i == j ? 1.f : 0.f; });
+    de::Matrix& R = de::CreateMatrixRef();
+    CHECK(de::cuda::PinMemory(S).error_type == 0);
+    CHECK(de::cuda::PinMemory(S).error_type == decx::DECX_FAIL_HOST_MEM_REGISTERED);
+    de::blas::cuda::GEMM(I, S, R);                                       // I(50x50) . S(50 rows x 40 cols)
+    CHECK(de::GetLastError()->error_type == 0 && R.Width() == 40 && R.Height() == 50);
+    same = true;
+    for (int i = 0; i < 50; ++i) for (int j = 0; j < 40; ++j) same &= (*R.ptr<float>(i, j) == *S.ptr<float>(i, j));
+    CHECK(same);
+    de::blas::cuda::GEMM(I, S, S, R);                                    // + C
+    same = true;
+    for (int i = 0; i < 50; ++i) for (int j = 0; j < 40; ++j) same &= (*R.ptr<float>(i, j) == 2 * *S.ptr<float>(i, j));
+    CHECK(same);
+    CHECK(de::cuda::UnpinMemory(S).error_type == 0);
+    CHECK(de::cuda::UnpinMemory(S).error_type == decx::DECX_FAIL_HOST_MEM_UNREGISTERED);
+    de::cuda::DECX_CUDA_exit();
+    return g_failures;
+}
+
+template <typename T> static bool read_into(de::Matrix& m, const std::string& path)
+{
+    std::ifstream f(path, std::ios::binary);
+    if (!f) return false;
+    for (uint32_t i = 0; i < m.Height(); ++i) f.read((char*)m.ptr<T>(i, 0), (std::streamsize)m.Width() * sizeof(T));
+    return (bool)f;
+}
+
+template <typename T> static int gemm_files(const std::string& dir, de::_DATA_TYPES_FLAGS_ ty, uint32_t M, uint32_t N,
+                                            uint32_t K, bool with_c, float alpha, float beta)
+{
+    de::InitCuda();
+    de::ResetLastError();
+    const de::Point2D O(0, 0);
+    de::Matrix& A = de::CreateMatrixRef(ty, K, M);
+    de::Matrix& B = de::CreateMatrixRef(ty, N, K);
+    de::Matrix& C = de::CreateMatrixRef(ty, N, M);
+    de::Matrix& D = de::CreateMatrixRef(ty, N, M);
+    if (!read_into<T>(A, dir + "/A.bin") || !read_into<T>(B, dir + "/B.bin")) return 2;
+    if (with_c && !read_into<T>(C, dir + "/C.bin")) return 2;
+    de::GPU_Matrix& dA = de::CreateGPUMatrixRef(ty, K, M);
+    de::GPU_Matrix& dB = de::CreateGPUMatrixRef(ty, N, K);
+    de::GPU_Matrix& dC = de::CreateGPUMatrixRef(ty, N, M);
+    de::GPU_Matrix& dD = de::CreateGPUMatrixRef(ty, N, M);
+    de::Memcpy(A, dA, O, O, de::Point2D(K, M), de::DECX_MEMCPY_H2D);
+    de::Memcpy(B, dB, O, O, de::Point2D(N, K), de::DECX_MEMCPY_H2D);
+    if (with_c) {
+        de::Memcpy(C, dC, O, O, de::Point2D(N, M), de::DECX_MEMCPY_H2D);
+        if (ty == de::_FP32_) de::blas::cuda::GEMM(dA, dB, dC, dD, de::Number(alpha), de::Number(beta));
+        else de::blas::cuda::GEMM(dA, dB, dC, dD, de::Number(de::Float2Half(alpha)), de::Number(de::Float2Half(beta)));
+    } else {
+        de::blas::cuda::GEMM(dA, dB, dD);
+    }
+    if (de::GetLastError()->error_type != 0) { std::cerr << de::GetLastError()->error_string << "\n"; return 3; }
+    de::Memcpy(D, dD, O, O, de::Point2D(N, M), de::DECX_MEMCPY_D2H);
+    std::ofstream out(dir + "/D.bin", std::ios::binary);
+    for (uint32_t i = 0; i < M; ++i) out.write((const char*)D.ptr<T>(i, 0), (std::streamsize)N * sizeof(T));
+    return out ? 0 : 2;
+}
+
+int main(int argc, char** argv)
+{
+    const std::string mode = argc > 1 ? argv[1] : "host";
+    int rc;
+    if (mode == "host") rc = host_checks();
+    else if (mode == "gpu") rc = gpu_checks();
+    else if (mode == "gemm" && argc == 10) {
+        const bool f16 = std::string(argv[3]) == "f16";
+        const uint32_t M = std::atoi(argv[4]), N = std::atoi(argv[5]), K = std::atoi(argv[6]);
+        const bool with_c = std::atoi(argv[7]) != 0;
+        const float alpha = (float)std::atof(argv[8]), beta = (float)std::atof(argv[9]);
+        rc = f16 ? gemm_files<de::Half>(argv[2], de::_FP16_, M, N, K, with_c, alpha, beta)
+                 : gemm_files<float>(argv[2], de::_FP32_, M, N, K, with_c, alpha, beta);
+    } else {
+        std::cerr << "usage: de_api_test host | gpu | gemm <dir> <f32|f16> M N K withC alpha beta\n";
+        return 64;
+    }
+    std::cout << (rc == 0 ? "de_api_test: all checks passed" : "de_api_test: FAILED") << " (" << mode << ")\n";
+    return rc;
+}

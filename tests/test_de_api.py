@@ -1,0 +1,74 @@
+"""The public C++ API (include/DECX.h) driven through tests/cpp/de_api_test, a program written
+the way the original library's sample uses it."""
+import os
+import subprocess
+import tempfile
+
+import numpy as np
+import pytest
+
+from decx_amd import synth
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EXE = os.path.join(ROOT, "tests", "cpp", "de_api_test")
+
+
+def run_exe(*args, timeout=300):
+    assert os.path.exists(EXE), "tests/cpp/de_api_test missing: run `python -m decx_amd.build`"
+    done = subprocess.run([EXE] + [str(a) for a in args], stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                          text=True, timeout=timeout)
+    return done.returncode, done.stdout
+
+
+def test_host_side_objects_and_error_codes():
+    rc, out = run_exe("host")
+    assert rc == 0, out
+
+
+def test_host_library_exports_the_public_entry_points():
+    lib = os.path.join(ROOT, "decx_amd", "lib", "libDECX_BLAS_HIP.so")
+    syms = subprocess.run(["nm", "-D", "-C", "--defined-only", lib], stdout=subprocess.PIPE, text=True).stdout
+    for needle in ["de::blas::cuda::GEMM(de::GPU_Matrix&, de::GPU_Matrix&, de::GPU_Matrix&)",
+                   "de::blas::cuda::GEMM(de::GPU_Matrix&, de::GPU_Matrix&, de::GPU_Matrix&, de::GPU_Matrix&, de::Number, de::Number)",
+                   "de::blas::cuda::GEMM(de::Matrix&, de::Matrix&, de::Matrix&)",
+                   "de::CreateGPUMatrixRef(de::_DATA_TYPES_FLAGS_, unsigned int, unsigned int, de::_DATA_FORMATS_)",
+                   "de::CreateMatrixRef(de::_DATA_TYPES_FLAGS_, unsigned int, unsigned int, de::_DATA_FORMATS_)",
+                   "de::Memcpy(de::Matrix&, de::GPU_Matrix&, de::Point2D, de::Point2D, de::Point2D, int)",
+                   "de::GetLastError()", "de::InitCuda()", "de::Float2Half(float const&)",
+                   "de::cuda::PinMemory(de::Matrix&)"]:
+        assert needle in syms, needle
+
+
+@pytest.mark.gpu
+def test_gpu_side_closed_forms_and_error_paths():
+    rc, out = run_exe("gpu")
+    assert rc == 0, out
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt,M,N,K,with_c,alpha,beta", [
+    ("f32", 1000, 1500, 777, False, 1.0, 1.0),
+    ("f32", 1000, 1500, 777, True, 1.0, 1.0),
+    ("f32", 300, 1, 500, True, -0.5, 2.0),          # N == 1: the row-dot path behind the same entry point
+    ("f16", 257, 130, 515, False, 1.0, 1.0),
+    ("f16", 257, 130, 515, True, 1.5, -0.5),
+])
+def test_gemm_through_the_objects_matches_oracle(oracle, dt, M, N, K, with_c, alpha, beta):
+    if dt == "f32":
+        A = synth.uniform_f32(M, K, 201); B = synth.uniform_f32(K, N, 202); C = synth.uniform_f32(M, N, 203)
+    else:
+        A = synth.normal_half(M, K, 201); B = synth.normal_half(K, N, 202); C = synth.normal_half(M, N, 203)
+    with tempfile.TemporaryDirectory() as tmp:
+        A.tofile(os.path.join(tmp, "A.bin")); B.tofile(os.path.join(tmp, "B.bin")); C.tofile(os.path.join(tmp, "C.bin"))
+        rc, out = run_exe("gemm", tmp, dt, M, N, K, int(with_c), alpha, beta)
+        assert rc == 0, out
+        D = np.fromfile(os.path.join(tmp, "D.bin"), A.dtype).reshape(M, N)
+    if dt == "f32":
+        ref = oracle.gemm_f32(A, B, C, alpha, beta) if with_c else oracle.gemm_f32(A, B)
+        tol = 1e-5
+    else:
+        ref = oracle.gemm_f16(A, B, C if with_c else None, alpha, beta)
+        tol = 2e-3
+    ref = ref.astype(np.float64)
+    err = np.max(np.abs(D.astype(np.float64) - ref)) / (np.max(np.abs(ref)) * np.sqrt(K))
+    assert err <= tol
