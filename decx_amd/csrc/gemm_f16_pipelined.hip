@@ -1,5 +1,7 @@
-// fp16 GEMM, the full-tile fast path for gfx950: 256 x 256 block tile, K slabs of 64,
-// global -> LDS by direct (LDS-DMA) 128-bit loads, B fragments by the transposing LDS read.
+// fp16 GEMM, the full-tile fast path for gfx950: 256 x 256 block tile, global -> LDS by
+// direct (LDS-DMA) 128-bit loads, B fragments by the transposing LDS read, and a hand-ordered
+// instruction stream in which every MFMA is followed by the LDS reads / direct loads that
+// should issue in its shadow.
 //
 // Why this shape.  v_mfma_f32_32x32x16_f16 takes 8 consecutive k per lane for BOTH
 // operands.  A (row-major M x K) has them contiguous.  B (row-major K x N) does not, and
@@ -15,18 +17,29 @@
 //     a lane needs.
 // Bank conflicts are removed by permuting 16-byte chunks inside each row -- done on the
 // global side of the copy, since the LDS side of a direct load is fixed:
-//   A slab  [256 rows][8 chunks]   chunk c of row r sits in slot c ^ ((r >> 1) & 7)
-//   B slab  [64 k-rows][32 chunks] chunk c of row k sits in slot c ^ (4 * (k & 3))
+//   A slab  [256 rows][CPR chunks]  chunk c of row r sits in slot c ^ ((r / RPB) % CPR)
+//   B slab  [BK k-rows][32 chunks]  chunk c of row k sits in slot c ^ (4 * (k & 3))
 // With these, 16 lanes reading one k-chunk of 16 consecutive A rows, and 32 lanes reading
 // four k-rows of B through the transposing read, each touch every bank exactly once.
 //
-// Pipeline: two LDS stages of 64 KB.  While slab s is multiplied, the direct loads of
-// slab s+1 are in flight into the other stage; one `s_waitcnt vmcnt(0)` + barrier per
-// slab.  Inside a slab the fragments of k-step i+1 are fetched while the 16 MFMAs of
-// k-step i run (two register sets).  4 wavefronts, each a 128 x 128 tile = 256 accumulator
-// registers; one workgroup per CU.
+// The MFMA is issued with its operands swapped (B fragment first): it then produces the
+// transposed 32x32 tile, in which a lane owns 4 *adjacent columns* of one output row per
+// register group, so the epilogue stores 8 bytes per lane instead of 2.
+//
+// Pipeline.  STAGES LDS stages of one K slab each.  The k-steps of all slabs form one
+// sequence of phases; phase p issues the 16 MFMAs of k-step p and, interleaved behind
+// them, the 12 fragment reads of k-step p+1 (two register sets) and 4 direct loads.  A
+// stage is free as soon as the fragments of its last k-step are in registers, so slab
+// s + STAGES is fetched from the last phase of slab s on; one wait + barrier per slab,
+// placed before that last phase.  Three things are taken out of the compiler's hands:
+// the direct loads are inline assembly (otherwise it puts `s_waitcnt vmcnt(0)` in front of
+// every LDS read that follows one, because it cannot prove the stages do not alias); the
+// barrier is a bare `s_barrier` with an explicit vmcnt wait (__syncthreads() drains all
+// loads); and `sched_group_barrier` pins the MFMA / LDS-read interleave (left alone it
+// issues all reads of a k-step in a clump in front of the MFMAs).
 #include "gemm_common.hpp"
 #include <cstdlib>
+#include <type_traits>
 
 namespace decx_hip {
 
@@ -46,18 +59,23 @@ __device__ __forceinline__ halfx8 join(shortx4 lo, shortx4 hi)
     return u.v;
 }
 
-// Waits until at most N of this wave's direct loads are still in flight, and until its LDS
-// reads have returned, then joins the workgroup barrier.  Deliberately not __syncthreads():
-// that carries a fence which drains every outstanding load and would undo the prefetch.
+#define DECX_DMA16(lds_dst, gptr) \
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(lds_dst), "v"(gptr) : "memory", "m0")
+
+// Waits until at most N of this wave's direct loads are in flight and all its LDS reads have
+// returned, then joins the workgroup barrier.  Not __syncthreads(): that carries a fence
+// which drains every outstanding load and would undo the prefetch.
 template <int N> __device__ __forceinline__ void wait_loads_and_barrier()
 {
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(N) : "memory");
 }
 
+// scheduling-group masks of __builtin_amdgcn_sched_group_barrier
+constexpr int SG_MFMA = 0x008, SG_DS_READ = 0x100;
+
 }  // namespace
 
-// BK: slab depth (32 or 64).  STAGES: LDS stages; slab s+STAGES-1 is fetched while slab s is
-// multiplied, so a direct load has (STAGES-1) slabs of MFMA time to land.
+// BK: slab depth (32 or 64).  STAGES: LDS stages.
 template <int BK, int STAGES>
 __global__ void __launch_bounds__(NT)
 gemm_f16_pipelined_kernel(const GemmArgs g)
@@ -71,11 +89,14 @@ gemm_f16_pipelined_kernel(const GemmArgs g)
     constexpr int A_LOADS = A_STAGE_BYTES / 1024 / 4;   // direct-load instructions per wave per slab
     constexpr int B_LOADS = B_STAGE_BYTES / 1024 / 4;
     constexpr int LOADS = A_LOADS + B_LOADS;
-    constexpr int KS = BK / 16;                      // MFMA k-steps per slab
+    constexpr int KS = BK / 16;                      // MFMA k-steps (= phases) per slab
+    constexpr int DMA_PER_PHASE = LOADS / KS;        // 4
     static_assert(STAGES >= 2 && STAGES * STAGE_BYTES <= 160 * 1024, "LDS budget");
     static_assert(LOADS * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
+    static_assert(KS % 2 == 0 && DMA_PER_PHASE == 4 && A_LOADS % DMA_PER_PHASE == 0, "phase plan");
 
     __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE_BYTES];
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)lds;
 
     uint32_t tile_m, tile_n;
     block_to_tile(g, tile_m, tile_n);
@@ -92,8 +113,6 @@ gemm_f16_pipelined_kernel(const GemmArgs g)
     // ---- global -> LDS copy plan.
     // A instruction I covers rows (64/CPR)*I ..: lane -> row (64/CPR)*I + lane/CPR, slot lane%CPR.
     // B instruction I covers k-rows 2I, 2I+1:    lane -> k 2I + lane/32, slot lane%32.
-    // Chunk permutation (see the file header): A slot = chunk ^ ((row / RPB) % CPR),
-    // B slot = chunk ^ (4 * (k & 3)).
     const unsigned char* a_src[A_LOADS];
     const unsigned char* b_src[B_LOADS];
 #pragma unroll
@@ -111,27 +130,28 @@ gemm_f16_pipelined_kernel(const GemmArgs g)
         b_src[i] = B + (size_t)k * ldb_b + (size_t)n0 * 2 + bchunk * 16;
     }
 
-    // The direct loads are issued from inline assembly on purpose: the compiler's wait-count
-    // pass cannot tell that a load into one LDS stage does not alias a read of another
-    // and would put `s_waitcnt vmcnt(0)` in front of every fragment read, serialising the
-    // copy with the arithmetic.  M0 carries the wave-uniform LDS destination.
-    auto issue_loads = [&](uint32_t slab) {
-        const uint32_t stage = slab % STAGES;
-        const uint32_t sa = stage * STAGE_BYTES;
-        const uint32_t sb = sa + A_STAGE_BYTES;
-        const uint32_t k0 = slab * BK;
-#pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) {
-            const uint32_t dst = __builtin_amdgcn_readfirstlane(sa + (uint32_t)(wave * A_LOADS + i) * 1024u);
-            const unsigned char* src = a_src[i] + (size_t)k0 * 2;
-            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
+    // One direct load: index q in [0, LOADS) of slab `slab` (A instructions first).
+    auto dma = [&](uint32_t slab, auto qc) {
+        constexpr int q = decltype(qc)::value;
+        const uint32_t stage_off = lds_base + (slab % STAGES) * STAGE_BYTES;
+        if constexpr (q < A_LOADS) {
+            const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + (uint32_t)(wave * A_LOADS + q) * 1024u);
+            const unsigned char* src = a_src[q] + (size_t)slab * (BK * 2);
+            DECX_DMA16(dst, src);
+        } else {
+            constexpr int qb = q - A_LOADS;
+            const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + A_STAGE_BYTES +
+                                                                (uint32_t)(wave * B_LOADS + qb) * 1024u);
+            const unsigned char* src = b_src[qb] + (size_t)slab * BK * ldb_b;
+            DECX_DMA16(dst, src);
         }
-#pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) {
-            const uint32_t dst = __builtin_amdgcn_readfirstlane(sb + (uint32_t)(wave * B_LOADS + i) * 1024u);
-            const unsigned char* src = b_src[i] + (size_t)k0 * ldb_b;
-            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
-        }
+    };
+    auto dma_batch = [&](uint32_t slab, auto bc) {       // batch b of KS: loads 4b .. 4b+3
+        constexpr int b = decltype(bc)::value;
+        dma(slab, std::integral_constant<int, 4 * b + 0>{});
+        dma(slab, std::integral_constant<int, 4 * b + 1>{});
+        dma(slab, std::integral_constant<int, 4 * b + 2>{});
+        dma(slab, std::integral_constant<int, 4 * b + 3>{});
     };
 
     // ---- fragment addressing (byte offsets inside a stage)
@@ -147,89 +167,162 @@ gemm_f16_pipelined_kernel(const GemmArgs g)
     const int b_krow = 8 * h + (s16 >> 2);                    // + 16 ks + 4 r
     const int b_col = wn0 + 16 * ((lane >> 4) & 1) + 4 * (s16 & 3);   // + 32 j ; in halves
     const int b_sw = 4 * (b_krow & 3);                        // k & 3 is unchanged by + 16 ks + 4 r
-
-    auto load_frags = [&](uint32_t stage, int ks, halfx8 (&af)[4], halfx8 (&bf)[4]) {
-        const unsigned char* sa = lds + stage * STAGE_BYTES;
-        const unsigned char* sb = sa + A_STAGE_BYTES;
+    int b_off[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            af[i] = *(const halfx8*)(sa + a_off + i * 32 * RB + (((2 * ks + h) ^ a_sw) * 16));
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int col = b_col + 32 * j;                    // halves
-            const int chunk = (col >> 3) ^ b_sw;
-            const int within = (col & 7) * 2;                  // bytes inside the 16-byte chunk (0 or 8)
-            const unsigned char* p0 = sb + (16 * ks + b_krow) * 512 + chunk * 16 + within;
-            const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)p0);
-            const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(p0 + 4 * 512));
-            bf[j] = join(lo, hi);
-        }
-    };
-
-    floatx16 acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-    auto multiply = [&](const halfx8 (&af)[4], const halfx8 (&bf)[4]) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
-    };
-
-    // Software pipeline.  Every phase = "fetch the next fragments, then issue 16 MFMAs on
-    // the current ones"; sched_barrier pins that order so the LDS latency of a fetch hides
-    // behind the 512 cycles of MFMA issue of the phase before it.  The last phase of a slab
-    // is multiplied after the barrier, under the first fetch of the next slab.
-    const uint32_t slabs = g.K / BK;
-#pragma unroll
-    for (int p = 0; p < STAGES - 1; ++p)
-        if ((uint32_t)p < slabs) issue_loads(p);
-    if (slabs >= (uint32_t)(STAGES - 1)) wait_loads_and_barrier<LOADS * (STAGES - 2)>();
-    else wait_loads_and_barrier<0>();
-
-    halfx8 afx[4], bfx[4], afy[4], bfy[4];
-    for (uint32_t s = 0; s < slabs; ++s) {
-        const uint32_t stage = s % STAGES;
-        const bool more = s + STAGES - 1 < slabs;
-        // the stage that held slab s-1 is free: every wave passed the barrier after reading it
-        if (more) issue_loads(s + STAGES - 1);
-#pragma unroll
-        for (int ks = 0; ks < KS; ks += 2) {
-            load_frags(stage, ks, afx, bfx);
-            __builtin_amdgcn_sched_barrier(0);
-            if (s > 0 || ks > 0) multiply(afy, bfy);           // the k-step before this one
-            __builtin_amdgcn_sched_barrier(0);
-            load_frags(stage, ks + 1, afy, bfy);
-            __builtin_amdgcn_sched_barrier(0);
-            multiply(afx, bfx);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        // slab s+1 must have landed (ours: vmcnt; everyone's: barrier).  Loads of the
-        // STAGES-2 slabs after it may stay in flight.
-        if (more) wait_loads_and_barrier<LOADS * (STAGES - 2)>(); else wait_loads_and_barrier<0>();
+    for (int j = 0; j < 4; ++j) {
+        const int col = b_col + 32 * j;
+        b_off[j] = A_STAGE_BYTES + b_krow * 512 + (((col >> 3) ^ b_sw) * 16) + (col & 7) * 2;
     }
-    multiply(afy, bfy);
 
-    // Epilogue: register r of lane (l32, h) is row 8*(r/4) + 4*h + r%4, column l32 of a tile.
+    struct Frags { halfx8 a[4], b[4]; };
+
+    auto read_a = [&](Frags& f, const unsigned char* st, int ks, int i) {
+        f.a[i] = *(const halfx8*)(st + a_off + i * 32 * RB + (((2 * ks + h) ^ a_sw) * 16));
+    };
+    auto read_b = [&](Frags& f, const unsigned char* st, int ks, int j) {
+        const unsigned char* p0 = st + b_off[j] + ks * 16 * 512;
+        const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)p0);
+        const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(p0 + 4 * 512));
+        f.b[j] = join(lo, hi);
+    };
+
+    // accT[j][i]: n-tile j, m-tile i, held transposed (see the file header)
+    floatx16 accT[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) accT[j][i][r] = 0.f;
+
+    auto mfma4 = [&](const Frags& cur, int j) {           // the 4 MFMAs of n-tile j
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            accT[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cur.b[j], cur.a[i], accT[j][i], 0, 0, 0);
+    };
+
+    // One phase: the 16 MFMAs of the current k-step, the 12 fragment reads of the next
+    // k-step (8 LDS instructions for B, 4 for A) spread behind them, and -- if `dma_ok` --
+    // one direct load in front of each quarter.  Source order = intended issue order; the
+    // group barriers make the scheduler keep the "one MFMA, one LDS read" alternation.
+    // Only the direct loads are conditional (tiny uniform branches): the arithmetic is
+    // never duplicated, so the 256 accumulators stay put.
+    auto quarter = [&](bool dma_ok, uint32_t dma_slab, auto qc) {
+        if (dma_ok) dma(dma_slab, qc);
+    };
+    auto phase = [&](const Frags& cur, Frags& nxt, const unsigned char* nst, int nks,
+                     bool dma_ok, uint32_t dma_slab, auto dbc) {
+        constexpr int db = decltype(dbc)::value;
+        quarter(dma_ok, dma_slab, std::integral_constant<int, 4 * db + 0>{});
+        read_b(nxt, nst, nks, 0); read_a(nxt, nst, nks, 0);
+        mfma4(cur, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        quarter(dma_ok, dma_slab, std::integral_constant<int, 4 * db + 1>{});
+        read_a(nxt, nst, nks, 1); read_a(nxt, nst, nks, 2); read_a(nxt, nst, nks, 3);
+        mfma4(cur, 1);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        quarter(dma_ok, dma_slab, std::integral_constant<int, 4 * db + 2>{});
+        read_b(nxt, nst, nks, 1); read_b(nxt, nst, nks, 2);
+        mfma4(cur, 2);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
+        quarter(dma_ok, dma_slab, std::integral_constant<int, 4 * db + 3>{});
+        read_b(nxt, nst, nks, 3);
+        mfma4(cur, 3);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 2, 0);
+    };
+    auto I0 = std::integral_constant<int, 0>{};
+
+    const uint32_t slabs = g.K / BK;
+
+    // ---- prologue: slabs 0 .. STAGES-2 entirely, plus the first batch of slab STAGES-1
+    // (its other batches are issued by phases 0 .. KS-2 of slab 0).
+#pragma unroll
+    for (int p = 0; p < STAGES - 1; ++p) {
+        if ((uint32_t)p < slabs) {
+            dma_batch(p, std::integral_constant<int, 0>{});
+            dma_batch(p, std::integral_constant<int, 1>{});
+            if constexpr (KS == 4) {
+                dma_batch(p, std::integral_constant<int, 2>{});
+                dma_batch(p, std::integral_constant<int, 3>{});
+            }
+        }
+    }
+    if ((uint32_t)(STAGES - 1) < slabs) dma_batch(STAGES - 1, std::integral_constant<int, 0>{});
+    wait_loads_and_barrier<0>();
+
+    Frags f0, f1;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) { read_a(f0, lds, 0, q); read_b(f0, lds, 0, q); }
+
+    for (uint32_t s = 0; s < slabs; ++s) {
+        const unsigned char* st = lds + (s % STAGES) * STAGE_BYTES;
+        const unsigned char* st_next = lds + ((s + 1) % STAGES) * STAGE_BYTES;
+        const bool dma_mid = s + STAGES - 1 < slabs;          // slab s+STAGES-1 exists (its batches 1..KS-1)
+        const bool dma_last = s + STAGES < slabs;             // slab s+STAGES exists (its batch 0)
+
+        // phases 0 .. KS-2: fetch k-step ks+1 of this slab
+        phase(f0, f1, st, 1, dma_mid, s + STAGES - 1, std::integral_constant<int, 1>{});
+        if constexpr (KS == 4) {
+            phase(f1, f0, st, 2, dma_mid, s + STAGES - 1, std::integral_constant<int, 2>{});
+            phase(f0, f1, st, 3, dma_mid, s + STAGES - 1, std::integral_constant<int, 3>{});
+        }
+
+        // Last phase of the slab.  Its fragments are in registers (lgkmcnt(0) in the wait), so
+        // every wave is done with this stage; slab s+1 must have landed: ours by vmcnt,
+        // everyone's by the barrier.  Loads of the STAGES-2 slabs behind it may stay in flight.
+        // It fetches k-step 0 of the next slab; after the final slab that read returns stale
+        // LDS contents which nothing uses.
+        if (dma_mid) wait_loads_and_barrier<LOADS * (STAGES - 2)>(); else wait_loads_and_barrier<0>();
+        phase(f1, f0, st_next, 0, dma_last, s + STAGES, I0);
+    }
+
+    // Epilogue.  Transposed tile layout: lane (l32, h) holds output row l32 of the m-tile;
+    // register 4 q + e is column 8 q + 4 h + e of the n-tile.
     const _Float16* __restrict__ C = (const _Float16*)g.C;
     _Float16* __restrict__ D = (_Float16*)g.D;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
+        const uint32_t row = m0 + wm0 + 32 * i + l32;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const uint32_t row = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+        for (int j = 0; j < 4; ++j) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t col = n0 + wn0 + 32 * j + l32;
-                float o = acc[i][j][r];
-                if (C) o = __builtin_fmaf((float)C[(size_t)row * g.ldc + col], g.beta, g.alpha * o);
-                D[(size_t)row * g.ldd + col] = (_Float16)o;
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t col = n0 + wn0 + 32 * j + 8 * q + 4 * h;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = accT[j][i][4 * q + e];
+                if (C) {
+                    const halfx4 cv = *(const halfx4*)(C + (size_t)row * g.ldc + col);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf((float)cv[e], g.beta, g.alpha * v[e]);
+                }
+                halfx4 out;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out[e] = (_Float16)v[e];
+                *(halfx4*)(D + (size_t)row * g.ldd + col) = out;
             }
         }
     }
