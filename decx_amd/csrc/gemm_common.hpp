@@ -82,6 +82,8 @@ __host__ inline TileInfo tile_info_f16(int shape)
 }
 
 int launch_gemm_f32(int shape, bool edge, const GemmArgs& args, hipStream_t stream);
+// 256 x 256 x 16 direct-to-LDS fp32 kernel; full tiles only (the caller checks divisibility and alignment)
+int launch_gemm_f32_pipelined(const GemmArgs& args, hipStream_t stream);
 int launch_gemm_f16(int shape, bool edge, const GemmArgs& args, hipStream_t stream);
 // 256 x 256 x 64 direct-to-LDS kernel; full tiles only (the caller checks divisibility and alignment)
 int launch_gemm_f16_pipelined(const GemmArgs& args, hipStream_t stream);

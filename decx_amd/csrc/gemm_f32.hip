@@ -24,7 +24,17 @@
 // do (GEMM_fp32_B128_kernels.cu:725-744).
 #include "gemm_common.hpp"
 
+#include <type_traits>
+
 namespace decx_hip {
+
+template <int I, int N, class F> __device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
 
 template <int TN> struct BFrag;
 template <> struct BFrag<1> { typedef float type; };
@@ -142,24 +152,43 @@ gemm_f32_kernel(const GemmArgs g)
         const int buf = s & 1;
         if (s + 1 < slabs) load_slab((s + 1) * BK);
 
+        // The slab is walked in k steps of 2 (one MFMA per tile each).  Fragments are fetched
+        // one step ahead into a second register set, and the group barriers keep every LDS
+        // read directly behind the first MFMA of the step before it, so its latency is
+        // covered by the remaining MFMAs instead of stalling the matrix pipe once per step.
         const float* a_base = As + buf * A_STAGE + (wm0 + l32) * A_STRIDE + 4 * h;
         const float* b_base = Bs + buf * B_STAGE + (4 * h) * BN + wn0 + TN * l32;
+        constexpr int STEPS = BK / 2, CHUNKS = BK / 8;
+        floatx4 af[2][TM];
+        bvec bf[2];
 #pragma unroll
-        for (int c = 0; c < BK / 8; ++c) {
-            floatx4 af[TM];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) af[i] = *(const floatx4*)(a_base + i * 32 * A_STRIDE + 8 * c);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const bvec bf = *(const bvec*)(b_base + (8 * c + e) * BN);
+        for (int i = 0; i < TM; ++i) af[0][i] = *(const floatx4*)(a_base + i * 32 * A_STRIDE);
+        bf[0] = *(const bvec*)(b_base);
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<0, STEPS>([&](auto stc) {
+            constexpr int st = decltype(stc)::value;
+            constexpr int c = st / 4, e = st % 4;
+            constexpr bool next_b = st + 1 < STEPS;
+            constexpr bool next_a = (e == 1) && (c + 1 < CHUNKS);
+            constexpr int reads = (next_b ? 1 : 0) + (next_a ? TM : 0);
+            if constexpr (next_b)
+                bf[(st + 1) & 1] = *(const bvec*)(b_base + (8 * ((st + 1) / 4) + (st + 1) % 4) * BN);
+            if constexpr (next_a) {
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][e], bfrag_get<TN>(bf, j),
-                                                                         acc[i][j], 0, 0, 0);
+                    af[(c + 1) & 1][i] = *(const floatx4*)(a_base + i * 32 * A_STRIDE + 8 * (c + 1));
             }
-        }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c & 1][i][e], bfrag_get<TN>(bf[st & 1], j),
+                                                                     acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                          // one MFMA
+            if constexpr (reads > 0) __builtin_amdgcn_sched_group_barrier(0x100, reads, 0);   // this step's LDS reads
+            if constexpr (TM * TN > 1) __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 1, 0);   // the other MFMAs
+            __builtin_amdgcn_sched_barrier(0);                                          // steps stay in order
+        });
 
         if (s + 1 < slabs) store_slab(buf ^ 1);
         __syncthreads();
@@ -226,6 +255,9 @@ static int launch_shape(bool edge, const GemmArgs& args, hipStream_t stream)
 
 int launch_gemm_f32(int shape, bool edge, const GemmArgs& args, hipStream_t stream)
 {
+    if (shape == TILE_256x256 && !edge && args.vec_ok && args.K > 0 &&
+        args.M % 256 == 0 && args.N % 256 == 0 && args.K % 16 == 0)
+        return launch_gemm_f32_pipelined(args, stream);
     switch (shape) {
     case TILE_256x256: return launch_shape<256, 256, 16, 4, 2>(edge, args, stream);
     case TILE_128x128: return launch_shape<128, 128, 16, 2, 2>(edge, args, stream);
