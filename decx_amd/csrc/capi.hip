@@ -254,8 +254,8 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
     const bool f16 = elem_bytes == 2;
     if (!f16 && N == 1 && K > 0) {
         out->path = DECX_HIP_PATH_GEMV;
-        out->tile_m = 8; out->tile_n = 1;
-        out->grid = (M + 7) / 8;
+        out->tile_m = 32; out->tile_n = 1;
+        out->grid = (M + 31) / 32;
         return DECX_HIP_OK;
     }
     const int shape = choose_tile(f16, M, N);

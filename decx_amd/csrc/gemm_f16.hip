@@ -74,13 +74,19 @@ gemm_f16_kernel(const GemmArgs g)
         return v;
     };
 
+    // Interior tiles and interior slabs of the predicated variant skip the per-element guards
+    // (uniform tests, scalar branches).
+    const bool rows_inside = g.vec_ok && (m0 + BM <= g.M);
+    const bool cols_inside = g.vec_ok && (n0 + BN <= g.N);
+
     auto load_slab = [&](uint32_t k0) {
+        const bool k_inside = k0 + BK <= g.K;
 #pragma unroll
         for (int i = 0; i < A_PER; ++i) {
             const int q = t + i * NT;
             const uint32_t gm = m0 + q / (BK / 8), gk = k0 + (q % (BK / 8)) * 8;
             const uint16_t* p = A + (size_t)gm * g.lda + gk;
-            if constexpr (!EDGE) ra[i] = *(const uintx4*)p;
+            if (!EDGE || (rows_inside && k_inside)) ra[i] = *(const uintx4*)p;
             else {
                 uintx4 v = {0u, 0u, 0u, 0u};
                 if (gm < g.M) v = load8(p, gk, g.K);
@@ -94,7 +100,7 @@ gemm_f16_kernel(const GemmArgs g)
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
                 const uint16_t* p = B + (size_t)(gk + r) * g.ldb + gn;
-                if constexpr (!EDGE) rb[i][r] = *(const uintx4*)p;
+                if (!EDGE || (cols_inside && k_inside)) rb[i][r] = *(const uintx4*)p;
                 else {
                     uintx4 v = {0u, 0u, 0u, 0u};
                     if (gk + r < g.K) v = load8(p, gn, g.N);
@@ -181,7 +187,7 @@ gemm_f16_kernel(const GemmArgs g)
             float v[TN];
 #pragma unroll
             for (int j = 0; j < TN; ++j) v[j] = acc[i][j][r];
-            if constexpr (!EDGE && TN > 1) {
+            if (TN > 1 && (!EDGE || (rows_inside && cols_inside))) {
                 if (C) {
                     const hvec cv = *(const hvec*)(C + (size_t)row * g.ldc + col0);
 #pragma unroll

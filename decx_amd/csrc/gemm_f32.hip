@@ -77,13 +77,20 @@ gemm_f32_kernel(const GemmArgs g)
 
     floatx4 ra[A_PER], rb[B_PER];
 
+    // In the predicated variant most of the work is still interior: a tile that lies fully
+    // inside M (or N) and a slab that lies fully inside K need no per-element guards.  These
+    // tests are uniform over the workgroup, so they cost a scalar branch.
+    const bool rows_inside = g.vec_ok && (m0 + BM <= g.M);
+    const bool cols_inside = g.vec_ok && (n0 + BN <= g.N);
+
     auto load_slab = [&](uint32_t k0) {
+        const bool k_inside = k0 + BK <= g.K;
 #pragma unroll
         for (int i = 0; i < A_PER; ++i) {
             const int q = t + i * NT;
             const uint32_t gm = m0 + q / (BK / 4), gk = k0 + (q % (BK / 4)) * 4;
             const float* p = A + (size_t)gm * g.lda + gk;
-            if constexpr (!EDGE) {
+            if (!EDGE || (rows_inside && k_inside)) {
                 ra[i] = *(const floatx4*)p;
             } else {
                 floatx4 v = {0.f, 0.f, 0.f, 0.f};
@@ -104,7 +111,7 @@ gemm_f32_kernel(const GemmArgs g)
             const int q = t + i * NT;
             const uint32_t gk = k0 + q / (BN / 4), gn = n0 + (q % (BN / 4)) * 4;
             const float* p = B + (size_t)gk * g.ldb + gn;
-            if constexpr (!EDGE) {
+            if (!EDGE || (cols_inside && k_inside)) {
                 rb[i] = *(const floatx4*)p;
             } else {
                 floatx4 v = {0.f, 0.f, 0.f, 0.f};
@@ -207,7 +214,7 @@ gemm_f32_kernel(const GemmArgs g)
             float v[TN];
 #pragma unroll
             for (int j = 0; j < TN; ++j) v[j] = acc[i][j][r];
-            if constexpr (!EDGE) {
+            if (!EDGE || (rows_inside && cols_inside)) {
                 if (C) {
                     const bvec cv = *(const bvec*)(C + (size_t)row * g.ldc + col0);
 #pragma unroll

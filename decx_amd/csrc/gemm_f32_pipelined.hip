@@ -17,6 +17,7 @@
 //     explicit vmcnt wait, because the compiler would otherwise wait for every outstanding
 //     load in front of each LDS read and at each __syncthreads().
 #include "gemm_common.hpp"
+#include <cstdlib>
 #include <type_traits>
 
 namespace decx_hip {
@@ -130,48 +131,67 @@ gemm_f32_pipelined_kernel(const GemmArgs g)
     if (slabs >= (uint32_t)(STAGES - 1)) wait_loads_and_barrier<LOADS * (STAGES - 2)>();
     else wait_loads_and_barrier<0>();
 
+    // Fragment registers: af[c & 1] holds chunk c of A (4 k per lane), bf[step & 1] the B values
+    // of a k step.  The MFMAs of the last step of a slab are issued after the slab barrier,
+    // behind the first fragment reads of the next slab, so the matrix pipe has work while
+    // those reads are in flight (before the first slab they multiply zeros).
+    constexpr int STEPS = BK / 2, CHUNKS = BK / 8;
+    floatx4 af[2][TM];
+    floatx4 bf[2];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) af[(CHUNKS - 1) & 1][i] = floatx4{0.f, 0.f, 0.f, 0.f};
+    bf[(STEPS - 1) & 1] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    auto multiply = [&](auto stc) {
+        constexpr int step = decltype(stc)::value;
+        constexpr int c = step / 4, e = step % 4;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c & 1][i][e], bf[step & 1][j], acc[i][j], 0, 0, 0);
+    };
+
     for (uint32_t s = 0; s < slabs; ++s) {
         const unsigned char* st = lds + (s % STAGES) * STAGE_BYTES;
         const bool more = s + STAGES - 1 < slabs;
-        // the stage that held slab s-1 is free: every wave passed the barrier after reading it
-        if (more) issue_loads(s + STAGES - 1);
 
-        // k steps of 2; fragments fetched one step ahead, each LDS read pinned behind the
-        // first MFMA of the step before the one that uses it
-        constexpr int STEPS = BK / 2, CHUNKS = BK / 8;
-        floatx4 af[2][TM];
-        floatx4 bf[2];
+        // first fragments of this slab, then the deferred last step of the previous one
 #pragma unroll
         for (int i = 0; i < TM; ++i) af[0][i] = *(const floatx4*)(st + a_off[0] + i * 32 * 64);
         bf[0] = *(const floatx4*)(st + b_off);
+        multiply(std::integral_constant<int, STEPS - 1>{});
+        __builtin_amdgcn_sched_group_barrier(0x100, TM + 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
         __builtin_amdgcn_sched_barrier(0);
-        static_for<0, STEPS>([&](auto stc) {
+        // the stage that held slab s-1 is free: every wave passed the barrier after reading it
+        if (more) issue_loads(s + STAGES - 1);
+
+        // steps 0 .. STEPS-2: fragments fetched one step ahead, each LDS read pinned behind
+        // the first MFMA of the step before the one that uses it
+        static_for<0, STEPS - 1>([&](auto stc) {
             constexpr int step = decltype(stc)::value;
             constexpr int c = step / 4, e = step % 4;
-            constexpr bool next_b = step + 1 < STEPS;
             constexpr bool next_a = (e == 1) && (c + 1 < CHUNKS);
-            constexpr int reads = (next_b ? 1 : 0) + (next_a ? TM : 0);
-            if constexpr (next_b)
-                bf[(step + 1) & 1] = *(const floatx4*)(st + b_off + (8 * ((step + 1) / 4) + (step + 1) % 4) * BN * 4);
+            constexpr int reads = 1 + (next_a ? TM : 0);
+            bf[(step + 1) & 1] = *(const floatx4*)(st + b_off + (8 * ((step + 1) / 4) + (step + 1) % 4) * BN * 4);
             if constexpr (next_a) {
 #pragma unroll
                 for (int i = 0; i < TM; ++i) af[(c + 1) & 1][i] = *(const floatx4*)(st + a_off[c + 1] + i * 32 * 64);
             }
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c & 1][i][e], bf[step & 1][j], acc[i][j], 0, 0, 0);
+            multiply(stc);
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if constexpr (reads > 0) __builtin_amdgcn_sched_group_barrier(0x100, reads, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, reads, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 1, 0);
             __builtin_amdgcn_sched_barrier(0);
         });
 
         // slab s+1 must have landed (ours: vmcnt; everyone's: barrier); the loads of the
-        // STAGES-2 slabs behind it may stay in flight
+        // STAGES-2 slabs behind it may stay in flight.  The fragments of the last step are in
+        // registers (lgkmcnt(0)), so the stage is free once every wave is here.
         if (more) wait_loads_and_barrier<LOADS * (STAGES - 2)>(); else wait_loads_and_barrier<0>();
     }
+    multiply(std::integral_constant<int, STEPS - 1>{});
 
     // Epilogue: register r of lane (l32, h) is row 8*(r/4) + 4*h + r%4 of a 32x32 tile; the
     // lane's TN tiles are TN adjacent columns.
@@ -205,7 +225,14 @@ int launch_gemm_f32_pipelined(const GemmArgs& args, hipStream_t stream)
     g.tiles_n = g.N / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
     g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
-    hipLaunchKernelGGL((gemm_f32_pipelined_kernel<4>), dim3(nb), dim3(NT), 0, stream, g);
+    static int variant = -1;
+    if (variant < 0) { const char* e = getenv("DECX_HIP_F32_STAGES"); variant = e ? atoi(e) : 4; }
+    switch (variant) {
+    case 3:  hipLaunchKernelGGL((gemm_f32_pipelined_kernel<3>), dim3(nb), dim3(NT), 0, stream, g); break;
+    case 5:  hipLaunchKernelGGL((gemm_f32_pipelined_kernel<5>), dim3(nb), dim3(NT), 0, stream, g); break;
+    case 2:  hipLaunchKernelGGL((gemm_f32_pipelined_kernel<2>), dim3(nb), dim3(NT), 0, stream, g); break;
+    default: hipLaunchKernelGGL((gemm_f32_pipelined_kernel<4>), dim3(nb), dim3(NT), 0, stream, g); break;
+    }
     return (int)hipGetLastError();
 }
 
