@@ -300,29 +300,46 @@ gemm_f16_pipelined_kernel(const GemmArgs g)
     }
 
     // Epilogue.  Transposed tile layout: lane (l32, h) holds output row l32 of the m-tile;
-    // register 4 q + e is column 8 q + 4 h + e of the n-tile.
+    // register 4 q + e is column 8 q + 4 h + e of the n-tile, so the two half-waves hold the
+    // two 4-column halves of every 8-column group of a row.  `v_permlane32_swap` trades the
+    // halves of an even and an odd group between lane l and lane l + 32; after it the lower
+    // lane owns all 8 columns of the even group and the upper lane those of the odd group,
+    // and each lane stores 16 bytes.
     const _Float16* __restrict__ C = (const _Float16*)g.C;
     _Float16* __restrict__ D = (_Float16*)g.D;
+    auto pack2 = [](float lo, float hi) -> uint32_t {
+        union { _Float16 f[2]; uint32_t u; } w;
+        w.f[0] = (_Float16)lo; w.f[1] = (_Float16)hi;
+        return w.u;
+    };
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const uint32_t row = m0 + wm0 + 32 * i + l32;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const uint32_t col = n0 + wn0 + 32 * j + 8 * q + 4 * h;
-                float v[4];
+            for (int qp = 0; qp < 2; ++qp) {
+                uint32_t w[2][2];                      // [even / odd group][dword]
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = accT[j][i][4 * q + e];
-                if (C) {
-                    const halfx4 cv = *(const halfx4*)(C + (size_t)row * g.ldc + col);
+                for (int o = 0; o < 2; ++o) {
+                    const int q = 2 * qp + o;
+                    float v[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf((float)cv[e], g.beta, g.alpha * v[e]);
+                    for (int e = 0; e < 4; ++e) v[e] = accT[j][i][4 * q + e];
+                    if (C) {
+                        const uint32_t col = n0 + wn0 + 32 * j + 8 * q + 4 * h;
+                        const halfx4 cv = *(const halfx4*)(C + (size_t)row * g.ldc + col);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf((float)cv[e], g.beta, g.alpha * v[e]);
+                    }
+                    w[o][0] = pack2(v[0], v[1]);
+                    w[o][1] = pack2(v[2], v[3]);
                 }
-                halfx4 out;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) out[e] = (_Float16)v[e];
-                *(halfx4*)(D + (size_t)row * g.ldd + col) = out;
+                const auto s0 = __builtin_amdgcn_permlane32_swap(w[0][0], w[1][0], false, false);
+                const auto s1 = __builtin_amdgcn_permlane32_swap(w[0][1], w[1][1], false, false);
+                const uintx4 out = {s0[0], s1[0], s0[1], s1[1]};
+                const uint32_t col = n0 + wn0 + 32 * j + 8 * (2 * qp + h);
+                *(uintx4*)(D + (size_t)row * g.ldd + col) = out;
             }
         }
     }
