@@ -87,7 +87,6 @@ int launch_gemm_f32_pipelined(const GemmArgs& args, hipStream_t stream);
 int launch_gemm_f16(int shape, bool edge, const GemmArgs& args, hipStream_t stream);
 // 256 x 256 x 64 direct-to-LDS kernel; full tiles only (the caller checks divisibility and alignment)
 int launch_gemm_f16_pipelined(const GemmArgs& args, hipStream_t stream);
-void set_f16_pipelined_variant(int v);   // tuning hook: 0 = 64-deep slabs x 2 stages, 1 = 32 x 4, 2 = 32 x 5
 int launch_gemv_f32(const float* A, const float* x, const float* c, float* y, uint32_t M, uint32_t K,
                     uint32_t lda, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta,
                     hipStream_t stream);

@@ -38,7 +38,6 @@
 // loads); and `sched_group_barrier` pins the MFMA / LDS-read interleave (left alone it
 // issues all reads of a k-step in a clump in front of the MFMAs).
 #include "gemm_common.hpp"
-#include <cstdlib>
 #include <type_traits>
 
 namespace decx_hip {
@@ -345,11 +344,9 @@ gemm_f16_pipelined_kernel(const GemmArgs g)
     }
 }
 
-static int g_variant = -1;
-void set_f16_pipelined_variant(int v) { g_variant = v; }
-
-// Full tiles only: M, N multiples of 256, K a positive multiple of 64, 16-byte aligned
-// bases and pitches.  The caller checks.
+// Full tiles only: M, N multiples of 256, K a positive multiple of 32, 16-byte aligned
+// bases and pitches.  The caller checks.  32-deep slabs in a ring of 4 stages measured best
+// (equal to 64 x 2 at 4096^3, 4 % faster at 8192^3; 32 x 5 is slower).
 int launch_gemm_f16_pipelined(const GemmArgs& args, hipStream_t stream)
 {
     GemmArgs g = args;
@@ -357,15 +354,7 @@ int launch_gemm_f16_pipelined(const GemmArgs& args, hipStream_t stream)
     g.tiles_n = g.N / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
     g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
-    if (g_variant < 0) {
-        const char* e = getenv("DECX_HIP_F16_VARIANT");
-        g_variant = e ? atoi(e) : 0;
-    }
-    switch (g_variant) {
-    case 1:  hipLaunchKernelGGL((gemm_f16_pipelined_kernel<32, 4>), dim3(nb), dim3(NT), 0, stream, g); break;
-    case 2:  hipLaunchKernelGGL((gemm_f16_pipelined_kernel<32, 5>), dim3(nb), dim3(NT), 0, stream, g); break;
-    default: hipLaunchKernelGGL((gemm_f16_pipelined_kernel<64, 2>), dim3(nb), dim3(NT), 0, stream, g); break;
-    }
+    hipLaunchKernelGGL((gemm_f16_pipelined_kernel<32, 4>), dim3(nb), dim3(NT), 0, stream, g);
     return (int)hipGetLastError();
 }
 

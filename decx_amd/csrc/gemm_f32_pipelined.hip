@@ -17,7 +17,6 @@
 //     explicit vmcnt wait, because the compiler would otherwise wait for every outstanding
 //     load in front of each LDS read and at each __syncthreads().
 #include "gemm_common.hpp"
-#include <cstdlib>
 #include <type_traits>
 
 namespace decx_hip {
@@ -225,14 +224,8 @@ int launch_gemm_f32_pipelined(const GemmArgs& args, hipStream_t stream)
     g.tiles_n = g.N / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
     g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
-    static int variant = -1;
-    if (variant < 0) { const char* e = getenv("DECX_HIP_F32_STAGES"); variant = e ? atoi(e) : 4; }
-    switch (variant) {
-    case 3:  hipLaunchKernelGGL((gemm_f32_pipelined_kernel<3>), dim3(nb), dim3(NT), 0, stream, g); break;
-    case 5:  hipLaunchKernelGGL((gemm_f32_pipelined_kernel<5>), dim3(nb), dim3(NT), 0, stream, g); break;
-    case 2:  hipLaunchKernelGGL((gemm_f32_pipelined_kernel<2>), dim3(nb), dim3(NT), 0, stream, g); break;
-    default: hipLaunchKernelGGL((gemm_f32_pipelined_kernel<4>), dim3(nb), dim3(NT), 0, stream, g); break;
-    }
+    // ring depth: 2, 3 and 4 stages measure the same, 5 is slower; 4 leaves slack for late loads
+    hipLaunchKernelGGL((gemm_f32_pipelined_kernel<4>), dim3(nb), dim3(NT), 0, stream, g);
     return (int)hipGetLastError();
 }
 
