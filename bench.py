@@ -42,6 +42,9 @@ WORKLOADS = {
     "fp32_ragged": ("f32", 1000, 1500, 777, "mfma", 2, "fp32 GEMM M=1000 N=1500 K=777, uniform[-1,1]"),
     "fp32_tall_skinny": ("f32", 65536, 256, 1024, "mfma", 5, "fp32 GEMM M=65536 N=256 K=1024, uniform[-1,1]"),
     "fp32_gemv": ("f32", 8192, 1, 8192, "hbm", 6, "fp32 GEMM M=8192 N=1 K=8192 (GEMV-like), uniform[-1,1]"),
+    "fp32_gevm": ("f32", 1, 8192, 8192, "hbm", 6, "fp32 GEMM M=1 N=8192 K=8192 (vector x matrix), uniform[-1,1]"),
+    "fp16_gemv": ("f16", 8192, 1, 8192, "hbm", 6, "fp16 GEMM M=8192 N=1 K=8192 (fp32 accumulate), normal(0,0.5)"),
+    "fp16_gevm": ("f16", 1, 8192, 8192, "hbm", 6, "fp16 GEMM M=1 N=8192 K=8192 (fp32 accumulate), normal(0,0.5)"),
 }
 
 

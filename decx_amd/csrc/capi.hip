@@ -58,9 +58,11 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
     if (rc != DECX_HIP_OK || M == 0 || N == 0) return rc;
     if (tile != DECX_HIP_TILE_AUTO && (tile < 0 || tile >= TILE_COUNT)) return DECX_HIP_E_INVALID_ARG;
 
-    if (!F16 && N == 1 && tile == DECX_HIP_TILE_AUTO && K > 0)
-        return launch_gemv_f32((const float*)A, (const float*)B, (const float*)C, (float*)D, M, K, lda,
-                               ldb, ldc, ldd, alpha, beta, as_stream(stream));
+    // the two vector corners are bandwidth-bound and have kernels of their own
+    if (N == 1 && tile == DECX_HIP_TILE_AUTO && K > 0)
+        return launch_gemv(F16, false, A, B, C, D, M, K, lda, ldb, ldc, ldd, alpha, beta, as_stream(stream));
+    if (M == 1 && tile == DECX_HIP_TILE_AUTO && K > 0)
+        return launch_gevm(F16, false, A, B, C, D, K, N, ldb, 1, 1, 1, alpha, beta, as_stream(stream));
 
     constexpr uint32_t per16 = F16 ? 8u : 4u;          // elements per 16 bytes
     GemmArgs g;
@@ -237,13 +239,47 @@ int decx_hip_gemm_f16_tile(const uint16_t* A, const uint16_t* B, const uint16_t*
     return run_gemm<true>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, tile, force_edge);
 }
 
-int decx_hip_gemv_f32(const float* A, const float* x, const float* c, float* y, uint32_t M, uint32_t K, uint32_t lda,
-                      uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, void* stream)
+static int run_gemv(bool f16, bool out_f32, const void* A, const void* x, const void* c, void* y, uint32_t M,
+                    uint32_t K, uint32_t lda, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta,
+                    void* stream)
 {
     if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
     if (M == 0) return DECX_HIP_OK;
     if (!A || !x || !y || lda < K || incx == 0 || incy == 0 || (c && incc == 0)) return DECX_HIP_E_INVALID_ARG;
-    return launch_gemv_f32(A, x, c, y, M, K, lda, incx, incc, incy, alpha, beta, as_stream(stream));
+    return launch_gemv(f16, out_f32, A, x, c, y, M, K, lda, incx, incc, incy, alpha, beta, as_stream(stream));
+}
+
+static int run_gevm(bool f16, bool out_f32, const void* x, const void* B, const void* c, void* y, uint32_t K,
+                    uint32_t N, uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta,
+                    void* stream)
+{
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    if (N == 0) return DECX_HIP_OK;
+    if (!x || !B || !y || ldb < N || incx == 0 || incy == 0 || (c && incc == 0)) return DECX_HIP_E_INVALID_ARG;
+    return launch_gevm(f16, out_f32, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, as_stream(stream));
+}
+
+int decx_hip_gemv_f32(const float* A, const float* x, const float* c, float* y, uint32_t M, uint32_t K, uint32_t lda,
+                      uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, void* stream)
+{
+    return run_gemv(false, true, A, x, c, y, M, K, lda, incx, incc, incy, alpha, beta, stream);
+}
+int decx_hip_gemv_f16(const uint16_t* A, const uint16_t* x, const uint16_t* c, void* y, uint32_t M, uint32_t K,
+                      uint32_t lda, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, int y_is_f32,
+                      void* stream)
+{
+    return run_gemv(true, y_is_f32 != 0, A, x, c, y, M, K, lda, incx, incc, incy, alpha, beta, stream);
+}
+int decx_hip_gevm_f32(const float* x, const float* B, const float* c, float* y, uint32_t K, uint32_t N, uint32_t ldb,
+                      uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, void* stream)
+{
+    return run_gevm(false, true, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream);
+}
+int decx_hip_gevm_f16(const uint16_t* x, const uint16_t* B, const uint16_t* c, void* y, uint32_t K, uint32_t N,
+                      uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, int y_is_f32,
+                      void* stream)
+{
+    return run_gevm(true, y_is_f32 != 0, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream);
 }
 
 int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int aligned, decx_hip_plan* out)
@@ -252,10 +288,16 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
     std::memset(out, 0, sizeof *out);
     if (M == 0 || N == 0) return DECX_HIP_OK;
     const bool f16 = elem_bytes == 2;
-    if (!f16 && N == 1 && K > 0) {
+    if (N == 1 && K > 0) {
         out->path = DECX_HIP_PATH_GEMV;
         out->tile_m = 32; out->tile_n = 1;
         out->grid = (M + 31) / 32;
+        return DECX_HIP_OK;
+    }
+    if (M == 1 && K > 0) {
+        out->path = DECX_HIP_PATH_GEVM;
+        out->tile_m = 1; out->tile_n = f16 ? 64 : 32;
+        out->grid = (N + out->tile_n - 1) / out->tile_n;
         return DECX_HIP_OK;
     }
     const int shape = choose_tile(f16, M, N);

@@ -87,8 +87,11 @@ int launch_gemm_f32_pipelined(const GemmArgs& args, hipStream_t stream);
 int launch_gemm_f16(int shape, bool edge, const GemmArgs& args, hipStream_t stream);
 // 256 x 256 x 64 direct-to-LDS kernel; full tiles only (the caller checks divisibility and alignment)
 int launch_gemm_f16_pipelined(const GemmArgs& args, hipStream_t stream);
-int launch_gemv_f32(const float* A, const float* x, const float* c, float* y, uint32_t M, uint32_t K,
-                    uint32_t lda, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta,
-                    hipStream_t stream);
+// y = alpha * A.x (+ beta * c) and y = alpha * x.B (+ beta * c); f16 inputs accumulate in fp32 and write
+// fp32 (out_f32) or fp16.  inc* are element strides.
+int launch_gemv(bool f16, bool out_f32, const void* A, const void* x, const void* c, void* y, uint32_t M, uint32_t K,
+                uint32_t lda, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream);
+int launch_gevm(bool f16, bool out_f32, const void* x, const void* B, const void* c, void* y, uint32_t K, uint32_t N,
+                uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream);
 
 }  // namespace decx_hip

@@ -1,0 +1,225 @@
+// The two vector corners of the GEMM entry point, both bound by HBM bandwidth (every
+// element of the matrix is used once):
+//
+//   gemv:  y (M) = alpha * A (M x K) . x (K)  (+ beta * c)      -- N == 1
+//   gevm:  y (N) = alpha * x (K) . B (K x N)  (+ beta * c)      -- M == 1
+//
+// They replace cu_mat_m_vec_fp32 / cu_vec_m_mat_fp32, their fp16 L1-L3 variants and the
+// second reduction pass those need (srcs/modules/BLAS/GEMM/CUDA/extreme_shapes/
+// VMM_fp32.cu:35-146, VMM_fp16.cu, VMM_callers.cuh:67-202): here a workgroup finishes its
+// outputs itself, so there are no partial sums to reduce in another kernel.  fp16 inputs
+// are always accumulated in fp32 (the reference's level 1); the result is written as fp32
+// or rounded once to fp16, whichever the caller asks for.
+//
+// gemv: 16 wavefronts per workgroup, two rows per wavefront (32 rows per workgroup: 8192
+//   rows give one workgroup per CU with 64 KB of A in flight); x is staged in LDS once per
+//   workgroup, as fp32, in chunks of 8192 -- x may be strided (the single column of a
+//   pitched K x 1 matrix puts every element in its own cache line), so staging it once per
+//   32 rows keeps that gather small; A is read with 128-bit loads; per lane an fp32 fma
+//   chain, then a butterfly over the 64 lanes.
+// gevm: a workgroup owns 128 bytes of columns (32 fp32 / 64 fp16); 8 lanes cover those with
+//   one 128-bit load each, the other lane bits and the 16 wavefronts stride over k
+//   (128 rows per sweep); partial sums meet in a shuffle over the row lanes and in LDS over
+//   the wavefronts.
+#include "gemm_common.hpp"
+
+namespace decx_hip {
+
+namespace {
+
+constexpr int GEMV_THREADS = 1024;
+constexpr int GEMV_WAVES = GEMV_THREADS / 64;
+constexpr int GEMV_ROWS_PER_BLOCK = 2 * GEMV_WAVES;
+constexpr int GEMV_KC = 8192;            // floats of x staged per chunk (32 KB of LDS)
+
+template <typename T> struct Per16 { static constexpr int n = 16 / sizeof(T); };
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(_Float16 v) { return (float)v; }
+
+// 16 bytes of T at p, widened to float
+template <typename T> __device__ __forceinline__ void load16(const T* p, float (&out)[Per16<T>::n])
+{
+    if constexpr (sizeof(T) == 4) {
+        const floatx4 v = *(const floatx4*)p;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[e] = v[e];
+    } else {
+        const halfx8 v = *(const halfx8*)p;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] = (float)v[e];
+    }
+}
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+template <typename T, typename TO>
+__global__ void __launch_bounds__(GEMV_THREADS)
+gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restrict__ c, TO* __restrict__ y,
+            uint32_t M, uint32_t K, uint32_t lda, uint32_t incx, uint32_t incc, uint32_t incy,
+            float alpha, float beta, uint32_t vec_ok)
+{
+    constexpr int N16 = Per16<T>::n;
+    __shared__ __attribute__((aligned(16))) float xs[GEMV_KC];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const uint32_t row0 = blockIdx.x * GEMV_ROWS_PER_BLOCK + wave * 2;
+    const bool has0 = row0 < M, has1 = row0 + 1 < M;
+    const T* a0 = A + (size_t)(has0 ? row0 : 0) * lda;
+    const T* a1 = A + (size_t)(has1 ? row0 + 1 : 0) * lda;
+    float s0 = 0.f, s1 = 0.f;
+
+    for (uint32_t kc = 0; kc < K; kc += GEMV_KC) {
+        const uint32_t len = (K - kc) < (uint32_t)GEMV_KC ? (K - kc) : (uint32_t)GEMV_KC;
+        __syncthreads();                                   // previous chunk fully consumed
+        for (uint32_t i = t; i < len; i += GEMV_THREADS) xs[i] = to_float(x[(size_t)(kc + i) * incx]);
+        __syncthreads();
+        const uint32_t lenv = vec_ok ? (len / N16) * N16 : 0u;   // part done with 128-bit loads
+        if (has0) {
+#pragma unroll 4
+            for (uint32_t k = lane * N16; k < lenv; k += 64 * N16) {
+                float av[N16], bv[N16];
+                load16<T>(a0 + kc + k, av);
+                if (has1) load16<T>(a1 + kc + k, bv);
+#pragma unroll
+                for (int e = 0; e < N16; ++e) {
+                    const float xv = xs[k + e];
+                    s0 = __builtin_fmaf(av[e], xv, s0);
+                    if (has1) s1 = __builtin_fmaf(bv[e], xv, s1);
+                }
+            }
+            for (uint32_t k = lenv + lane; k < len; k += 64) {
+                s0 = __builtin_fmaf(to_float(a0[kc + k]), xs[k], s0);
+                if (has1) s1 = __builtin_fmaf(to_float(a1[kc + k]), xs[k], s1);
+            }
+        }
+    }
+    s0 = wave_sum(s0);
+    s1 = wave_sum(s1);
+    if (lane == 0) {
+        if (has0) {
+            float o = s0;
+            if (c) o = __builtin_fmaf(to_float(c[(size_t)row0 * incc]), beta, alpha * o);
+            y[(size_t)row0 * incy] = (TO)o;
+        }
+        if (has1) {
+            float o = s1;
+            if (c) o = __builtin_fmaf(to_float(c[(size_t)(row0 + 1) * incc]), beta, alpha * o);
+            y[(size_t)(row0 + 1) * incy] = (TO)o;
+        }
+    }
+}
+
+template <typename T, typename TO>
+__global__ void __launch_bounds__(GEMV_THREADS)
+gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restrict__ c, TO* __restrict__ y,
+            uint32_t K, uint32_t N, uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy,
+            float alpha, float beta, uint32_t vec_ok)
+{
+    constexpr int N16 = Per16<T>::n;
+    constexpr int CB = 8 * N16;                            // columns per workgroup (128 bytes of a row)
+    __shared__ __attribute__((aligned(16))) float xs[GEMV_KC];
+    __shared__ float red[GEMV_WAVES][CB];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int col_lane = lane & 7, row_lane = lane >> 3;   // 8 column groups x 8 rows per wavefront
+    const uint32_t n0 = blockIdx.x * CB + col_lane * N16;
+    const bool whole = vec_ok && (n0 + N16 <= N);
+    float acc[N16];
+#pragma unroll
+    for (int e = 0; e < N16; ++e) acc[e] = 0.f;
+
+    for (uint32_t kc = 0; kc < K; kc += GEMV_KC) {
+        const uint32_t len = (K - kc) < (uint32_t)GEMV_KC ? (K - kc) : (uint32_t)GEMV_KC;
+        __syncthreads();
+        for (uint32_t i = t; i < len; i += GEMV_THREADS) xs[i] = to_float(x[(size_t)(kc + i) * incx]);
+        __syncthreads();
+        if (n0 < N) {
+#pragma unroll 4
+            for (uint32_t k = wave * 8 + row_lane; k < len; k += GEMV_WAVES * 8) {
+                const T* p = B + (size_t)(kc + k) * ldb + n0;
+                const float xv = xs[k];
+                if (whole) {
+                    float bv[N16];
+                    load16<T>(p, bv);
+#pragma unroll
+                    for (int e = 0; e < N16; ++e) acc[e] = __builtin_fmaf(xv, bv[e], acc[e]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < N16; ++e)
+                        if (n0 + e < N) acc[e] = __builtin_fmaf(xv, to_float(p[e]), acc[e]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < N16; ++e) {
+        float v = acc[e];
+        v += __shfl_xor(v, 8, 64);
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        if (row_lane == 0) red[wave][col_lane * N16 + e] = v;
+    }
+    __syncthreads();
+    if (t < CB) {
+        const uint32_t n = blockIdx.x * CB + t;
+        if (n < N) {
+            float o = 0.f;
+#pragma unroll
+            for (int w = 0; w < GEMV_WAVES; ++w) o += red[w][t];
+            if (c) o = __builtin_fmaf(to_float(c[(size_t)n * incc]), beta, alpha * o);
+            y[(size_t)n * incy] = (TO)o;
+        }
+    }
+}
+
+template <typename T> uint32_t rows_vectorisable(const void* base, uint32_t ld)
+{
+    return (((uintptr_t)base & 15u) == 0 && (ld * sizeof(T)) % 16 == 0) ? 1u : 0u;
+}
+
+}  // namespace
+
+int launch_gemv(bool f16, bool out_f32, const void* A, const void* x, const void* c, void* y, uint32_t M, uint32_t K,
+                uint32_t lda, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream)
+{
+    const dim3 grid((M + GEMV_ROWS_PER_BLOCK - 1) / GEMV_ROWS_PER_BLOCK), block(GEMV_THREADS);
+    if (!f16)
+        hipLaunchKernelGGL((gemv_kernel<float, float>), grid, block, 0, stream, (const float*)A, (const float*)x,
+                           (const float*)c, (float*)y, M, K, lda, incx, incc, incy, alpha, beta,
+                           rows_vectorisable<float>(A, lda));
+    else if (out_f32)
+        hipLaunchKernelGGL((gemv_kernel<_Float16, float>), grid, block, 0, stream, (const _Float16*)A,
+                           (const _Float16*)x, (const _Float16*)c, (float*)y, M, K, lda, incx, incc, incy, alpha, beta,
+                           rows_vectorisable<_Float16>(A, lda));
+    else
+        hipLaunchKernelGGL((gemv_kernel<_Float16, _Float16>), grid, block, 0, stream, (const _Float16*)A,
+                           (const _Float16*)x, (const _Float16*)c, (_Float16*)y, M, K, lda, incx, incc, incy, alpha,
+                           beta, rows_vectorisable<_Float16>(A, lda));
+    return (int)hipGetLastError();
+}
+
+int launch_gevm(bool f16, bool out_f32, const void* x, const void* B, const void* c, void* y, uint32_t K, uint32_t N,
+                uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream)
+{
+    const uint32_t cb = f16 ? 64u : 32u;
+    const dim3 grid((N + cb - 1) / cb), block(GEMV_THREADS);
+    if (!f16)
+        hipLaunchKernelGGL((gevm_kernel<float, float>), grid, block, 0, stream, (const float*)x, (const float*)B,
+                           (const float*)c, (float*)y, K, N, ldb, incx, incc, incy, alpha, beta,
+                           rows_vectorisable<float>(B, ldb));
+    else if (out_f32)
+        hipLaunchKernelGGL((gevm_kernel<_Float16, float>), grid, block, 0, stream, (const _Float16*)x,
+                           (const _Float16*)B, (const _Float16*)c, (float*)y, K, N, ldb, incx, incc, incy, alpha, beta,
+                           rows_vectorisable<_Float16>(B, ldb));
+    else
+        hipLaunchKernelGGL((gevm_kernel<_Float16, _Float16>), grid, block, 0, stream, (const _Float16*)x,
+                           (const _Float16*)B, (const _Float16*)c, (_Float16*)y, K, N, ldb, incx, incc, incy, alpha,
+                           beta, rows_vectorisable<_Float16>(B, ldb));
+    return (int)hipGetLastError();
+}
+
+}  // namespace decx_hip

@@ -9,7 +9,7 @@ import numpy as np
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "lib", "libdecx_hip.so")
 
-TILE_AUTO, TILE_256, TILE_128, TILE_64, PATH_GEMV = -1, 0, 1, 2, 16
+TILE_AUTO, TILE_256, TILE_128, TILE_64, PATH_GEMV, PATH_GEVM = -1, 0, 1, 2, 16, 17
 
 _vp = ctypes.c_void_p
 _u32 = ctypes.c_uint32
@@ -52,6 +52,9 @@ SYMBOLS = {
     "decx_hip_gemm_f32": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp]),
     "decx_hip_gemm_f16": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp]),
     "decx_hip_gemv_f32": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _vp]),
+    "decx_hip_gemv_f16": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _int, _vp]),
+    "decx_hip_gevm_f32": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _vp]),
+    "decx_hip_gevm_f16": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _int, _vp]),
     "decx_hip_gemm_f32_tile": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, _int, _int]),
     "decx_hip_gemm_f16_tile": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, _int, _int]),
     "decx_hip_gemm_plan": (_int, [_int, _u32, _u32, _u32, _int, ctypes.POINTER(Plan)]),
@@ -180,6 +183,47 @@ def gemm(A, B, D, C=None, alpha=1.0, beta=1.0, stream=None, tile=TILE_AUTO, forc
     else:
         rc = (L.decx_hip_gemm_f16_tile if f16 else L.decx_hip_gemm_f32_tile)(*args, tile, 1 if force_edge else 0)
     check(rc, "gemm")
+
+
+def _as_vector(V, n):
+    """(pointer, element stride) of a DeviceMatrix used as a vector of n elements: 1 x n is contiguous,
+    n x 1 strides by the pitch."""
+    if V.rows == 1 and V.cols == n:
+        return V.ptr, 1
+    assert V.cols == 1 and V.rows == n, "vector operand must be 1 x n or n x 1"
+    return V.ptr, V.pitch
+
+
+def gemv(A, x, y, c=None, alpha=1.0, beta=1.0, stream=None):
+    """y (M) = alpha * A (M x K) . x (K) + beta * c through decx_hip_gemv_f32 / _f16; y may be fp32 for fp16 inputs."""
+    M, K = A.rows, A.cols
+    (xp, incx), (yp, incy) = _as_vector(x, K), _as_vector(y, M)
+    cp, incc = _as_vector(c, M) if c is not None else (None, 0)
+    L = lib()
+    if A.dtype == np.float16:
+        assert x.dtype == np.float16 and y.dtype in (np.float16, np.float32)
+        rc = L.decx_hip_gemv_f16(A.ptr, xp, cp, yp, M, K, A.pitch, incx, incc, incy, alpha, beta,
+                                 1 if y.dtype == np.float32 else 0, stream)
+    else:
+        assert x.dtype == y.dtype == np.float32
+        rc = L.decx_hip_gemv_f32(A.ptr, xp, cp, yp, M, K, A.pitch, incx, incc, incy, alpha, beta, stream)
+    check(rc, "gemv")
+
+
+def gevm(x, B, y, c=None, alpha=1.0, beta=1.0, stream=None):
+    """y (N) = alpha * x (K) . B (K x N) + beta * c through decx_hip_gevm_f32 / _f16."""
+    K, N = B.rows, B.cols
+    (xp, incx), (yp, incy) = _as_vector(x, K), _as_vector(y, N)
+    cp, incc = _as_vector(c, N) if c is not None else (None, 0)
+    L = lib()
+    if B.dtype == np.float16:
+        assert x.dtype == np.float16 and y.dtype in (np.float16, np.float32)
+        rc = L.decx_hip_gevm_f16(xp, B.ptr, cp, yp, K, N, B.pitch, incx, incc, incy, alpha, beta,
+                                 1 if y.dtype == np.float32 else 0, stream)
+    else:
+        assert x.dtype == y.dtype == np.float32
+        rc = L.decx_hip_gevm_f32(xp, B.ptr, cp, yp, K, N, B.pitch, incx, incc, incy, alpha, beta, stream)
+    check(rc, "gevm")
 
 
 def sync(stream=None):

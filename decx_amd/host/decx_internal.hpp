@@ -99,6 +99,61 @@ public:
     bool re_construct(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height);
 };
 
+// Host vector.  Storage rule of the original (srcs/modules/core/classes/Vector.cxx): the
+// allocation is the length rounded up to 32 bytes of elements, zero-filled.
+class _Vector : public de::Vector {
+    size_t _length, _capacity;          // elements asked for / elements allocated
+    de::_DATA_TYPES_FLAGS_ _type;
+    uint32_t _element_size;
+    std::shared_ptr<HostBlock> _block;
+    void* _data;
+    void assign(de::_DATA_TYPES_FLAGS_ type, size_t length);
+    bool allocate();
+
+public:
+    _Vector();
+    _Vector(de::_DATA_TYPES_FLAGS_ type, size_t length);
+    virtual size_t Len() const;
+    virtual void release();
+    virtual de::Vector& SoftCopy(de::Vector& src);
+    virtual de::_DATA_TYPES_FLAGS_ Type() const;
+    virtual void Reinterpret(const de::_DATA_TYPES_FLAGS_ new_type);
+    virtual ~_Vector();
+
+    bool is_init() const { return _data != nullptr; }
+    void* data() const { return _data; }
+    uint32_t element_bytes() const { return _element_size; }
+    size_t capacity_bytes() const { return _block ? _block->bytes : 0; }
+    bool re_construct(de::_DATA_TYPES_FLAGS_ type, size_t length);      // grows only
+    bool is_pinned() const { return _block && _block->pinned; }
+    int move_storage(bool pinned);
+};
+
+// Device vector: same length rule, storage in HBM.
+class _GPU_Vector : public de::GPU_Vector {
+    size_t _length, _capacity;
+    de::_DATA_TYPES_FLAGS_ _type;
+    uint32_t _element_size;
+    std::shared_ptr<DeviceBlock> _block;
+    void assign(de::_DATA_TYPES_FLAGS_ type, size_t length);
+    bool allocate();
+
+public:
+    _GPU_Vector();
+    _GPU_Vector(de::_DATA_TYPES_FLAGS_ type, size_t length);
+    virtual size_t Len() const;
+    virtual void release();
+    virtual de::GPU_Vector& SoftCopy(de::GPU_Vector& src);
+    virtual de::_DATA_TYPES_FLAGS_ Type() const;
+    virtual void Reinterpret(const de::_DATA_TYPES_FLAGS_ new_type);
+    virtual ~_GPU_Vector();
+
+    bool is_init() const { return _block && _block->ptr; }
+    void* data() const { return _block ? _block->ptr : nullptr; }
+    uint32_t element_bytes() const { return _element_size; }
+    bool re_construct(de::_DATA_TYPES_FLAGS_ type, size_t length);
+};
+
 // One stream for the module, created on first use; one mutex around every GEMM call
 // (the original guards its cached planner with a plain flag).
 void* module_stream();

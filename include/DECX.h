@@ -230,12 +230,63 @@ _DECX_API_ GPU_Matrix* CreateGPUMatrixPtr(const _DATA_TYPES_FLAGS_ type, const u
 _DECX_API_ GPU_Matrix& CreateGPUMatrixRef(const _DATA_TYPES_FLAGS_ type, const uint32_t _width, const uint32_t _height,
                                           const _DATA_FORMATS_ format = _NA_);
 
+/* ------------------------------------------------------------------ host and device vectors */
+
+/* A zero-filled array of Len() elements whose storage is rounded up to 32 bytes. */
+class _DECX_API_ Vector {
+protected:
+    _SHADOW_ATTRIBUTE_(void*) _exp_data_ptr;               /* -> the implementation's data pointer */
+
+public:
+    Vector() {}
+    virtual size_t Len() const = 0;
+
+    template <typename _ptr_type> _ptr_type* ptr(const uint64_t _idx) { return ((_ptr_type*)*this->_exp_data_ptr) + _idx; }
+
+    virtual void release() = 0;
+    virtual Vector& SoftCopy(Vector& src) = 0;
+    virtual _DATA_TYPES_FLAGS_ Type() const = 0;
+    virtual void Reinterpret(const _DATA_TYPES_FLAGS_ _new_type) = 0;
+    ~Vector() {}
+};
+typedef const Vector& InputVector;
+typedef Vector& OutputVector;
+typedef Vector& InOutVector;
+
+_DECX_API_ Vector& CreateVectorRef();
+_DECX_API_ Vector* CreateVectorPtr();
+_DECX_API_ Vector& CreateVectorRef(const _DATA_TYPES_FLAGS_ _type, size_t len);
+_DECX_API_ Vector* CreateVectorPtr(const _DATA_TYPES_FLAGS_ _type, size_t len);
+
+class _DECX_API_ GPU_Vector {
+public:
+    GPU_Vector() {}
+    virtual size_t Len() const = 0;
+    virtual void release() = 0;
+    virtual GPU_Vector& SoftCopy(GPU_Vector& src) = 0;
+    virtual _DATA_TYPES_FLAGS_ Type() const = 0;
+    virtual void Reinterpret(const _DATA_TYPES_FLAGS_ _new_type) = 0;
+    ~GPU_Vector() {}
+};
+
+_DECX_API_ GPU_Vector& CreateGPUVectorRef();
+_DECX_API_ GPU_Vector* CreateGPUVectorPtr();
+_DECX_API_ GPU_Vector& CreateGPUVectorRef(const _DATA_TYPES_FLAGS_ _type, const size_t _length);
+_DECX_API_ GPU_Vector* CreateGPUVectorPtr(const _DATA_TYPES_FLAGS_ _type, const size_t _length);
+
+/* How fp16 vector products accumulate.  Every level accumulates in fp32 here (the most
+ * accurate of the three); the level only selects the element type of the result, as it does
+ * in the original: level 1 writes fp32, levels 2 and 3 write fp16 (rounded once). */
+enum Fp16_Accuracy_Levels { Fp16_Accurate_L1 = 0, Fp16_Accurate_L2 = 1, Fp16_Accurate_L3 = 2 };
+
 namespace cuda {
 /* Makes the host matrix's storage page-locked (faster, asynchronous-capable transfers) and
  * back.  The storage is moved, not registered in place; pointers obtained from ptr<T>()
  * before the call must be re-read. */
 _DECX_API_ DH PinMemory(Matrix& src);
 _DECX_API_ DH UnpinMemory(Matrix& src);
+_DECX_API_ DH PinMemory(Vector& src);
+_DECX_API_ DH UnpinMemory(Vector& src);
 }
 
 /* ------------------------------------------------------------------ transfers */
@@ -247,6 +298,11 @@ enum DECX_Memcpy_Flags { DECX_MEMCPY_H2D = 0, DECX_MEMCPY_D2H = 1 };
  * device matrix for D2H.  Blocks until the copy has finished. */
 _DECX_API_ DH Memcpy(Matrix& __host, GPU_Matrix& __device, const Point2D start_src, Point2D start_dst,
                      const Point2D cpy_size, const int _memcpy_flag);
+
+/* Copies cpy_len elements from element start_src of the source to element start_dst of the
+ * destination (source = host vector for H2D, device vector for D2H). */
+_DECX_API_ DH Memcpy(Vector& __host, GPU_Vector& __device, const uint64_t start_src, const uint64_t start_dst,
+                     const uint64_t cpy_len, const int _memcpy_flag);
 
 /* ------------------------------------------------------------------ the product */
 namespace blas {
@@ -260,6 +316,13 @@ _DECX_API_ void GEMM(GPU_Matrix& A, GPU_Matrix& B, GPU_Matrix& C, GPU_Matrix& ds
 /* Host-matrix forms: operands are staged through device memory around the same kernels. */
 _DECX_API_ void GEMM(Matrix& A, Matrix& B, Matrix& dst);
 _DECX_API_ void GEMM(Matrix& A, Matrix& B, Matrix& C, Matrix& dst);
+/* Vector forms on host objects.  dst <- A . B with A a row vector of B.Height() elements
+ * (result: B.Width() elements), or with B a column vector of A.Width() elements (result:
+ * A.Height() elements).  For fp16 operands _fp16_accu (Fp16_Accuracy_Levels) selects an fp32
+ * (level 1) or fp16 result.  dst keeps its storage when the result fits and is re-created
+ * with the result's type and length otherwise. */
+_DECX_API_ void GEMM(Vector& A, Matrix& B, Vector& dst, const uint32_t _fp16_accu = 0);
+_DECX_API_ void GEMM(Matrix& A, Vector& B, Vector& dst, const uint32_t _fp16_accu = 0);
 }  // namespace cuda
 }  // namespace blas
 

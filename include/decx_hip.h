@@ -53,7 +53,8 @@ enum {
     DECX_HIP_TILE_256x256 = 0,
     DECX_HIP_TILE_128x128 = 1,
     DECX_HIP_TILE_64x64   = 2,
-    DECX_HIP_PATH_GEMV    = 16     /* N == 1: bandwidth-bound row-dot kernel */
+    DECX_HIP_PATH_GEMV    = 16,    /* N == 1: bandwidth-bound row-dot kernel */
+    DECX_HIP_PATH_GEVM    = 17     /* M == 1: bandwidth-bound column-sum kernel */
 };
 
 typedef struct decx_hip_plan {
@@ -100,8 +101,7 @@ DECX_HIP_API int decx_hip_event_elapsed_ms(void* start, void* stop, float* ms);
  * fp32: products and sums in fp32 on the matrix cores.  Replaces the kernels launched by
  * cuda_GEMM_LS_planner<float>::run (srcs/modules/BLAS/GEMM/CUDA/large_squares/fp32/
  * GEMM_fp32_callers.cu:56-122) behind de::blas::cuda::GEMM (GEMM_LS.cu:62-109,315-393).
- * N == 1 is routed to the row-dot kernel that replaces cu_mat_m_vec_fp32
- * (extreme_shapes/VMM_fp32.cu:104-146). */
+ * N == 1 and M == 1 are routed to the bandwidth-bound vector kernels below. */
 DECX_HIP_API int decx_hip_gemm_f32(const float* A, const float* B, const float* C, float* D,
                                    uint32_t M, uint32_t N, uint32_t K,
                                    uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
@@ -114,13 +114,30 @@ DECX_HIP_API int decx_hip_gemm_f16(const uint16_t* A, const uint16_t* B, const u
                                    uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
                                    float alpha, float beta, void* stream);
 
-/* y (M) = A (M x K) . x (K), optionally y = fma(c, beta, alpha * A.x).  incx / incc / incy
- * are element strides (a K x 1 pitched matrix has incx = its pitch).  This is what
- * decx_hip_gemm_f32 runs for N == 1; exported for callers that hold vectors. */
+/* The two vector corners, exported for callers that hold vectors (the GEMM entry points above
+ * route N == 1 and M == 1 here themselves).  inc* are element strides (a K x 1 pitched matrix
+ * has incx = its pitch); c == NULL -> no accumulate term.
+ *   gemv:  y (M) = alpha * A (M x K) . x (K) + beta * c     replaces cu_mat_m_vec_fp32 / _fp16_L1..L3
+ *   gevm:  y (N) = alpha * x (K) . B (K x N) + beta * c     replaces cu_vec_m_mat_fp32 / _fp16_L1..L3
+ * (srcs/modules/BLAS/GEMM/CUDA/extreme_shapes/VMM_fp32.cu:35-146, VMM_fp16.cu) and their second
+ * reduction pass.  fp16 inputs are accumulated in fp32; y is fp32 when y_is_f32 != 0 (the
+ * reference's accuracy level 1) and fp16, rounded once, otherwise. */
 DECX_HIP_API int decx_hip_gemv_f32(const float* A, const float* x, const float* c, float* y,
                                    uint32_t M, uint32_t K, uint32_t lda,
                                    uint32_t incx, uint32_t incc, uint32_t incy,
                                    float alpha, float beta, void* stream);
+DECX_HIP_API int decx_hip_gemv_f16(const uint16_t* A, const uint16_t* x, const uint16_t* c, void* y,
+                                   uint32_t M, uint32_t K, uint32_t lda,
+                                   uint32_t incx, uint32_t incc, uint32_t incy,
+                                   float alpha, float beta, int y_is_f32, void* stream);
+DECX_HIP_API int decx_hip_gevm_f32(const float* x, const float* B, const float* c, float* y,
+                                   uint32_t K, uint32_t N, uint32_t ldb,
+                                   uint32_t incx, uint32_t incc, uint32_t incy,
+                                   float alpha, float beta, void* stream);
+DECX_HIP_API int decx_hip_gevm_f16(const uint16_t* x, const uint16_t* B, const uint16_t* c, void* y,
+                                   uint32_t K, uint32_t N, uint32_t ldb,
+                                   uint32_t incx, uint32_t incc, uint32_t incy,
+                                   float alpha, float beta, int y_is_f32, void* stream);
 
 /* Same as decx_hip_gemm_f32 / _f16 with the planner's choice overridden (`tile` = one of
  * DECX_HIP_TILE_*; AUTO = planner) and, with force_edge != 0, the predicated kernel

@@ -6,6 +6,10 @@
 //   de_api_test gpu                       self-contained GPU checks (closed forms, error paths)
 //   de_api_test gemm <dir> <f32|f16> M N K <withC 0|1> <alpha> <beta>
 //                                         reads dense A.bin B.bin [C.bin] from <dir>, writes D.bin
+//   de_api_test vmm <dir> <f32|f16> <mv|vm> W H <level 0|1|2>
+//                                         reads M.bin (H rows x W) and V.bin, writes Y.bin (fp32 for f32
+//                                         and for f16 at level 0, fp16 otherwise) through the host-object
+//                                         vector forms of GEMM
 #include "DECX.h"
 
 #include <cmath>
@@ -197,6 +201,163 @@ static int gpu_checks()
     return g_failures;
 }
 
+static int vector_host_checks()
+{
+    // storage rule of vectors: length rounded up to 32 bytes, zero-filled, 32-byte aligned
+    de::Vector& v = de::CreateVectorRef(de::_FP32_, 13);
+    CHECK(v.Len() == 13 && v.Type() == de::_FP32_ && ((uintptr_t)v.ptr<float>(0) & 31u) == 0);
+    bool zero = true;
+    for (int i = 0; i < 16; ++i) zero &= (*v.ptr<float>(i) == 0.f);          // 13 -> 16 elements allocated
+    CHECK(zero);
+    de::Vector* e = de::CreateVectorPtr();
+    CHECK(e->Len() == 0 && e->Type() == de::_VOID_);
+    de::Vector& alias = de::CreateVectorRef();
+    alias.SoftCopy(v);
+    *v.ptr<float>(5) = 7.f;
+    CHECK(alias.Len() == 13 && *alias.ptr<float>(5) == 7.f);
+    v.release();
+    CHECK(*alias.ptr<float>(5) == 7.f);
+    alias.Reinterpret(de::_INT32_);
+    CHECK(alias.Type() == de::_INT32_ && alias.Len() == 13);
+    CHECK(de::Fp16_Accurate_L1 == 0 && de::Fp16_Accurate_L2 == 1 && de::Fp16_Accurate_L3 == 2);
+
+    // without InitCuda every GPU-facing vector call reports 0x16 and does nothing else
+    de::Vector& x = de::CreateVectorRef(de::_FP32_, 4);
+    de::Vector& y = de::CreateVectorRef(de::_FP32_, 4);
+    de::Matrix& m = de::CreateMatrixRef(de::_FP32_, 4, 4);
+    de::GPU_Vector& g = de::CreateGPUVectorRef();
+    CHECK(de::Memcpy(x, g, 0, 0, 4, de::DECX_MEMCPY_H2D).error_type == decx::DECX_FAIL_CUDA_not_init);
+    de::blas::cuda::GEMM(x, m, y);
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_CUDA_not_init);
+    de::blas::cuda::GEMM(m, x, y);
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_CUDA_not_init);
+    CHECK(de::cuda::PinMemory(x).error_type == decx::DECX_FAIL_CUDA_not_init);
+    de::ResetLastError();
+    return g_failures;
+}
+
+static int vector_gpu_checks()
+{
+    de::InitCuda();
+    de::ResetLastError();
+    // transfers with offsets, and their range / type checks
+    de::Vector& a = de::CreateVectorRef(de::_FP32_, 100);
+    de::Vector& b = de::CreateVectorRef(de::_FP32_, 100);
+    for (int i = 0; i < 100; ++i) *a.ptr<float>(i) = (float)i;
+    de::GPU_Vector& g = de::CreateGPUVectorRef(de::_FP32_, 60);
+    CHECK(g.Len() == 60 && g.Type() == de::_FP32_);
+    CHECK(de::Memcpy(a, g, 10, 20, 30, de::DECX_MEMCPY_H2D).error_type == 0);        // a[10..40) -> g[20..50)
+    CHECK(de::Memcpy(b, g, 0, 5, 60, de::DECX_MEMCPY_D2H).error_type == 0);          // g[0..60)  -> b[5..65)
+    bool same = true;
+    for (int i = 0; i < 100; ++i) {
+        const float want = (i >= 25 && i < 55) ? (float)(i - 25 + 10) : 0.f;         // device storage starts zeroed
+        same &= (*b.ptr<float>(i) == want);
+    }
+    CHECK(same);
+    CHECK(de::Memcpy(a, g, 0, 31, 30, de::DECX_MEMCPY_H2D).error_type == decx::DECX_FAIL_MEMCPY_OVERRANGED);
+    CHECK(de::Memcpy(a, g, 90, 0, 11, de::DECX_MEMCPY_H2D).error_type == decx::DECX_FAIL_MEMCPY_OVERRANGED);
+    CHECK(de::Memcpy(b, g, 41, 0, 20, de::DECX_MEMCPY_D2H).error_type == decx::DECX_FAIL_MEMCPY_OVERRANGED);
+    de::GPU_Vector& gh = de::CreateGPUVectorRef(de::_FP16_, 60);
+    CHECK(de::Memcpy(a, gh, 0, 0, 1, de::DECX_MEMCPY_H2D).error_type == decx::DECX_FAIL_TYPE_MOT_MATCH);
+    de::GPU_Vector& galias = de::CreateGPUVectorRef();
+    galias.SoftCopy(g);
+    g.release();
+    CHECK(galias.Len() == 60 && de::Memcpy(b, galias, 20, 0, 1, de::DECX_MEMCPY_D2H).error_type == 0 && *b.ptr<float>(0) == 10.f);
+
+    // closed forms: ones . M sums columns, M . ones sums rows (small integers: exact)
+    const uint32_t W = 300, H = 200;
+    de::Matrix& M = de::CreateMatrixRef(de::_FP32_, W, H);
+    for (uint32_t i = 0; i < H; ++i) for (uint32_t j = 0; j < W; ++j) *M.ptr<float>(i, j) = (float)((int)((i * 7 + j * 3) % 11) - 5);
+    de::Vector& onesH = de::CreateVectorRef(de::_FP32_, H);
+    de::Vector& onesW = de::CreateVectorRef(de::_FP32_, W);
+    for (uint32_t i = 0; i < H; ++i) *onesH.ptr<float>(i) = 1.f;
+    for (uint32_t j = 0; j < W; ++j) *onesW.ptr<float>(j) = 1.f;
+    de::Vector& cols = de::CreateVectorRef();                                        // empty: created by the call
+    de::blas::cuda::GEMM(onesH, M, cols);
+    CHECK(de::GetLastError()->error_type == 0 && cols.Len() == W && cols.Type() == de::_FP32_);
+    same = true;
+    for (uint32_t j = 0; j < W; ++j) { float s = 0; for (uint32_t i = 0; i < H; ++i) s += *M.ptr<float>(i, j); same &= (*cols.ptr<float>(j) == s); }
+    CHECK(same);
+    de::Vector& rows = de::CreateVectorRef(de::_FP32_, H);                           // exact size: storage kept
+    float* before = rows.ptr<float>(0);
+    de::blas::cuda::GEMM(M, onesW, rows);
+    CHECK(de::GetLastError()->error_type == 0 && rows.Len() == H && rows.ptr<float>(0) == before);
+    same = true;
+    for (uint32_t i = 0; i < H; ++i) { float s = 0; for (uint32_t j = 0; j < W; ++j) s += *M.ptr<float>(i, j); same &= (*rows.ptr<float>(i) == s); }
+    CHECK(same);
+
+    // fp16: level 1 gives an fp32 result, level 2 an fp16 one
+    de::Matrix& Mh = de::CreateMatrixRef(de::_FP16_, W, H);
+    for (uint32_t i = 0; i < H; ++i) for (uint32_t j = 0; j < W; ++j) *Mh.ptr<de::Half>(i, j) = de::Float2Half((float)((int)((i + j) % 5) - 2));
+    de::Vector& hx = de::CreateVectorRef(de::_FP16_, W);
+    for (uint32_t j = 0; j < W; ++j) *hx.ptr<de::Half>(j) = de::Float2Half((float)((int)(j % 3) - 1));
+    de::Vector& r1 = de::CreateVectorRef();
+    de::Vector& r2 = de::CreateVectorRef();
+    de::blas::cuda::GEMM(Mh, hx, r1, de::Fp16_Accurate_L1);
+    CHECK(de::GetLastError()->error_type == 0 && r1.Len() == H && r1.Type() == de::_FP32_);
+    de::blas::cuda::GEMM(Mh, hx, r2, de::Fp16_Accurate_L2);
+    CHECK(de::GetLastError()->error_type == 0 && r2.Len() == H && r2.Type() == de::_FP16_);
+    same = true;
+    for (uint32_t i = 0; i < H; ++i) {
+        float s = 0;
+        for (uint32_t j = 0; j < W; ++j) s += (float)((int)((i + j) % 5) - 2) * (float)((int)(j % 3) - 1);
+        same &= (*r1.ptr<float>(i) == s) && (de::Half2Float(*r2.ptr<de::Half>(i)) == s);
+    }
+    CHECK(same);
+
+    // error paths: nothing is launched, dst is left alone
+    de::Vector& shortv = de::CreateVectorRef(de::_FP32_, W - 1);
+    de::blas::cuda::GEMM(M, shortv, rows);
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_DimsNotMatching);
+    de::blas::cuda::GEMM(onesW, M, cols);                                            // needs H elements
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_DimsNotMatching);
+    de::blas::cuda::GEMM(Mh, onesW, rows);
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_TYPE_MOT_MATCH);
+    de::Matrix& Mi = de::CreateMatrixRef(de::_INT32_, W, H);
+    de::Vector& vi = de::CreateVectorRef(de::_INT32_, W);
+    de::blas::cuda::GEMM(Mi, vi, rows);
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_UNSUPPORTED_TYPE);
+    de::Vector& none = de::CreateVectorRef();
+    de::blas::cuda::GEMM(M, none, rows);
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_CLASS_NOT_INIT);
+    de::blas::cuda::GEMM(Mh, hx, r2, 3);
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_INVALID_PARAM);
+    de::blas::cuda::GEMM(M, onesW, rows);                                            // and a good call clears the status
+    CHECK(de::GetLastError()->error_type == 0);
+
+    // pinned host vectors behave the same
+    CHECK(de::cuda::PinMemory(onesW).error_type == 0);
+    CHECK(de::cuda::PinMemory(onesW).error_type == decx::DECX_FAIL_HOST_MEM_REGISTERED);
+    de::blas::cuda::GEMM(M, onesW, rows);
+    CHECK(de::GetLastError()->error_type == 0 && *onesW.ptr<float>(W - 1) == 1.f);
+    CHECK(de::cuda::UnpinMemory(onesW).error_type == 0);
+    CHECK(de::cuda::UnpinMemory(onesW).error_type == decx::DECX_FAIL_HOST_MEM_UNREGISTERED);
+    de::cuda::DECX_CUDA_exit();
+    return g_failures;
+}
+
+template <typename T> static int vmm_files(const std::string& dir, de::_DATA_TYPES_FLAGS_ ty, bool mat_times_vec,
+                                           uint32_t W, uint32_t H, uint32_t level)
+{
+    de::InitCuda();
+    de::ResetLastError();
+    de::Matrix& M = de::CreateMatrixRef(ty, W, H);
+    de::Vector& V = de::CreateVectorRef(ty, mat_times_vec ? W : H);
+    de::Vector& Y = de::CreateVectorRef();
+    std::ifstream fm(dir + "/M.bin", std::ios::binary), fv(dir + "/V.bin", std::ios::binary);
+    if (!fm || !fv) return 2;
+    for (uint32_t i = 0; i < H; ++i) fm.read((char*)M.ptr<T>(i, 0), (std::streamsize)W * sizeof(T));
+    fv.read((char*)V.ptr<T>(0), (std::streamsize)V.Len() * sizeof(T));
+    if (!fm || !fv) return 2;
+    if (mat_times_vec) de::blas::cuda::GEMM(M, V, Y, level); else de::blas::cuda::GEMM(V, M, Y, level);
+    if (de::GetLastError()->error_type != 0) { std::cerr << de::GetLastError()->error_string << "\n"; return 3; }
+    const size_t es = Y.Type() == de::_FP32_ ? 4 : 2;
+    if (Y.Len() != (mat_times_vec ? H : W)) return 4;
+    std::ofstream out(dir + "/Y.bin", std::ios::binary);
+    out.write((const char*)Y.ptr<char>(0), (std::streamsize)(Y.Len() * es));
+    return out ? 0 : 2;
+}
+
 template <typename T> static bool read_into(de::Matrix& m, const std::string& path)
 {
     std::ifstream f(path, std::ios::binary);
@@ -243,6 +404,14 @@ int main(int argc, char** argv)
     int rc;
     if (mode == "host") rc = host_checks();
     else if (mode == "gpu") rc = gpu_checks();
+    else if (mode == "vector_host") rc = vector_host_checks();
+    else if (mode == "vector_gpu") rc = vector_gpu_checks();
+    else if (mode == "vmm" && argc == 8) {
+        const bool f16 = std::string(argv[3]) == "f16", mv = std::string(argv[4]) == "mv";
+        const uint32_t W = std::atoi(argv[5]), H = std::atoi(argv[6]), level = std::atoi(argv[7]);
+        rc = f16 ? vmm_files<de::Half>(argv[2], de::_FP16_, mv, W, H, level)
+                 : vmm_files<float>(argv[2], de::_FP32_, mv, W, H, level);
+    }
     else if (mode == "gemm" && argc == 10) {
         const bool f16 = std::string(argv[3]) == "f16";
         const uint32_t M = std::atoi(argv[4]), N = std::atoi(argv[5]), K = std::atoi(argv[6]);
@@ -251,7 +420,8 @@ int main(int argc, char** argv)
         rc = f16 ? gemm_files<de::Half>(argv[2], de::_FP16_, M, N, K, with_c, alpha, beta)
                  : gemm_files<float>(argv[2], de::_FP32_, M, N, K, with_c, alpha, beta);
     } else {
-        std::cerr << "usage: de_api_test host | gpu | gemm <dir> <f32|f16> M N K withC alpha beta\n";
+        std::cerr << "usage: de_api_test host | gpu | vector_host | vector_gpu | gemm <dir> <f32|f16> M N K withC alpha beta"
+                     " | vmm <dir> <f32|f16> <mv|vm> W H level\n";
         return 64;
     }
     std::cout << (rc == 0 ? "de_api_test: all checks passed" : "de_api_test: FAILED") << " (" << mode << ")\n";

@@ -65,9 +65,12 @@ def test_planner_choices():
     assert p.edge == 1 and p.tile_m < 256 and p.grid == -(-1000 // p.tile_m) * -(-1500 // p.tile_n)
     assert hip.plan(4, 1024, 1024, 1024).tile_m < 256
     assert hip.plan(4, 1024, 1024, 1024, aligned=False).edge == 1
-    # N == 1 goes to the row-dot kernel (fp32 only)
-    assert hip.plan(4, 8192, 1, 8192).path == hip.PATH_GEMV
-    assert hip.plan(2, 8192, 1, 8192).path != hip.PATH_GEMV
+    # N == 1 goes to the row-dot kernel and M == 1 to the column-sum kernel, in both element types
+    for eb in (4, 2):
+        p = hip.plan(eb, 8192, 1, 8192)
+        assert (p.path, p.grid) == (hip.PATH_GEMV, 8192 // 32)
+        p = hip.plan(eb, 1, 8192, 8192)
+        assert (p.path, p.grid) == (hip.PATH_GEVM, 8192 // (128 // eb))
     assert hip.plan(4, 0, 5, 5).grid == 0
     bad = hip.Plan()
     assert hip.lib().decx_hip_gemm_plan(3, 4, 4, 4, 1, ctypes.byref(bad)) == -1
@@ -84,6 +87,9 @@ def test_compute_entry_points_refuse_to_run_uninitialised():
         "assert L.decx_hip_gemm_f32(p, p, None, p, 4, 4, 4, 4, 4, 0, 4, 1.0, 1.0, None) == -2;"
         "assert L.decx_hip_gemm_f16(p, p, None, p, 4, 4, 4, 4, 4, 0, 4, 1.0, 1.0, None) == -2;"
         "assert L.decx_hip_gemv_f32(p, p, None, p, 4, 4, 4, 1, 1, 1, 1.0, 1.0, None) == -2;"
+        "assert L.decx_hip_gevm_f32(p, p, None, p, 4, 4, 4, 1, 1, 1, 1.0, 1.0, None) == -2;"
+        "assert L.decx_hip_gemv_f16(p, p, None, p, 4, 4, 4, 1, 1, 1, 1.0, 1.0, 1, None) == -2;"
+        "assert L.decx_hip_gevm_f16(p, p, None, p, 4, 4, 4, 1, 1, 1, 1.0, 1.0, 0, None) == -2;"
         "assert L.decx_hip_malloc(ctypes.byref(q), 64) == -2;"
         "assert L.decx_hip_stream_create(ctypes.byref(q)) == -2;"
         "assert b'init' in L.decx_hip_error_string(-2)" % ROOT)

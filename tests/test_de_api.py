@@ -25,6 +25,11 @@ def test_host_side_objects_and_error_codes():
     assert rc == 0, out
 
 
+def test_host_side_vectors_and_error_codes():
+    rc, out = run_exe("vector_host")
+    assert rc == 0, out
+
+
 def test_host_library_exports_the_public_entry_points():
     lib = os.path.join(ROOT, "decx_amd", "lib", "libDECX_BLAS_HIP.so")
     syms = subprocess.run(["nm", "-D", "-C", "--defined-only", lib], stdout=subprocess.PIPE, text=True).stdout
@@ -35,7 +40,12 @@ def test_host_library_exports_the_public_entry_points():
                    "de::CreateMatrixRef(de::_DATA_TYPES_FLAGS_, unsigned int, unsigned int, de::_DATA_FORMATS_)",
                    "de::Memcpy(de::Matrix&, de::GPU_Matrix&, de::Point2D, de::Point2D, de::Point2D, int)",
                    "de::GetLastError()", "de::InitCuda()", "de::Float2Half(float const&)",
-                   "de::cuda::PinMemory(de::Matrix&)"]:
+                   "de::cuda::PinMemory(de::Matrix&)", "de::cuda::PinMemory(de::Vector&)",
+                   "de::blas::cuda::GEMM(de::Vector&, de::Matrix&, de::Vector&, unsigned int)",
+                   "de::blas::cuda::GEMM(de::Matrix&, de::Vector&, de::Vector&, unsigned int)",
+                   "de::CreateVectorRef(de::_DATA_TYPES_FLAGS_, unsigned long)",
+                   "de::CreateGPUVectorRef(de::_DATA_TYPES_FLAGS_, unsigned long)",
+                   "de::Memcpy(de::Vector&, de::GPU_Vector&, unsigned long, unsigned long, unsigned long, int)"]:
         assert needle in syms, needle
 
 
@@ -72,3 +82,41 @@ def test_gemm_through_the_objects_matches_oracle(oracle, dt, M, N, K, with_c, al
     ref = ref.astype(np.float64)
     err = np.max(np.abs(D.astype(np.float64) - ref)) / (np.max(np.abs(ref)) * np.sqrt(K))
     assert err <= tol
+
+
+@pytest.mark.gpu
+def test_gpu_side_vectors_closed_forms_and_error_paths():
+    rc, out = run_exe("vector_gpu")
+    assert rc == 0, out
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt,form,W,H,level", [
+    ("f32", "mv", 1030, 700, 0), ("f32", "vm", 1030, 700, 0),
+    ("f32", "mv", 8200, 33, 0), ("f32", "vm", 33, 8200, 0),
+    ("f16", "mv", 1030, 700, 0), ("f16", "vm", 1030, 700, 0),      # level 1: fp32 result
+    ("f16", "mv", 1030, 700, 1), ("f16", "vm", 1030, 700, 2),      # levels 2, 3: fp16 result
+])
+def test_vector_forms_through_the_objects_match_oracle(oracle, dt, form, W, H, level):
+    """de::blas::cuda::GEMM(Matrix, Vector, Vector) / (Vector, Matrix, Vector) on host objects against the
+    oracle's GEMM with one column / one row (fp16 inputs widened exactly to fp32)."""
+    n_in = W if form == "mv" else H
+    if dt == "f32":
+        M = synth.uniform_f32(H, W, 301); V = synth.uniform_f32(1, n_in, 302).reshape(-1)
+    else:
+        M = synth.normal_half(H, W, 301); V = synth.normal_half(1, n_in, 302).reshape(-1)
+    out_f32 = dt == "f32" or level == 0
+    with tempfile.TemporaryDirectory() as tmp:
+        M.tofile(os.path.join(tmp, "M.bin")); V.tofile(os.path.join(tmp, "V.bin"))
+        rc, out = run_exe("vmm", tmp, dt, form, W, H, level)
+        assert rc == 0, out
+        Y = np.fromfile(os.path.join(tmp, "Y.bin"), np.float32 if out_f32 else np.float16)
+    Mf, Vf = M.astype(np.float32), V.astype(np.float32)
+    ref = (oracle.gemm_f32(Mf, Vf.reshape(-1, 1)) if form == "mv" else oracle.gemm_f32(Vf.reshape(1, -1), Mf)).reshape(-1)
+    K = n_in
+    assert Y.shape == ref.shape
+    if not out_f32:
+        ref = ref.astype(np.float16)
+    ref = ref.astype(np.float64)
+    err = np.max(np.abs(Y.astype(np.float64) - ref)) / (np.max(np.abs(ref)) * np.sqrt(K))
+    assert err <= (1e-5 if out_f32 else 2e-3)
