@@ -25,12 +25,12 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 // Picks the block tile: cost = (tiles the busiest CU runs) x (tile area) / (relative speed
 // of that shape).  Big tiles win once they fill the chip; small tiles win while the grid
 // would otherwise leave CUs idle.  Ties go to the larger tile.
-int choose_tile(bool f16, uint32_t M, uint32_t N)
+int choose_tile(bool f16, uint32_t M, uint32_t N, bool aligned)
 {
     int best = TILE_64x64;
     double best_cost = 1e300;
     for (int s = TILE_COUNT - 1; s >= 0; --s) {
-        const TileInfo ti = f16 ? tile_info_f16(s) : tile_info_f32(s);
+        const TileInfo ti = f16 ? tile_info_f16(s) : tile_info_f32(s, aligned);
         const uint64_t tiles = (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
         const uint64_t per_cu = (tiles + g_dev.compute_units - 1) / g_dev.compute_units;
         const double cost = (double)per_cu * ti.bm * ti.bn / ti.rel_speed;
@@ -73,7 +73,7 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
     g.alpha = alpha; g.beta = beta;
     g.vec_ok = (aligned16(A) && aligned16(B) && aligned16(D) && (!C || aligned16(C)) &&
                 lda % per16 == 0 && ldb % per16 == 0 && ldd % per16 == 0 && (!C || ldc % per16 == 0)) ? 1u : 0u;
-    const int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile(F16, M, N) : tile;
+    const int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile(F16, M, N, g.vec_ok != 0) : tile;
     const bool edge = force_edge != 0 || K == 0;
     return F16 ? launch_gemm_f16(shape, edge, g, as_stream(stream))
                : launch_gemm_f32(shape, edge, g, as_stream(stream));
@@ -300,13 +300,14 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
         out->grid = (N + out->tile_n - 1) / out->tile_n;
         return DECX_HIP_OK;
     }
-    const int shape = choose_tile(f16, M, N);
+    const int shape = choose_tile(f16, M, N, aligned != 0);
     const TileInfo ti = f16 ? tile_info_f16(shape) : tile_info_f32(shape);
-    const uint32_t bk = f16 ? 64u : 16u;
     out->path = shape;
     out->tile_m = ti.bm; out->tile_n = ti.bn;
     out->grid = ((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
-    out->edge = (M % ti.bm || N % ti.bn || K % bk || K == 0 || !aligned) ? 1 : 0;
+    // fp32: the direct-to-LDS kernels take every aligned shape; fp16: full tiles only
+    if (f16) out->edge = (M % ti.bm || N % ti.bn || K % 64u || K == 0 || !aligned) ? 1 : 0;
+    else out->edge = (K == 0 || !aligned) ? 1 : 0;
     return DECX_HIP_OK;
 }
 

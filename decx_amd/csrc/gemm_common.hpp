@@ -60,30 +60,34 @@ enum TileShape : int {
     TILE_COUNT   = 3,
 };
 
-struct TileInfo { int bm, bn, threads; float rel_speed; int blocks_per_cu; };
+struct TileInfo { int bm, bn, threads; float rel_speed; };
 
 // rel_speed: per-CU throughput of the shape relative to the largest one once the chip is
-// full (smaller tiles re-read more operand data per flop and keep fewer MFMAs in flight).
-__host__ inline TileInfo tile_info_f32(int shape)
+// full (smaller tiles fetch more operand bytes per flop).  fp32, measured on MI355X at 2048^3 /
+// 3000^3: direct-to-LDS kernels 144 : 129 : 121 TFLOP/s, predicated register-staged kernels
+// (operands that are not 16-byte aligned) about 1 : 0.8 : 0.7.
+__host__ inline TileInfo tile_info_f32(int shape, bool aligned = true)
 {
     switch (shape) {
-    case TILE_256x256: return {256, 256, 512, 1.00f, 1};
-    case TILE_128x128: return {128, 128, 256, 0.80f, 2};
-    default:           return { 64,  64, 256, 0.45f, 4};
+    case TILE_256x256: return {256, 256, 512, 1.00f};
+    case TILE_128x128: return {128, 128, 256, aligned ? 0.90f : 0.80f};
+    default:           return { 64,  64, 256, aligned ? 0.85f : 0.70f};
     }
 }
 __host__ inline TileInfo tile_info_f16(int shape)
 {
     switch (shape) {
-    case TILE_256x256: return {256, 256, 256, 1.00f, 1};
-    case TILE_128x128: return {128, 128, 128, 0.60f, 2};
-    default:           return { 64,  64,  64, 0.25f, 4};
+    case TILE_256x256: return {256, 256, 256, 1.00f};
+    case TILE_128x128: return {128, 128, 128, 0.60f};
+    default:           return { 64,  64,  64, 0.25f};
     }
 }
 
 int launch_gemm_f32(int shape, bool edge, const GemmArgs& args, hipStream_t stream);
 // 256 x 256 x 16 direct-to-LDS fp32 kernel; full tiles only (the caller checks divisibility and alignment)
 int launch_gemm_f32_pipelined(const GemmArgs& args, hipStream_t stream);
+// direct-to-LDS fp32 kernel for any M, N, K >= 1 on 16-byte aligned bases and pitches, in the three tile shapes
+int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream);
 int launch_gemm_f16(int shape, bool edge, const GemmArgs& args, hipStream_t stream);
 // 256 x 256 x 64 direct-to-LDS kernel; full tiles only (the caller checks divisibility and alignment)
 int launch_gemm_f16_pipelined(const GemmArgs& args, hipStream_t stream);

@@ -1,4 +1,7 @@
-// fp32 GEMM for gfx950 on the fp32 matrix cores (v_mfma_f32_32x32x2_f32).
+// fp32 GEMM for gfx950 on the fp32 matrix cores (v_mfma_f32_32x32x2_f32): the register-staged
+// kernel.  It takes operands of any alignment (element loads where 128-bit ones would be
+// misaligned) and K == 0; 16-byte aligned operands, the usual case, go to the direct-to-LDS
+// kernels instead (launch_gemm_f32 below routes).
 //
 // Replaces the reference's SIMT kernels cu_GEMM_fp32_[F_]kernel_* and their transposed-A
 // variants (srcs/modules/BLAS/GEMM/CUDA/large_squares/fp32/GEMM_fp32_B128_kernels.cu,
@@ -251,6 +254,7 @@ static int launch_shape(bool edge, const GemmArgs& args, hipStream_t stream)
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
     g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
+    // the unpredicated variant serves full tiles only; with `edge` the caller asks for the predicated one anyway
     const bool full = (g.M % BM == 0) && (g.N % BN == 0) && (g.K % BK == 0) && g.vec_ok;
     const dim3 grid(nb), block(WAVES_M * WAVES_N * 64);
     if (edge || !full)
@@ -262,9 +266,11 @@ static int launch_shape(bool edge, const GemmArgs& args, hipStream_t stream)
 
 int launch_gemm_f32(int shape, bool edge, const GemmArgs& args, hipStream_t stream)
 {
-    if (shape == TILE_256x256 && !edge && args.vec_ok && args.K > 0 &&
-        args.M % 256 == 0 && args.N % 256 == 0 && args.K % 16 == 0)
-        return launch_gemm_f32_pipelined(args, stream);
+    if (!edge && args.vec_ok && args.K > 0) {
+        if (shape == TILE_256x256 && args.M % 256 == 0 && args.N % 256 == 0 && args.K % 16 == 0)
+            return launch_gemm_f32_pipelined(args, stream);
+        return launch_gemm_f32_dma(shape, args, stream);
+    }
     switch (shape) {
     case TILE_256x256: return launch_shape<256, 256, 16, 4, 2>(edge, args, stream);
     case TILE_128x128: return launch_shape<128, 128, 16, 2, 2>(edge, args, stream);

@@ -1,0 +1,373 @@
+// fp32 GEMM for gfx950, any M, N, K on 16-byte aligned operands: BM x BN block tiles whose K
+// slabs are copied global -> LDS by direct (LDS-DMA) 128-bit loads into a ring of STAGES
+// stages, ragged edges included.
+//
+// The arithmetic and the fragment scheme are those of the full-tile 256 x 256 kernel
+// (v_mfma_f32_32x32x2_f32; the lower / upper half-wave take k and k + 4 of each 8-deep
+// chunk; a lane's TN column tiles are TN adjacent columns).  What this kernel adds:
+//   * tile shapes down to 64 x 64 (four wavefronts of 32 x 32), so that small problems
+//     still put a workgroup on every CU; wave tiles that small issue one MFMA per k step,
+//     less than an LDS read takes, so their fragments are fetched a whole 8-deep chunk ahead;
+//   * ragged M and N without predicated loads: a copy lane whose row or column chunk
+//     lies outside the matrix fetches the last valid row / chunk instead (always mapped
+//     memory); what it brings lands in accumulators of rows / columns that are never stored;
+//   * ragged K: the last, partial slab goes through registers (zero-filled beyond K) into
+//     its LDS stage, so no product ever sees bytes from outside the operands.
+//
+// LDS layout of a stage: A as [BM rows][BK / 4 chunks of 16 bytes], chunk c of row r in
+// slot c ^ ((r / RP) % CPR) (CPR chunks per row, RP = 16 / CPR rows per 256 bytes): the
+// 128-bit fragment reads of 16 consecutive rows then cover 16 distinct 16-byte bank
+// groups.  B as [BK][BN] floats; for 32-column wave tiles the chunks of k rows 4..7 (mod 8)
+// are shifted by 128 bytes so the two half-waves read different banks.  Both permutations
+// are applied on the global side of the copy: a direct load always writes 1 KB contiguous.
+#include "gemm_common.hpp"
+#include <type_traits>
+
+namespace decx_hip {
+
+namespace {
+
+typedef __attribute__((address_space(3))) void lds_void;
+
+template <int I, int N, class F> __device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+template <int N> __device__ __forceinline__ void wait_loads_and_barrier()
+{
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(N) : "memory");
+}
+
+template <int TN> struct BFrag;
+template <> struct BFrag<1> { typedef float type; };
+template <> struct BFrag<2> { typedef floatx2 type; };
+template <> struct BFrag<4> { typedef floatx4 type; };
+
+template <int TN> __device__ __forceinline__ float lane_of(const typename BFrag<TN>::type& v, int j)
+{
+    if constexpr (TN == 1) return v; else return v[j];
+}
+
+}  // namespace
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD>
+__global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
+gemm_f32_dma_kernel(const GemmArgs g)
+{
+    constexpr int WAVES = WAVES_M * WAVES_N, NT = WAVES * 64;
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
+    constexpr int CPR = BK / 4, RP = 16 / CPR;                    // A chunks per row, rows per 256 bytes
+    constexpr int CB = BN / 4, RB = 64 / CB;                      // B chunks per k row, k rows per direct load
+    constexpr int A_STAGE_BYTES = BM * BK * 4, B_STAGE_BYTES = BK * BN * 4, STAGE_BYTES = A_STAGE_BYTES + B_STAGE_BYTES;
+    constexpr int A_LOADS = A_STAGE_BYTES / 1024 / WAVES, B_LOADS = B_STAGE_BYTES / 1024 / WAVES, LOADS = A_LOADS + B_LOADS;
+    constexpr int B_SHIFT = (TN == 1) ? 8 : 0;                    // chunk shift of k rows with bit 2 set
+    static_assert(TM >= 1 && (TN == 1 || TN == 2 || TN == 4), "wave tile");
+    static_assert(BK == 16 || BK == 32, "slab depth");
+    static_assert(CB <= 64 && 64 % CB == 0 && (B_SHIFT == 0 || CB >= 16), "B copy plan");
+    static_assert(A_LOADS >= 1 && B_LOADS >= 1 && A_LOADS * WAVES * 1024 == A_STAGE_BYTES &&
+                  B_LOADS * WAVES * 1024 == B_STAGE_BYTES, "copy plan must divide evenly");
+    static_assert(STAGES >= 2 && STAGES * STAGE_BYTES <= 160 * 1024, "LDS budget");
+    static_assert(LOADS * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE_BYTES];
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)lds;
+
+    uint32_t tile_m, tile_n;
+    block_to_tile(g, tile_m, tile_n);
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
+    const int l32 = lane & 31, h = lane >> 5;
+
+    const unsigned char* __restrict__ A = (const unsigned char*)g.A;
+    const unsigned char* __restrict__ B = (const unsigned char*)g.B;
+    const size_t lda_b = (size_t)g.lda * 4, ldb_b = (size_t)g.ldb * 4;
+
+    // ---- copy plan.  A direct load I covers rows (64 / CPR) I ..: lane -> row I * 64 / CPR + lane / CPR,
+    // slot lane % CPR, fetching chunk slot ^ ((row / RP) % CPR).  B direct load I covers k rows RB I ..:
+    // lane -> k row RB I + lane / CB, slot lane % CB, fetching column chunk slot ^ (B_SHIFT if k row & 4).
+    // Rows beyond M and column chunks beyond N are replaced by the last valid ones.
+    const unsigned char* a_src[A_LOADS];
+    const unsigned char* b_src[B_LOADS];
+    int a_chunk[A_LOADS], b_krow[B_LOADS];
+    const uint32_t last_row = g.M - 1, last_col_chunk = (g.N - 1) / 4;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+        const int I = wave * A_LOADS + i;
+        const int row = I * (64 / CPR) + lane / CPR;
+        a_chunk[i] = (lane % CPR) ^ ((row / RP) % CPR);
+        const uint32_t grow = (m0 + row) < last_row ? (m0 + row) : last_row;
+        a_src[i] = A + (size_t)grow * lda_b + a_chunk[i] * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+        const int I = wave * B_LOADS + i;
+        b_krow[i] = I * RB + lane / CB;
+        const int chunk = (lane % CB) ^ ((b_krow[i] & 4) ? B_SHIFT : 0);
+        const uint32_t gchunk = (n0 / 4 + chunk) < last_col_chunk ? (n0 / 4 + chunk) : last_col_chunk;
+        b_src[i] = B + (size_t)b_krow[i] * ldb_b + (size_t)gchunk * 16;
+    }
+
+    const uint32_t full_slabs = g.K / BK, k_tail = g.K % BK;
+    const uint32_t slabs = full_slabs + (k_tail ? 1u : 0u);
+
+    auto issue_loads = [&](uint32_t slab) {
+        const uint32_t stage = slab % STAGES;
+        if (slab < full_slabs) {
+            const uint32_t stage_off = lds_base + stage * STAGE_BYTES;
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) {
+                const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u);
+                const unsigned char* src = a_src[i] + (size_t)slab * (BK * 4);
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
+            }
+#pragma unroll
+            for (int i = 0; i < B_LOADS; ++i) {
+                const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + A_STAGE_BYTES +
+                                                                    (uint32_t)(wave * B_LOADS + i) * 1024u);
+                const unsigned char* src = b_src[i] + (size_t)slab * BK * ldb_b;
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
+            }
+        } else {
+            // the partial last slab: through registers, zero beyond K
+            unsigned char* st = lds + stage * STAGE_BYTES;
+            const uint32_t k0 = full_slabs * BK;
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) {
+                const uint32_t k = k0 + a_chunk[i] * 4;
+                floatx4 v = floatx4{0.f, 0.f, 0.f, 0.f};
+                if (k < g.K) {
+                    v = *(const floatx4*)(a_src[i] + (size_t)k0 * 4);      // inside the pitch: lda is a multiple of 4
+#pragma unroll
+                    for (int e = 1; e < 4; ++e) if (k + e >= g.K) v[e] = 0.f;
+                }
+                *(floatx4*)(st + (wave * A_LOADS + i) * 1024 + lane * 16) = v;
+            }
+#pragma unroll
+            for (int i = 0; i < B_LOADS; ++i) {
+                floatx4 v = floatx4{0.f, 0.f, 0.f, 0.f};
+                if (k0 + b_krow[i] < g.K) v = *(const floatx4*)(b_src[i] + (size_t)k0 * ldb_b);
+                *(floatx4*)(st + A_STAGE_BYTES + (wave * B_LOADS + i) * 1024 + lane * 16) = v;
+            }
+        }
+    };
+
+    // ---- fragment addressing inside a stage
+    const int a_row = wm0 + l32;                       // + 32 i leaves (row / RP) % CPR unchanged
+    const int a_sw = (a_row / RP) % CPR;
+    int a_off[BK / 8];                                 // byte offset of chunk 2 c + h of this lane's row
+#pragma unroll
+    for (int c = 0; c < BK / 8; ++c) a_off[c] = a_row * (BK * 4) + (((2 * c + h) ^ a_sw) * 16);
+    const int b_col = wn0 + TN * l32;
+    const int b_off = A_STAGE_BYTES + (4 * h) * BN * 4 + (((b_col / 4) ^ (h ? B_SHIFT : 0)) * 16) + (b_col % 4) * 4;
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+#pragma unroll
+    for (int p = 0; p < STAGES - 1; ++p)
+        if ((uint32_t)p < slabs) issue_loads(p);
+    if (slabs >= (uint32_t)(STAGES - 1)) wait_loads_and_barrier<LOADS * (STAGES - 2)>();
+    else wait_loads_and_barrier<0>();
+
+    constexpr int STEPS = BK / 2, CHUNKS = BK / 8;
+    typedef typename BFrag<TN>::type bfrag;
+
+    if constexpr (!CHUNK_AHEAD) {
+        // Large wave tiles: a k step is TM * TN MFMAs, long enough to hide an LDS read, so fragments
+        // are fetched one step ahead.  af[c & 1] holds chunk c of A (4 k per lane), bf[step & 1] the
+        // B values of a k step.  The MFMAs of the last step of a slab are issued after the slab
+        // barrier, behind the first fragment reads of the next slab (before the first slab they
+        // multiply zeros).
+        floatx4 af[2][TM];
+        bfrag bf[2];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) af[(CHUNKS - 1) & 1][i] = floatx4{0.f, 0.f, 0.f, 0.f};
+        bf[(STEPS - 1) & 1] = bfrag{};
+
+        auto multiply = [&](auto stc) {
+            constexpr int step = decltype(stc)::value;
+            constexpr int c = step / 4, e = step % 4;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c & 1][i][e], lane_of<TN>(bf[step & 1], j), acc[i][j], 0, 0, 0);
+        };
+
+        for (uint32_t s = 0; s < slabs; ++s) {
+            const unsigned char* st = lds + (s % STAGES) * STAGE_BYTES;
+            const bool more = s + STAGES - 1 < slabs;
+
+#pragma unroll
+            for (int i = 0; i < TM; ++i) af[0][i] = *(const floatx4*)(st + a_off[0] + i * 32 * BK * 4);
+            bf[0] = *(const bfrag*)(st + b_off);
+            multiply(std::integral_constant<int, STEPS - 1>{});
+            __builtin_amdgcn_sched_group_barrier(0x100, TM + 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            // the stage that held slab s-1 is free: every wave passed the barrier after reading it
+            if (more) issue_loads(s + STAGES - 1);
+
+            static_for<0, STEPS - 1>([&](auto stc) {
+                constexpr int step = decltype(stc)::value;
+                constexpr int c = step / 4, e = step % 4;
+                constexpr bool next_a = (e == 1) && (c + 1 < CHUNKS);
+                constexpr int reads = 1 + (next_a ? TM : 0);
+                bf[(step + 1) & 1] = *(const bfrag*)(st + b_off + (8 * ((step + 1) / 4) + (step + 1) % 4) * BN * 4);
+                if constexpr (next_a) {
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) af[(c + 1) & 1][i] = *(const floatx4*)(st + a_off[c + 1] + i * 32 * BK * 4);
+                }
+                multiply(stc);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, reads, 0);
+                if constexpr (TM * TN > 1) __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 1, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+
+            // slab s+1 must have landed (ours: vmcnt; everyone's: barrier); the loads of the
+            // STAGES-2 slabs behind it may stay in flight.
+            if (more) wait_loads_and_barrier<LOADS * (STAGES - 2)>(); else wait_loads_and_barrier<0>();
+        }
+        multiply(std::integral_constant<int, STEPS - 1>{});
+    } else {
+        // Small wave tiles: a k step is one or two MFMAs, shorter than an LDS read, so fragments are
+        // fetched a whole 8-deep chunk (4 steps) ahead: fa[c & 1] / fb[c & 1] hold chunk c.  The last
+        // chunk of a slab is multiplied after the slab barrier, behind the reads of the next slab's
+        // first chunk.
+        floatx4 fa[2][TM];
+        bfrag fb[2][4];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[(CHUNKS - 1) & 1][i] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) fb[(CHUNKS - 1) & 1][e] = bfrag{};
+
+        auto read_chunk = [&](const unsigned char* st, auto cc) {
+            constexpr int c = decltype(cc)::value;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) fa[c & 1][i] = *(const floatx4*)(st + a_off[c] + i * 32 * BK * 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) fb[c & 1][e] = *(const bfrag*)(st + b_off + (8 * c + e) * BN * 4);
+        };
+        auto multiply_chunk = [&](auto cc) {
+            constexpr int c = decltype(cc)::value;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[c & 1][i][e], lane_of<TN>(fb[c & 1][e], j), acc[i][j], 0, 0, 0);
+        };
+        constexpr int READS = TM + 4, MFMAS = 4 * TM * TN;
+
+        for (uint32_t s = 0; s < slabs; ++s) {
+            const unsigned char* st = lds + (s % STAGES) * STAGE_BYTES;
+            const bool more = s + STAGES - 1 < slabs;
+
+            read_chunk(st, std::integral_constant<int, 0>{});
+            multiply_chunk(std::integral_constant<int, CHUNKS - 1>{});
+            __builtin_amdgcn_sched_group_barrier(0x100, READS, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (more) issue_loads(s + STAGES - 1);
+
+            static_for<0, CHUNKS - 1>([&](auto cc) {
+                constexpr int c = decltype(cc)::value;
+                read_chunk(st, std::integral_constant<int, c + 1>{});
+                multiply_chunk(cc);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, READS, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - 1, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+
+            if (more) wait_loads_and_barrier<LOADS * (STAGES - 2)>(); else wait_loads_and_barrier<0>();
+        }
+        multiply_chunk(std::integral_constant<int, CHUNKS - 1>{});
+    }
+
+    // Epilogue: register r of lane (l32, h) is row 8*(r/4) + 4*h + r%4 of a 32x32 tile; the
+    // lane's TN tiles are TN adjacent columns.
+    const float* __restrict__ C = (const float*)g.C;
+    float* __restrict__ D = (float*)g.D;
+    const uint32_t col0 = n0 + b_col;
+    const bool interior = (m0 + BM <= g.M) && (n0 + BN <= g.N);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const uint32_t row = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+            float v[TN];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) v[j] = acc[i][j][r];
+            if (interior) {
+                if (C) {
+                    const bfrag cv = *(const bfrag*)(C + (size_t)row * g.ldc + col0);
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) v[j] = __builtin_fmaf(lane_of<TN>(cv, j), g.beta, g.alpha * v[j]);
+                }
+                bfrag o;
+                if constexpr (TN == 1) o = v[0];
+                else {
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) o[j] = v[j];
+                }
+                *(bfrag*)(D + (size_t)row * g.ldd + col0) = o;
+            } else if (row < g.M) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    if (col0 + j < g.N) {
+                        float o = v[j];
+                        if (C) o = __builtin_fmaf(C[(size_t)row * g.ldc + col0 + j], g.beta, g.alpha * o);
+                        D[(size_t)row * g.ldd + col0 + j] = o;
+                    }
+                }
+            }
+        }
+    }
+}
+
+namespace {
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD>
+int launch_dma(const GemmArgs& args, hipStream_t stream)
+{
+    GemmArgs g = args;
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    const uint32_t nb = g.tiles_m * g.tiles_n;
+    g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
+    hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD>), dim3(nb), dim3(WAVES_M * WAVES_N * 64),
+                       0, stream, g);
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
+// M, N, K >= 1; 16-byte aligned bases and pitches (the caller checks).  Measured on MI355X: the
+// 64 x 64 tile runs best with 32-deep slabs in a 4-stage ring (two workgroups per CU) and
+// chunk-ahead fragments; deeper rings and a second accumulator chain changed nothing, its ceiling
+// is the L2 -> LDS rate (16 flop per byte fetched).  The 128 x 128 tile measures the same with 4 or
+// 8 wavefronts and 16- or 32-deep slabs.
+int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
+{
+    switch (shape) {
+    case TILE_256x256: return launch_dma<256, 256, 4, 2, 16, 4, false>(args, stream);
+    case TILE_128x128: return launch_dma<128, 128, 2, 2, 16, 4, true>(args, stream);
+    case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 32, 4, true>(args, stream);
+    default:           return (int)hipErrorInvalidValue;
+    }
+}
+
+}  // namespace decx_hip

@@ -13,7 +13,7 @@
 //
 // gemv: 16 wavefronts per workgroup, two rows per wavefront (32 rows per workgroup: 8192
 //   rows give one workgroup per CU with 64 KB of A in flight); x is staged in LDS once per
-//   workgroup, as fp32, in chunks of 8192 -- x may be strided (the single column of a
+//   workgroup, as fp32, in chunks of 4096 -- x may be strided (the single column of a
 //   pitched K x 1 matrix puts every element in its own cache line), so staging it once per
 //   32 rows keeps that gather small; A is read with 128-bit loads; per lane an fp32 fma
 //   chain, then a butterfly over the 64 lanes.
@@ -30,7 +30,7 @@ namespace {
 constexpr int GEMV_THREADS = 1024;
 constexpr int GEMV_WAVES = GEMV_THREADS / 64;
 constexpr int GEMV_ROWS_PER_BLOCK = 2 * GEMV_WAVES;
-constexpr int GEMV_KC = 8192;            // floats of x staged per chunk (32 KB of LDS)
+constexpr int GEMV_KC = 4096;            // floats of x staged per chunk (16 KB of LDS)
 
 template <typename T> struct Per16 { static constexpr int n = 16 / sizeof(T); };
 
@@ -73,23 +73,37 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
     const T* a1 = A + (size_t)(has1 ? row0 + 1 : 0) * lda;
     float s0 = 0.f, s1 = 0.f;
 
-    for (uint32_t kc = 0; kc < K; kc += GEMV_KC) {
+    // Every workgroup walks the same K range of rows that lie a whole number of pitches apart; started
+    // together at k = 0 they would all pull on the same memory channels at the same time.  So each
+    // workgroup starts at another chunk and each wavefront at another step inside it (sums commute).
+    const uint32_t chunks = (K + GEMV_KC - 1) / GEMV_KC;
+    const uint32_t chunk0 = chunks ? (blockIdx.x * 3u) % chunks : 0u;
+    for (uint32_t ci = 0; ci < chunks; ++ci) {
+        const uint32_t chunk = chunk0 + ci < chunks ? chunk0 + ci : chunk0 + ci - chunks;
+        const uint32_t kc = chunk * GEMV_KC;
         const uint32_t len = (K - kc) < (uint32_t)GEMV_KC ? (K - kc) : (uint32_t)GEMV_KC;
         __syncthreads();                                   // previous chunk fully consumed
         for (uint32_t i = t; i < len; i += GEMV_THREADS) xs[i] = to_float(x[(size_t)(kc + i) * incx]);
         __syncthreads();
         const uint32_t lenv = vec_ok ? (len / N16) * N16 : 0u;   // part done with 128-bit loads
         if (has0) {
+            constexpr uint32_t STEP = 64 * N16;
+            const uint32_t steps = (lenv + STEP - 1) / STEP;
+            const uint32_t step0 = steps ? ((blockIdx.x * GEMV_WAVES + wave) * 5u) % steps : 0u;
 #pragma unroll 4
-            for (uint32_t k = lane * N16; k < lenv; k += 64 * N16) {
-                float av[N16], bv[N16];
-                load16<T>(a0 + kc + k, av);
-                if (has1) load16<T>(a1 + kc + k, bv);
+            for (uint32_t i = 0; i < steps; ++i) {
+                const uint32_t step = step0 + i < steps ? step0 + i : step0 + i - steps;
+                const uint32_t k = step * STEP + lane * N16;
+                if (k < lenv) {
+                    float av[N16], bv[N16];
+                    load16<T>(a0 + kc + k, av);
+                    if (has1) load16<T>(a1 + kc + k, bv);
 #pragma unroll
-                for (int e = 0; e < N16; ++e) {
-                    const float xv = xs[k + e];
-                    s0 = __builtin_fmaf(av[e], xv, s0);
-                    if (has1) s1 = __builtin_fmaf(bv[e], xv, s1);
+                    for (int e = 0; e < N16; ++e) {
+                        const float xv = xs[k + e];
+                        s0 = __builtin_fmaf(av[e], xv, s0);
+                        if (has1) s1 = __builtin_fmaf(bv[e], xv, s1);
+                    }
                 }
             }
             for (uint32_t k = lenv + lane; k < len; k += 64) {
@@ -138,7 +152,7 @@ gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restric
         for (uint32_t i = t; i < len; i += GEMV_THREADS) xs[i] = to_float(x[(size_t)(kc + i) * incx]);
         __syncthreads();
         if (n0 < N) {
-#pragma unroll 4
+#pragma unroll 2
             for (uint32_t k = wave * 8 + row_lane; k < len; k += GEMV_WAVES * 8) {
                 const T* p = B + (size_t)(kc + k) * ldb + n0;
                 const float xv = xs[k];

@@ -185,6 +185,28 @@ def test_f32_ragged_shapes_every_tile(hip, oracle, M, N, K, tile):
     assert rel_err(run(hip, A, B, C, 1.5, -0.5, tile=tile), oracle.gemm_f32(A, B, C, 1.5, -0.5), K) <= TOL_F32
 
 
+@pytest.mark.parametrize("K", [2, 5, 8, 15, 16, 17, 31, 32, 33, 47, 48, 63, 64, 65, 101, 130])
+@pytest.mark.parametrize("tile", [0, 1, 2])
+def test_f32_every_k_remainder(hip, oracle, K, tile):
+    """K around the slab depths (16 and 32): full slabs only, a partial last slab only, both; the pitch
+    padding next to the last k holds NaN, so a product that reads past K shows."""
+    M, N = 70, 91
+    A = synth.uniform_f32(M, K, 161); B = synth.uniform_f32(K, N, 162); C = synth.uniform_f32(M, N, 163)
+    assert rel_err(run(hip, A, B, tile=tile), oracle.gemm_f32(A, B), K) <= TOL_F32
+    assert rel_err(run(hip, A, B, C, -1.0, 0.5, tile=tile), oracle.gemm_f32(A, B, C, -1.0, 0.5), K) <= TOL_F32
+
+
+def test_f32_large_ragged_sampled(hip, oracle):
+    """A ragged problem large enough for several rounds of workgroups per CU, planner's choice of tile."""
+    M, N, K = 3001, 2903, 3107
+    A = synth.uniform_f32(M, K, 171); B = synth.uniform_f32(K, N, 172)
+    rows = sample_rows(M, 192, 7)
+    got = run(hip, A, B)
+    assert rel_err(got[rows], oracle.gemm_f32(A, B, rows=rows), K) <= TOL_F32
+    colsum = A.astype(np.float64).sum(axis=0) @ B.astype(np.float64)       # checksum over all rows
+    assert np.max(np.abs(got.astype(np.float64).sum(axis=0) - colsum)) / np.max(np.abs(colsum)) < 1e-5
+
+
 @pytest.mark.parametrize("M,N,K", SHAPES)
 @pytest.mark.parametrize("tile", [0, 1, 2])
 def test_f16_ragged_shapes_every_tile(hip, oracle, M, N, K, tile):
