@@ -30,7 +30,7 @@ int choose_tile(bool f16, uint32_t M, uint32_t N, bool aligned)
     int best = TILE_64x64;
     double best_cost = 1e300;
     for (int s = TILE_COUNT - 1; s >= 0; --s) {
-        const TileInfo ti = f16 ? tile_info_f16(s) : tile_info_f32(s, aligned);
+        const TileInfo ti = f16 ? tile_info_f16(s, aligned) : tile_info_f32(s, aligned);
         const uint64_t tiles = (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
         const uint64_t per_cu = (tiles + g_dev.compute_units - 1) / g_dev.compute_units;
         const double cost = (double)per_cu * ti.bm * ti.bn / ti.rel_speed;
@@ -305,9 +305,8 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
     out->path = shape;
     out->tile_m = ti.bm; out->tile_n = ti.bn;
     out->grid = ((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
-    // fp32: the direct-to-LDS kernels take every aligned shape; fp16: full tiles only
-    if (f16) out->edge = (M % ti.bm || N % ti.bn || K % 64u || K == 0 || !aligned) ? 1 : 0;
-    else out->edge = (K == 0 || !aligned) ? 1 : 0;
+    // the direct-to-LDS kernels take every aligned shape
+    out->edge = (K == 0 || !aligned) ? 1 : 0;
     return DECX_HIP_OK;
 }
 

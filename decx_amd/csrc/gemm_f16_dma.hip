@@ -1,0 +1,364 @@
+// fp16 GEMM (fp32 accumulate, fp16 out) for gfx950, any M, N, K on 16-byte aligned operands:
+// BM x BN block tiles whose K slabs are copied global -> LDS by direct (LDS-DMA) 128-bit
+// loads into a ring of STAGES stages, ragged edges included.
+//
+// Replaces the reference's cu_GEMM_fp16_[F_]kernel_* family and the transpose pass in front of
+// its "_T" kernels (srcs/modules/BLAS/GEMM/CUDA/large_squares/fp16/, srcs/common/Basic_process/
+// transpose/CUDA/transpose_kernels.cuh:204-236).
+//
+// v_mfma_f32_32x32x16_f16 takes 8 consecutive k per lane for BOTH operands.  A (row-major M x K)
+// has them contiguous: A fragments are 128-bit LDS reads.  B (row-major K x N) does not; its
+// fragments come from the transposing read `ds_read_b64_tr_b16` straight out of the row-major B
+// slab: a group of 16 lanes hands in the addresses of a 4 (k) x 16 (n) block (lane s: row s / 4,
+// 8-byte segment s % 4) and lane i receives column i of it, 4 consecutive k of one n; two such
+// reads give the 8 k a lane needs.  So neither a transpose pass nor a register shuffle is needed.
+// The MFMA is issued with its operands swapped (B fragment first): it then produces the transposed
+// 32 x 32 tile, in which a lane owns adjacent columns of one output row, and the epilogue stores
+// 16 bytes per lane after one `v_permlane32_swap`.
+//
+// Slabs reach LDS by `global_load_lds_dwordx4` (no VGPRs, no ds_write).  These are inline assembly
+// and the slab barrier is a bare `s_barrier` behind an explicit vmcnt wait, because the compiler
+// would otherwise drain every outstanding load in front of each LDS read and at each
+// __syncthreads(); `sched_group_barrier` pins the MFMA / LDS-read alternation.
+//   * tile shapes from 256 x 256 down to 64 x 64, so small problems still cover the chip;
+//   * ragged M and N without predicated loads: a copy lane whose row or column chunk lies outside
+//     the matrix fetches the last valid row / chunk (mapped memory); what it brings only reaches
+//     accumulators of rows / columns that are never stored;
+//   * ragged K: the partial last slab goes through registers, zero-filled beyond K.
+//
+// LDS layout of a stage.  A: [BM rows][CPR chunks of 16 bytes], chunk c of row r in slot
+// c ^ ((r / RPB) % CPR).  B: [BK k rows][BN / 8 chunks], chunk c of row k in slot c ^ key(k),
+// key(k) = 4 (k & 3) for rows of 256 bytes or more and 4 ((k >> 1) & 1) for 128-byte rows, so
+// that the 4 k rows x 64 bytes a half-wave reads through the transposing read cover all banks
+// once.  Both permutations are applied on the global side of the copy.
+#include "gemm_common.hpp"
+#include <type_traits>
+
+namespace decx_hip {
+
+namespace {
+
+typedef __attribute__((address_space(3))) void lds_void;
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
+
+__device__ __forceinline__ halfx8 join(shortx4 lo, shortx4 hi)
+{
+    union { struct { shortx4 a, b; } s; halfx8 v; } u;
+    u.s.a = lo; u.s.b = hi;
+    return u.v;
+}
+
+template <int I, int N, class F> __device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+template <int N> __device__ __forceinline__ void wait_loads_and_barrier()
+{
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(N) : "memory");
+}
+
+constexpr int SG_MFMA = 0x008, SG_DS_READ = 0x100;
+
+// `mfmas` MFMAs and `reads` LDS reads, alternating one to one while both last
+template <int MFMAS, int READS> __device__ __forceinline__ void interleave()
+{
+    constexpr int PAIRS = MFMAS < READS ? MFMAS : READS;
+    static_for<0, PAIRS>([&](auto) {
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(SG_DS_READ, 1, 0);
+    });
+    if constexpr (READS > PAIRS) __builtin_amdgcn_sched_group_barrier(SG_DS_READ, READS - PAIRS, 0);
+    if constexpr (MFMAS > PAIRS) __builtin_amdgcn_sched_group_barrier(SG_MFMA, MFMAS - PAIRS, 0);
+}
+
+}  // namespace
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES>
+__global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
+gemm_f16_dma_kernel(const GemmArgs g)
+{
+    constexpr int WAVES = WAVES_M * WAVES_N;
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
+    constexpr int RB = BK * 2, CPR = RB / 16, RPB = 16 / CPR;         // A row bytes, chunks per row, rows per 256 bytes
+    constexpr int BRB = BN * 2, CBR = BRB / 16, BROWS = 1024 / BRB;   // B row bytes, chunks per row, k rows per direct load
+    constexpr int A_STAGE_BYTES = BM * RB, B_STAGE_BYTES = BK * BRB, STAGE_BYTES = A_STAGE_BYTES + B_STAGE_BYTES;
+    constexpr int A_LOADS = A_STAGE_BYTES / 1024 / WAVES, B_LOADS = B_STAGE_BYTES / 1024 / WAVES, LOADS = A_LOADS + B_LOADS;
+    constexpr int KS = BK / 16;                                       // MFMA k steps per slab
+    static_assert(TM >= 1 && TN >= 1 && (BK == 32 || BK == 64) && KS % 2 == 0, "shape");
+    static_assert(BN == 64 || BN == 128 || BN == 256, "B row must be 128, 256 or 512 bytes");
+    static_assert(A_LOADS >= 1 && B_LOADS >= 1 && A_LOADS * WAVES * 1024 == A_STAGE_BYTES &&
+                  B_LOADS * WAVES * 1024 == B_STAGE_BYTES, "copy plan must divide evenly");
+    static_assert(STAGES >= 2 && STAGES * STAGE_BYTES <= 160 * 1024, "LDS budget");
+    static_assert(LOADS * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE_BYTES];
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)lds;
+
+    uint32_t tile_m, tile_n;
+    block_to_tile(g, tile_m, tile_n);
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
+    const int l32 = lane & 31, h = lane >> 5;
+
+    const unsigned char* __restrict__ A = (const unsigned char*)g.A;
+    const unsigned char* __restrict__ B = (const unsigned char*)g.B;
+    const size_t lda_b = (size_t)g.lda * 2, ldb_b = (size_t)g.ldb * 2;
+
+    auto b_key = [](int k) { return BN >= 128 ? 4 * (k & 3) : 4 * ((k >> 1) & 1); };
+
+    // ---- copy plan (rows beyond M and column chunks beyond N are replaced by the last valid ones)
+    const unsigned char* a_src[A_LOADS];
+    const unsigned char* b_src[B_LOADS];
+    int a_chunk[A_LOADS], b_krow[B_LOADS];
+    const uint32_t last_row = g.M - 1, last_col_chunk = (g.N - 1) / 8;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+        const int I = wave * A_LOADS + i;
+        const int row = (64 / CPR) * I + lane / CPR;
+        a_chunk[i] = (lane % CPR) ^ ((row / RPB) % CPR);
+        const uint32_t grow = (m0 + row) < last_row ? (m0 + row) : last_row;
+        a_src[i] = A + (size_t)grow * lda_b + a_chunk[i] * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+        const int I = wave * B_LOADS + i;
+        b_krow[i] = BROWS * I + lane / CBR;
+        const int chunk = (lane % CBR) ^ b_key(b_krow[i]);
+        const uint32_t gchunk = (n0 / 8 + chunk) < last_col_chunk ? (n0 / 8 + chunk) : last_col_chunk;
+        b_src[i] = B + (size_t)b_krow[i] * ldb_b + (size_t)gchunk * 16;
+    }
+
+    const uint32_t full_slabs = g.K / BK, k_tail = g.K % BK;
+    const uint32_t slabs = full_slabs + (k_tail ? 1u : 0u);
+
+    auto issue_loads = [&](uint32_t slab) {
+        const uint32_t stage = slab % STAGES;
+        if (slab < full_slabs) {
+            const uint32_t stage_off = lds_base + stage * STAGE_BYTES;
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) {
+                const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u);
+                const unsigned char* src = a_src[i] + (size_t)slab * RB;
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
+            }
+#pragma unroll
+            for (int i = 0; i < B_LOADS; ++i) {
+                const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + A_STAGE_BYTES +
+                                                                    (uint32_t)(wave * B_LOADS + i) * 1024u);
+                const unsigned char* src = b_src[i] + (size_t)slab * BK * ldb_b;
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
+            }
+        } else {
+            // the partial last slab: through registers, zero beyond K
+            unsigned char* st = lds + stage * STAGE_BYTES;
+            const uint32_t k0 = full_slabs * BK;
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) {
+                const uint32_t k = k0 + a_chunk[i] * 8;
+                halfx8 v = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
+                if (k < g.K) {
+                    v = *(const halfx8*)(a_src[i] + (size_t)k0 * 2);      // inside the pitch: lda is a multiple of 8
+#pragma unroll
+                    for (int e = 1; e < 8; ++e) if (k + e >= g.K) v[e] = (_Float16)0;
+                }
+                *(halfx8*)(st + (wave * A_LOADS + i) * 1024 + lane * 16) = v;
+            }
+#pragma unroll
+            for (int i = 0; i < B_LOADS; ++i) {
+                halfx8 v = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
+                if (k0 + b_krow[i] < g.K) v = *(const halfx8*)(b_src[i] + (size_t)k0 * ldb_b);
+                *(halfx8*)(st + A_STAGE_BYTES + (wave * B_LOADS + i) * 1024 + lane * 16) = v;
+            }
+        }
+    };
+
+    // ---- fragment addressing (byte offsets inside a stage)
+    // A fragment (tile i, k step ks): row = wm0 + 32 i + l32, chunk = 2 ks + h.
+    const int a_row = wm0 + l32;
+    const int a_sw = (a_row / RPB) % CPR;
+    const int a_off = a_row * RB;
+    // B fragment (tile j, k step ks, half r): a 16-lane group handles the n half (lane >> 4) & 1;
+    // lane s = lane & 15 supplies k = 16 ks + 8 h + 4 r + s / 4 and the 8-byte segment s % 4 of the
+    // 16 columns starting at wn0 + 32 j + 16 * nhalf.
+    const int s16 = lane & 15;
+    const int bk_row = 8 * h + (s16 >> 2);
+    const int bk_col = wn0 + 16 * ((lane >> 4) & 1) + 4 * (s16 & 3);
+    const int bk_sw = b_key(bk_row);                       // unchanged by + 16 ks + 4 r
+    int b_off[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int col = bk_col + 32 * j;
+        b_off[j] = A_STAGE_BYTES + bk_row * BRB + (((col >> 3) ^ bk_sw) * 16) + (col & 7) * 2;
+    }
+
+    struct Frags { halfx8 a[TM], b[TN]; };
+    auto read_frags = [&](Frags& f, const unsigned char* st, int ks) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) f.a[i] = *(const halfx8*)(st + a_off + i * 32 * RB + (((2 * ks + h) ^ a_sw) * 16));
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const unsigned char* p0 = st + b_off[j] + ks * 16 * BRB;
+            const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)p0);
+            const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(p0 + 4 * BRB));
+            f.b[j] = join(lo, hi);
+        }
+    };
+
+    floatx16 accT[TN][TM];                                 // n tile j, m tile i, transposed
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) accT[j][i][r] = 0.f;
+
+    auto multiply = [&](const Frags& f) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                accT[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.b[j], f.a[i], accT[j][i], 0, 0, 0);
+    };
+    constexpr int MFMAS = TM * TN, READS = TM + 2 * TN;
+
+#pragma unroll
+    for (int p = 0; p < STAGES - 1; ++p)
+        if ((uint32_t)p < slabs) issue_loads(p);
+    if (slabs >= (uint32_t)(STAGES - 1)) wait_loads_and_barrier<LOADS * (STAGES - 2)>();
+    else wait_loads_and_barrier<0>();
+
+    // fr[ks & 1] holds the fragments of k step ks.  The last step of a slab is multiplied after
+    // the slab barrier, behind the fragment reads of the next slab's first step (before the first
+    // slab it multiplies zeros).
+    Frags fr[2];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fr[(KS - 1) & 1].a[i] = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fr[(KS - 1) & 1].b[j] = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
+
+    for (uint32_t s = 0; s < slabs; ++s) {
+        const unsigned char* st = lds + (s % STAGES) * STAGE_BYTES;
+        const bool more = s + STAGES - 1 < slabs;
+
+        read_frags(fr[0], st, 0);
+        multiply(fr[(KS - 1) & 1]);
+        interleave<MFMAS, READS>();
+        __builtin_amdgcn_sched_barrier(0);
+        // the stage that held slab s-1 is free: every wave passed the barrier after reading it
+        if (more) issue_loads(s + STAGES - 1);
+
+        static_for<0, KS - 1>([&](auto kc) {
+            constexpr int ks = decltype(kc)::value;
+            read_frags(fr[(ks + 1) & 1], st, ks + 1);
+            multiply(fr[ks & 1]);
+            interleave<MFMAS, READS>();
+            __builtin_amdgcn_sched_barrier(0);
+        });
+
+        if (more) wait_loads_and_barrier<LOADS * (STAGES - 2)>(); else wait_loads_and_barrier<0>();
+    }
+    multiply(fr[(KS - 1) & 1]);
+
+    // Epilogue.  Lane (l32, h) holds output row l32 of the m tile; register 4 q + e is column
+    // 8 q + 4 h + e of the n tile.  Interior tiles: `v_permlane32_swap` trades the halves of an even
+    // and an odd 8-column group between lane l and lane l + 32, after which each lane stores 16 bytes.
+    const _Float16* __restrict__ C = (const _Float16*)g.C;
+    _Float16* __restrict__ D = (_Float16*)g.D;
+    auto pack2 = [](float lo, float hi) -> uint32_t {
+        union { _Float16 f[2]; uint32_t u; } w;
+        w.f[0] = (_Float16)lo; w.f[1] = (_Float16)hi;
+        return w.u;
+    };
+    const bool interior = (m0 + BM <= g.M) && (n0 + BN <= g.N);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const uint32_t row = m0 + wm0 + 32 * i + l32;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            if (interior) {
+#pragma unroll
+                for (int qp = 0; qp < 2; ++qp) {
+                    uint32_t w[2][2];                      // [even / odd group][dword]
+#pragma unroll
+                    for (int o = 0; o < 2; ++o) {
+                        const int q = 2 * qp + o;
+                        float v[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = accT[j][i][4 * q + e];
+                        if (C) {
+                            const uint32_t col = n0 + wn0 + 32 * j + 8 * q + 4 * h;
+                            const halfx4 cv = *(const halfx4*)(C + (size_t)row * g.ldc + col);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf((float)cv[e], g.beta, g.alpha * v[e]);
+                        }
+                        w[o][0] = pack2(v[0], v[1]);
+                        w[o][1] = pack2(v[2], v[3]);
+                    }
+                    const auto s0 = __builtin_amdgcn_permlane32_swap(w[0][0], w[1][0], false, false);
+                    const auto s1 = __builtin_amdgcn_permlane32_swap(w[0][1], w[1][1], false, false);
+                    const uintx4 out = {s0[0], s1[0], s0[1], s1[1]};
+                    const uint32_t col = n0 + wn0 + 32 * j + 8 * (2 * qp + h);
+                    *(uintx4*)(D + (size_t)row * g.ldd + col) = out;
+                }
+            } else if (row < g.M) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t col = n0 + wn0 + 32 * j + 8 * q + 4 * h + e;
+                        if (col < g.N) {
+                            float v = accT[j][i][4 * q + e];
+                            if (C) v = __builtin_fmaf((float)C[(size_t)row * g.ldc + col], g.beta, g.alpha * v);
+                            D[(size_t)row * g.ldd + col] = (_Float16)v;
+                        }
+                    }
+            }
+        }
+    }
+}
+
+namespace {
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES>
+int launch_dma(const GemmArgs& args, hipStream_t stream)
+{
+    GemmArgs g = args;
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    const uint32_t nb = g.tiles_m * g.tiles_n;
+    g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
+    hipLaunchKernelGGL((gemm_f16_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES>), dim3(nb), dim3(WAVES_M * WAVES_N * 64),
+                       0, stream, g);
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
+// M, N, K >= 1; 16-byte aligned bases and pitches (the caller checks).  Shapes measured on MI355X:
+//   256 x 256: 8 wavefronts of 128 x 64 on 64-deep slabs in 2 stages (1177 TFLOP/s at 4096^3, 1222 at
+//     8192^3); 4 wavefronts of 128 x 128 reach 1075-1124, 16 wavefronts 1144, 32-deep slabs 1100-1124.
+//     Two wavefronts per SIMD take turns on the matrix pipe while the other waits for LDS or the barrier.
+//   128 x 128: 4 wavefronts of 64 x 64; 64-deep slabs in 4 stages when there is at most one workgroup
+//     per CU (751 TFLOP/s at 2048^3), else 32-deep so that two workgroups share a CU (640 at 3000^3).
+//   64 x 64: 4 wavefronts of 32 x 32, 64-deep slabs in 4 stages (287 TFLOP/s at 1024^3).
+int launch_gemm_f16_dma(int shape, const GemmArgs& args, hipStream_t stream)
+{
+    switch (shape) {
+    case TILE_256x256: return launch_dma<256, 256, 2, 4, 64, 2>(args, stream);
+    case TILE_128x128: {
+        const uint64_t blocks = (uint64_t)((args.M + 127) / 128) * ((args.N + 127) / 128);
+        return blocks <= 256 ? launch_dma<128, 128, 2, 2, 64, 4>(args, stream)
+                             : launch_dma<128, 128, 2, 2, 32, 4>(args, stream);
+    }
+    case TILE_64x64:   return launch_dma<64, 64, 2, 2, 64, 4>(args, stream);
+    default:           return (int)hipErrorInvalidValue;
+    }
+}
+
+}  // namespace decx_hip

@@ -59,8 +59,8 @@ enum {
 
 typedef struct decx_hip_plan {
     int32_t  path;                 /* one of the enum above */
-    int32_t  edge;                 /* 1: the predicated register-staged kernel runs (fp32: unaligned operands or
-                                      K == 0; fp16: also any ragged M, N, K); 0: a direct-to-LDS kernel */
+    int32_t  edge;                 /* 1: the predicated register-staged kernel runs (operands not 16-byte
+                                      aligned, or K == 0); 0: a direct-to-LDS kernel */
     uint32_t tile_m, tile_n;       /* block tile */
     uint32_t grid;                 /* workgroups launched */
 } decx_hip_plan;

@@ -60,12 +60,13 @@ def test_planner_choices():
         p = hip.plan(eb, M, N, K)
         assert (p.path, p.edge, p.tile_m, p.tile_n) == (hip.TILE_256, 0, 256, 256)
         assert p.grid == (M // 256) * (N // 256)
-    # small and ragged problems take smaller tiles so the chip fills; fp32 stays on the direct-to-LDS
-    # kernels as long as the operands are 16-byte aligned, fp16 falls to the predicated variant
+    # small and ragged problems take smaller tiles so the chip fills; they stay on the direct-to-LDS
+    # kernels as long as the operands are 16-byte aligned
     p = hip.plan(4, 1000, 1500, 777)
     assert p.edge == 0 and p.tile_m < 256 and p.grid == -(-1000 // p.tile_m) * -(-1500 // p.tile_n)
     assert hip.plan(4, 1000, 1500, 777, aligned=False).edge == 1
-    assert hip.plan(2, 1000, 1500, 777).edge == 1
+    assert hip.plan(2, 1000, 1500, 777).edge == 0 and hip.plan(2, 1000, 1500, 777).tile_m == 64
+    assert hip.plan(2, 2048, 2048, 2048).tile_m == 128 and hip.plan(2, 1000, 1500, 777, aligned=False).edge == 1
     assert hip.plan(4, 1024, 1024, 1024).tile_m == 64
     assert hip.plan(4, 2048, 2048, 2048).tile_m == 128
     assert hip.plan(4, 3000, 3000, 3000).tile_m == 64
