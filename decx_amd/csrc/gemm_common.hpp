@@ -86,8 +86,6 @@ __host__ inline TileInfo tile_info_f16(int shape, bool aligned = true)
 }
 
 int launch_gemm_f32(int shape, bool edge, const GemmArgs& args, hipStream_t stream);
-// 256 x 256 x 16 direct-to-LDS fp32 kernel; full tiles only (the caller checks divisibility and alignment)
-int launch_gemm_f32_pipelined(const GemmArgs& args, hipStream_t stream);
 // direct-to-LDS fp32 kernel for any M, N, K >= 1 on 16-byte aligned bases and pitches, in the three tile shapes
 int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream);
 int launch_gemm_f16(int shape, bool edge, const GemmArgs& args, hipStream_t stream);

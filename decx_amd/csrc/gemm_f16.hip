@@ -1,5 +1,7 @@
 // fp16 GEMM for gfx950: half inputs, fp32 accumulation on the matrix cores
-// (v_mfma_f32_32x32x16_f16), one round-to-nearest-even conversion to half at the end.
+// (v_mfma_f32_32x32x16_f16), one round-to-nearest-even conversion to half at the end.  This is
+// the register-staged, fully predicated kernel for operands of any alignment and K == 0;
+// 16-byte aligned operands go to the direct-to-LDS kernels (launch_gemm_f16 below routes).
 //
 // Replaces the reference's cu_GEMM_fp16_[F_]kernel_* (srcs/modules/BLAS/GEMM/CUDA/
 // large_squares/fp16/GEMM_fp16_B128_kernels.cu), which accumulate each K chunk in fp16 and
@@ -32,7 +34,7 @@ __device__ __forceinline__ uint32_t pack_hi(uint32_t even_row, uint32_t odd_row)
     return __builtin_amdgcn_perm(odd_row, even_row, 0x07060302u);
 }
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool EDGE>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_f16_kernel(const GemmArgs g)
 {
@@ -86,7 +88,7 @@ gemm_f16_kernel(const GemmArgs g)
             const int q = t + i * NT;
             const uint32_t gm = m0 + q / (BK / 8), gk = k0 + (q % (BK / 8)) * 8;
             const uint16_t* p = A + (size_t)gm * g.lda + gk;
-            if (!EDGE || (rows_inside && k_inside)) ra[i] = *(const uintx4*)p;
+            if (rows_inside && k_inside) ra[i] = *(const uintx4*)p;
             else {
                 uintx4 v = {0u, 0u, 0u, 0u};
                 if (gm < g.M) v = load8(p, gk, g.K);
@@ -100,7 +102,7 @@ gemm_f16_kernel(const GemmArgs g)
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
                 const uint16_t* p = B + (size_t)(gk + r) * g.ldb + gn;
-                if (!EDGE || (cols_inside && k_inside)) rb[i][r] = *(const uintx4*)p;
+                if (cols_inside && k_inside) rb[i][r] = *(const uintx4*)p;
                 else {
                     uintx4 v = {0u, 0u, 0u, 0u};
                     if (gk + r < g.K) v = load8(p, gn, g.N);
@@ -187,7 +189,7 @@ gemm_f16_kernel(const GemmArgs g)
             float v[TN];
 #pragma unroll
             for (int j = 0; j < TN; ++j) v[j] = acc[i][j][r];
-            if (TN > 1 && (!EDGE || (rows_inside && cols_inside))) {
+            if (TN > 1 && (rows_inside && cols_inside)) {
                 if (C) {
                     const hvec cv = *(const hvec*)(C + (size_t)row * g.ldc + col0);
 #pragma unroll
@@ -214,19 +216,14 @@ gemm_f16_kernel(const GemmArgs g)
 }
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
-static int launch_shape(bool edge, const GemmArgs& args, hipStream_t stream)
+static int launch_shape(const GemmArgs& args, hipStream_t stream)
 {
     GemmArgs g = args;
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
     g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
-    const bool full = (g.M % BM == 0) && (g.N % BN == 0) && (g.K % BK == 0) && g.vec_ok;
-    const dim3 grid(nb), block(WAVES_M * WAVES_N * 64);
-    if (edge || !full)
-        hipLaunchKernelGGL((gemm_f16_kernel<BM, BN, BK, WAVES_M, WAVES_N, true>), grid, block, 0, stream, g);
-    else
-        hipLaunchKernelGGL((gemm_f16_kernel<BM, BN, BK, WAVES_M, WAVES_N, false>), grid, block, 0, stream, g);
+    hipLaunchKernelGGL((gemm_f16_kernel<BM, BN, BK, WAVES_M, WAVES_N>), dim3(nb), dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
     return (int)hipGetLastError();
 }
 
@@ -234,9 +231,9 @@ int launch_gemm_f16(int shape, bool edge, const GemmArgs& args, hipStream_t stre
 {
     if (!edge && args.vec_ok && args.K > 0) return launch_gemm_f16_dma(shape, args, stream);
     switch (shape) {
-    case TILE_256x256: return launch_shape<256, 256, 64, 2, 2>(edge, args, stream);
-    case TILE_128x128: return launch_shape<128, 128, 64, 2, 1>(edge, args, stream);
-    case TILE_64x64:   return launch_shape< 64,  64, 64, 1, 1>(edge, args, stream);
+    case TILE_256x256: return launch_shape<256, 256, 64, 2, 2>(args, stream);
+    case TILE_128x128: return launch_shape<128, 128, 64, 2, 1>(args, stream);
+    case TILE_64x64:   return launch_shape< 64,  64, 64, 1, 1>(args, stream);
     default:           return (int)hipErrorInvalidValue;
     }
 }

@@ -1,12 +1,8 @@
-// fp32 GEMM for gfx950 on the fp32 matrix cores (v_mfma_f32_32x32x2_f32): the register-staged
-// kernel.  It takes operands of any alignment (element loads where 128-bit ones would be
-// misaligned) and K == 0; 16-byte aligned operands, the usual case, go to the direct-to-LDS
-// kernels instead (launch_gemm_f32 below routes).
-//
-// Replaces the reference's SIMT kernels cu_GEMM_fp32_[F_]kernel_* and their transposed-A
-// variants (srcs/modules/BLAS/GEMM/CUDA/large_squares/fp32/GEMM_fp32_B128_kernels.cu,
-// GEMM_fp32_B64_kernels.cu) and the separate A-transpose pass: one kernel family, no
-// scratch, no reliance on zero-filled pitch padding.
+// fp32 GEMM for gfx950 on the fp32 matrix cores (v_mfma_f32_32x32x2_f32): the register-staged,
+// fully predicated kernel.  It takes operands of any alignment (element loads where 128-bit
+// ones would be misaligned; tiles that lie inside aligned matrices still take 128-bit loads)
+// and K == 0.  16-byte aligned operands, the usual case (the reference's device pitch rule
+// guarantees them), go to the direct-to-LDS kernels instead; launch_gemm_f32 below routes.
 //
 // Structure of one workgroup (BM x BN output tile, WAVES_M x WAVES_N wavefronts):
 //   * K is walked in slabs of BK.  Slab s+1 travels global -> registers (128-bit loads)
@@ -49,7 +45,7 @@ template <int TN> __device__ __forceinline__ float bfrag_get(const typename BFra
     if constexpr (TN == 1) return v; else return v[i];
 }
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool EDGE>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_f32_kernel(const GemmArgs g)
 {
@@ -93,7 +89,7 @@ gemm_f32_kernel(const GemmArgs g)
             const int q = t + i * NT;
             const uint32_t gm = m0 + q / (BK / 4), gk = k0 + (q % (BK / 4)) * 4;
             const float* p = A + (size_t)gm * g.lda + gk;
-            if (!EDGE || (rows_inside && k_inside)) {
+            if (rows_inside && k_inside) {
                 ra[i] = *(const floatx4*)p;
             } else {
                 floatx4 v = {0.f, 0.f, 0.f, 0.f};
@@ -114,7 +110,7 @@ gemm_f32_kernel(const GemmArgs g)
             const int q = t + i * NT;
             const uint32_t gk = k0 + q / (BN / 4), gn = n0 + (q % (BN / 4)) * 4;
             const float* p = B + (size_t)gk * g.ldb + gn;
-            if (!EDGE || (cols_inside && k_inside)) {
+            if (cols_inside && k_inside) {
                 rb[i] = *(const floatx4*)p;
             } else {
                 floatx4 v = {0.f, 0.f, 0.f, 0.f};
@@ -217,7 +213,7 @@ gemm_f32_kernel(const GemmArgs g)
             float v[TN];
 #pragma unroll
             for (int j = 0; j < TN; ++j) v[j] = acc[i][j][r];
-            if (!EDGE || (rows_inside && cols_inside)) {
+            if (rows_inside && cols_inside) {
                 if (C) {
                     const bvec cv = *(const bvec*)(C + (size_t)row * g.ldc + col0);
 #pragma unroll
@@ -247,35 +243,24 @@ gemm_f32_kernel(const GemmArgs g)
 }
 
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
-static int launch_shape(bool edge, const GemmArgs& args, hipStream_t stream)
+static int launch_shape(const GemmArgs& args, hipStream_t stream)
 {
     GemmArgs g = args;
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
     g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
-    // the unpredicated variant serves full tiles only; with `edge` the caller asks for the predicated one anyway
-    const bool full = (g.M % BM == 0) && (g.N % BN == 0) && (g.K % BK == 0) && g.vec_ok;
-    const dim3 grid(nb), block(WAVES_M * WAVES_N * 64);
-    if (edge || !full)
-        hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, BK, WAVES_M, WAVES_N, true>), grid, block, 0, stream, g);
-    else
-        hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, BK, WAVES_M, WAVES_N, false>), grid, block, 0, stream, g);
+    hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, BK, WAVES_M, WAVES_N>), dim3(nb), dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
     return (int)hipGetLastError();
 }
 
 int launch_gemm_f32(int shape, bool edge, const GemmArgs& args, hipStream_t stream)
 {
-    if (!edge && args.vec_ok && args.K > 0) {
-        // full tiles: the same scheme without the edge bookkeeping measures 3 % faster (143 vs 138 TFLOP/s at 8192^3)
-        if (shape == TILE_256x256 && args.M % 256 == 0 && args.N % 256 == 0 && args.K % 16 == 0)
-            return launch_gemm_f32_pipelined(args, stream);
-        return launch_gemm_f32_dma(shape, args, stream);
-    }
+    if (!edge && args.vec_ok && args.K > 0) return launch_gemm_f32_dma(shape, args, stream);
     switch (shape) {
-    case TILE_256x256: return launch_shape<256, 256, 16, 4, 2>(edge, args, stream);
-    case TILE_128x128: return launch_shape<128, 128, 16, 2, 2>(edge, args, stream);
-    case TILE_64x64:   return launch_shape< 64,  64, 16, 2, 2>(edge, args, stream);
+    case TILE_256x256: return launch_shape<256, 256, 16, 4, 2>(args, stream);
+    case TILE_128x128: return launch_shape<128, 128, 16, 2, 2>(args, stream);
+    case TILE_64x64:   return launch_shape< 64,  64, 16, 2, 2>(args, stream);
     default:           return (int)hipErrorInvalidValue;
     }
 }
