@@ -202,6 +202,10 @@ int decx_hip_event_record(void* event, void* stream)
 {
     return event ? hip_rc(hipEventRecord((hipEvent_t)event, as_stream(stream))) : DECX_HIP_E_INVALID_ARG;
 }
+int decx_hip_stream_wait_event(void* stream, void* event)
+{
+    return event ? hip_rc(hipStreamWaitEvent(as_stream(stream), (hipEvent_t)event, 0)) : DECX_HIP_E_INVALID_ARG;
+}
 int decx_hip_event_sync(void* event)
 {
     return event ? hip_rc(hipEventSynchronize((hipEvent_t)event)) : DECX_HIP_E_INVALID_ARG;

@@ -47,6 +47,7 @@ SYMBOLS = {
     "decx_hip_event_create": (_int, [ctypes.POINTER(_vp)]),
     "decx_hip_event_destroy": (_int, [_vp]),
     "decx_hip_event_record": (_int, [_vp, _vp]),
+    "decx_hip_stream_wait_event": (_int, [_vp, _vp]),
     "decx_hip_event_sync": (_int, [_vp]),
     "decx_hip_event_elapsed_ms": (_int, [_vp, _vp, ctypes.POINTER(_f)]),
     "decx_hip_gemm_f32": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp]),

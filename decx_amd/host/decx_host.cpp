@@ -434,8 +434,33 @@ _DECX_API_ void de::blas::cuda::GEMM(de::GPU_Matrix& A, de::GPU_Matrix& B, de::G
 
 namespace {
 
-// Host-matrix form: stage through device memory.  The original declares these overloads
-// (srcs/includes/DECX/BLAS/BLAS.h:69-70) and defines them nowhere.
+// Streams and events of the host-matrix form, created on first use and kept.
+struct HostPipe {
+    void* in = nullptr;        // host -> device copies
+    void* out = nullptr;       // device -> host copies
+    bool ok = false;
+};
+HostPipe& host_pipe()
+{
+    static HostPipe p;
+    if (!p.ok && decx::gpu_ready()) {
+        p.ok = decx_hip_stream_create(&p.in) == DECX_HIP_OK && decx_hip_stream_create(&p.out) == DECX_HIP_OK;
+    }
+    return p;
+}
+
+struct EventList {
+    void* ev[64];
+    int n = 0;
+    void* make() { void* e = nullptr; if (n < 64 && decx_hip_event_create(&e) == DECX_HIP_OK) ev[n++] = e; return e; }
+    ~EventList() { for (int i = 0; i < n; ++i) decx_hip_event_destroy(ev[i]); }
+};
+
+// Host-matrix form.  The original declares these overloads (srcs/includes/DECX/BLAS/BLAS.h:69-70) and defines
+// them nowhere.  Here the operands are staged through device memory in row panels of A (and C): panel p + 1
+// travels host -> device while panel p is multiplied and panel p - 1 of the result travels back, on three
+// streams chained by events.  The copies are asynchronous when the host matrices are page-locked
+// (de::cuda::PinMemory); with pageable memory the runtime stages them and the overlap is partial.
 void gemm_host(de::Matrix& A, de::Matrix& B, de::Matrix* C, de::Matrix& dst)
 {
     de::DH* h = de::GetLastError();
@@ -447,25 +472,68 @@ void gemm_host(de::Matrix& A, de::Matrix& B, de::Matrix* C, de::Matrix& dst)
     if (!a || !b || !d || !a->is_init() || !b->is_init() || (C && (!c || !c->is_init()))) {
         decx::err::set(h, decx::DECX_FAIL_CLASS_NOT_INIT, kClassNotInit); return;
     }
+    // device twins: they carry the shapes through the same checks as the device form
     decx::_GPU_Matrix dA(a->Type(), a->Width(), a->Height(), de::_NA_);
     decx::_GPU_Matrix dB(b->Type(), b->Width(), b->Height(), de::_NA_);
     decx::_GPU_Matrix dC, dD;
     if (!dA.is_init() || !dB.is_init()) return;
-    const de::Point2D zero(0, 0);
-    de::DH r = de::Memcpy(A, dA, zero, zero, de::Point2D(a->Width(), a->Height()), de::DECX_MEMCPY_H2D);
-    if (r.error_type == decx::DECX_SUCCESS)
-        r = de::Memcpy(B, dB, zero, zero, de::Point2D(b->Width(), b->Height()), de::DECX_MEMCPY_H2D);
-    if (r.error_type == decx::DECX_SUCCESS && c) {
-        dC.re_construct(c->Type(), c->Width(), c->Height());
-        if (!dC.is_init()) return;
-        r = de::Memcpy(*C, dC, zero, zero, de::Point2D(c->Width(), c->Height()), de::DECX_MEMCPY_H2D);
-    }
-    if (r.error_type != decx::DECX_SUCCESS) { *h = r; return; }
+    if (c) { dC.re_construct(c->Type(), c->Width(), c->Height()); if (!dC.is_init()) return; }
     if (!validate(&dA, &dB, c ? &dC : nullptr, &dD, nullptr, nullptr, h)) return;
-    if (!gemm_device(&dA, &dB, c ? &dC : nullptr, &dD, 1.f, 1.f, h)) return;
-    d->re_construct(a->Type(), b->Width(), a->Height());
-    r = de::Memcpy(dst, dD, zero, zero, de::Point2D(dD.Width(), dD.Height()), de::DECX_MEMCPY_D2H);
-    if (r.error_type != decx::DECX_SUCCESS) *h = r;
+    const uint32_t M = a->Height(), N = b->Width(), K = a->Width();
+    // C may be dst: take what is needed of it before dst is reshaped
+    const char* c_host = c ? (const char*)c->data() : nullptr;
+    const size_t c_host_pitch = c ? (size_t)c->Pitch() : 0;
+    // (when C is dst the reshape below changes nothing: C already has the result's shape)
+    d->re_construct(a->Type(), N, M);
+    if (!dD.re_construct(a->Type(), N, M)) return;
+    if (M == 0 || N == 0) return;
+
+    std::lock_guard<std::mutex> guard(decx::module_mutex());
+    HostPipe& pipe = host_pipe();
+    void* S = decx::module_stream();
+    if (!pipe.ok || !S) { decx::err::set(h, decx::DECX_FAIL_CUDA_STREAM, "error: Fail to create the staging streams"); return; }
+    const size_t es = (size_t)a->get_layout()._single_element_size;
+    const bool f16 = a->Type() == de::_FP16_;
+    // panels of at least 256 rows, at most 16 of them
+    uint32_t rows_per = (M + 15) / 16;
+    rows_per = (rows_per + 255) / 256 * 256;
+    const uint32_t panels = (M + rows_per - 1) / rows_per;
+
+    EventList events;
+    int rc = DECX_HIP_OK;
+    auto copy = [&](void* dp, size_t dpitch, const void* hp, size_t hpitch, size_t width, size_t rows, int kind, void* st) {
+        if (rc == DECX_HIP_OK && width && rows)
+            rc = decx_hip_memcpy2d_async(kind == 0 ? dp : const_cast<void*>(hp), (kind == 0 ? dpitch : hpitch) * es,
+                                         kind == 0 ? hp : dp, (kind == 0 ? hpitch : dpitch) * es, width * es, rows, kind, st);
+    };
+    copy(dB.data(), dB.Pitch(), b->data(), b->Pitch(), N, K, 0, pipe.in);
+    for (uint32_t p = 0; p < panels && rc == DECX_HIP_OK; ++p) {
+        const uint32_t r0 = p * rows_per, rows = (M - r0) < rows_per ? (M - r0) : rows_per;
+        char* a_dev = (char*)dA.data() + (size_t)r0 * dA.Pitch() * es;
+        char* d_dev = (char*)dD.data() + (size_t)r0 * dD.Pitch() * es;
+        char* c_dev = c ? (char*)dC.data() + (size_t)r0 * dC.Pitch() * es : nullptr;
+        copy(a_dev, dA.Pitch(), (const char*)a->data() + (size_t)r0 * a->Pitch() * es, a->Pitch(), K, rows, 0, pipe.in);
+        if (c) copy(c_dev, dC.Pitch(), c_host + (size_t)r0 * c_host_pitch * es, c_host_pitch, N, rows, 0, pipe.in);
+        void* arrived = events.make();
+        void* done = events.make();
+        if (!arrived || !done) { rc = DECX_HIP_E_INVALID_ARG; break; }
+        if (rc == DECX_HIP_OK) rc = decx_hip_event_record(arrived, pipe.in);
+        if (rc == DECX_HIP_OK) rc = decx_hip_stream_wait_event(S, arrived);
+        if (rc == DECX_HIP_OK)
+            rc = f16 ? decx_hip_gemm_f16((const uint16_t*)a_dev, (const uint16_t*)dB.data(), (const uint16_t*)c_dev,
+                                         (uint16_t*)d_dev, rows, N, K, dA.Pitch(), dB.Pitch(), c ? dC.Pitch() : 0,
+                                         dD.Pitch(), 1.f, 1.f, S)
+                     : decx_hip_gemm_f32((const float*)a_dev, (const float*)dB.data(), (const float*)c_dev,
+                                         (float*)d_dev, rows, N, K, dA.Pitch(), dB.Pitch(), c ? dC.Pitch() : 0,
+                                         dD.Pitch(), 1.f, 1.f, S);
+        if (rc == DECX_HIP_OK) rc = decx_hip_event_record(done, S);
+        if (rc == DECX_HIP_OK) rc = decx_hip_stream_wait_event(pipe.out, done);
+        copy(d_dev, dD.Pitch(), (char*)d->data() + (size_t)r0 * d->Pitch() * es, d->Pitch(), N, rows, 1, pipe.out);
+    }
+    // drain all three streams whatever happened, so that nothing is in flight when the device twins die
+    const int r1 = decx_hip_stream_sync(pipe.in), r2 = decx_hip_stream_sync(S), r3 = decx_hip_stream_sync(pipe.out);
+    if (rc == DECX_HIP_OK) rc = r1 != DECX_HIP_OK ? r1 : (r2 != DECX_HIP_OK ? r2 : r3);
+    decx::err::from_hip(h, rc, "GEMM");
 }
 
 }  // namespace

@@ -93,6 +93,8 @@ DECX_HIP_API int decx_hip_event_create(void** event);
 DECX_HIP_API int decx_hip_event_destroy(void* event);
 DECX_HIP_API int decx_hip_event_record(void* event, void* stream);
 DECX_HIP_API int decx_hip_event_sync(void* event);
+/* work submitted to `stream` after this call starts only once `event` has completed */
+DECX_HIP_API int decx_hip_stream_wait_event(void* stream, void* event);
 DECX_HIP_API int decx_hip_event_elapsed_ms(void* start, void* stop, float* ms);
 
 /* ---- the contraction -------------------------------------------------------------------

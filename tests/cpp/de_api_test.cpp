@@ -6,12 +6,16 @@
 //   de_api_test gpu                       self-contained GPU checks (closed forms, error paths)
 //   de_api_test gemm <dir> <f32|f16> M N K <withC 0|1> <alpha> <beta>
 //                                         reads dense A.bin B.bin [C.bin] from <dir>, writes D.bin
+//   de_api_test hostgemm <dir> <f32|f16> M N K <withC 0|1|2> <pinned 0|1> <repeats>
+//                                         the same through the host-matrix overloads (withC = 2: C is dst);
+//                                         prints the wall time of each repeat
 //   de_api_test vmm <dir> <f32|f16> <mv|vm> W H <level 0|1|2>
 //                                         reads M.bin (H rows x W) and V.bin, writes Y.bin (fp32 for f32
 //                                         and for f16 at level 0, fp16 otherwise) through the host-object
 //                                         vector forms of GEMM
 #include "DECX.h"
 
+#include <chrono>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -398,12 +402,49 @@ template <typename T> static int gemm_files(const std::string& dir, de::_DATA_TY
     return out ? 0 : 2;
 }
 
+template <typename T> static int hostgemm_files(const std::string& dir, de::_DATA_TYPES_FLAGS_ ty, uint32_t M, uint32_t N,
+                                                uint32_t K, int with_c, bool pinned, int repeats)
+{
+    de::InitCuda();
+    de::ResetLastError();
+    de::Matrix& A = de::CreateMatrixRef(ty, K, M);
+    de::Matrix& B = de::CreateMatrixRef(ty, N, K);
+    de::Matrix& C = de::CreateMatrixRef(ty, N, M);
+    // dst: C itself, an empty matrix the call has to create, or (pinned) one made page-locked beforehand
+    de::Matrix& D = with_c == 2 ? C : (pinned ? de::CreateMatrixRef(ty, N, M) : de::CreateMatrixRef());
+    if (!read_into<T>(A, dir + "/A.bin") || !read_into<T>(B, dir + "/B.bin")) return 2;
+    if (pinned) {
+        if (de::cuda::PinMemory(A).error_type || de::cuda::PinMemory(B).error_type || de::cuda::PinMemory(C).error_type) return 5;
+        if (with_c != 2 && de::cuda::PinMemory(D).error_type) return 5;
+    }
+    for (int r = 0; r < repeats; ++r) {
+        if (with_c && !read_into<T>(C, dir + "/C.bin")) return 2;           // C is overwritten when it is dst
+        const auto t0 = std::chrono::steady_clock::now();
+        if (with_c) de::blas::cuda::GEMM(A, B, C, D); else de::blas::cuda::GEMM(A, B, D);
+        const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+        std::cout << "hostgemm repeat " << r << ": " << ms << " ms\n";
+        if (de::GetLastError()->error_type != 0) { std::cerr << de::GetLastError()->error_string << "\n"; return 3; }
+    }
+    if (D.Width() != N || D.Height() != M) return 4;
+    std::ofstream out(dir + "/D.bin", std::ios::binary);
+    for (uint32_t i = 0; i < M; ++i) out.write((const char*)D.ptr<T>(i, 0), (std::streamsize)N * sizeof(T));
+    return out ? 0 : 2;
+}
+
 int main(int argc, char** argv)
 {
     const std::string mode = argc > 1 ? argv[1] : "host";
     int rc;
     if (mode == "host") rc = host_checks();
     else if (mode == "gpu") rc = gpu_checks();
+    else if (mode == "hostgemm" && argc == 10) {
+        const bool f16 = std::string(argv[3]) == "f16";
+        const uint32_t M = std::atoi(argv[4]), N = std::atoi(argv[5]), K = std::atoi(argv[6]);
+        const int with_c = std::atoi(argv[7]), repeats = std::atoi(argv[9]);
+        const bool pinned = std::atoi(argv[8]) != 0;
+        rc = f16 ? hostgemm_files<de::Half>(argv[2], de::_FP16_, M, N, K, with_c, pinned, repeats)
+                 : hostgemm_files<float>(argv[2], de::_FP32_, M, N, K, with_c, pinned, repeats);
+    }
     else if (mode == "vector_host") rc = vector_host_checks();
     else if (mode == "vector_gpu") rc = vector_gpu_checks();
     else if (mode == "vmm" && argc == 8) {

@@ -120,3 +120,36 @@ def test_vector_forms_through_the_objects_match_oracle(oracle, dt, form, W, H, l
     ref = ref.astype(np.float64)
     err = np.max(np.abs(Y.astype(np.float64) - ref)) / (np.max(np.abs(ref)) * np.sqrt(K))
     assert err <= (1e-5 if out_f32 else 2e-3)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt,M,N,K,with_c,pinned", [
+    ("f32", 1000, 1500, 777, 0, 0),        # 4 row panels, the last one ragged
+    ("f32", 1000, 1500, 777, 1, 1),
+    ("f32", 1000, 1500, 777, 2, 1),        # C is dst
+    ("f32", 5000, 300, 260, 2, 0),         # 10 panels of 512 rows, the last one ragged
+    ("f32", 100, 70, 33, 1, 0),            # a single panel
+    ("f16", 1300, 520, 515, 0, 1),
+    ("f16", 1300, 520, 515, 2, 0),
+])
+def test_host_matrix_forms_match_oracle(oracle, dt, M, N, K, with_c, pinned):
+    """de::blas::cuda::GEMM(Matrix, Matrix[, Matrix], Matrix): operands staged in row panels on three streams;
+    pageable and page-locked host storage, C as a separate matrix and as dst."""
+    if dt == "f32":
+        A = synth.uniform_f32(M, K, 401); B = synth.uniform_f32(K, N, 402); C = synth.uniform_f32(M, N, 403)
+    else:
+        A = synth.normal_half(M, K, 401); B = synth.normal_half(K, N, 402); C = synth.normal_half(M, N, 403)
+    with tempfile.TemporaryDirectory() as tmp:
+        A.tofile(os.path.join(tmp, "A.bin")); B.tofile(os.path.join(tmp, "B.bin")); C.tofile(os.path.join(tmp, "C.bin"))
+        rc, out = run_exe("hostgemm", tmp, dt, M, N, K, with_c, pinned, 2)
+        assert rc == 0, out
+        D = np.fromfile(os.path.join(tmp, "D.bin"), A.dtype).reshape(M, N)
+    if dt == "f32":
+        ref = oracle.gemm_f32(A, B, C, 1.0, 1.0) if with_c else oracle.gemm_f32(A, B)
+        tol = 1e-5
+    else:
+        ref = oracle.gemm_f16(A, B, C if with_c else None, 1.0, 1.0)
+        tol = 2e-3
+    ref = ref.astype(np.float64)
+    err = np.max(np.abs(D.astype(np.float64) - ref)) / (np.max(np.abs(ref)) * np.sqrt(K))
+    assert err <= tol
