@@ -85,6 +85,24 @@ __global__ void __launch_bounds__(256) calibration_copy_kernel(uintx4* __restric
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
 }
 
+// kmat[(kh * k_w + kw) * img_dpitch + ic][oc] = kernel oc at (kh, kw, ic); zero where ic >= depth or oc >= out_c
+__global__ void __launch_bounds__(256) conv2d_pack_kernels_kernel(const float* __restrict__ kernels, float* __restrict__ kmat,
+                                                                  uint32_t k_w, uint32_t k_h, uint32_t depth,
+                                                                  uint32_t k_dpitch, uint32_t k_wpitch, uint64_t tensor_stride,
+                                                                  uint32_t out_c, uint32_t kmat_pitch, uint32_t img_dpitch)
+{
+    const uint64_t total = (uint64_t)k_h * k_w * img_dpitch * kmat_pitch;
+    for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (uint64_t)gridDim.x * 256) {
+        const uint32_t oc = (uint32_t)(i % kmat_pitch);
+        const uint64_t k = i / kmat_pitch;
+        const uint32_t ic = (uint32_t)(k % img_dpitch);
+        const uint32_t kw = (uint32_t)((k / img_dpitch) % k_w), kh = (uint32_t)(k / img_dpitch / k_w);
+        float v = 0.f;
+        if (oc < out_c && ic < depth) v = kernels[oc * tensor_stride + ((uint64_t)kh * k_wpitch + kw) * k_dpitch + ic];
+        kmat[i] = v;
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -284,6 +302,49 @@ int decx_hip_gevm_f16(const uint16_t* x, const uint16_t* B, const uint16_t* c, v
                       void* stream)
 {
     return run_gevm(true, y_is_f32 != 0, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream);
+}
+
+int decx_hip_conv2d_pack_kernels_f32(const float* kernels, float* kmat, uint32_t k_w, uint32_t k_h, uint32_t depth,
+                                     uint32_t k_dpitch, uint32_t k_wpitch, uint64_t tensor_stride, uint32_t out_c,
+                                     uint32_t kmat_pitch, uint32_t img_dpitch, void* stream)
+{
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    if (!kernels || !kmat || !k_w || !k_h || !depth || !out_c || k_dpitch < depth || k_wpitch < k_w ||
+        img_dpitch < depth || kmat_pitch < out_c || tensor_stride < (uint64_t)k_dpitch * k_wpitch * (k_h - 1) + (uint64_t)k_dpitch * (k_w - 1) + depth)
+        return DECX_HIP_E_INVALID_ARG;
+    const uint64_t total = (uint64_t)k_h * k_w * img_dpitch * kmat_pitch;
+    const uint64_t want = (total + 255) / 256;
+    hipLaunchKernelGGL(conv2d_pack_kernels_kernel, dim3((unsigned)(want < 4096 ? want : 4096)), dim3(256), 0, as_stream(stream),
+                       kernels, kmat, k_w, k_h, depth, k_dpitch, k_wpitch, tensor_stride, out_c, kmat_pitch, img_dpitch);
+    return (int)hipGetLastError();
+}
+
+int decx_hip_conv2d_f32(const float* image, const float* kmat, float* dst, uint32_t out_w, uint32_t out_h, uint32_t out_c,
+                        uint32_t k_w, uint32_t k_h, uint32_t img_dpitch, uint32_t img_wpitch, uint32_t stride_x,
+                        uint32_t stride_y, uint32_t kmat_pitch, uint32_t dst_dpitch, uint32_t dst_wpitch, void* stream)
+{
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    if (!out_w || !out_h || !out_c) return DECX_HIP_OK;
+    if (!image || !kmat || !dst || !k_w || !k_h || !stride_x || !stride_y || !img_dpitch || img_dpitch % 4 || kmat_pitch % 4 ||
+        dst_dpitch % 4 || kmat_pitch < out_c || dst_dpitch < out_c || dst_wpitch < out_w ||
+        img_wpitch < (uint64_t)(out_w - 1) * stride_x + k_w || !aligned16(image) || !aligned16(kmat) || !aligned16(dst) ||
+        (uint64_t)out_w * out_h > 0xffffffffull || (uint64_t)k_w * img_dpitch * 4 > 0xffffffffull ||
+        (uint64_t)k_h * k_w * img_dpitch > 0xffffffffull)
+        return DECX_HIP_E_INVALID_ARG;
+    GemmArgs g;
+    std::memset(&g, 0, sizeof g);
+    g.A = image; g.B = kmat; g.C = nullptr; g.D = dst;
+    g.M = out_w * out_h; g.N = out_c; g.K = k_h * k_w * img_dpitch;
+    g.lda = g.K; g.ldb = kmat_pitch; g.ldc = 0; g.ldd = dst_dpitch;
+    g.alpha = 1.f; g.beta = 1.f;
+    g.vec_ok = 1;
+    g.conv_wout = out_w;
+    g.conv_seg_bytes = k_w * img_dpitch * 4u;
+    g.conv_px_bytes = stride_x * img_dpitch * 4u;
+    g.conv_dst_row = dst_wpitch * dst_dpitch;
+    g.conv_seg_stride = (uint64_t)img_wpitch * img_dpitch * 4u;
+    g.conv_py_bytes = (uint64_t)stride_y * img_wpitch * img_dpitch * 4u;
+    return launch_conv2d_f32_dma(choose_tile(false, g.M, g.N, true), g, as_stream(stream));
 }
 
 int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int aligned, decx_hip_plan* out)

@@ -28,6 +28,16 @@ struct GemmArgs {
     uint32_t tiles_m, tiles_n;   // number of block tiles along M and N
     uint32_t xcd_remap;          // 1: grid size is a multiple of 8, use the per-XCD ordering
     uint32_t vec_ok;             // 1: every base pointer is 16-byte aligned and every pitch a multiple of 16 bytes
+    // Convolution as an implicit GEMM (used by the CONV instantiations only): row p of the A operand is the
+    // patch under output pixel (p / conv_wout, p % conv_wout) of an image stored [row][column][channel]; its K
+    // elements are KH runs of conv_seg_bytes contiguous bytes (KW columns x channel pitch), conv_seg_stride bytes
+    // apart (one image row).  D row p lands at pixel pitch ldd inside image rows of conv_dst_row floats.
+    uint32_t conv_wout;
+    uint32_t conv_seg_bytes;
+    uint32_t conv_px_bytes;      // bytes between patches of horizontally adjacent output pixels
+    uint32_t conv_dst_row;       // floats per output image row
+    uint64_t conv_seg_stride;
+    uint64_t conv_py_bytes;      // bytes between patches of vertically adjacent output pixels
 };
 
 constexpr int kXcds = 8;        // MI355X: 8 accelerator complex dies, blocks are dealt to them round-robin
@@ -88,6 +98,8 @@ __host__ inline TileInfo tile_info_f16(int shape, bool aligned = true)
 int launch_gemm_f32(int shape, bool edge, const GemmArgs& args, hipStream_t stream);
 // direct-to-LDS fp32 kernel for any M, N, K >= 1 on 16-byte aligned bases and pitches, in the three tile shapes
 int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream);
+// the same kernels with the A operand gathered from an image (GemmArgs::conv_*): 2-D convolution without an im2col buffer
+int launch_conv2d_f32_dma(int shape, const GemmArgs& args, hipStream_t stream);
 int launch_gemm_f16(int shape, bool edge, const GemmArgs& args, hipStream_t stream);
 // direct-to-LDS fp16 kernel for any M, N, K >= 1 on 16-byte aligned bases and pitches, in the three tile shapes
 int launch_gemm_f16_dma(int shape, const GemmArgs& args, hipStream_t stream);

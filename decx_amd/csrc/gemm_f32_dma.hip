@@ -71,7 +71,7 @@ template <int TN> __device__ __forceinline__ float lane_of(const typename BFrag<
 
 }  // namespace
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, bool CONV = false>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_f32_dma_kernel(const GemmArgs g)
 {
@@ -108,9 +108,13 @@ gemm_f32_dma_kernel(const GemmArgs g)
     // slot lane % CPR, fetching chunk slot ^ ((row / RP) % CPR).  B direct load I covers k rows RB I ..:
     // lane -> k row RB I + lane / CB, slot lane % CB, fetching column chunk slot ^ (B_SHIFT if k row & 4).
     // Rows beyond M and column chunks beyond N are replaced by the last valid ones.
+    // CONV: the A operand is gathered from an image.  a_src[i] then walks along the patch of the lane's output
+    // pixel: a_seg[i] is its byte position inside the current run of contiguous bytes (one kernel row), and
+    // every slab issued moves it on by BK floats, hopping to the next image row at the end of a run.
     const unsigned char* a_src[A_LOADS];
     const unsigned char* b_src[B_LOADS];
     int a_chunk[A_LOADS], b_krow[B_LOADS];
+    uint32_t a_seg[CONV ? A_LOADS : 1];
     const uint32_t last_row = g.M - 1, last_col_chunk = (g.N - 1) / 4;
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
@@ -118,8 +122,27 @@ gemm_f32_dma_kernel(const GemmArgs g)
         const int row = I * (64 / CPR) + lane / CPR;
         a_chunk[i] = (lane % CPR) ^ ((row / RP) % CPR);
         const uint32_t grow = (m0 + row) < last_row ? (m0 + row) : last_row;
-        a_src[i] = A + (size_t)grow * lda_b + a_chunk[i] * 16;
+        if constexpr (CONV) {
+            const uint32_t py = grow / g.conv_wout, px = grow % g.conv_wout;
+            const uint32_t k_bytes = a_chunk[i] * 16;
+            a_seg[i] = k_bytes % g.conv_seg_bytes;
+            a_src[i] = A + (size_t)py * g.conv_py_bytes + (size_t)px * g.conv_px_bytes +
+                       (size_t)(k_bytes / g.conv_seg_bytes) * g.conv_seg_stride + a_seg[i];
+        } else {
+            a_src[i] = A + (size_t)grow * lda_b + a_chunk[i] * 16;
+        }
     }
+    auto conv_advance = [&]() {                        // CONV: on to the next slab
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) {
+            a_seg[i] += BK * 4;
+            a_src[i] += BK * 4;
+            while (a_seg[i] >= g.conv_seg_bytes) {
+                a_seg[i] -= g.conv_seg_bytes;
+                a_src[i] += g.conv_seg_stride - g.conv_seg_bytes;
+            }
+        }
+    };
 #pragma unroll
     for (int i = 0; i < B_LOADS; ++i) {
         const int I = wave * B_LOADS + i;
@@ -139,9 +162,10 @@ gemm_f32_dma_kernel(const GemmArgs g)
 #pragma unroll
             for (int i = 0; i < A_LOADS; ++i) {
                 const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u);
-                const unsigned char* src = a_src[i] + (size_t)slab * (BK * 4);
+                const unsigned char* src = CONV ? a_src[i] : a_src[i] + (size_t)slab * (BK * 4);
                 asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
             }
+            if constexpr (CONV) conv_advance();
 #pragma unroll
             for (int i = 0; i < B_LOADS; ++i) {
                 const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + A_STAGE_BYTES +
@@ -158,7 +182,7 @@ gemm_f32_dma_kernel(const GemmArgs g)
                 const uint32_t k = k0 + a_chunk[i] * 4;
                 floatx4 v = floatx4{0.f, 0.f, 0.f, 0.f};
                 if (k < g.K) {
-                    v = *(const floatx4*)(a_src[i] + (size_t)k0 * 4);      // inside the pitch: lda is a multiple of 4
+                    v = *(const floatx4*)(CONV ? a_src[i] : a_src[i] + (size_t)k0 * 4);   // inside the pitch: lda is a multiple of 4
 #pragma unroll
                     for (int e = 1; e < 4; ++e) if (k + e >= g.K) v[e] = 0.f;
                 }
@@ -325,6 +349,9 @@ gemm_f32_dma_kernel(const GemmArgs g)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const uint32_t row = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+            size_t d_row;                              // offset of the row's first element in D
+            if constexpr (CONV) d_row = (size_t)(row / g.conv_wout) * g.conv_dst_row + (size_t)(row % g.conv_wout) * g.ldd;
+            else d_row = (size_t)row * g.ldd;
             float v[TN];
 #pragma unroll
             for (int j = 0; j < TN; ++j) v[j] = acc[i][j][r];
@@ -340,14 +367,14 @@ gemm_f32_dma_kernel(const GemmArgs g)
 #pragma unroll
                     for (int j = 0; j < TN; ++j) o[j] = v[j];
                 }
-                *(bfrag*)(D + (size_t)row * g.ldd + col0) = o;
+                *(bfrag*)(D + d_row + col0) = o;
             } else if (row < g.M) {
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
                     if (col0 + j < g.N) {
                         float o = v[j];
                         if (C) o = __builtin_fmaf(C[(size_t)row * g.ldc + col0 + j], g.beta, g.alpha * o);
-                        D[(size_t)row * g.ldd + col0 + j] = o;
+                        D[d_row + col0 + j] = o;
                     }
                 }
             }
@@ -357,7 +384,7 @@ gemm_f32_dma_kernel(const GemmArgs g)
 
 namespace {
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, bool CONV = false>
 int launch_dma(const GemmArgs& args, hipStream_t stream)
 {
     GemmArgs g = args;
@@ -365,7 +392,7 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
     g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
-    hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD>), dim3(nb), dim3(WAVES_M * WAVES_N * 64),
+    hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD, CONV>), dim3(nb), dim3(WAVES_M * WAVES_N * 64),
                        0, stream, g);
     return (int)hipGetLastError();
 }
@@ -385,6 +412,19 @@ int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
     case TILE_256x256: return launch_dma<256, 256, 2, 4, 16, 4, false>(args, stream);
     case TILE_128x128: return launch_dma<128, 128, 2, 2, 16, 4, true>(args, stream);
     case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 32, 4, true>(args, stream);
+    default:           return (int)hipErrorInvalidValue;
+    }
+}
+
+// 2-D convolution as an implicit GEMM: M = output pixels, N = output channels, K = kernel rows x (kernel columns x
+// channel pitch); B is the kernel set packed [K][N].  Replaces cu_im2col_*_fp32 + cu_im2col_GEMM_fp32
+// (srcs/modules/NN/convolution/CUDA/fp32/im2col_fp32.cu, im2col_GEMM_fp32.cu:40-106) and their im2col buffer.
+int launch_conv2d_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
+{
+    switch (shape) {
+    case TILE_256x256: return launch_dma<256, 256, 2, 4, 16, 4, false, true>(args, stream);
+    case TILE_128x128: return launch_dma<128, 128, 2, 2, 16, 4, true, true>(args, stream);
+    case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 32, 4, true, true>(args, stream);
     default:           return (int)hipErrorInvalidValue;
     }
 }

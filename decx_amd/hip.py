@@ -56,6 +56,8 @@ SYMBOLS = {
     "decx_hip_gemv_f16": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _int, _vp]),
     "decx_hip_gevm_f32": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _vp]),
     "decx_hip_gevm_f16": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _int, _vp]),
+    "decx_hip_conv2d_pack_kernels_f32": (_int, [_vp, _vp] + [_u32] * 5 + [ctypes.c_uint64] + [_u32] * 3 + [_vp]),
+    "decx_hip_conv2d_f32": (_int, [_vp] * 3 + [_u32] * 12 + [_vp]),
     "decx_hip_gemm_f32_tile": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, _int, _int]),
     "decx_hip_gemm_f16_tile": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, _int, _int]),
     "decx_hip_gemm_plan": (_int, [_int, _u32, _u32, _u32, _int, ctypes.POINTER(Plan)]),
@@ -225,6 +227,55 @@ def gevm(x, B, y, c=None, alpha=1.0, beta=1.0, stream=None):
         assert x.dtype == y.dtype == np.float32
         rc = L.decx_hip_gevm_f32(xp, B.ptr, cp, yp, K, N, B.pitch, incx, incc, incy, alpha, beta, stream)
     check(rc, "gevm")
+
+
+def _align(v, a):
+    return (v + a - 1) // a * a
+
+
+def conv2d(image, kernels, stride_x=1, stride_y=1, extend=False, stream=None, pad_value=np.nan):
+    """dst[oy][ox][oc] = sum image[oy*sy+kh][ox*sx+kw][ic] * kernels[oc][kh][kw][ic] through decx_hip_conv2d_f32.
+    image [H][W][C], kernels [OC][KH][KW][C] (numpy fp32).  Device layouts follow the original's device tensors:
+    channel pitch = C rounded up to 4, row pitch = W rounded up to 8 columns; unused columns hold `pad_value`,
+    unused channels zero.  extend: zero-extended borders, output W/sx x H/sy."""
+    image = np.ascontiguousarray(image, np.float32); kernels = np.ascontiguousarray(kernels, np.float32)
+    H, W, C = image.shape
+    OC, KH, KW, _ = kernels.shape
+    L = lib()
+    dp = _align(C, 4)
+    if extend:
+        ow, oh = W // stride_x, H // stride_y
+        left, top = KW // 2, KH // 2
+        PW = max((ow - 1) * stride_x + KW, W + left) if ow else W + left
+        PH = max((oh - 1) * stride_y + KH, H + top) if oh else H + top
+        host_img = np.zeros((PH, PW, C), np.float32)
+        host_img[top:top + H, left:left + W] = image
+    else:
+        ow, oh = (W - KW + 1) // stride_x, (H - KH + 1) // stride_y
+        PH, PW, host_img = H, W, image
+    wp = _align(PW, 8)
+    raw = np.full((PH, wp, dp), pad_value, np.float32)
+    raw[:, :PW, :] = 0
+    raw[:, :PW, :C] = host_img
+    d_img = DeviceMatrix(PH, wp * dp, np.float32, data=raw.reshape(PH, wp * dp))
+    kdp, kwp = _align(C, 4), _align(KW, 8)
+    kraw = np.zeros((OC, KH, kwp, kdp), np.float32)
+    kraw[:, :, :KW, :C] = kernels
+    d_ker = DeviceMatrix(OC, KH * kwp * kdp, np.float32, data=kraw.reshape(OC, -1))
+    kp = _align(OC, 4)
+    d_kmat = DeviceMatrix(KH * KW * dp, kp, np.float32)
+    check(L.decx_hip_conv2d_pack_kernels_f32(d_ker.ptr, d_kmat.ptr, KW, KH, C, kdp, kwp, KH * kwp * kdp, OC, kp, dp, stream),
+          "conv2d pack")
+    odp, owp = _align(OC, 4), _align(max(ow, 1), 8)
+    d_out = DeviceMatrix(max(oh, 1), owp * odp, np.float32)
+    d_out.upload_raw(np.full((max(oh, 1), owp * odp), -555.0, np.float32))
+    check(L.decx_hip_conv2d_f32(d_img.ptr, d_kmat.ptr, d_out.ptr, ow, oh, OC, KW, KH, dp, wp, stride_x, stride_y, kp, odp, owp,
+                                stream), "conv2d")
+    check(L.decx_hip_stream_sync(stream))
+    out_raw = d_out.download_raw().reshape(max(oh, 1), owp, odp)
+    for d in (d_img, d_ker, d_kmat, d_out):
+        d.free()
+    return out_raw[:oh, :ow, :OC].copy(), out_raw
 
 
 def sync(stream=None):

@@ -142,6 +142,29 @@ DECX_HIP_API int decx_hip_gevm_f16(const uint16_t* x, const uint16_t* B, const u
                                    uint32_t incx, uint32_t incc, uint32_t incy,
                                    float alpha, float beta, int y_is_f32, void* stream);
 
+/* ---- 2-D convolution as an implicit GEMM ---------------------------------------------------
+ * Replaces the planner, the im2col kernels, the im2col buffer and cu_im2col_GEMM_fp32 behind
+ * de::nn::cuda::Conv2D (srcs/modules/NN/convolution/CUDA/fp32/cuda_conv2D_fp32_im2col_planner.cu:
+ * 212-552, im2col_fp32.cu, im2col_GEMM_fp32.cu:40-106).  Images are stored [row][column][channel]
+ * with a channel pitch (multiple of 4 floats) and a row pitch in columns; all pointers 16-byte
+ * aligned.
+ *
+ *   dst(y, x, oc) = sum over kh, kw, ic of image(y * stride_y + kh, x * stride_x + kw, ic) * kernel_oc(kh, kw, ic)
+ *
+ * (no flip: a cross-correlation, as the original computes).  `image` points at the pixel under
+ * kernel element (0, 0) of output pixel (0, 0): for zero-extended borders pass a zero-padded copy.
+ * The kernel set comes packed as kmat[(kh * k_w + kw) * img_dpitch + ic][oc] (row pitch kmat_pitch,
+ * zero rows for ic >= depth); decx_hip_conv2d_pack_kernels_f32 builds it from out_c kernels stored
+ * like images, tensor_stride floats apart. */
+DECX_HIP_API int decx_hip_conv2d_pack_kernels_f32(const float* kernels, float* kmat, uint32_t k_w, uint32_t k_h,
+                                                  uint32_t depth, uint32_t k_dpitch, uint32_t k_wpitch,
+                                                  uint64_t tensor_stride, uint32_t out_c, uint32_t kmat_pitch,
+                                                  uint32_t img_dpitch, void* stream);
+DECX_HIP_API int decx_hip_conv2d_f32(const float* image, const float* kmat, float* dst,
+                                     uint32_t out_w, uint32_t out_h, uint32_t out_c, uint32_t k_w, uint32_t k_h,
+                                     uint32_t img_dpitch, uint32_t img_wpitch, uint32_t stride_x, uint32_t stride_y,
+                                     uint32_t kmat_pitch, uint32_t dst_dpitch, uint32_t dst_wpitch, void* stream);
+
 /* Same as decx_hip_gemm_f32 / _f16 with the planner's choice overridden (`tile` = one of
  * DECX_HIP_TILE_*; AUTO = planner) and, with force_edge != 0, the predicated kernel
  * variant forced even for shapes that are tile multiples.  For tests and tuning. */

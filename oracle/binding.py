@@ -44,6 +44,8 @@ def lib():
         L.cpu_port_max_threads.restype = _u32
         L.cpu_port_gemm_f32.restype = ctypes.c_int
         L.cpu_port_gemm_f32.argtypes = [_f32p, _f32p, _f32p, _f32p] + [_u32] * 7 + [_f32p, _u32]
+        L.oracle_conv2d_out_dims.argtypes = [_u32] * 6 + [ctypes.c_int, _u32p, _u32p]
+        L.oracle_conv2d_f32.argtypes = [_f32p] + [_u32] * 3 + [_f32p] + [_u32] * 5 + [ctypes.c_int, _f32p]
         _lib = L
     return _lib
 
@@ -201,3 +203,21 @@ def reference_cpu_gemm_f32(A, B, C=None, threads=8):
             if done.returncode == 0:
                 return np.load(os.path.join(tmp, "D.npy")), int(open(os.path.join(tmp, "err")).read())
         raise RuntimeError("the compiled reference crashed on %s x %s, %d threads" % (A.shape, B.shape, threads))
+
+
+def conv2d_out_dims(W, H, KW, KH, sx=1, sy=1, extend=False):
+    ow, oh = _u32(), _u32()
+    lib().oracle_conv2d_out_dims(W, H, KW, KH, sx, sy, int(extend), ctypes.byref(ow), ctypes.byref(oh))
+    return ow.value, oh.value
+
+
+def conv2d_f32(image, kernels, sx=1, sy=1, extend=False):
+    """image [H][W][C], kernels [OC][KH][KW][C] -> [OH][OW][OC]; fmaf chain over (kh, kw, ic)."""
+    image = np.ascontiguousarray(image, np.float32); kernels = np.ascontiguousarray(kernels, np.float32)
+    H, W, C = image.shape
+    OC, KH, KW, C2 = kernels.shape
+    assert C == C2
+    ow, oh = conv2d_out_dims(W, H, KW, KH, sx, sy, extend)
+    out = np.empty((oh, ow, OC), np.float32)
+    lib().oracle_conv2d_f32(_p(image, _f32p), W, H, C, _p(kernels, _f32p), OC, KW, KH, sx, sy, int(extend), _p(out, _f32p))
+    return out
