@@ -112,6 +112,53 @@ def run_workload(name, steps, warmup, keep_inputs=False, settle_s=0.0):
     return result
 
 
+CONV = {"W": 256, "H": 256, "C": 112, "OC": 256, "KW": 3, "KH": 3}     # 64 516 pixels x 256 channels x 1008 taps
+
+
+def run_conv(steps, warmup, settle_s=0.25):
+    """fp32 3 x 3 convolution of a 256 x 256 x 112 image with 256 kernels through decx_hip_conv2d_f32 (implicit GEMM,
+    operands resident): the workload BASELINE's tall-skinny GEMM shape stands for."""
+    from decx_amd import hip, synth
+    c = CONV
+    L = hip.lib()
+    dp, wp = (c["C"] + 3) // 4 * 4, (c["W"] + 7) // 8 * 8
+    img = np.zeros((c["H"], wp, dp), np.float32)
+    img[:, :c["W"], :c["C"]] = synth.uniform_f32(c["H"], c["W"] * c["C"], 0xA007).reshape(c["H"], c["W"], c["C"])
+    d_img = hip.DeviceMatrix(c["H"], wp * dp, np.float32, data=img.reshape(c["H"], -1))
+    K = c["KH"] * c["KW"] * dp
+    kmat = np.zeros((K, c["OC"]), np.float32)
+    kmat.reshape(c["KH"] * c["KW"], dp, c["OC"])[:, :c["C"], :] = synth.uniform_f32(c["KH"] * c["KW"] * c["C"], c["OC"], 0xB007).reshape(-1, c["C"], c["OC"])
+    d_kmat = hip.DeviceMatrix(K, c["OC"], np.float32, data=kmat)
+    ow, oh = c["W"] - c["KW"] + 1, c["H"] - c["KH"] + 1
+    owp = (ow + 7) // 8 * 8
+    d_out = hip.DeviceMatrix(oh, owp * c["OC"], np.float32)
+    call = lambda: hip.check(L.decx_hip_conv2d_f32(d_img.ptr, d_kmat.ptr, d_out.ptr, ow, oh, c["OC"], c["KW"], c["KH"], dp, wp,
+                                                   1, 1, c["OC"], c["OC"], owp, None))
+    for _ in range(warmup):
+        call()
+    hip.sync()
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < settle_s:
+        for _ in range(10):
+            call()
+        hip.sync()
+    timer = hip.Timer(); timer.start()
+    for _ in range(steps):
+        call()
+    ms = timer.stop() / steps
+    flops = 2.0 * ow * oh * c["OC"] * c["KH"] * c["KW"] * c["C"]
+    abytes = 4.0 * (c["H"] * c["W"] * c["C"] + c["KH"] * c["KW"] * c["C"] * c["OC"] + ow * oh * c["OC"])
+    tf = flops / (ms * 1e-3) / 1e12
+    out = {"workload": "fp32 conv2D 3x3, image 256x256x112, 256 kernels (implicit GEMM 64516 x 256 x 1008), uniform[-1,1]",
+           "dtype": "f32", "value": round(tf, 3), "unit": "TFLOP/s", "hbm_gbs_algorithmic": round(abytes / (ms * 1e-3) / 1e9, 1),
+           "kernel_ms": round(ms, 5),
+           "roofline": {"bound": "mfma", "achieved": round(tf, 3), "peak": PEAK_F32_TFLOPS, "unit": "TFLOP/s",
+                        "frac": round(tf / PEAK_F32_TFLOPS, 4), "traffic": None}}
+    for d in (d_img, d_kmat, d_out):
+        d.free()
+    return out
+
+
 def cpu_baseline(name, A, B):
     """Times the AVX2 restatement of the reference CPU GEMM once on this host and checks it
     bit-for-bit against the scalar fma chain on sampled rows."""
@@ -144,7 +191,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="fp32_8192", choices=sorted(WORKLOADS) + ["copy_1GiB"])
+    ap.add_argument("--workload", default="fp32_8192", choices=sorted(WORKLOADS) + ["copy_1GiB", "conv2d"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     args = ap.parse_args()
@@ -170,6 +217,10 @@ def main():
         print(json.dumps({"workload": "calibration copy 1 GiB", "kernel_ms": ms, "GB/s_read_plus_write": 2 * n / ms / 1e6}))
         return
 
+    if args.workload == "conv2d":
+        print(json.dumps(run_conv(args.steps, args.warmup)))
+        return
+
     main_out, inputs = run_workload(args.workload, args.steps, args.warmup, keep_inputs=not args.no_cpu,
                                     settle_s=0.25 if args.workload != "fp32_8192" else 0.0)
     line = {
@@ -191,6 +242,7 @@ def main():
             if name != args.workload:
                 small = WORKLOADS[name][1] * WORKLOADS[name][2] * WORKLOADS[name][3] < 2 ** 38
                 others.append(run_workload(name, 200 if small else args.steps, args.warmup, settle_s=0.25)[0])
+        others.append(run_conv(200, args.warmup))
         line["other_workloads"] = others
     if not args.no_cpu:
         if main_out["dtype"] == "f32":

@@ -154,6 +154,117 @@ public:
     bool re_construct(de::_DATA_TYPES_FLAGS_ type, size_t length);
 };
 
+// Tensor layouts of the original (srcs/modules/core/classes/Tensor.cxx:35-69, GPU_Tensor.cu:35-86): depth padded
+// to 16 bytes of elements, width padded to 4 columns on the host and 8 on the device.
+void assign_tensor_layout(de::TensorLayout& L, de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height,
+                          uint32_t depth, bool device);
+
+class _Tensor : public de::Tensor {
+    de::TensorLayout _layout;
+    de::_DATA_TYPES_FLAGS_ _type;
+    std::shared_ptr<HostBlock> _block;
+    void* _data;
+
+public:
+    _Tensor();
+    _Tensor(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height, uint32_t depth);
+    virtual uint32_t Width() const;
+    virtual uint32_t Height() const;
+    virtual uint32_t Depth() const;
+    virtual de::Tensor& SoftCopy(de::Tensor& src);
+    virtual void release();
+    virtual de::_DATA_TYPES_FLAGS_ Type() const;
+    virtual void Reinterpret(const de::_DATA_TYPES_FLAGS_ new_type);
+    virtual ~_Tensor();
+
+    const de::TensorLayout& get_layout() const { return _layout; }
+    bool is_init() const { return _data != nullptr; }
+    void* data() const { return _data; }
+    // makes this tensor a view of `bytes_offset` into `block` with the given shape
+    void alias(const std::shared_ptr<HostBlock>& block, size_t bytes_offset, de::_DATA_TYPES_FLAGS_ type,
+               uint32_t width, uint32_t height, uint32_t depth);
+};
+
+class _GPU_Tensor : public de::GPU_Tensor {
+    de::TensorLayout _layout;
+    de::_DATA_TYPES_FLAGS_ _type;
+    std::shared_ptr<DeviceBlock> _block;
+    void* _data;
+
+public:
+    _GPU_Tensor();
+    _GPU_Tensor(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height, uint32_t depth);
+    virtual uint Width() const;
+    virtual uint Height() const;
+    virtual uint Depth() const;
+    virtual de::GPU_Tensor& SoftCopy(de::GPU_Tensor& src);
+    virtual void release();
+    virtual de::_DATA_TYPES_FLAGS_ Type() const;
+    virtual void Reinterpret(const de::_DATA_TYPES_FLAGS_ new_type);
+    virtual de::DH Extract_SoftCopy(const uint32_t index, de::GPU_Tensor& dst) const;
+    virtual ~_GPU_Tensor();
+
+    const de::TensorLayout& get_layout() const { return _layout; }
+    bool is_init() const { return _data != nullptr; }
+    void* data() const { return _data; }
+    size_t total_bytes() const { return (size_t)_layout.dp_x_wp * _layout.height * _layout._single_element_size; }
+    bool re_construct(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height, uint32_t depth);   // grows only
+    void alias(const std::shared_ptr<DeviceBlock>& block, size_t bytes_offset, de::_DATA_TYPES_FLAGS_ type,
+               uint32_t width, uint32_t height, uint32_t depth);
+};
+
+class _TensorArray : public de::TensorArray {
+    de::TensorLayout _layout;
+    de::_DATA_TYPES_FLAGS_ _type;
+    uint32_t _count;
+    std::shared_ptr<HostBlock> _block;
+    std::shared_ptr<void*> _table;      // per-tensor pointers
+    void** _table_ptr;
+
+public:
+    _TensorArray();
+    _TensorArray(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height, uint32_t depth, uint32_t count);
+    virtual uint Width() const;
+    virtual uint Height() const;
+    virtual uint Depth() const;
+    virtual uint TensorNum() const;
+    virtual de::TensorArray& SoftCopy(de::TensorArray& src);
+    virtual de::_DATA_TYPES_FLAGS_ Type() const;
+    virtual void Reinterpret(const de::_DATA_TYPES_FLAGS_ new_type);
+    virtual de::DH Extract_SoftCopy(const uint32_t index, de::Tensor& dst) const;
+    virtual void release();
+    virtual ~_TensorArray();
+
+    size_t gap_bytes() const { return (size_t)_layout.dp_x_wp * _layout.height * _layout._single_element_size; }
+    bool is_init() const { return _block && _block->ptr; }
+};
+
+class _GPU_TensorArray : public de::GPU_TensorArray {
+    de::TensorLayout _layout;
+    de::_DATA_TYPES_FLAGS_ _type;
+    uint32_t _count;
+    std::shared_ptr<DeviceBlock> _block;
+
+public:
+    _GPU_TensorArray();
+    _GPU_TensorArray(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint32_t height, uint32_t depth, uint32_t count);
+    virtual uint Width() const;
+    virtual uint Height() const;
+    virtual uint Depth() const;
+    virtual uint TensorNum() const;
+    virtual de::_DATA_TYPES_FLAGS_ Type() const;
+    virtual void Reinterpret(const de::_DATA_TYPES_FLAGS_ new_type);
+    virtual de::GPU_TensorArray& SoftCopy(const de::GPU_TensorArray& src);
+    virtual de::DH Extract_SoftCopy(const uint32_t index, de::GPU_Tensor& dst) const;
+    virtual void release();
+    virtual ~_GPU_TensorArray();
+
+    const de::TensorLayout& get_layout() const { return _layout; }
+    size_t gap_bytes() const { return (size_t)_layout.dp_x_wp * _layout.height * _layout._single_element_size; }
+    bool is_init() const { return _block && _block->ptr; }
+    void* data() const { return _block ? _block->ptr : nullptr; }
+};
+
 // One stream for the module, created on first use; one mutex around every GEMM call
 // (the original guards its cached planner with a plain flag).
 void* module_stream();

@@ -115,6 +115,16 @@ struct __attribute__((aligned(8))) Point2D {         /* [x = along the width, y 
     Point2D() {}
 };
 
+struct __attribute__((aligned(16))) Point3D {        /* tensors: [x = depth, y = width, z = height] */
+    int32_t x, y, z;
+    Point3D(const int32_t _x, const int32_t _y, const int32_t _z) : x(_x), y(_y), z(_z) {}
+    Point3D(const uint32_t _x, const uint32_t _y, const uint32_t _z) : x((int32_t)_x), y((int32_t)_y), z((int32_t)_z) {}
+    Point3D() {}
+};
+
+/* How the borders of an image are treated by a convolution. */
+enum extend_label { _EXTEND_NONE_ = 0, _EXTEND_REFLECT_ = 1, _EXTEND_CONSTANT_ = 2 };
+
 _DECX_API_ Half  Float2Half(const float& __x);       /* round to nearest even */
 _DECX_API_ float Half2Float(const Half& __x);
 
@@ -289,6 +299,113 @@ _DECX_API_ DH PinMemory(Vector& src);
 _DECX_API_ DH UnpinMemory(Vector& src);
 }
 
+/* ------------------------------------------------------------------ tensors (images with channels) */
+
+/* Element (row x, column y, channel z) of a tensor lives at x * dp_x_wp + y * dpitch + z.  Host tensors pad
+ * the width to 4 columns, device tensors to 8; both pad the depth to 16 bytes of elements; zero-filled. */
+struct TensorLayout {
+    uint32_t width, height, depth;
+    uint32_t dpitch;               /* channel pitch in elements */
+    uint32_t wpitch;               /* row pitch in columns */
+    uint64_t dp_x_wp;              /* dpitch * wpitch */
+    uint8_t  _single_element_size;
+    uint64_t plane[3];             /* active elements of the WH, WD and HD planes */
+};
+
+class _DECX_API_ Tensor {
+protected:
+    _SHADOW_ATTRIBUTE_(void*)        _exp_data_ptr;
+    _SHADOW_ATTRIBUTE_(TensorLayout) _exp_tensor_dscr;
+
+public:
+    Tensor() {}
+    virtual uint32_t Width() const = 0;
+    virtual uint32_t Height() const = 0;
+    virtual uint32_t Depth() const = 0;
+
+    template <typename _ptr_type> _ptr_type* ptr(const int x, const int y, const int z) {
+        return ((_ptr_type*)(*this->_exp_data_ptr)) +
+               (x * this->_exp_tensor_dscr->dp_x_wp + y * this->_exp_tensor_dscr->dpitch + z);
+    }
+
+    virtual Tensor& SoftCopy(Tensor& src) = 0;
+    virtual void release() = 0;
+    virtual _DATA_TYPES_FLAGS_ Type() const = 0;
+    virtual void Reinterpret(const _DATA_TYPES_FLAGS_ _new_type) = 0;
+};
+
+_DECX_API_ Tensor* CreateTensorPtr();
+_DECX_API_ Tensor& CreateTensorRef();
+_DECX_API_ Tensor* CreateTensorPtr(const _DATA_TYPES_FLAGS_ _type, const uint _width, const uint _height, const uint _depth);
+_DECX_API_ Tensor& CreateTensorRef(const _DATA_TYPES_FLAGS_ _type, const uint _width, const uint _height, const uint _depth);
+
+class _DECX_API_ GPU_Tensor {
+public:
+    GPU_Tensor() {}
+    virtual uint Width() const = 0;
+    virtual uint Height() const = 0;
+    virtual uint Depth() const = 0;
+    virtual GPU_Tensor& SoftCopy(GPU_Tensor& src) = 0;
+    virtual void release() = 0;
+    virtual _DATA_TYPES_FLAGS_ Type() const = 0;
+    virtual void Reinterpret(const _DATA_TYPES_FLAGS_ _new_type) = 0;
+    virtual DH Extract_SoftCopy(const uint32_t index, GPU_Tensor& dst) const = 0;   /* one channel plane: not provided here */
+};
+
+_DECX_API_ GPU_Tensor* CreateGPUTensorPtr();
+_DECX_API_ GPU_Tensor& CreateGPUTensorRef();
+_DECX_API_ GPU_Tensor* CreateGPUTensorPtr(const _DATA_TYPES_FLAGS_ _type, const uint _width, const uint _height, const uint32_t _depth);
+_DECX_API_ GPU_Tensor& CreateGPUTensorRef(const _DATA_TYPES_FLAGS_ _type, const uint _width, const uint _height, const uint32_t _depth);
+
+/* tensor_num tensors of one shape in one allocation (a set of convolution kernels). */
+class _DECX_API_ TensorArray {
+protected:
+    _SHADOW_ATTRIBUTE_(void**)       _exp_data_ptr;        /* -> the table of per-tensor pointers */
+    _SHADOW_ATTRIBUTE_(TensorLayout) _exp_tensor_dscr;
+
+public:
+    TensorArray() {}
+    virtual uint Width() const = 0;
+    virtual uint Height() const = 0;
+    virtual uint Depth() const = 0;
+    virtual uint TensorNum() const = 0;
+
+    template <typename _ptr_type> _ptr_type* ptr(const int x, const int y, const int z, const int tensor_id) {
+        return ((_ptr_type*)(*this->_exp_data_ptr)[tensor_id]) + x * this->_exp_tensor_dscr->dp_x_wp +
+               y * this->_exp_tensor_dscr->dpitch + z;
+    }
+
+    virtual TensorArray& SoftCopy(TensorArray& src) = 0;
+    virtual _DATA_TYPES_FLAGS_ Type() const = 0;
+    virtual void Reinterpret(const _DATA_TYPES_FLAGS_ _new_type) = 0;
+    virtual DH Extract_SoftCopy(const uint32_t index, Tensor& dst) const = 0;        /* dst aliases tensor `index` */
+    virtual void release() = 0;
+};
+
+_DECX_API_ TensorArray& CreateTensorArrayRef();
+_DECX_API_ TensorArray* CreateTensorArrayPtr();
+_DECX_API_ TensorArray& CreateTensorArrayRef(const _DATA_TYPES_FLAGS_ _type, const uint width, const uint height, const uint depth, const uint tensor_num);
+_DECX_API_ TensorArray* CreateTensorArrayPtr(const _DATA_TYPES_FLAGS_ _type, const uint width, const uint height, const uint depth, const uint tensor_num);
+
+class _DECX_API_ GPU_TensorArray {
+public:
+    GPU_TensorArray() {}
+    virtual uint Width() const = 0;
+    virtual uint Height() const = 0;
+    virtual uint Depth() const = 0;
+    virtual uint TensorNum() const = 0;
+    virtual _DATA_TYPES_FLAGS_ Type() const = 0;
+    virtual void Reinterpret(const _DATA_TYPES_FLAGS_ _new_type) = 0;
+    virtual GPU_TensorArray& SoftCopy(const GPU_TensorArray& src) = 0;
+    virtual DH Extract_SoftCopy(const uint32_t index, GPU_Tensor& dst) const = 0;    /* dst aliases tensor `index` */
+    virtual void release() = 0;
+};
+
+_DECX_API_ GPU_TensorArray& CreateGPUTensorArrayRef();
+_DECX_API_ GPU_TensorArray* CreateGPUTensorArrayPtr();
+_DECX_API_ GPU_TensorArray& CreateGPUTensorArrayRef(const _DATA_TYPES_FLAGS_ _type, const uint width, const uint height, const uint depth, const uint32_t _array_length);
+_DECX_API_ GPU_TensorArray* CreateGPUTensorArrayPtr(const _DATA_TYPES_FLAGS_ _type, const uint width, const uint height, const uint depth, const uint32_t _array_length);
+
 /* ------------------------------------------------------------------ transfers */
 
 enum DECX_Memcpy_Flags { DECX_MEMCPY_H2D = 0, DECX_MEMCPY_D2H = 1 };
@@ -303,6 +420,11 @@ _DECX_API_ DH Memcpy(Matrix& __host, GPU_Matrix& __device, const Point2D start_s
  * destination (source = host vector for H2D, device vector for D2H). */
 _DECX_API_ DH Memcpy(Vector& __host, GPU_Vector& __device, const uint64_t start_src, const uint64_t start_dst,
                      const uint64_t cpy_len, const int _memcpy_flag);
+
+/* Copies the cpy_size = [D, W, H] box that starts at start_src = [depth, column, row] of the source to start_dst
+ * of the destination (source = host tensor for H2D, device tensor for D2H). */
+_DECX_API_ DH Memcpy(Tensor& __host, GPU_Tensor& __device, const Point3D start_src, const Point3D start_dst,
+                     const Point3D cpy_size, const int _memcpy_flag);
 
 /* ------------------------------------------------------------------ the product */
 namespace blas {
@@ -325,6 +447,19 @@ _DECX_API_ void GEMM(Vector& A, Matrix& B, Vector& dst, const uint32_t _fp16_acc
 _DECX_API_ void GEMM(Matrix& A, Vector& B, Vector& dst, const uint32_t _fp16_accu = 0);
 }  // namespace cuda
 }  // namespace blas
+
+/* ------------------------------------------------------------------ convolution on the product */
+namespace nn {
+namespace cuda {
+/* dst(y, x, n) <- sum over kh, kw, c of src(y * strides.y + kh, x * strides.x + kw, c) * kernel_n(kh, kw, c)   (fp32).
+ * _EXTEND_NONE_: dst is ((W - KW + 1) / strides.x) x ((H - KH + 1) / strides.y); _EXTEND_CONSTANT_: src is
+ * zero-extended (KW / 2 columns on the left, KH / 2 rows on top) and dst is (W / strides.x) x (H / strides.y).
+ * dst is reshaped to that size with depth = kernel.TensorNum().  Computed as one GEMM on the matrix cores whose
+ * left operand is read straight out of the image (no im2col buffer). */
+_DECX_API_ DH Conv2D(GPU_Tensor& src, GPU_TensorArray& kernel, GPU_Tensor& dst, const Point2D strides = {1, 1},
+                     const extend_label extend = _EXTEND_NONE_);
+}  // namespace cuda
+}  // namespace nn
 
 }  // namespace de
 

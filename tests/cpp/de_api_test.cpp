@@ -9,6 +9,10 @@
 //   de_api_test hostgemm <dir> <f32|f16> M N K <withC 0|1|2> <pinned 0|1> <repeats>
 //                                         the same through the host-matrix overloads (withC = 2: C is dst);
 //                                         prints the wall time of each repeat
+//   de_api_test tensor_host               tensor / tensor-array layouts and views, no GPU
+//   de_api_test conv <dir> W H C OC KW KH sx sy <extend 0|2>
+//                                         reads image.bin [H][W][C] and kernels.bin [OC][KH][KW][C] (dense fp32),
+//                                         runs de::nn::cuda::Conv2D, writes out.bin [OH][OW][OC] and prints OW OH
 //   de_api_test vmm <dir> <f32|f16> <mv|vm> W H <level 0|1|2>
 //                                         reads M.bin (H rows x W) and V.bin, writes Y.bin (fp32 for f32
 //                                         and for f16 at level 0, fp16 otherwise) through the host-object
@@ -402,6 +406,87 @@ template <typename T> static int gemm_files(const std::string& dir, de::_DATA_TY
     return out ? 0 : 2;
 }
 
+static int tensor_host_checks()
+{
+    // host tensors: width padded to 4 columns, depth to 16 bytes of elements; element (row, column, channel)
+    de::Tensor& t = de::CreateTensorRef(de::_FP32_, 10, 6, 3);
+    CHECK(t.Width() == 10 && t.Height() == 6 && t.Depth() == 3 && t.Type() == de::_FP32_);
+    CHECK(t.ptr<float>(0, 1, 0) - t.ptr<float>(0, 0, 0) == 4);            // dpitch
+    CHECK(t.ptr<float>(1, 0, 0) - t.ptr<float>(0, 0, 0) == 4 * 12);       // dpitch * wpitch
+    bool zero = true;
+    for (int i = 0; i < 6 * 12 * 4; ++i) zero &= (t.ptr<float>(0, 0, 0)[i] == 0.f);
+    CHECK(zero);
+    de::Tensor& th = de::CreateTensorRef(de::_FP16_, 3, 2, 9);
+    CHECK(th.ptr<de::Half>(0, 1, 0) - th.ptr<de::Half>(0, 0, 0) == 16 && th.ptr<de::Half>(1, 0, 0) - th.ptr<de::Half>(0, 0, 0) == 64);
+    de::Tensor& alias = de::CreateTensorRef();
+    alias.SoftCopy(t);
+    *t.ptr<float>(2, 3, 1) = 5.f;
+    CHECK(alias.Width() == 10 && *alias.ptr<float>(2, 3, 1) == 5.f);
+    // tensor arrays: tensors back to back, views by Extract_SoftCopy
+    de::TensorArray& a = de::CreateTensorArrayRef(de::_FP32_, 3, 3, 5, 7);
+    CHECK(a.Width() == 3 && a.Height() == 3 && a.Depth() == 5 && a.TensorNum() == 7);
+    CHECK(a.ptr<float>(0, 0, 0, 1) - a.ptr<float>(0, 0, 0, 0) == 8 * 4 * 3);          // dpitch 8, wpitch 4, 3 rows
+    *a.ptr<float>(1, 2, 4, 6) = 9.f;
+    de::Tensor& view = de::CreateTensorRef();
+    CHECK(a.Extract_SoftCopy(6, view).error_type == 0 && view.Depth() == 5 && *view.ptr<float>(1, 2, 4) == 9.f);
+    CHECK(a.Extract_SoftCopy(7, view).error_type == decx::DECX_FAIL_INVALID_PARAM);
+    a.release();
+    CHECK(*view.ptr<float>(1, 2, 4) == 9.f);                              // the view keeps the storage alive
+    CHECK(sizeof(de::Point3D) == 16 && de::_EXTEND_CONSTANT_ == 2);
+    // without InitCuda
+    de::GPU_Tensor& g = de::CreateGPUTensorRef();
+    de::GPU_TensorArray& gk = de::CreateGPUTensorArrayRef();
+    CHECK(de::Memcpy(t, g, de::Point3D(0, 0, 0), de::Point3D(0, 0, 0), de::Point3D(1, 1, 1), de::DECX_MEMCPY_H2D).error_type == decx::DECX_FAIL_CUDA_not_init);
+    CHECK(de::nn::cuda::Conv2D(g, gk, g).error_type == decx::DECX_FAIL_CUDA_not_init);
+    de::ResetLastError();
+    return g_failures;
+}
+
+static int conv_files(const std::string& dir, uint32_t W, uint32_t H, uint32_t C, uint32_t OC, uint32_t KW, uint32_t KH,
+                      int sx, int sy, int extend)
+{
+    de::InitCuda();
+    de::ResetLastError();
+    de::Tensor& img = de::CreateTensorRef(de::_FP32_, W, H, C);
+    de::TensorArray& ker = de::CreateTensorArrayRef(de::_FP32_, KW, KH, C, OC);
+    std::ifstream fi(dir + "/image.bin", std::ios::binary), fk(dir + "/kernels.bin", std::ios::binary);
+    if (!fi || !fk) return 2;
+    for (uint32_t y = 0; y < H; ++y) for (uint32_t x = 0; x < W; ++x) fi.read((char*)img.ptr<float>(y, x, 0), C * 4);
+    for (uint32_t o = 0; o < OC; ++o) for (uint32_t y = 0; y < KH; ++y) for (uint32_t x = 0; x < KW; ++x) fk.read((char*)ker.ptr<float>(y, x, 0, o), C * 4);
+    if (!fi || !fk) return 2;
+    de::GPU_Tensor& dimg = de::CreateGPUTensorRef(de::_FP32_, W, H, C);
+    de::GPU_TensorArray& dker = de::CreateGPUTensorArrayRef(de::_FP32_, KW, KH, C, OC);
+    de::GPU_Tensor& dout = de::CreateGPUTensorRef();
+    const de::Point3D O(0, 0, 0);
+    if (de::Memcpy(img, dimg, O, O, de::Point3D(C, W, H), de::DECX_MEMCPY_H2D).error_type) return 3;
+    de::Tensor& hv = de::CreateTensorRef();
+    de::GPU_Tensor& dv = de::CreateGPUTensorRef();
+    for (uint32_t o = 0; o < OC; ++o) {                                   // kernels go up one by one through views
+        if (ker.Extract_SoftCopy(o, hv).error_type || dker.Extract_SoftCopy(o, dv).error_type) return 3;
+        if (de::Memcpy(hv, dv, O, O, de::Point3D(C, KW, KH), de::DECX_MEMCPY_H2D).error_type) return 3;
+    }
+    de::DH r = de::nn::cuda::Conv2D(dimg, dker, dout, de::Point2D(sx, sy), (de::extend_label)extend);
+    if (r.error_type) { std::cerr << r.error_string << "\n"; return 4; }
+    r = de::nn::cuda::Conv2D(dimg, dker, dout, de::Point2D(sx, sy), (de::extend_label)extend);    // again: scratch reused
+    if (r.error_type) return 4;
+    const uint32_t OW = dout.Width(), OH = dout.Height();
+    if (dout.Depth() != OC) return 5;
+    de::Tensor& out = de::CreateTensorRef(de::_FP32_, OW, OH, OC);
+    if (OW && OH && de::Memcpy(out, dout, O, O, de::Point3D(OC, OW, OH), de::DECX_MEMCPY_D2H).error_type) return 3;
+    std::ofstream fo(dir + "/out.bin", std::ios::binary);
+    for (uint32_t y = 0; y < OH; ++y) for (uint32_t x = 0; x < OW; ++x) fo.write((const char*)out.ptr<float>(y, x, 0), OC * 4);
+    std::cout << "conv out " << OW << " " << OH << "\n";
+    // error paths
+    de::GPU_TensorArray& bad = de::CreateGPUTensorArrayRef(de::_FP32_, KW, KH, C + 1, OC);
+    if (de::nn::cuda::Conv2D(dimg, bad, dout, de::Point2D(sx, sy), (de::extend_label)extend).error_type != decx::DECX_FAIL_DimsNotMatching) return 6;
+    if (de::nn::cuda::Conv2D(dimg, dker, dout, de::Point2D(sx, sy), de::_EXTEND_REFLECT_).error_type != decx::DECX_FAIL_ErrorFlag) return 6;
+    if (de::nn::cuda::Conv2D(dimg, dker, dout, de::Point2D(0, sy), (de::extend_label)extend).error_type != decx::DECX_FAIL_INVALID_PARAM) return 6;
+    de::GPU_Tensor& half_img = de::CreateGPUTensorRef(de::_FP16_, W, H, C);
+    if (de::nn::cuda::Conv2D(half_img, dker, dout).error_type != decx::DECX_FAIL_TYPE_MOT_MATCH) return 6;
+    if (dout.Width() != OW || dout.Height() != OH) return 6;             // failed calls left dst alone
+    return fo ? 0 : 2;
+}
+
 template <typename T> static int hostgemm_files(const std::string& dir, de::_DATA_TYPES_FLAGS_ ty, uint32_t M, uint32_t N,
                                                 uint32_t K, int with_c, bool pinned, int repeats)
 {
@@ -445,6 +530,10 @@ int main(int argc, char** argv)
         rc = f16 ? hostgemm_files<de::Half>(argv[2], de::_FP16_, M, N, K, with_c, pinned, repeats)
                  : hostgemm_files<float>(argv[2], de::_FP32_, M, N, K, with_c, pinned, repeats);
     }
+    else if (mode == "tensor_host") rc = tensor_host_checks();
+    else if (mode == "conv" && argc == 12)
+        rc = conv_files(argv[2], std::atoi(argv[3]), std::atoi(argv[4]), std::atoi(argv[5]), std::atoi(argv[6]), std::atoi(argv[7]),
+                        std::atoi(argv[8]), std::atoi(argv[9]), std::atoi(argv[10]), std::atoi(argv[11]));
     else if (mode == "vector_host") rc = vector_host_checks();
     else if (mode == "vector_gpu") rc = vector_gpu_checks();
     else if (mode == "vmm" && argc == 8) {

@@ -30,6 +30,11 @@ def test_host_side_vectors_and_error_codes():
     assert rc == 0, out
 
 
+def test_host_side_tensors_and_views():
+    rc, out = run_exe("tensor_host")
+    assert rc == 0, out
+
+
 def test_host_library_exports_the_public_entry_points():
     lib = os.path.join(ROOT, "decx_amd", "lib", "libDECX_BLAS_HIP.so")
     syms = subprocess.run(["nm", "-D", "-C", "--defined-only", lib], stdout=subprocess.PIPE, text=True).stdout
@@ -44,6 +49,9 @@ def test_host_library_exports_the_public_entry_points():
                    "de::blas::cuda::GEMM(de::Vector&, de::Matrix&, de::Vector&, unsigned int)",
                    "de::blas::cuda::GEMM(de::Matrix&, de::Vector&, de::Vector&, unsigned int)",
                    "de::CreateVectorRef(de::_DATA_TYPES_FLAGS_, unsigned long)",
+                   "de::nn::cuda::Conv2D(de::GPU_Tensor&, de::GPU_TensorArray&, de::GPU_Tensor&, de::Point2D, de::extend_label)",
+                   "de::CreateGPUTensorArrayRef(de::_DATA_TYPES_FLAGS_, unsigned int, unsigned int, unsigned int, unsigned int)",
+                   "de::Memcpy(de::Tensor&, de::GPU_Tensor&, de::Point3D, de::Point3D, de::Point3D, int)",
                    "de::CreateGPUVectorRef(de::_DATA_TYPES_FLAGS_, unsigned long)",
                    "de::Memcpy(de::Vector&, de::GPU_Vector&, unsigned long, unsigned long, unsigned long, int)"]:
         assert needle in syms, needle
@@ -153,3 +161,24 @@ def test_host_matrix_forms_match_oracle(oracle, dt, M, N, K, with_c, pinned):
     ref = ref.astype(np.float64)
     err = np.max(np.abs(D.astype(np.float64) - ref)) / (np.max(np.abs(ref)) * np.sqrt(K))
     assert err <= tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("W,H,C,OC,KW,KH,sx,sy,extend", [
+    (20, 17, 5, 3, 4, 2, 2, 1, 0), (20, 17, 5, 3, 4, 2, 2, 1, 2),
+    (57, 43, 13, 70, 3, 3, 1, 1, 0), (57, 43, 13, 70, 3, 3, 1, 1, 2),
+    (64, 48, 16, 64, 5, 5, 2, 2, 2), (9, 9, 4, 8, 9, 9, 1, 1, 0),
+])
+def test_conv2d_through_the_objects_matches_oracle(oracle, W, H, C, OC, KW, KH, sx, sy, extend):
+    """de::nn::cuda::Conv2D on GPU_Tensor / GPU_TensorArray objects filled through de::Memcpy and views."""
+    image = synth.uniform_f32(H, W * C, 601).reshape(H, W, C)
+    kernels = synth.uniform_f32(OC, KH * KW * C, 602).reshape(OC, KH, KW, C)
+    ref = oracle.conv2d_f32(image, kernels, sx, sy, extend == 2)
+    with tempfile.TemporaryDirectory() as tmp:
+        image.tofile(os.path.join(tmp, "image.bin")); kernels.tofile(os.path.join(tmp, "kernels.bin"))
+        rc, out = run_exe("conv", tmp, W, H, C, OC, KW, KH, sx, sy, extend)
+        assert rc == 0, out
+        got = np.fromfile(os.path.join(tmp, "out.bin"), np.float32).reshape(ref.shape)
+    assert ("conv out %d %d" % (ref.shape[1], ref.shape[0])) in out
+    r = ref.astype(np.float64)
+    assert np.max(np.abs(got - r)) / (np.max(np.abs(r)) * np.sqrt(KW * KH * C)) <= 1e-5
