@@ -24,6 +24,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_F32_TFLOPS = 157.3      # MI355X dense fp32 matrix
 PEAK_F16_TFLOPS = 2500.0     # MI355X dense fp16 matrix
+PEAK_F64_TFLOPS = 78.6       # MI355X dense fp64 matrix
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by a
@@ -39,6 +40,7 @@ WORKLOADS = {
     # name: (dtype, M, N, K, bound, config number for seeds, description)
     "fp32_8192": ("f32", 8192, 8192, 8192, "mfma", 4, "fp32 GEMM C=A.B M=N=K=8192, uniform[-1,1]"),
     "fp16_4096": ("f16", 4096, 4096, 4096, "mfma", 3, "fp16 GEMM (fp32 accumulate, fp16 out) M=N=K=4096, normal(0,0.5) clipped to [-4,4]"),
+    "fp64_4096": ("f64", 4096, 4096, 4096, "mfma", 7, "fp64 GEMM M=N=K=4096, uniform[-1,1]"),
     "fp32_1024": ("f32", 1024, 1024, 1024, "mfma", 1, "fp32 GEMM M=N=K=1024, uniform[-1,1]"),
     "fp32_ragged": ("f32", 1000, 1500, 777, "mfma", 2, "fp32 GEMM M=1000 N=1500 K=777, uniform[-1,1]"),
     "fp32_tall_skinny": ("f32", 65536, 256, 1024, "mfma", 5, "fp32 GEMM M=65536 N=256 K=1024, uniform[-1,1]"),
@@ -55,6 +57,8 @@ def make_inputs(name):
     sa, sb, _ = synth.seeds(cfg)
     if dt == "f32":
         return synth.uniform_f32(M, K, sa), synth.uniform_f32(K, N, sb)
+    if dt == "f64":
+        return synth.uniform_f64(M, K, sa), synth.uniform_f64(K, N, sb)
     return synth.normal_half(M, K, sa), synth.normal_half(K, N, sb)
 
 
@@ -66,7 +70,7 @@ def device_pitch(cols, itemsize):
 def run_workload(name, steps, warmup, keep_inputs=False, settle_s=0.0):
     from decx_amd import hip
     dt, M, N, K, bound, _, desc = WORKLOADS[name]
-    npdt = np.float32 if dt == "f32" else np.float16
+    npdt = {"f32": np.float32, "f16": np.float16, "f64": np.float64}[dt]
     A, B = make_inputs(name)
     isz = np.dtype(npdt).itemsize
     dA = hip.DeviceMatrix(M, K, npdt, device_pitch(K, isz), A)
@@ -95,7 +99,7 @@ def run_workload(name, steps, warmup, keep_inputs=False, settle_s=0.0):
     tflops = flops / (kernel_ms * 1e-3) / 1e12
     gbs = abytes / (kernel_ms * 1e-3) / 1e9
     if bound == "mfma":
-        peak = PEAK_F32_TFLOPS if dt == "f32" else PEAK_F16_TFLOPS
+        peak = {"f32": PEAK_F32_TFLOPS, "f16": PEAK_F16_TFLOPS, "f64": PEAK_F64_TFLOPS}[dt]
         roof = {"bound": "mfma", "achieved": round(tflops, 3), "peak": peak, "unit": "TFLOP/s",
                 "frac": round(tflops / peak, 4), "traffic": MEASURED_TRAFFIC.get(name)}
     else:

@@ -25,6 +25,20 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 // Picks the block tile: cost = (tiles the busiest CU runs) x (tile area) / (relative speed
 // of that shape).  Big tiles win once they fill the chip; small tiles win while the grid
 // would otherwise leave CUs idle.  Ties go to the larger tile.
+int choose_tile_f64(uint32_t M, uint32_t N)
+{
+    int best = TILE_64x64;
+    double best_cost = 1e300;
+    for (int s = TILE_COUNT - 1; s >= 0; --s) {
+        const TileInfo ti = tile_info_f64(s);
+        const uint64_t tiles = (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
+        const uint64_t per_cu = (tiles + g_dev.compute_units - 1) / g_dev.compute_units;
+        const double cost = (double)per_cu * ti.bm * ti.bn / ti.rel_speed;
+        if (cost <= best_cost) { best_cost = cost; best = s; }
+    }
+    return best;
+}
+
 int choose_tile(bool f16, uint32_t M, uint32_t N, bool aligned)
 {
     int best = TILE_64x64;
@@ -247,6 +261,40 @@ int decx_hip_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, u
     return run_gemm<true>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0);
 }
 
+static int run_gemm_f64(const double* A, const double* B, const double* C, double* D, uint32_t M, uint32_t N, uint32_t K,
+                        uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, double alpha, double beta, void* stream,
+                        int tile, int force_plain)
+{
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    const int rc = check_gemm(A, B, C, D, M, N, K, lda, ldb, ldc, ldd);
+    if (rc != DECX_HIP_OK || M == 0 || N == 0) return rc;
+    if (tile != DECX_HIP_TILE_AUTO && (tile < 0 || tile >= TILE_COUNT)) return DECX_HIP_E_INVALID_ARG;
+    GemmArgs g;
+    std::memset(&g, 0, sizeof g);
+    g.A = A; g.B = B; g.C = C; g.D = D;
+    g.M = M; g.N = N; g.K = K;
+    g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldd = ldd;
+    g.alpha = (float)alpha; g.beta = (float)beta;
+    g.alpha64 = alpha; g.beta64 = beta;
+    g.vec_ok = (aligned16(A) && aligned16(B) && aligned16(D) && (!C || aligned16(C)) &&
+                lda % 2 == 0 && ldb % 2 == 0 && ldd % 2 == 0 && (!C || ldc % 2 == 0)) ? 1u : 0u;
+    const int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile_f64(M, N) : tile;
+    return launch_gemm_f64(shape, force_plain != 0, g, as_stream(stream));
+}
+
+int decx_hip_gemm_f64(const double* A, const double* B, const double* C, double* D, uint32_t M, uint32_t N, uint32_t K,
+                      uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, double alpha, double beta, void* stream)
+{
+    return run_gemm_f64(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0);
+}
+
+int decx_hip_gemm_f64_tile(const double* A, const double* B, const double* C, double* D, uint32_t M, uint32_t N,
+                           uint32_t K, uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, double alpha,
+                           double beta, void* stream, int tile, int force_plain)
+{
+    return run_gemm_f64(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, tile, force_plain);
+}
+
 int decx_hip_gemm_f32_tile(const float* A, const float* B, const float* C, float* D, uint32_t M, uint32_t N,
                            uint32_t K, uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha,
                            float beta, void* stream, int tile, int force_edge)
@@ -349,9 +397,19 @@ int decx_hip_conv2d_f32(const float* image, const float* kmat, float* dst, uint3
 
 int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int aligned, decx_hip_plan* out)
 {
-    if (!out || (elem_bytes != 4 && elem_bytes != 2)) return DECX_HIP_E_INVALID_ARG;
+    if (!out || (elem_bytes != 4 && elem_bytes != 2 && elem_bytes != 8)) return DECX_HIP_E_INVALID_ARG;
     std::memset(out, 0, sizeof *out);
     if (M == 0 || N == 0) return DECX_HIP_OK;
+    if (elem_bytes == 8) {                      // fp64 has no vector-corner kernels: N == 1 / M == 1 run as thin GEMMs
+        const int shape = choose_tile_f64(M, N);
+        const TileInfo ti = tile_info_f64(shape);
+        out->path = shape;
+        out->tile_m = ti.bm; out->tile_n = ti.bn;
+        out->grid = ((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
+        out->edge = (K == 0 || !aligned) ? 1 : 0;
+        if (out->edge) { out->tile_m = out->tile_n = 16; out->grid = ((M + 15) / 16) * ((N + 15) / 16); }
+        return DECX_HIP_OK;
+    }
     const bool f16 = elem_bytes == 2;
     if (N == 1 && K > 0) {
         out->path = DECX_HIP_PATH_GEMV;

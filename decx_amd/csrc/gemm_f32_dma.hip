@@ -83,7 +83,8 @@ gemm_f32_dma_kernel(const GemmArgs g)
     constexpr int A_LOADS = A_STAGE_BYTES / 1024 / WAVES, B_LOADS = B_STAGE_BYTES / 1024 / WAVES, LOADS = A_LOADS + B_LOADS;
     constexpr int B_SHIFT = (TN == 1) ? 8 : 0;                    // chunk shift of k rows with bit 2 set
     static_assert(TM >= 1 && (TN == 1 || TN == 2 || TN == 4), "wave tile");
-    static_assert(BK == 16 || BK == 32, "slab depth");
+    static_assert(BK == 16 || BK == 32, "slab depth");     // an even number of 8-deep chunks: the fragments of a slab's last
+                                                            // chunk and of the next slab's first one sit in different registers
     static_assert(CB <= 64 && 64 % CB == 0 && (B_SHIFT == 0 || CB >= 16), "B copy plan");
     static_assert(A_LOADS >= 1 && B_LOADS >= 1 && A_LOADS * WAVES * 1024 == A_STAGE_BYTES &&
                   B_LOADS * WAVES * 1024 == B_STAGE_BYTES, "copy plan must divide evenly");

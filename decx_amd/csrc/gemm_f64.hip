@@ -1,0 +1,310 @@
+// fp64 GEMM for gfx950 on the fp64 matrix cores (v_mfma_f64_16x16x4_f64).
+//
+// Replaces the reference's cu_GEMM_fp64_*_16_64_64 kernels and their runner
+// (srcs/modules/BLAS/GEMM/CUDA/large_squares/GEMM_kernels.cuh:182-189, GEMM_LS.cu:164-211).
+// Same data movement as the fp32 / fp16 kernels: K slabs go global -> LDS by direct 128-bit
+// loads into a ring of STAGES stages (inline assembly, bare s_barrier behind an explicit vmcnt
+// wait), ragged M / N by fetching the last valid row / column chunk, ragged K through registers
+// with zero fill.
+//
+// Fragment scheme.  One MFMA multiplies a 16 x 4 by a 4 x 16 block: lane l supplies A(l % 16, q)
+// and B(q, l % 16) with q = l / 16, and holds D(4 i + q, l % 16) in result element i.  A lane
+// fetches two consecutive k of its A row with one 128-bit LDS read and uses them in two
+// successive k steps: step 2 t + e takes k = 8 t + 2 q + e (any assignment of k's to steps is valid
+// as long as A and B agree).  Columns are dealt to lanes in pairs (lane c owns columns
+// 32 jj + 2 c, 32 jj + 2 c + 1 of the wave tile), so B fragments are 128-bit reads of adjacent
+// lanes and the epilogue stores 16 bytes per lane.
+//
+// LDS layout of a stage: A as [BM rows][BK / 2 chunks of 16 bytes], chunk c of row r in slot
+// c ^ ((r / RP) % CPR); B as [BK][BN] doubles, straight.
+//
+// A plain one-thread-per-element kernel serves operands that are not 16-byte aligned, and K == 0.
+#include "gemm_common.hpp"
+#include <type_traits>
+
+namespace decx_hip {
+
+namespace {
+
+typedef double doublex2 __attribute__((ext_vector_type(2)));
+typedef double doublex4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void lds_void;
+
+template <int I, int N, class F> __device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+template <int N> __device__ __forceinline__ void wait_loads_and_barrier()
+{
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(N) : "memory");
+}
+
+}  // namespace
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES>
+__global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
+gemm_f64_dma_kernel(const GemmArgs g)
+{
+    constexpr int WAVES = WAVES_M * WAVES_N;
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 16, TN = WN / 16, TP = TN / 2;
+    constexpr int RBYTES = BK * 8, CPR = RBYTES / 16, RP = 16 / CPR;       // A row bytes, chunks per row, rows per 256 bytes
+    constexpr int CB = BN / 2, RB = 64 / CB;                               // B chunks per k row, k rows per direct load
+    constexpr int A_STAGE_BYTES = BM * RBYTES, B_STAGE_BYTES = BK * BN * 8, STAGE_BYTES = A_STAGE_BYTES + B_STAGE_BYTES;
+    constexpr int A_LOADS = A_STAGE_BYTES / 1024 / WAVES, B_LOADS = B_STAGE_BYTES / 1024 / WAVES, LOADS = A_LOADS + B_LOADS;
+    constexpr int STEPS = BK / 4, GROUPS = BK / 8;                          // MFMA k steps, 8-deep k groups per slab
+    // GROUPS must be even: the A pairs of a slab's last k group (af[1]) have to survive the reads of the next
+    // slab's first group (af[0]) until the deferred last step is issued
+    static_assert(TM >= 1 && TN >= 2 && TN % 2 == 0 && BK == 16, "shape");
+    static_assert(CB <= 64 && 64 % CB == 0, "B copy plan");
+    static_assert(A_LOADS >= 1 && B_LOADS >= 1 && A_LOADS * WAVES * 1024 == A_STAGE_BYTES &&
+                  B_LOADS * WAVES * 1024 == B_STAGE_BYTES, "copy plan must divide evenly");
+    static_assert(STAGES >= 2 && STAGES * STAGE_BYTES <= 160 * 1024, "LDS budget");
+    static_assert(LOADS * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE_BYTES];
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)lds;
+
+    uint32_t tile_m, tile_n;
+    block_to_tile(g, tile_m, tile_n);
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
+    const int l16 = lane & 15, q = lane >> 4;
+
+    const unsigned char* __restrict__ A = (const unsigned char*)g.A;
+    const unsigned char* __restrict__ B = (const unsigned char*)g.B;
+    const size_t lda_b = (size_t)g.lda * 8, ldb_b = (size_t)g.ldb * 8;
+
+    // ---- copy plan (rows beyond M and column chunks beyond N are replaced by the last valid ones)
+    const unsigned char* a_src[A_LOADS];
+    const unsigned char* b_src[B_LOADS];
+    int a_chunk[A_LOADS], b_krow[B_LOADS];
+    const uint32_t last_row = g.M - 1, last_col_chunk = (g.N - 1) / 2;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+        const int I = wave * A_LOADS + i;
+        const int row = I * (64 / CPR) + lane / CPR;
+        a_chunk[i] = (lane % CPR) ^ ((row / RP) % CPR);
+        const uint32_t grow = (m0 + row) < last_row ? (m0 + row) : last_row;
+        a_src[i] = A + (size_t)grow * lda_b + a_chunk[i] * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+        const int I = wave * B_LOADS + i;
+        b_krow[i] = I * RB + lane / CB;
+        const uint32_t chunk = lane % CB;
+        const uint32_t gchunk = (n0 / 2 + chunk) < last_col_chunk ? (n0 / 2 + chunk) : last_col_chunk;
+        b_src[i] = B + (size_t)b_krow[i] * ldb_b + (size_t)gchunk * 16;
+    }
+
+    const uint32_t full_slabs = g.K / BK, k_tail = g.K % BK;
+    const uint32_t slabs = full_slabs + (k_tail ? 1u : 0u);
+
+    auto issue_loads = [&](uint32_t slab) {
+        const uint32_t stage = slab % STAGES;
+        if (slab < full_slabs) {
+            const uint32_t stage_off = lds_base + stage * STAGE_BYTES;
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) {
+                const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u);
+                const unsigned char* src = a_src[i] + (size_t)slab * RBYTES;
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
+            }
+#pragma unroll
+            for (int i = 0; i < B_LOADS; ++i) {
+                const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + A_STAGE_BYTES +
+                                                                    (uint32_t)(wave * B_LOADS + i) * 1024u);
+                const unsigned char* src = b_src[i] + (size_t)slab * BK * ldb_b;
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
+            }
+        } else {
+            // the partial last slab: through registers, zero beyond K
+            unsigned char* st = lds + stage * STAGE_BYTES;
+            const uint32_t k0 = full_slabs * BK;
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i) {
+                const uint32_t k = k0 + a_chunk[i] * 2;
+                doublex2 v = doublex2{0.0, 0.0};
+                if (k < g.K) {
+                    v = *(const doublex2*)(a_src[i] + (size_t)k0 * 8);      // inside the pitch: lda is a multiple of 2
+                    if (k + 1 >= g.K) v[1] = 0.0;
+                }
+                *(doublex2*)(st + (wave * A_LOADS + i) * 1024 + lane * 16) = v;
+            }
+#pragma unroll
+            for (int i = 0; i < B_LOADS; ++i) {
+                doublex2 v = doublex2{0.0, 0.0};
+                if (k0 + b_krow[i] < g.K) v = *(const doublex2*)(b_src[i] + (size_t)k0 * ldb_b);
+                *(doublex2*)(st + A_STAGE_BYTES + (wave * B_LOADS + i) * 1024 + lane * 16) = v;
+            }
+        }
+    };
+
+    // ---- fragment addressing inside a stage
+    const int a_row = wm0 + l16;                       // + 16 i leaves (row / RP) % CPR unchanged
+    const int a_sw = (a_row / RP) % CPR;
+    int a_off[GROUPS];                                 // byte offset of chunk 4 t + q of this lane's row
+#pragma unroll
+    for (int tt = 0; tt < GROUPS; ++tt) a_off[tt] = a_row * RBYTES + (((4 * tt + q) ^ a_sw) * 16);
+    const int b_col = wn0 + 2 * l16;                   // + 32 jj
+    const int b_off = A_STAGE_BYTES + (2 * q) * BN * 8 + b_col * 8;       // + (8 t + e) rows
+
+    doublex4 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = doublex4{0.0, 0.0, 0.0, 0.0};
+
+#pragma unroll
+    for (int p = 0; p < STAGES - 1; ++p)
+        if ((uint32_t)p < slabs) issue_loads(p);
+    if (slabs >= (uint32_t)(STAGES - 1)) wait_loads_and_barrier<LOADS * (STAGES - 2)>();
+    else wait_loads_and_barrier<0>();
+
+    // af[t & 1] holds the A pairs of k group t, bf[step & 1] the B pairs of a k step.  Fragments are fetched one
+    // step ahead; the MFMAs of the last step of a slab are issued after the slab barrier, behind the first
+    // fragment reads of the next slab (before the first slab they multiply zeros).
+    doublex2 af[2][TM];
+    doublex2 bf[2][TP];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) af[(GROUPS - 1) & 1][i] = doublex2{0.0, 0.0};
+#pragma unroll
+    for (int jj = 0; jj < TP; ++jj) bf[(STEPS - 1) & 1][jj] = doublex2{0.0, 0.0};
+
+    auto multiply = [&](auto stc) {
+        constexpr int step = decltype(stc)::value;
+        constexpr int tt = step / 2, e = step % 2;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[tt & 1][i][e], bf[step & 1][j / 2][j % 2], acc[i][j], 0, 0, 0);
+    };
+    auto read_b = [&](const unsigned char* st, auto stc) {
+        constexpr int step = decltype(stc)::value;
+#pragma unroll
+        for (int jj = 0; jj < TP; ++jj)
+            bf[step & 1][jj] = *(const doublex2*)(st + b_off + (8 * (step / 2) + step % 2) * BN * 8 + jj * 32 * 8);
+    };
+    auto read_a = [&](const unsigned char* st, auto tc) {
+        constexpr int tt = decltype(tc)::value;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) af[tt & 1][i] = *(const doublex2*)(st + a_off[tt] + i * 16 * RBYTES);
+    };
+
+    for (uint32_t s = 0; s < slabs; ++s) {
+        const unsigned char* st = lds + (s % STAGES) * STAGE_BYTES;
+        const bool more = s + STAGES - 1 < slabs;
+
+        read_a(st, std::integral_constant<int, 0>{});
+        read_b(st, std::integral_constant<int, 0>{});
+        multiply(std::integral_constant<int, STEPS - 1>{});
+        __builtin_amdgcn_sched_group_barrier(0x100, TM + TP, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        // the stage that held slab s-1 is free: every wave passed the barrier after reading it
+        if (more) issue_loads(s + STAGES - 1);
+
+        static_for<0, STEPS - 1>([&](auto stc) {
+            constexpr int step = decltype(stc)::value;
+            constexpr bool next_a = (step % 2 == 1);                   // step + 1 opens the next k group
+            read_b(st, std::integral_constant<int, step + 1>{});
+            if constexpr (next_a) read_a(st, std::integral_constant<int, (step + 1) / 2>{});
+            multiply(stc);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, TP + (next_a ? TM : 0), 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 1, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+
+        if (more) wait_loads_and_barrier<LOADS * (STAGES - 2)>(); else wait_loads_and_barrier<0>();
+    }
+    multiply(std::integral_constant<int, STEPS - 1>{});
+
+    // Epilogue: element i of tile (ti, tj) is row 16 ti + 4 i + q; tiles 2 jj, 2 jj + 1 are the adjacent columns
+    // 32 jj + 2 l16, + 1.
+    const double* __restrict__ C = (const double*)g.C;
+    double* __restrict__ D = (double*)g.D;
+    const bool interior = (m0 + BM <= g.M) && (n0 + BN <= g.N);
+#pragma unroll
+    for (int ti = 0; ti < TM; ++ti) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t row = m0 + wm0 + 16 * ti + 4 * i + q;
+#pragma unroll
+            for (int jj = 0; jj < TP; ++jj) {
+                const uint32_t col = n0 + b_col + 32 * jj;
+                double v0 = acc[ti][2 * jj][i], v1 = acc[ti][2 * jj + 1][i];
+                if (interior) {
+                    if (C) {
+                        const doublex2 cv = *(const doublex2*)(C + (size_t)row * g.ldc + col);
+                        v0 = __builtin_fma(cv[0], g.beta64, g.alpha64 * v0);
+                        v1 = __builtin_fma(cv[1], g.beta64, g.alpha64 * v1);
+                    }
+                    *(doublex2*)(D + (size_t)row * g.ldd + col) = doublex2{v0, v1};
+                } else if (row < g.M) {
+                    if (col < g.N) {
+                        if (C) v0 = __builtin_fma(C[(size_t)row * g.ldc + col], g.beta64, g.alpha64 * v0);
+                        D[(size_t)row * g.ldd + col] = v0;
+                    }
+                    if (col + 1 < g.N) {
+                        if (C) v1 = __builtin_fma(C[(size_t)row * g.ldc + col + 1], g.beta64, g.alpha64 * v1);
+                        D[(size_t)row * g.ldd + col + 1] = v1;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// One thread per output element, k ascending: any alignment, any K (also 0).
+__global__ void __launch_bounds__(256) gemm_f64_plain_kernel(const GemmArgs g)
+{
+    const uint32_t col = blockIdx.x * 16 + (threadIdx.x & 15), row = blockIdx.y * 16 + (threadIdx.x >> 4);
+    if (row >= g.M || col >= g.N) return;
+    const double* a = (const double*)g.A + (size_t)row * g.lda;
+    const double* b = (const double*)g.B + col;
+    double acc = 0.0;
+    for (uint32_t k = 0; k < g.K; ++k) acc = __builtin_fma(a[k], b[(size_t)k * g.ldb], acc);
+    if (g.C) acc = __builtin_fma(((const double*)g.C)[(size_t)row * g.ldc + col], g.beta64, g.alpha64 * acc);
+    ((double*)g.D)[(size_t)row * g.ldd + col] = acc;
+}
+
+namespace {
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES>
+int launch_dma(const GemmArgs& args, hipStream_t stream)
+{
+    GemmArgs g = args;
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    const uint32_t nb = g.tiles_m * g.tiles_n;
+    g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
+    hipLaunchKernelGGL((gemm_f64_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES>), dim3(nb), dim3(WAVES_M * WAVES_N * 64),
+                       0, stream, g);
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
+// shape: TILE_256x256 stands for the largest fp64 tile, 256 x 128 (eight wavefronts of 64 x 64).
+int launch_gemm_f64(int shape, bool plain, const GemmArgs& args, hipStream_t stream)
+{
+    if (plain || !args.vec_ok || args.K == 0) {
+        const dim3 grid((args.N + 15) / 16, (args.M + 15) / 16);
+        hipLaunchKernelGGL(gemm_f64_plain_kernel, grid, dim3(256), 0, stream, args);
+        return (int)hipGetLastError();
+    }
+    switch (shape) {
+    case TILE_256x256: return launch_dma<256, 128, 4, 2, 16, 3>(args, stream);
+    case TILE_128x128: return launch_dma<128, 128, 2, 2, 16, 3>(args, stream);
+    case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 16, 4>(args, stream);
+    default:           return (int)hipErrorInvalidValue;
+    }
+}
+
+}  // namespace decx_hip

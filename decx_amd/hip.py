@@ -58,6 +58,8 @@ SYMBOLS = {
     "decx_hip_gevm_f16": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _int, _vp]),
     "decx_hip_conv2d_pack_kernels_f32": (_int, [_vp, _vp] + [_u32] * 5 + [ctypes.c_uint64] + [_u32] * 3 + [_vp]),
     "decx_hip_conv2d_f32": (_int, [_vp] * 3 + [_u32] * 12 + [_vp]),
+    "decx_hip_gemm_f64": (_int, [_vp] * 4 + [_u32] * 7 + [ctypes.c_double, ctypes.c_double, _vp]),
+    "decx_hip_gemm_f64_tile": (_int, [_vp] * 4 + [_u32] * 7 + [ctypes.c_double, ctypes.c_double, _vp, _int, _int]),
     "decx_hip_gemm_f32_tile": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, _int, _int]),
     "decx_hip_gemm_f16_tile": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, _int, _int]),
     "decx_hip_gemm_plan": (_int, [_int, _u32, _u32, _u32, _int, ctypes.POINTER(Plan)]),
@@ -181,6 +183,12 @@ def gemm(A, B, D, C=None, alpha=1.0, beta=1.0, stream=None, tile=TILE_AUTO, forc
     f16 = A.dtype == np.float16
     args = [A.ptr, B.ptr, C.ptr if C is not None else None, D.ptr, M, N, K, A.pitch, B.pitch,
             C.pitch if C is not None else 0, D.pitch, alpha, beta, stream]
+    if A.dtype == np.float64:
+        if tile == TILE_AUTO and not force_edge:
+            check(L.decx_hip_gemm_f64(*args), "gemm")
+        else:
+            check(L.decx_hip_gemm_f64_tile(*args, tile, 1 if force_edge else 0), "gemm")
+        return
     if tile == TILE_AUTO and not force_edge:
         rc = (L.decx_hip_gemm_f16 if f16 else L.decx_hip_gemm_f32)(*args)
     else:

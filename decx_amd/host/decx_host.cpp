@@ -376,14 +376,14 @@ bool validate(const decx::_GPU_Matrix* A, const decx::_GPU_Matrix* B, const decx
                        "The input scalar alpha and beta must match the type of input matrices");
         return false;
     }
-    if (A->Type() != de::_FP32_ && A->Type() != de::_FP16_) {
+    if (A->Type() != de::_FP32_ && A->Type() != de::_FP16_ && A->Type() != de::_FP64_) {
         decx::err::set(h, decx::DECX_FAIL_UNSUPPORTED_TYPE, kUnsupportedType); return false;
     }
     return true;
 }
 
 bool gemm_device(decx::_GPU_Matrix* A, decx::_GPU_Matrix* B, decx::_GPU_Matrix* C, decx::_GPU_Matrix* dst,
-                 float alpha, float beta, de::DH* h)
+                 double alpha, double beta, de::DH* h)
 {
     std::lock_guard<std::mutex> guard(decx::module_mutex());
     // C may be the same object as dst: keep its storage alive and its pitch in hand across the reshape
@@ -395,18 +395,24 @@ bool gemm_device(decx::_GPU_Matrix* A, decx::_GPU_Matrix* B, decx::_GPU_Matrix* 
     if (A->Type() == de::_FP32_)
         rc = decx_hip_gemm_f32((const float*)A->data(), (const float*)B->data(), (const float*)c_ptr,
                                (float*)dst->data(), A->Height(), B->Width(), A->Width(),
+                               A->Pitch(), B->Pitch(), ldc, dst->Pitch(), (float)alpha, (float)beta, S);
+    else if (A->Type() == de::_FP64_)
+        rc = decx_hip_gemm_f64((const double*)A->data(), (const double*)B->data(), (const double*)c_ptr,
+                               (double*)dst->data(), A->Height(), B->Width(), A->Width(),
                                A->Pitch(), B->Pitch(), ldc, dst->Pitch(), alpha, beta, S);
     else
         rc = decx_hip_gemm_f16((const uint16_t*)A->data(), (const uint16_t*)B->data(), (const uint16_t*)c_ptr,
                                (uint16_t*)dst->data(), A->Height(), B->Width(), A->Width(),
-                               A->Pitch(), B->Pitch(), ldc, dst->Pitch(), alpha, beta, S);
+                               A->Pitch(), B->Pitch(), ldc, dst->Pitch(), (float)alpha, (float)beta, S);
     if (rc == DECX_HIP_OK) rc = decx_hip_stream_sync(S);                     // result complete on return
     return !decx::err::from_hip(h, rc, "GEMM");
 }
 
-float scalar_of(const de::Number& n)
+double scalar_of(const de::Number& n)
 {
-    return n.Type() == de::_FP16_ ? de::Half2Float(n.get_data_ref<de::Half>()) : n.get_data_ref<float>();
+    if (n.Type() == de::_FP16_) return de::Half2Float(n.get_data_ref<de::Half>());
+    if (n.Type() == de::_FP64_) return n.get_data_ref<double>();
+    return n.get_data_ref<float>();
 }
 
 }  // namespace
@@ -417,7 +423,7 @@ _DECX_API_ void de::blas::cuda::GEMM(de::GPU_Matrix& A, de::GPU_Matrix& B, de::G
     decx::_GPU_Matrix* b = dynamic_cast<decx::_GPU_Matrix*>(&B);
     decx::_GPU_Matrix* d = dynamic_cast<decx::_GPU_Matrix*>(&dst);
     if (!validate(a, b, nullptr, d, nullptr, nullptr, de::GetLastError())) return;
-    gemm_device(a, b, nullptr, d, 1.f, 1.f, de::GetLastError());
+    gemm_device(a, b, nullptr, d, 1.0, 1.0, de::GetLastError());
 }
 
 _DECX_API_ void de::blas::cuda::GEMM(de::GPU_Matrix& A, de::GPU_Matrix& B, de::GPU_Matrix& C, de::GPU_Matrix& dst,
@@ -519,7 +525,10 @@ void gemm_host(de::Matrix& A, de::Matrix& B, de::Matrix* C, de::Matrix& dst)
         if (!arrived || !done) { rc = DECX_HIP_E_INVALID_ARG; break; }
         if (rc == DECX_HIP_OK) rc = decx_hip_event_record(arrived, pipe.in);
         if (rc == DECX_HIP_OK) rc = decx_hip_stream_wait_event(S, arrived);
-        if (rc == DECX_HIP_OK)
+        if (rc == DECX_HIP_OK && a->Type() == de::_FP64_)
+            rc = decx_hip_gemm_f64((const double*)a_dev, (const double*)dB.data(), (const double*)c_dev, (double*)d_dev, rows, N, K,
+                                   dA.Pitch(), dB.Pitch(), c ? dC.Pitch() : 0, dD.Pitch(), 1.0, 1.0, S);
+        else if (rc == DECX_HIP_OK)
             rc = f16 ? decx_hip_gemm_f16((const uint16_t*)a_dev, (const uint16_t*)dB.data(), (const uint16_t*)c_dev,
                                          (uint16_t*)d_dev, rows, N, K, dA.Pitch(), dB.Pitch(), c ? dC.Pitch() : 0,
                                          dD.Pitch(), 1.f, 1.f, S)

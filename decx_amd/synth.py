@@ -31,6 +31,17 @@ def uniform_f32(rows: int, cols: int, seed: int) -> np.ndarray:
     return out
 
 
+def uniform_f64(rows: int, cols: int, seed: int) -> np.ndarray:
+    """iid uniform in [-1, 1), fp64 (52 random mantissa bits), shape (rows, cols), row-major and dense."""
+    out = np.empty((rows, cols), np.float64)
+    step = max(1, (1 << 22) // max(cols, 1))
+    for r0 in range(0, rows, step):
+        r1 = min(rows, r0 + step)
+        u = _mix(seed, (r1 - r0) * cols, r0 * cols) >> np.uint64(12)
+        out[r0:r1] = (u.astype(np.float64) * (1.0 / 2251799813685248.0) - 1.0).reshape(r1 - r0, cols)
+    return out
+
+
 def normal_half(rows: int, cols: int, seed: int, sigma: float = 0.5, clip: float = 4.0) -> np.ndarray:
     """iid N(0, sigma) drawn in fp32 (Box-Muller on two counter streams), clipped to
     [-clip, clip], rounded to nearest-even binary16.  Returns float16, shape (rows, cols)."""

@@ -117,6 +117,15 @@ DECX_HIP_API int decx_hip_gemm_f16(const uint16_t* A, const uint16_t* B, const u
                                    uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
                                    float alpha, float beta, void* stream);
 
+/* fp64: D = A.B or fma(C, beta, alpha * (A.B)) in double precision on the fp64 matrix cores.
+ * Replaces the body of decx::blas::GEMM_fp64 (srcs/modules/BLAS/GEMM/CUDA/GEMM_LS.cu:164-211) and
+ * cu_GEMM_fp64_*_16_64_64 (large_squares/GEMM_kernels.cuh:182-189).  Operands that are not 16-byte
+ * aligned (base or pitch), and K == 0, take a plain one-thread-per-element kernel. */
+DECX_HIP_API int decx_hip_gemm_f64(const double* A, const double* B, const double* C, double* D,
+                                   uint32_t M, uint32_t N, uint32_t K,
+                                   uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                                   double alpha, double beta, void* stream);
+
 /* The two vector corners, exported for callers that hold vectors (the GEMM entry points above
  * route N == 1 and M == 1 here themselves).  inc* are element strides (a K x 1 pitched matrix
  * has incx = its pitch); c == NULL -> no accumulate term.
@@ -176,8 +185,14 @@ DECX_HIP_API int decx_hip_gemm_f16_tile(const uint16_t* A, const uint16_t* B, co
                                         uint32_t M, uint32_t N, uint32_t K,
                                         uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
                                         float alpha, float beta, void* stream, int tile, int force_edge);
+/* fp64: DECX_HIP_TILE_256x256 selects the largest fp64 tile (256 x 128); force_plain != 0 forces the
+ * one-thread-per-element kernel. */
+DECX_HIP_API int decx_hip_gemm_f64_tile(const double* A, const double* B, const double* C, double* D,
+                                        uint32_t M, uint32_t N, uint32_t K,
+                                        uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                                        double alpha, double beta, void* stream, int tile, int force_plain);
 
-/* What the planner would run for this problem (no GPU work).  elem_bytes: 4 = fp32, 2 = fp16.
+/* What the planner would run for this problem (no GPU work).  elem_bytes: 4 = fp32, 2 = fp16, 8 = fp64.
  * `aligned` != 0 promises 16-byte aligned bases and pitches.  Replaces the scoring of
  * cuda_GEMM_LS_planner<T>::plan (large_squares/common/cuda_GEMM_LS_planner.cu:108-224).
  * Works without a GPU: before decx_hip_init() it assumes 256 compute units. */

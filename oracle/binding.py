@@ -44,6 +44,9 @@ def lib():
         L.cpu_port_max_threads.restype = _u32
         L.cpu_port_gemm_f32.restype = ctypes.c_int
         L.cpu_port_gemm_f32.argtypes = [_f32p, _f32p, _f32p, _f32p] + [_u32] * 7 + [_f32p, _u32]
+        L.oracle_gemm_f64_chain.argtypes = [_f64p, _f64p, _f64p, _f64p] + [_u32] * 7 + [_u32p, _u32]
+        L.oracle_gemm_f64_axpby.argtypes = ([_f64p, _f64p, _f64p, _f64p] + [_u32] * 7 +
+                                            [ctypes.c_double, ctypes.c_double, _u32p, _u32])
         L.oracle_conv2d_out_dims.argtypes = [_u32] * 6 + [ctypes.c_int, _u32p, _u32p]
         L.oracle_conv2d_f32.argtypes = [_f32p] + [_u32] * 3 + [_f32p] + [_u32] * 5 + [ctypes.c_int, _f32p]
         _lib = L
@@ -82,6 +85,23 @@ def gemm_f32(A, B, C=None, alpha=None, beta=None, rows=None):
     else:
         assert C is not None
         lib().oracle_gemm_f32_axpby(_p(A, _f32p), _p(B, _f32p), _p(C, _f32p), _p(out, _f32p), M, N, K,
+                                    _ld(A), _ld(B), _ld(C), N, alpha, beta, rp, nr)
+    return out
+
+
+def gemm_f64(A, B, C=None, alpha=None, beta=None, rows=None):
+    """Double-precision chain oracle; same conventions as gemm_f32."""
+    M, K = A.shape
+    K2, N = B.shape
+    assert K == K2 and A.dtype == np.float64 and B.dtype == np.float64
+    keep, rp, nr = _rows(rows)
+    out = np.empty((nr if rows is not None else M, N), np.float64)
+    if alpha is None:
+        lib().oracle_gemm_f64_chain(_p(A, _f64p), _p(B, _f64p), _p(C, _f64p), _p(out, _f64p), M, N, K,
+                                    _ld(A), _ld(B), _ld(C) if C is not None else 0, N, rp, nr)
+    else:
+        assert C is not None
+        lib().oracle_gemm_f64_axpby(_p(A, _f64p), _p(B, _f64p), _p(C, _f64p), _p(out, _f64p), M, N, K,
                                     _ld(A), _ld(B), _ld(C), N, alpha, beta, rp, nr)
     return out
 
@@ -162,22 +182,31 @@ def reference_available():
 
 
 def _reference_call(A, B, C, threads):
+    """Element type by A.dtype: float32 or float64."""
     global _ref_fn
     if _ref_fn is None:
         ld = ctypes.CDLL(os.path.join(_HERE, "_ref", "libref_loader.so"))
         ld.ref_loader_sym.restype = ctypes.c_void_p
         ld.ref_loader_sym.argtypes = [ctypes.c_char_p, ctypes.c_char_p]
-        addr = ld.ref_loader_sym(os.path.join(_HERE, "_ref", "libdecx_ref_cpu.so").encode(), b"ref_cpu_gemm_f32")
-        assert addr, "could not load the compiled reference"
-        _ref_fn = ctypes.CFUNCTYPE(ctypes.c_int, _f32p, _f32p, _f32p, _f32p, _u32, _u32, _u32, _u32)(addr)
+        path = os.path.join(_HERE, "_ref", "libdecx_ref_cpu.so").encode()
+        a32, a64 = ld.ref_loader_sym(path, b"ref_cpu_gemm_f32"), ld.ref_loader_sym(path, b"ref_cpu_gemm_f64")
+        assert a32 and a64, "could not load the compiled reference"
+        _ref_fn = {np.dtype(np.float32): (ctypes.CFUNCTYPE(ctypes.c_int, _f32p, _f32p, _f32p, _f32p, _u32, _u32, _u32, _u32)(a32), _f32p),
+                   np.dtype(np.float64): (ctypes.CFUNCTYPE(ctypes.c_int, _f64p, _f64p, _f64p, _f64p, _u32, _u32, _u32, _u32)(a64), _f64p)}
+    fn, pt = _ref_fn[A.dtype]
     M, K = A.shape
     N = B.shape[1]
-    out = np.empty((M, N), np.float32)
-    err = _ref_fn(_p(A, _f32p), _p(B, _f32p), _p(C, _f32p), _p(out, _f32p), M, N, K, threads)
+    out = np.empty((M, N), A.dtype)
+    err = fn(_p(A, pt), _p(B, pt), _p(C, pt), _p(out, pt), M, N, K, threads)
     return out, err
 
 
-def reference_cpu_gemm_f32(A, B, C=None, threads=8):
+def reference_cpu_gemm_f64(A, B, C=None, threads=8):
+    """The same for the reference's double-precision CPU GEMM."""
+    return reference_cpu_gemm_f32(A, B, C, threads, dtype=np.float64)
+
+
+def reference_cpu_gemm_f32(A, B, C=None, threads=8, dtype=np.float32):
     """de::blas::cpu::GEMM of the compiled reference (build container only).  Every call runs
     in a process of its own: the reference's cached planner does not survive a change of
     shape or thread count reliably, and a crash must not take the test run with it.  Some
@@ -186,12 +215,12 @@ def reference_cpu_gemm_f32(A, B, C=None, threads=8):
     then with one 64x64x64 single-thread call in front, up to three times each (the crashes
     are intermittent).  Returns (D, error_type); raises RuntimeError if every child died."""
     import tempfile
-    A = np.ascontiguousarray(A, np.float32); B = np.ascontiguousarray(B, np.float32)
+    A = np.ascontiguousarray(A, dtype); B = np.ascontiguousarray(B, dtype)
     with tempfile.TemporaryDirectory() as tmp:
         np.save(os.path.join(tmp, "A.npy"), A)
         np.save(os.path.join(tmp, "B.npy"), B)
         if C is not None:
-            np.save(os.path.join(tmp, "C.npy"), np.ascontiguousarray(C, np.float32))
+            np.save(os.path.join(tmp, "C.npy"), np.ascontiguousarray(C, dtype))
         for warm in ("", "w = np.zeros((64, 64), np.float32); b._reference_call(w, w, None, 1);") * 3:
             code = ("import sys, os, numpy as np; sys.path.insert(0, %r); from oracle import binding as b; t = %r;"
                     "A = np.load(t + '/A.npy'); B = np.load(t + '/B.npy');"

@@ -238,3 +238,50 @@ void oracle_gemm_f64_brute(const float* A, const float* B, const float* C, doubl
             D[(size_t)i * ldd + j] = alpha * s + (C ? beta * (double)C[(size_t)i * ldc + j] : 0.0);
         }
 }
+
+/* ---------------------------------------------------------------- fp64 */
+
+/*
+ * Double precision: the same k-ascending chain with fma in double, seeded with 0 or C[i][j]
+ * (what the reference's fp64 CPU GEMM computes: srcs/modules/BLAS/GEMM/CPU/fp64/, same structure as the
+ * fp32 path), and the GPU entry point's D = fma(C, beta, alpha * chain0)
+ * (srcs/modules/BLAS/GEMM/CUDA/GEMM_LS.cu:164-211).  Pinned by tests/test_oracle.py: exact rational
+ * arithmetic on tiny shapes, integer closed forms, and bit-for-bit against the compiled reference and its
+ * committed outputs (tests/golden/ref_f64_*.npz).
+ */
+void oracle_gemm_f64_chain(const double* A, const double* B, const double* C, double* D,
+                           uint32_t M, uint32_t N, uint32_t K,
+                           uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                           const uint32_t* rows, uint32_t nrows)
+{
+    const uint32_t count = rows ? nrows : M;
+#pragma omp parallel for schedule(dynamic, 1)
+    for (uint32_t r = 0; r < count; ++r) {
+        const uint32_t i = rows ? rows[r] : r;
+        double* __restrict acc = D + (size_t)r * ldd;
+        if (C) for (uint32_t j = 0; j < N; ++j) acc[j] = C[(size_t)i * ldc + j];
+        else   for (uint32_t j = 0; j < N; ++j) acc[j] = 0.0;
+        for (uint32_t k = 0; k < K; ++k) {
+            const double a = A[(size_t)i * lda + k];
+            const double* __restrict b = B + (size_t)k * ldb;
+            for (uint32_t j = 0; j < N; ++j) acc[j] = fma(a, b[j], acc[j]);
+        }
+    }
+}
+
+void oracle_gemm_f64_axpby(const double* A, const double* B, const double* C, double* D,
+                           uint32_t M, uint32_t N, uint32_t K,
+                           uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                           double alpha, double beta,
+                           const uint32_t* rows, uint32_t nrows)
+{
+    oracle_gemm_f64_chain(A, B, NULL, D, M, N, K, lda, ldb, 0, ldd, rows, nrows);
+    const uint32_t count = rows ? nrows : M;
+    for (uint32_t r = 0; r < count; ++r) {
+        const uint32_t i = rows ? rows[r] : r;
+        for (uint32_t j = 0; j < N; ++j) {
+            const double t = alpha * D[(size_t)r * ldd + j];
+            D[(size_t)r * ldd + j] = fma(C[(size_t)i * ldc + j], beta, t);
+        }
+    }
+}

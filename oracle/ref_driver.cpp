@@ -28,3 +28,26 @@ extern "C" int ref_cpu_gemm_f32(const float* A, const float* B, const float* C, 
     mA.release(); mB.release(); mD.release();
     return err;
 }
+
+extern "C" int ref_cpu_gemm_f64(const double* A, const double* B, const double* C, double* D,
+                                uint32_t M, uint32_t N, uint32_t K, uint32_t threads)
+{
+    de::cpu::DecxSetThreadingNum(threads);
+    de::Matrix& mA = de::CreateMatrixRef(de::_FP64_, K, M);
+    de::Matrix& mB = de::CreateMatrixRef(de::_FP64_, N, K);
+    de::Matrix& mD = de::CreateMatrixRef(de::_FP64_, N, M);
+    for (uint32_t i = 0; i < M; ++i) std::memcpy(mA.ptr<double>(i, 0), A + (size_t)i * K, K * sizeof(double));
+    for (uint32_t i = 0; i < K; ++i) std::memcpy(mB.ptr<double>(i, 0), B + (size_t)i * N, N * sizeof(double));
+    if (C) {
+        de::Matrix& mC = de::CreateMatrixRef(de::_FP64_, N, M);
+        for (uint32_t i = 0; i < M; ++i) std::memcpy(mC.ptr<double>(i, 0), C + (size_t)i * N, N * sizeof(double));
+        de::blas::cpu::GEMM(mA, mB, mC, mD);
+        mC.release();
+    } else {
+        de::blas::cpu::GEMM(mA, mB, mD);
+    }
+    const int err = de::GetLastError()->error_type;
+    for (uint32_t i = 0; i < M; ++i) std::memcpy(D + (size_t)i * N, mD.ptr<double>(i, 0), N * sizeof(double));
+    mA.release(); mB.release(); mD.release();
+    return err;
+}

@@ -162,9 +162,30 @@ static int gpu_checks()
     de::blas::cuda::GEMM(dA, dB, dS, dD, de::Number(1.f), de::Number(1.f));    // C has the wrong shape
     CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_DimsNotMatching);
     de::ResetLastError();
-    de::GPU_Matrix& d64 = de::CreateGPUMatrixRef(de::_FP64_, 8, 8);
-    de::blas::cuda::GEMM(d64, d64, dD);
+    de::GPU_Matrix& dcx = de::CreateGPUMatrixRef(de::_COMPLEX_F32_, 8, 8);
+    de::blas::cuda::GEMM(dcx, dcx, dD);
     CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_UNSUPPORTED_TYPE);
+    de::ResetLastError();
+    // double precision: identity, and alpha / beta carried as doubles
+    de::Matrix& I64 = de::CreateMatrixRef(de::_FP64_, 24, 24);
+    de::Matrix& X64 = de::CreateMatrixRef(de::_FP64_, 17, 24);
+    for (int i = 0; i < 24; ++i) { *I64.ptr<double>(i, i) = 1.0; for (int j = 0; j < 17; ++j) *X64.ptr<double>(i, j) = 1.0 / 3.0 + i * 17 + j; }
+    CHECK(I64.ptr<double>(1, 0) - I64.ptr<double>(0, 0) == 24 && X64.ptr<double>(1, 0) - X64.ptr<double>(0, 0) == 20);   // 32-byte rule
+    de::GPU_Matrix& dI64 = de::CreateGPUMatrixRef(de::_FP64_, 24, 24);
+    de::GPU_Matrix& dX64 = de::CreateGPUMatrixRef(de::_FP64_, 17, 24);
+    de::GPU_Matrix& dR64 = de::CreateGPUMatrixRef();
+    CHECK(de::Memcpy(I64, dI64, O, O, de::Point2D(24, 24), de::DECX_MEMCPY_H2D).error_type == 0);
+    CHECK(de::Memcpy(X64, dX64, O, O, de::Point2D(17, 24), de::DECX_MEMCPY_H2D).error_type == 0);
+    de::blas::cuda::GEMM(dI64, dX64, dX64, dR64, de::Number(2.0), de::Number(-0.5));        // 2 I X - X / 2 = 1.5 X
+    CHECK(de::GetLastError()->error_type == 0 && dR64.Type() == de::_FP64_ && dR64.Width() == 17 && dR64.Height() == 24);
+    de::Matrix& R64 = de::CreateMatrixRef(de::_FP64_, 17, 24);
+    CHECK(de::Memcpy(R64, dR64, O, O, de::Point2D(17, 24), de::DECX_MEMCPY_D2H).error_type == 0);
+    bool same64 = true;
+    for (int i = 0; i < 24; ++i) for (int j = 0; j < 17; ++j) same64 &= (*R64.ptr<double>(i, j) == 1.5 * *X64.ptr<double>(i, j));
+    CHECK(same64);
+    de::blas::cuda::GEMM(dI64, dX64, dX64, dR64, de::Number(2.0f), de::Number(-0.5f));      // float scalars for double matrices
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_TYPE_MOT_MATCH);
+    de::ResetLastError();
     de::ResetLastError();
     CHECK(de::Memcpy(A, dH, O, O, de::Point2D(1, 1), de::DECX_MEMCPY_H2D).error_type == decx::DECX_FAIL_TYPE_MOT_MATCH);
     CHECK(dD.Width() == W && dD.Height() == H);                          // failed calls left dst alone
@@ -395,6 +416,7 @@ template <typename T> static int gemm_files(const std::string& dir, de::_DATA_TY
     if (with_c) {
         de::Memcpy(C, dC, O, O, de::Point2D(N, M), de::DECX_MEMCPY_H2D);
         if (ty == de::_FP32_) de::blas::cuda::GEMM(dA, dB, dC, dD, de::Number(alpha), de::Number(beta));
+        else if (ty == de::_FP64_) de::blas::cuda::GEMM(dA, dB, dC, dD, de::Number((double)alpha), de::Number((double)beta));
         else de::blas::cuda::GEMM(dA, dB, dC, dD, de::Number(de::Float2Half(alpha)), de::Number(de::Float2Half(beta)));
     } else {
         de::blas::cuda::GEMM(dA, dB, dD);
@@ -528,6 +550,7 @@ int main(int argc, char** argv)
         const int with_c = std::atoi(argv[7]), repeats = std::atoi(argv[9]);
         const bool pinned = std::atoi(argv[8]) != 0;
         rc = f16 ? hostgemm_files<de::Half>(argv[2], de::_FP16_, M, N, K, with_c, pinned, repeats)
+                 : std::string(argv[3]) == "f64" ? hostgemm_files<double>(argv[2], de::_FP64_, M, N, K, with_c, pinned, repeats)
                  : hostgemm_files<float>(argv[2], de::_FP32_, M, N, K, with_c, pinned, repeats);
     }
     else if (mode == "tensor_host") rc = tensor_host_checks();
@@ -548,6 +571,7 @@ int main(int argc, char** argv)
         const bool with_c = std::atoi(argv[7]) != 0;
         const float alpha = (float)std::atof(argv[8]), beta = (float)std::atof(argv[9]);
         rc = f16 ? gemm_files<de::Half>(argv[2], de::_FP16_, M, N, K, with_c, alpha, beta)
+                 : std::string(argv[3]) == "f64" ? gemm_files<double>(argv[2], de::_FP64_, M, N, K, with_c, alpha, beta)
                  : gemm_files<float>(argv[2], de::_FP32_, M, N, K, with_c, alpha, beta);
     } else {
         std::cerr << "usage: de_api_test host | gpu | vector_host | vector_gpu | gemm <dir> <f32|f16> M N K withC alpha beta"

@@ -2,7 +2,7 @@
 
     python tests/golden/make_golden.py
 
-`ref_f32_*.npz` hold outputs of the *reference's own* CPU GEMM (de::blas::cpu::GEMM,
+`ref_f32_*.npz` / `ref_f64_*.npz` hold outputs of the *reference's own* CPU GEMM (de::blas::cpu::GEMM,
 compiled from the mounted reference tree by oracle/build_ref.sh) at shapes and thread
 counts inside the envelope where it is correct; the inputs are regenerated from the seeds
 stored beside them (fp16 fixtures store their inputs, which pass through libm).  `orc_*.npz` hold outputs the reference cannot produce (fp16, the
@@ -26,6 +26,12 @@ REF_CASES = [  # (M, N, K, threads)
     (96, 80, 72, 4),      # wrong at 1 and 2 threads
     (128, 64, 96, 2),
     (200, 112, 136, 4),   # (200, 120, 136) is outside the envelope: the reference gets it wrong at every thread count
+]
+REF64_CASES = [  # (M, N, K, threads, with_C): the reference's double-precision CPU GEMM, correct also with C
+    (64, 64, 64, 1, False),
+    (96, 80, 72, 4, True),
+    (100, 150, 77, 4, False),
+    (200, 112, 136, 4, True),
 ]
 ORC_F32 = [  # (M, N, K, with_C, alpha, beta)   alpha None => chain seeded with C
     (37, 53, 29, False, None, None),
@@ -56,6 +62,15 @@ def main():
         assert err == 0
         np.savez(os.path.join(HERE, f"ref_f32_{M}x{N}x{K}.npz"), M=M, N=N, K=K, threads=T,
                  seed_a=sa, seed_b=sb, D=D, crc=crc(D))
+    for idx, (M, N, K, T, with_c) in enumerate(REF64_CASES):
+        sa, sb, sc = 0x6400 + idx, 0x7400 + idx, 0x8400 + idx
+        A = synth.uniform_f64(M, K, sa)
+        B = synth.uniform_f64(K, N, sb)
+        C = synth.uniform_f64(M, N, sc) if with_c else None
+        D, err = orc.reference_cpu_gemm_f64(A, B, C, threads=T)
+        assert err == 0
+        np.savez(os.path.join(HERE, f"ref_f64_{'abc' if with_c else 'ab'}_{M}x{N}x{K}.npz"), M=M, N=N, K=K, threads=T,
+                 with_c=with_c, seed_a=sa, seed_b=sb, seed_c=sc, D=D, crc=crc(D))
     for idx, (M, N, K, with_c, alpha, beta) in enumerate(ORC_F32):
         sa, sb, sc = 0x6100 + idx, 0x7100 + idx, 0x8100 + idx
         A = synth.uniform_f32(M, K, sa)

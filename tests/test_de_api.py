@@ -70,10 +70,14 @@ def test_gpu_side_closed_forms_and_error_paths():
     ("f32", 300, 1, 500, True, -0.5, 2.0),          # N == 1: the row-dot path behind the same entry point
     ("f16", 257, 130, 515, False, 1.0, 1.0),
     ("f16", 257, 130, 515, True, 1.5, -0.5),
+    ("f64", 1000, 700, 333, False, 1.0, 1.0),
+    ("f64", 1000, 700, 333, True, -0.5, 2.0),
 ])
 def test_gemm_through_the_objects_matches_oracle(oracle, dt, M, N, K, with_c, alpha, beta):
     if dt == "f32":
         A = synth.uniform_f32(M, K, 201); B = synth.uniform_f32(K, N, 202); C = synth.uniform_f32(M, N, 203)
+    elif dt == "f64":
+        A = synth.uniform_f64(M, K, 201); B = synth.uniform_f64(K, N, 202); C = synth.uniform_f64(M, N, 203)
     else:
         A = synth.normal_half(M, K, 201); B = synth.normal_half(K, N, 202); C = synth.normal_half(M, N, 203)
     with tempfile.TemporaryDirectory() as tmp:
@@ -84,6 +88,9 @@ def test_gemm_through_the_objects_matches_oracle(oracle, dt, M, N, K, with_c, al
     if dt == "f32":
         ref = oracle.gemm_f32(A, B, C, alpha, beta) if with_c else oracle.gemm_f32(A, B)
         tol = 1e-5
+    elif dt == "f64":
+        ref = oracle.gemm_f64(A, B, C, alpha, beta) if with_c else oracle.gemm_f64(A, B)
+        tol = 1e-14
     else:
         ref = oracle.gemm_f16(A, B, C if with_c else None, alpha, beta)
         tol = 2e-3
@@ -139,12 +146,15 @@ def test_vector_forms_through_the_objects_match_oracle(oracle, dt, form, W, H, l
     ("f32", 100, 70, 33, 1, 0),            # a single panel
     ("f16", 1300, 520, 515, 0, 1),
     ("f16", 1300, 520, 515, 2, 0),
+    ("f64", 700, 300, 129, 1, 1),
 ])
 def test_host_matrix_forms_match_oracle(oracle, dt, M, N, K, with_c, pinned):
     """de::blas::cuda::GEMM(Matrix, Matrix[, Matrix], Matrix): operands staged in row panels on three streams;
     pageable and page-locked host storage, C as a separate matrix and as dst."""
     if dt == "f32":
         A = synth.uniform_f32(M, K, 401); B = synth.uniform_f32(K, N, 402); C = synth.uniform_f32(M, N, 403)
+    elif dt == "f64":
+        A = synth.uniform_f64(M, K, 401); B = synth.uniform_f64(K, N, 402); C = synth.uniform_f64(M, N, 403)
     else:
         A = synth.normal_half(M, K, 401); B = synth.normal_half(K, N, 402); C = synth.normal_half(M, N, 403)
     with tempfile.TemporaryDirectory() as tmp:
@@ -155,6 +165,9 @@ def test_host_matrix_forms_match_oracle(oracle, dt, M, N, K, with_c, pinned):
     if dt == "f32":
         ref = oracle.gemm_f32(A, B, C, 1.0, 1.0) if with_c else oracle.gemm_f32(A, B)
         tol = 1e-5
+    elif dt == "f64":
+        ref = oracle.gemm_f64(A, B, C, 1.0, 1.0) if with_c else oracle.gemm_f64(A, B)
+        tol = 1e-14
     else:
         ref = oracle.gemm_f16(A, B, C if with_c else None, 1.0, 1.0)
         tol = 2e-3

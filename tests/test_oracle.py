@@ -280,8 +280,60 @@ def test_oracle_regression_fixtures_f16(oracle, path):
     assert np.array_equal(got.view(np.uint16), g["D"])
 
 
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLD, "ref_f64_*.npz"))))
+def test_f64_oracle_reproduces_reference_outputs(oracle, path):
+    """Outputs of the reference's double-precision de::blas::cpu::GEMM (three- and four-matrix form)."""
+    g = np.load(path)
+    M, N, K = int(g["M"]), int(g["N"]), int(g["K"])
+    A = synth.uniform_f64(M, K, int(g["seed_a"])); B = synth.uniform_f64(K, N, int(g["seed_b"]))
+    C = synth.uniform_f64(M, N, int(g["seed_c"])) if bool(g["with_c"]) else None
+    assert zlib.crc32(g["D"].tobytes()) & 0xFFFFFFFF == int(g["crc"])
+    assert np.array_equal(oracle.gemm_f64(A, B, C).view(np.uint64), g["D"].view(np.uint64))
+
+
+def test_f64_chain_against_exact_rationals(oracle):
+    """fma in exact arithmetic: float(Fraction) rounds to nearest even, so acc = float(a * b + acc) over
+    Fractions is the fused chain; a dropped fma (separate multiply and add) or a reversed k order differs."""
+    from fractions import Fraction
+    rng = np.random.default_rng(17)
+    M, N, K = 5, 4, 23
+    A = rng.uniform(-1, 1, (M, K)); B = rng.uniform(-1, 1, (K, N)); C = rng.uniform(-1, 1, (M, N))
+    for seed_c, alpha, beta in ((False, None, None), (True, None, None), (True, 0.75, -1.25)):
+        want = np.empty((M, N))
+        for i in range(M):
+            for j in range(N):
+                acc = C[i, j] if (seed_c and alpha is None) else 0.0
+                for k in range(K):
+                    acc = float(Fraction(A[i, k]) * Fraction(B[k, j]) + Fraction(acc))
+                if alpha is not None:
+                    acc = float(Fraction(C[i, j]) * Fraction(beta) + Fraction(alpha * acc))
+                want[i, j] = acc
+        got = oracle.gemm_f64(A, B, C if seed_c else None, alpha, beta)
+        assert np.array_equal(got.view(np.uint64), want.view(np.uint64))
+    rows = [4, 0]
+    assert np.array_equal(oracle.gemm_f64(A, B, rows=rows), oracle.gemm_f64(A, B)[rows])
+    ints_a = rng.integers(-9, 10, (30, 40)).astype(np.float64); ints_b = rng.integers(-9, 10, (40, 20)).astype(np.float64)
+    assert np.array_equal(oracle.gemm_f64(ints_a, ints_b), (ints_a.astype(np.int64) @ ints_b.astype(np.int64)).astype(np.float64))
+
+
+@pytest.mark.parametrize("M,N,K,threads", [(64, 64, 64, 1), (256, 256, 256, 8), (100, 150, 77, 4), (1024, 1024, 1024, 8)])  # 1000 x 1500 x 777 at 8 threads: the reference is wrong
+def test_f64_chain_bit_equal_to_compiled_reference(oracle, M, N, K, threads):
+    if not oracle.reference_available():
+        pytest.skip("compiled reference (oracle/_ref) not present on this host")
+    A = synth.uniform_f64(M, K, 95); B = synth.uniform_f64(K, N, 96); C = synth.uniform_f64(M, N, 97)
+    try:
+        D, err = oracle.reference_cpu_gemm_f64(A, B, None, threads)
+        Dc, errc = oracle.reference_cpu_gemm_f64(A, B, C, threads)
+    except RuntimeError as e:
+        pytest.skip(str(e))
+    assert err == 0 and errc == 0
+    assert np.array_equal(D.view(np.uint64), oracle.gemm_f64(A, B).view(np.uint64))
+    assert np.array_equal(Dc.view(np.uint64), oracle.gemm_f64(A, B, C).view(np.uint64))
+
+
 def test_golden_set_is_complete():
     assert len(glob.glob(os.path.join(GOLD, "ref_f32_*.npz"))) == 4
+    assert len(glob.glob(os.path.join(GOLD, "ref_f64_*.npz"))) == 4
     assert len(glob.glob(os.path.join(GOLD, "orc_f32_*.npz"))) == 5
     assert len(glob.glob(os.path.join(GOLD, "orc_f16_*.npz"))) == 3
 
