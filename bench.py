@@ -34,6 +34,7 @@ MEASURED_TRAFFIC = {
     "fp16_4096": 2.35e8,     # FETCH_SIZE 98 461 x 2.0 KiB + WRITE_SIZE 32 793 KiB
     "fp32_gemv": 2.77e8,     # FETCH_SIZE 135 189 x 2.0 KiB + WRITE_SIZE 256 KiB
     "fp32_gevm": 2.69e8,     # FETCH_SIZE 131 224 x 2.0 KiB + WRITE_SIZE 32 KiB
+    "fp64_4096": 1.21e9,     # FETCH_SIZE 524 415 x 2.0 KiB + WRITE_SIZE 131 072 KiB
 }
 
 WORKLOADS = {
@@ -157,7 +158,8 @@ def run_conv(steps, warmup, settle_s=0.25):
            "dtype": "f32", "value": round(tf, 3), "unit": "TFLOP/s", "hbm_gbs_algorithmic": round(abytes / (ms * 1e-3) / 1e9, 1),
            "kernel_ms": round(ms, 5),
            "roofline": {"bound": "mfma", "achieved": round(tf, 3), "peak": PEAK_F32_TFLOPS, "unit": "TFLOP/s",
-                        "frac": round(tf / PEAK_F32_TFLOPS, 4), "traffic": None}}
+                        "frac": round(tf / PEAK_F32_TFLOPS, 4),
+                        "traffic": 1.80e8}}      # FETCH_SIZE 55 474 x 2.0 KiB + WRITE_SIZE 64 516 KiB
     for d in (d_img, d_kmat, d_out):
         d.free()
     return out
