@@ -295,6 +295,57 @@ int decx_hip_gemm_f64_tile(const double* A, const double* B, const double* C, do
     return run_gemm_f64(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, tile, force_plain);
 }
 
+size_t decx_hip_gemm_complex_workspace(int real_bytes, uint32_t N, uint32_t K)
+{
+    if (real_bytes != 4 && real_bytes != 8) return 0;
+    const size_t ldx = ((size_t)2 * N + 15) / 16 * 16;           // 64 / 128 bytes per row at least
+    return (size_t)2 * K * ldx * (size_t)real_bytes;
+}
+
+extern "C++" {
+template <typename T>
+static int run_gemm_complex(const T* A, const T* B, const T* C, T* D, uint32_t M, uint32_t N, uint32_t K, uint32_t lda,
+                            uint32_t ldb, uint32_t ldc, uint32_t ldd, T ar, T ai, T br, T bi, void* workspace,
+                            size_t workspace_bytes, void* stream)
+{
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    const int rc0 = check_gemm(A, B, C, D, M, N, K, lda, ldb, ldc, ldd);
+    if (rc0 != DECX_HIP_OK || M == 0 || N == 0) return rc0;
+    if (N > 0x7fffffffu || K > 0x7fffffffu || lda > 0x7fffffffu || ldd > 0x7fffffffu) return DECX_HIP_E_INVALID_ARG;
+    const size_t need = decx_hip_gemm_complex_workspace((int)sizeof(T), N, K);
+    if (K > 0 && (!workspace || workspace_bytes < need || !aligned16(workspace))) return DECX_HIP_E_INVALID_ARG;
+    hipStream_t S = as_stream(stream);
+    int rc = DECX_HIP_OK;
+    if (C) rc = launch_complex_scale<T>(C, D, M, N, ldc, ldd, br, bi, S);
+    const uint32_t ldx = (uint32_t)(((size_t)2 * N + 15) / 16 * 16);
+    if (rc == DECX_HIP_OK && K > 0) rc = launch_complex_expand_b<T>(B, (T*)workspace, K, N, ldb, ldx, ar, ai, S);
+    if (rc != DECX_HIP_OK) return rc;
+    // real GEMM M x 2N x 2K accumulating onto D when C was given (K == 0 leaves D = beta * C, or zero)
+    if constexpr (sizeof(T) == 4)
+        return run_gemm<false>(A, workspace, C ? D : nullptr, D, M, 2 * N, 2 * K, 2 * lda, ldx, 2 * ldd, 2 * ldd, 1.f, 1.f, stream,
+                               DECX_HIP_TILE_AUTO, 0);
+    else
+        return run_gemm_f64((const double*)A, (const double*)workspace, C ? (const double*)D : nullptr, (double*)D, M, 2 * N, 2 * K,
+                            2 * lda, ldx, 2 * ldd, 2 * ldd, 1.0, 1.0, stream, DECX_HIP_TILE_AUTO, 0);
+}
+}  // extern "C++"
+
+int decx_hip_gemm_c32(const float* A, const float* B, const float* C, float* D, uint32_t M, uint32_t N, uint32_t K,
+                      uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha_re, float alpha_im, float beta_re,
+                      float beta_im, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return run_gemm_complex<float>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha_re, alpha_im, beta_re, beta_im, workspace,
+                                   workspace_bytes, stream);
+}
+
+int decx_hip_gemm_c64(const double* A, const double* B, const double* C, double* D, uint32_t M, uint32_t N, uint32_t K,
+                      uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, double alpha_re, double alpha_im, double beta_re,
+                      double beta_im, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return run_gemm_complex<double>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha_re, alpha_im, beta_re, beta_im, workspace,
+                                    workspace_bytes, stream);
+}
+
 int decx_hip_gemm_f32_tile(const float* A, const float* B, const float* C, float* D, uint32_t M, uint32_t N,
                            uint32_t K, uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha,
                            float beta, void* stream, int tile, int force_edge)

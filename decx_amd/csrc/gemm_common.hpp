@@ -116,6 +116,12 @@ int launch_conv2d_f32_dma(int shape, const GemmArgs& args, hipStream_t stream);
 int launch_gemm_f16(int shape, bool edge, const GemmArgs& args, hipStream_t stream);
 // direct-to-LDS fp16 kernel for any M, N, K >= 1 on 16-byte aligned bases and pitches, in the three tile shapes
 int launch_gemm_f16_dma(int shape, const GemmArgs& args, hipStream_t stream);
+// complex GEMM helpers: B -> the real 2K x 2N expansion of alpha * B; D = beta * C (interleaved complex)
+template <typename T>
+int launch_complex_expand_b(const T* B, T* Bx, uint32_t K, uint32_t N, uint32_t ldb, uint32_t ldx, T ar, T ai, hipStream_t stream);
+template <typename T>
+int launch_complex_scale(const T* C, T* D, uint32_t M, uint32_t N, uint32_t ldc, uint32_t ldd, T br, T bi, hipStream_t stream);
+
 // y = alpha * A.x (+ beta * c) and y = alpha * x.B (+ beta * c); f16 inputs accumulate in fp32 and write
 // fp32 (out_f32) or fp16.  inc* are element strides.
 int launch_gemv(bool f16, bool out_f32, const void* A, const void* x, const void* c, void* y, uint32_t M, uint32_t K,

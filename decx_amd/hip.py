@@ -60,6 +60,9 @@ SYMBOLS = {
     "decx_hip_conv2d_f32": (_int, [_vp] * 3 + [_u32] * 12 + [_vp]),
     "decx_hip_gemm_f64": (_int, [_vp] * 4 + [_u32] * 7 + [ctypes.c_double, ctypes.c_double, _vp]),
     "decx_hip_gemm_f64_tile": (_int, [_vp] * 4 + [_u32] * 7 + [ctypes.c_double, ctypes.c_double, _vp, _int, _int]),
+    "decx_hip_gemm_complex_workspace": (ctypes.c_size_t, [_int, _u32, _u32]),
+    "decx_hip_gemm_c32": (_int, [_vp] * 4 + [_u32] * 7 + [_f] * 4 + [_vp, ctypes.c_size_t, _vp]),
+    "decx_hip_gemm_c64": (_int, [_vp] * 4 + [_u32] * 7 + [ctypes.c_double] * 4 + [_vp, ctypes.c_size_t, _vp]),
     "decx_hip_gemm_f32_tile": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, _int, _int]),
     "decx_hip_gemm_f16_tile": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, _int, _int]),
     "decx_hip_gemm_plan": (_int, [_int, _u32, _u32, _u32, _int, ctypes.POINTER(Plan)]),
@@ -183,6 +186,18 @@ def gemm(A, B, D, C=None, alpha=1.0, beta=1.0, stream=None, tile=TILE_AUTO, forc
     f16 = A.dtype == np.float16
     args = [A.ptr, B.ptr, C.ptr if C is not None else None, D.ptr, M, N, K, A.pitch, B.pitch,
             C.pitch if C is not None else 0, D.pitch, alpha, beta, stream]
+    if A.dtype in (np.complex64, np.complex128):
+        real_bytes = 4 if A.dtype == np.complex64 else 8
+        need = L.decx_hip_gemm_complex_workspace(real_bytes, N, K)
+        ws = DeviceMatrix(1, max(need // 16, 1), np.complex128)
+        a, b = complex(alpha), complex(beta)
+        fn = L.decx_hip_gemm_c32 if real_bytes == 4 else L.decx_hip_gemm_c64
+        rc = fn(A.ptr, B.ptr, C.ptr if C is not None else None, D.ptr, M, N, K, A.pitch, B.pitch,
+                C.pitch if C is not None else 0, D.pitch, a.real, a.imag, b.real, b.imag, ws.ptr, need, stream)
+        check(lib().decx_hip_stream_sync(stream))          # the workspace dies with this call
+        ws.free()
+        check(rc, "gemm")
+        return
     if A.dtype == np.float64:
         if tile == TILE_AUTO and not force_edge:
             check(L.decx_hip_gemm_f64(*args), "gemm")

@@ -376,15 +376,22 @@ bool validate(const decx::_GPU_Matrix* A, const decx::_GPU_Matrix* B, const decx
                        "The input scalar alpha and beta must match the type of input matrices");
         return false;
     }
-    if (A->Type() != de::_FP32_ && A->Type() != de::_FP16_ && A->Type() != de::_FP64_) {
+    if (A->Type() != de::_FP32_ && A->Type() != de::_FP16_ && A->Type() != de::_FP64_ &&
+        A->Type() != de::_COMPLEX_F32_ && A->Type() != de::_COMPLEX_F64_) {
         decx::err::set(h, decx::DECX_FAIL_UNSUPPORTED_TYPE, kUnsupportedType); return false;
     }
     return true;
 }
 
+// workspace of the complex forms (the real expansion of B), kept between calls; guarded by the module mutex
+std::shared_ptr<decx::DeviceBlock>& complex_workspace() { static std::shared_ptr<decx::DeviceBlock> w; return w; }
+
+struct Scalar { double re, im; };
+
 bool gemm_device(decx::_GPU_Matrix* A, decx::_GPU_Matrix* B, decx::_GPU_Matrix* C, decx::_GPU_Matrix* dst,
-                 double alpha, double beta, de::DH* h)
+                 Scalar alpha_c, Scalar beta_c, de::DH* h)
 {
+    const double alpha = alpha_c.re, beta = beta_c.re;
     std::lock_guard<std::mutex> guard(decx::module_mutex());
     // C may be the same object as dst: keep its storage alive and its pitch in hand across the reshape
     const uint32_t ldc = C ? C->Pitch() : 0;
@@ -392,7 +399,27 @@ bool gemm_device(decx::_GPU_Matrix* A, decx::_GPU_Matrix* B, decx::_GPU_Matrix* 
     if (!dst->re_construct(A->Type(), B->Width(), A->Height())) return false;   // status already set
     void* S = decx::module_stream();
     int rc;
-    if (A->Type() == de::_FP32_)
+    if (A->Type() == de::_COMPLEX_F32_ || A->Type() == de::_COMPLEX_F64_) {
+        const bool single = A->Type() == de::_COMPLEX_F32_;
+        const size_t need = decx_hip_gemm_complex_workspace(single ? 4 : 8, B->Width(), A->Width());
+        std::shared_ptr<decx::DeviceBlock>& ws = complex_workspace();
+        if (!ws || ws->bytes < need) {
+            auto block = std::make_shared<decx::DeviceBlock>();
+            block->bytes = need ? need : 64;
+            if (decx_hip_malloc(&block->ptr, block->bytes) != DECX_HIP_OK) {
+                block->ptr = nullptr;
+                decx::err::set(h, decx::DECX_FAIL_CUDA_ALLOCATION, kDevAllocFail); return false;
+            }
+            ws = block;
+        }
+        rc = single ? decx_hip_gemm_c32((const float*)A->data(), (const float*)B->data(), (const float*)c_ptr, (float*)dst->data(),
+                                        A->Height(), B->Width(), A->Width(), A->Pitch(), B->Pitch(), ldc, dst->Pitch(),
+                                        (float)alpha_c.re, (float)alpha_c.im, (float)beta_c.re, (float)beta_c.im, ws->ptr, ws->bytes, S)
+                    : decx_hip_gemm_c64((const double*)A->data(), (const double*)B->data(), (const double*)c_ptr, (double*)dst->data(),
+                                        A->Height(), B->Width(), A->Width(), A->Pitch(), B->Pitch(), ldc, dst->Pitch(),
+                                        alpha_c.re, alpha_c.im, beta_c.re, beta_c.im, ws->ptr, ws->bytes, S);
+    }
+    else if (A->Type() == de::_FP32_)
         rc = decx_hip_gemm_f32((const float*)A->data(), (const float*)B->data(), (const float*)c_ptr,
                                (float*)dst->data(), A->Height(), B->Width(), A->Width(),
                                A->Pitch(), B->Pitch(), ldc, dst->Pitch(), (float)alpha, (float)beta, S);
@@ -408,11 +435,13 @@ bool gemm_device(decx::_GPU_Matrix* A, decx::_GPU_Matrix* B, decx::_GPU_Matrix* 
     return !decx::err::from_hip(h, rc, "GEMM");
 }
 
-double scalar_of(const de::Number& n)
+Scalar scalar_of(const de::Number& n)
 {
-    if (n.Type() == de::_FP16_) return de::Half2Float(n.get_data_ref<de::Half>());
-    if (n.Type() == de::_FP64_) return n.get_data_ref<double>();
-    return n.get_data_ref<float>();
+    if (n.Type() == de::_FP16_) return {de::Half2Float(n.get_data_ref<de::Half>()), 0.0};
+    if (n.Type() == de::_FP64_) return {n.get_data_ref<double>(), 0.0};
+    if (n.Type() == de::_COMPLEX_F32_) return {n.get_data_ref<de::CPf>().real, n.get_data_ref<de::CPf>().image};
+    if (n.Type() == de::_COMPLEX_F64_) return {n.get_data_ref<de::CPd>().real, n.get_data_ref<de::CPd>().image};
+    return {n.get_data_ref<float>(), 0.0};
 }
 
 }  // namespace
@@ -423,7 +452,7 @@ _DECX_API_ void de::blas::cuda::GEMM(de::GPU_Matrix& A, de::GPU_Matrix& B, de::G
     decx::_GPU_Matrix* b = dynamic_cast<decx::_GPU_Matrix*>(&B);
     decx::_GPU_Matrix* d = dynamic_cast<decx::_GPU_Matrix*>(&dst);
     if (!validate(a, b, nullptr, d, nullptr, nullptr, de::GetLastError())) return;
-    gemm_device(a, b, nullptr, d, 1.0, 1.0, de::GetLastError());
+    gemm_device(a, b, nullptr, d, Scalar{1.0, 0.0}, Scalar{1.0, 0.0}, de::GetLastError());
 }
 
 _DECX_API_ void de::blas::cuda::GEMM(de::GPU_Matrix& A, de::GPU_Matrix& B, de::GPU_Matrix& C, de::GPU_Matrix& dst,
@@ -485,6 +514,9 @@ void gemm_host(de::Matrix& A, de::Matrix& B, de::Matrix* C, de::Matrix& dst)
     if (!dA.is_init() || !dB.is_init()) return;
     if (c) { dC.re_construct(c->Type(), c->Width(), c->Height()); if (!dC.is_init()) return; }
     if (!validate(&dA, &dB, c ? &dC : nullptr, &dD, nullptr, nullptr, h)) return;
+    if (a->Type() == de::_COMPLEX_F32_ || a->Type() == de::_COMPLEX_F64_) {   // complex: device-matrix forms only
+        decx::err::set(h, decx::DECX_FAIL_UNSUPPORTED_TYPE, kUnsupportedType); return;
+    }
     const uint32_t M = a->Height(), N = b->Width(), K = a->Width();
     // C may be dst: take what is needed of it before dst is reshaped
     const char* c_host = c ? (const char*)c->data() : nullptr;

@@ -126,6 +126,23 @@ DECX_HIP_API int decx_hip_gemm_f64(const double* A, const double* B, const doubl
                                    uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
                                    double alpha, double beta, void* stream);
 
+/* Complex (interleaved re, im) single / double precision: D = alpha * (A . B) [+ beta * C], all pitches in
+ * complex elements, C may alias D.  Replaces decx::blas::GEMM_cplxf / GEMM_cplxd (GEMM_LS.cu:214-312).  Runs as
+ * one real GEMM on the matrix cores over the real expansion of alpha * B, which is written into `workspace`
+ * (device memory, 16-byte aligned, at least decx_hip_gemm_complex_workspace(4 or 8, N, K) bytes; the library
+ * never allocates). */
+DECX_HIP_API size_t decx_hip_gemm_complex_workspace(int real_bytes, uint32_t N, uint32_t K);
+DECX_HIP_API int decx_hip_gemm_c32(const float* A, const float* B, const float* C, float* D,
+                                   uint32_t M, uint32_t N, uint32_t K,
+                                   uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                                   float alpha_re, float alpha_im, float beta_re, float beta_im,
+                                   void* workspace, size_t workspace_bytes, void* stream);
+DECX_HIP_API int decx_hip_gemm_c64(const double* A, const double* B, const double* C, double* D,
+                                   uint32_t M, uint32_t N, uint32_t K,
+                                   uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                                   double alpha_re, double alpha_im, double beta_re, double beta_im,
+                                   void* workspace, size_t workspace_bytes, void* stream);
+
 /* The two vector corners, exported for callers that hold vectors (the GEMM entry points above
  * route N == 1 and M == 1 here themselves).  inc* are element strides (a K x 1 pitched matrix
  * has incx = its pitch); c == NULL -> no accumulate term.

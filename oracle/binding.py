@@ -106,6 +106,27 @@ def gemm_f64(A, B, C=None, alpha=None, beta=None, rows=None):
     return out
 
 
+def complex_embed(B):
+    """The real 2K x 2N matrix whose product with an interleaved complex row gives the interleaved complex result."""
+    K, N = B.shape
+    rt = np.float32 if B.dtype == np.complex64 else np.float64
+    X = np.empty((2 * K, 2 * N), rt)
+    X[0::2, 0::2] = B.real; X[0::2, 1::2] = B.imag
+    X[1::2, 0::2] = -B.imag; X[1::2, 1::2] = B.real
+    return X
+
+
+def gemm_complex(A, B, C=None):
+    """Complex A.B (+ C): per element re = chain of fma(ar, br, .), fma(ai, -bi, .) and im = chain of fma(ar, bi, .),
+    fma(ai, br, .), k ascending, seeded with 0 or C -- i.e. the real chain oracle on the real expansion of B."""
+    assert A.dtype == B.dtype and A.dtype in (np.complex64, np.complex128)
+    rt = np.float32 if A.dtype == np.complex64 else np.float64
+    Ar = np.ascontiguousarray(A).view(rt)
+    Cr = np.ascontiguousarray(C).view(rt) if C is not None else None
+    fn = gemm_f32 if rt == np.float32 else gemm_f64
+    return np.ascontiguousarray(fn(Ar, complex_embed(B), Cr)).view(A.dtype)
+
+
 def gemm_f32_scalar(A, B, C=None):
     M, K = A.shape
     N = B.shape[1]
@@ -190,15 +211,23 @@ def _reference_call(A, B, C, threads):
         ld.ref_loader_sym.argtypes = [ctypes.c_char_p, ctypes.c_char_p]
         path = os.path.join(_HERE, "_ref", "libdecx_ref_cpu.so").encode()
         a32, a64 = ld.ref_loader_sym(path, b"ref_cpu_gemm_f32"), ld.ref_loader_sym(path, b"ref_cpu_gemm_f64")
-        assert a32 and a64, "could not load the compiled reference"
-        _ref_fn = {np.dtype(np.float32): (ctypes.CFUNCTYPE(ctypes.c_int, _f32p, _f32p, _f32p, _f32p, _u32, _u32, _u32, _u32)(a32), _f32p),
-                   np.dtype(np.float64): (ctypes.CFUNCTYPE(ctypes.c_int, _f64p, _f64p, _f64p, _f64p, _u32, _u32, _u32, _u32)(a64), _f64p)}
+        ac32 = ld.ref_loader_sym(path, b"ref_cpu_gemm_c32")
+        assert a32 and a64 and ac32, "could not load the compiled reference"
+        f32sig = ctypes.CFUNCTYPE(ctypes.c_int, _f32p, _f32p, _f32p, _f32p, _u32, _u32, _u32, _u32)
+        _ref_fn = {np.dtype(np.float32): (f32sig(a32), _f32p),
+                   np.dtype(np.float64): (ctypes.CFUNCTYPE(ctypes.c_int, _f64p, _f64p, _f64p, _f64p, _u32, _u32, _u32, _u32)(a64), _f64p),
+                   np.dtype(np.complex64): (f32sig(ac32), _f32p)}
     fn, pt = _ref_fn[A.dtype]
     M, K = A.shape
     N = B.shape[1]
     out = np.empty((M, N), A.dtype)
     err = fn(_p(A, pt), _p(B, pt), _p(C, pt), _p(out, pt), M, N, K, threads)
     return out, err
+
+
+def reference_cpu_gemm_c32(A, B, C=None, threads=8):
+    """The same for the reference's single-precision complex CPU GEMM (complex64 arrays)."""
+    return reference_cpu_gemm_f32(A, B, C, threads, dtype=np.complex64)
 
 
 def reference_cpu_gemm_f64(A, B, C=None, threads=8):

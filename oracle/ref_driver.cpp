@@ -51,3 +51,27 @@ extern "C" int ref_cpu_gemm_f64(const double* A, const double* B, const double* 
     mA.release(); mB.release(); mD.release();
     return err;
 }
+
+// complex single precision, interleaved (re, im); pitches of the dense inputs in complex elements
+extern "C" int ref_cpu_gemm_c32(const float* A, const float* B, const float* C, float* D,
+                                uint32_t M, uint32_t N, uint32_t K, uint32_t threads)
+{
+    de::cpu::DecxSetThreadingNum(threads);
+    de::Matrix& mA = de::CreateMatrixRef(de::_COMPLEX_F32_, K, M);
+    de::Matrix& mB = de::CreateMatrixRef(de::_COMPLEX_F32_, N, K);
+    de::Matrix& mD = de::CreateMatrixRef(de::_COMPLEX_F32_, N, M);
+    for (uint32_t i = 0; i < M; ++i) std::memcpy(mA.ptr<de::CPf>(i, 0), A + (size_t)i * K * 2, K * sizeof(de::CPf));
+    for (uint32_t i = 0; i < K; ++i) std::memcpy(mB.ptr<de::CPf>(i, 0), B + (size_t)i * N * 2, N * sizeof(de::CPf));
+    if (C) {
+        de::Matrix& mC = de::CreateMatrixRef(de::_COMPLEX_F32_, N, M);
+        for (uint32_t i = 0; i < M; ++i) std::memcpy(mC.ptr<de::CPf>(i, 0), C + (size_t)i * N * 2, N * sizeof(de::CPf));
+        de::blas::cpu::GEMM(mA, mB, mC, mD);
+        mC.release();
+    } else {
+        de::blas::cpu::GEMM(mA, mB, mD);
+    }
+    const int err = de::GetLastError()->error_type;
+    for (uint32_t i = 0; i < M; ++i) std::memcpy(D + (size_t)i * N * 2, mD.ptr<de::CPf>(i, 0), N * sizeof(de::CPf));
+    mA.release(); mB.release(); mD.release();
+    return err;
+}

@@ -162,8 +162,40 @@ static int gpu_checks()
     de::blas::cuda::GEMM(dA, dB, dS, dD, de::Number(1.f), de::Number(1.f));    // C has the wrong shape
     CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_DimsNotMatching);
     de::ResetLastError();
-    de::GPU_Matrix& dcx = de::CreateGPUMatrixRef(de::_COMPLEX_F32_, 8, 8);
-    de::blas::cuda::GEMM(dcx, dcx, dD);
+    de::GPU_Matrix& dint = de::CreateGPUMatrixRef(de::_INT32_, 8, 8);
+    de::blas::cuda::GEMM(dint, dint, dD);
+    CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_UNSUPPORTED_TYPE);
+    de::ResetLastError();
+    // complex single precision: (1 + i) I . X = (1 + i) X, then alpha = i, beta = 2: i (1 + i) X + 2 X = (1 + i) X
+    de::Matrix& Ic = de::CreateMatrixRef(de::_COMPLEX_F32_, 20, 20);
+    de::Matrix& Xc = de::CreateMatrixRef(de::_COMPLEX_F32_, 9, 20);
+    for (int i = 0; i < 20; ++i) { *Ic.ptr<de::CPf>(i, i) = de::CPf(1.f, 1.f); for (int j = 0; j < 9; ++j) *Xc.ptr<de::CPf>(i, j) = de::CPf((float)(i - 7), (float)(2 * j - 5)); }
+    CHECK(Xc.ptr<de::CPf>(1, 0) - Xc.ptr<de::CPf>(0, 0) == 12);                               // 32-byte rule: 4 complex
+    de::GPU_Matrix& dIc = de::CreateGPUMatrixRef(de::_COMPLEX_F32_, 20, 20);
+    de::GPU_Matrix& dXc = de::CreateGPUMatrixRef(de::_COMPLEX_F32_, 9, 20);
+    de::GPU_Matrix& dRc = de::CreateGPUMatrixRef();
+    CHECK(de::Memcpy(Ic, dIc, O, O, de::Point2D(20, 20), de::DECX_MEMCPY_H2D).error_type == 0);
+    CHECK(de::Memcpy(Xc, dXc, O, O, de::Point2D(9, 20), de::DECX_MEMCPY_H2D).error_type == 0);
+    de::blas::cuda::GEMM(dIc, dXc, dRc);
+    CHECK(de::GetLastError()->error_type == 0 && dRc.Type() == de::_COMPLEX_F32_ && dRc.Width() == 9 && dRc.Height() == 20);
+    de::Matrix& Rc = de::CreateMatrixRef(de::_COMPLEX_F32_, 9, 20);
+    CHECK(de::Memcpy(Rc, dRc, O, O, de::Point2D(9, 20), de::DECX_MEMCPY_D2H).error_type == 0);
+    bool samec = true;
+    for (int i = 0; i < 20; ++i) for (int j = 0; j < 9; ++j) {
+        const de::CPf x = *Xc.ptr<de::CPf>(i, j), r = *Rc.ptr<de::CPf>(i, j);
+        samec &= (r.real == x.real - x.image) && (r.image == x.real + x.image);
+    }
+    CHECK(samec);
+    de::blas::cuda::GEMM(dIc, dXc, dXc, dRc, de::Number(de::CPf(0.f, 1.f)), de::Number(de::CPf(2.f, 0.f)));
+    CHECK(de::GetLastError()->error_type == 0);
+    CHECK(de::Memcpy(Rc, dRc, O, O, de::Point2D(9, 20), de::DECX_MEMCPY_D2H).error_type == 0);
+    samec = true;
+    for (int i = 0; i < 20; ++i) for (int j = 0; j < 9; ++j) {
+        const de::CPf x = *Xc.ptr<de::CPf>(i, j), r = *Rc.ptr<de::CPf>(i, j);
+        samec &= (r.real == x.real - x.image) && (r.image == x.real + x.image);
+    }
+    CHECK(samec);
+    de::blas::cuda::GEMM(Ic, Xc, Rc);                                                         // host-matrix form: real types only
     CHECK(de::GetLastError()->error_type == decx::DECX_FAIL_UNSUPPORTED_TYPE);
     de::ResetLastError();
     // double precision: identity, and alpha / beta carried as doubles

@@ -33,6 +33,10 @@ REF64_CASES = [  # (M, N, K, threads, with_C): the reference's double-precision 
     (100, 150, 77, 4, False),
     (200, 112, 136, 4, True),
 ]
+REFC32_CASES = [  # (M, N, K, threads): the reference's single-precision complex CPU GEMM (compared with a tolerance:
+    (64, 64, 64, 1),   #  its blocked complex arithmetic rounds in another order than the oracle's chain)
+    (96, 80, 72, 4),
+]
 ORC_F32 = [  # (M, N, K, with_C, alpha, beta)   alpha None => chain seeded with C
     (37, 53, 29, False, None, None),
     (37, 53, 29, True, None, None),
@@ -71,6 +75,13 @@ def main():
         assert err == 0
         np.savez(os.path.join(HERE, f"ref_f64_{'abc' if with_c else 'ab'}_{M}x{N}x{K}.npz"), M=M, N=N, K=K, threads=T,
                  with_c=with_c, seed_a=sa, seed_b=sb, seed_c=sc, D=D, crc=crc(D))
+    for idx, (M, N, K, T) in enumerate(REFC32_CASES):
+        sa, sb = 0x6500 + idx, 0x7500 + idx
+        A = synth.uniform_f32(M, 2 * K, sa).view(np.complex64)
+        B = synth.uniform_f32(K, 2 * N, sb).view(np.complex64)
+        D, err = orc.reference_cpu_gemm_c32(A, B, None, threads=T)
+        assert err == 0
+        np.savez(os.path.join(HERE, f"ref_c32_{M}x{N}x{K}.npz"), M=M, N=N, K=K, threads=T, seed_a=sa, seed_b=sb, D=D, crc=crc(D))
     for idx, (M, N, K, with_c, alpha, beta) in enumerate(ORC_F32):
         sa, sb, sc = 0x6100 + idx, 0x7100 + idx, 0x8100 + idx
         A = synth.uniform_f32(M, K, sa)
