@@ -90,6 +90,8 @@ gemm_f32_dma_kernel(const GemmArgs g)
                   B_LOADS * WAVES * 1024 == B_STAGE_BYTES, "copy plan must divide evenly");
     static_assert(STAGES >= 2 && STAGES * STAGE_BYTES <= 160 * 1024, "LDS budget");
     static_assert(LOADS * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
+    static_assert(CHUNK_AHEAD || LOADS <= BK / 2 - 1, "one direct load per k step, the deferred last step excepted");
+    
     __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE_BYTES];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)lds;
 
@@ -97,7 +99,8 @@ gemm_f32_dma_kernel(const GemmArgs g)
     block_to_tile(g, tile_m, tile_n);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
 
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);      // uniform: LDS destinations stay in scalar registers
     const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
     const int l32 = lane & 31, h = lane >> 5;
 
@@ -133,17 +136,6 @@ gemm_f32_dma_kernel(const GemmArgs g)
             a_src[i] = A + (size_t)grow * lda_b + a_chunk[i] * 16;
         }
     }
-    auto conv_advance = [&]() {                        // CONV: on to the next slab
-#pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) {
-            a_seg[i] += BK * 4;
-            a_src[i] += BK * 4;
-            while (a_seg[i] >= g.conv_seg_bytes) {
-                a_seg[i] -= g.conv_seg_bytes;
-                a_src[i] += g.conv_seg_stride - g.conv_seg_bytes;
-            }
-        }
-    };
 #pragma unroll
     for (int i = 0; i < B_LOADS; ++i) {
         const int I = wave * B_LOADS + i;
@@ -156,46 +148,55 @@ gemm_f32_dma_kernel(const GemmArgs g)
     const uint32_t full_slabs = g.K / BK, k_tail = g.K % BK;
     const uint32_t slabs = full_slabs + (k_tail ? 1u : 0u);
 
-    auto issue_loads = [&](uint32_t slab) {
-        const uint32_t stage = slab % STAGES;
-        if (slab < full_slabs) {
-            const uint32_t stage_off = lds_base + stage * STAGE_BYTES;
-#pragma unroll
-            for (int i = 0; i < A_LOADS; ++i) {
-                const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u);
-                const unsigned char* src = CONV ? a_src[i] : a_src[i] + (size_t)slab * (BK * 4);
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
-            }
-            if constexpr (CONV) conv_advance();
-#pragma unroll
-            for (int i = 0; i < B_LOADS; ++i) {
-                const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + A_STAGE_BYTES +
-                                                                    (uint32_t)(wave * B_LOADS + i) * 1024u);
-                const unsigned char* src = b_src[i] + (size_t)slab * BK * ldb_b;
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
+    // Slabs are issued in ascending order, so a_src / b_src simply run along K: each direct load
+    // leaves its pointer at the next slab (CONV: hopping to the next image row at the end of a run).
+    const size_t b_step = (size_t)BK * ldb_b;
+    auto issue_one = [&](uint32_t stage, auto ic) {        // direct load ic of a full slab: A first, then B
+        constexpr int idx = decltype(ic)::value;
+        const uint32_t stage_off = lds_base + stage * STAGE_BYTES;
+        if constexpr (idx < A_LOADS) {
+            constexpr int i = idx;
+            const uint32_t dst = stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u;
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(a_src[i]) : "memory", "m0");
+            a_src[i] += BK * 4;
+            if constexpr (CONV) {
+                a_seg[i] += BK * 4;
+                while (a_seg[i] >= g.conv_seg_bytes) {
+                    a_seg[i] -= g.conv_seg_bytes;
+                    a_src[i] += g.conv_seg_stride - g.conv_seg_bytes;
+                }
             }
         } else {
-            // the partial last slab: through registers, zero beyond K
-            unsigned char* st = lds + stage * STAGE_BYTES;
-            const uint32_t k0 = full_slabs * BK;
-#pragma unroll
-            for (int i = 0; i < A_LOADS; ++i) {
-                const uint32_t k = k0 + a_chunk[i] * 4;
-                floatx4 v = floatx4{0.f, 0.f, 0.f, 0.f};
-                if (k < g.K) {
-                    v = *(const floatx4*)(CONV ? a_src[i] : a_src[i] + (size_t)k0 * 4);   // inside the pitch: lda is a multiple of 4
-#pragma unroll
-                    for (int e = 1; e < 4; ++e) if (k + e >= g.K) v[e] = 0.f;
-                }
-                *(floatx4*)(st + (wave * A_LOADS + i) * 1024 + lane * 16) = v;
-            }
-#pragma unroll
-            for (int i = 0; i < B_LOADS; ++i) {
-                floatx4 v = floatx4{0.f, 0.f, 0.f, 0.f};
-                if (k0 + b_krow[i] < g.K) v = *(const floatx4*)(b_src[i] + (size_t)k0 * ldb_b);
-                *(floatx4*)(st + A_STAGE_BYTES + (wave * B_LOADS + i) * 1024 + lane * 16) = v;
-            }
+            constexpr int i = idx - A_LOADS;
+            const uint32_t dst = stage_off + A_STAGE_BYTES + (uint32_t)(wave * B_LOADS + i) * 1024u;
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(b_src[i]) : "memory", "m0");
+            b_src[i] += b_step;
         }
+    };
+    auto issue_tail = [&](uint32_t stage) {                // the partial last slab: through registers, zero beyond K
+        unsigned char* st = lds + stage * STAGE_BYTES;
+        const uint32_t k0 = full_slabs * BK;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) {
+            const uint32_t k = k0 + a_chunk[i] * 4;
+            floatx4 v = floatx4{0.f, 0.f, 0.f, 0.f};
+            if (k < g.K) {
+                v = *(const floatx4*)a_src[i];             // inside the pitch: lda is a multiple of 4
+#pragma unroll
+                for (int e = 1; e < 4; ++e) if (k + e >= g.K) v[e] = 0.f;
+            }
+            *(floatx4*)(st + (wave * A_LOADS + i) * 1024 + lane * 16) = v;
+        }
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) {
+            floatx4 v = floatx4{0.f, 0.f, 0.f, 0.f};
+            if (k0 + b_krow[i] < g.K) v = *(const floatx4*)b_src[i];
+            *(floatx4*)(st + A_STAGE_BYTES + (wave * B_LOADS + i) * 1024 + lane * 16) = v;
+        }
+    };
+    auto issue_loads = [&](uint32_t slab) {                // a whole slab in one burst
+        if (slab < full_slabs) static_for<0, LOADS>([&](auto ic) { issue_one(slab % STAGES, ic); });
+        else issue_tail(slab % STAGES);
     };
 
     // ---- fragment addressing inside a stage
@@ -226,24 +227,34 @@ gemm_f32_dma_kernel(const GemmArgs g)
 
     if constexpr (!CHUNK_AHEAD) {
         // Large wave tiles: a k step is TM * TN MFMAs, long enough to hide an LDS read, so fragments
-        // are fetched one step ahead.  af[c & 1] holds chunk c of A (4 k per lane), bf[step & 1] the
-        // B values of a k step.  The MFMAs of the last step of a slab are issued after the slab
-        // barrier, behind the first fragment reads of the next slab (before the first slab they
-        // multiply zeros).
+        // are fetched a few steps ahead, one or a few reads behind the first MFMA of each step (bursts
+        // of reads, and reads only one step ahead, both measure slower: LDS reads are held up while
+        // direct loads land).  af[c & 1] holds chunk c of A (4 k per lane), read 3 steps before its
+        // first use; bf[step & 3] the B values of a k step, read 2 steps ahead.  The MFMAs of the last
+        // step of a slab are issued after the slab barrier, behind the first fragment reads of the next
+        // slab (before the first slab they multiply zeros).
         floatx4 af[2][TM];
-        bfrag bf[2];
+        constexpr int BF_AHEAD = 2, BFM = 3;               // B fragments are read 2 k steps ahead into a ring of 4
+        bfrag bf[BFM + 1];
 #pragma unroll
         for (int i = 0; i < TM; ++i) af[(CHUNKS - 1) & 1][i] = floatx4{0.f, 0.f, 0.f, 0.f};
-        bf[(STEPS - 1) & 1] = bfrag{};
+        bf[(STEPS - 1) & BFM] = bfrag{};
 
-        auto multiply = [&](auto stc) {
+        // MFMAs FIRST .. LAST-1 (in i-major order) of a k step
+        auto multiply_part = [&](auto stc, auto firstc, auto lastc) {
             constexpr int step = decltype(stc)::value;
             constexpr int c = step / 4, e = step % 4;
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c & 1][i][e], lane_of<TN>(bf[step & 1], j), acc[i][j], 0, 0, 0);
+            static_for<decltype(firstc)::value, decltype(lastc)::value>([&](auto nc) {
+                constexpr int i = decltype(nc)::value / TN, j = decltype(nc)::value % TN;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c & 1][i][e], lane_of<TN>(bf[step & BFM], j), acc[i][j], 0, 0, 0);
+            });
+        };
+        auto multiply = [&](auto stc) {
+            multiply_part(stc, std::integral_constant<int, 0>{}, std::integral_constant<int, TM * TN>{});
+        };
+        auto read_b = [&](const unsigned char* st, auto stc) {
+            constexpr int step = decltype(stc)::value;
+            bf[step & BFM] = *(const bfrag*)(st + b_off + (8 * (step / 4) + step % 4) * BN * 4);
         };
 
         for (uint32_t s = 0; s < slabs; ++s) {
@@ -252,28 +263,36 @@ gemm_f32_dma_kernel(const GemmArgs g)
 
 #pragma unroll
             for (int i = 0; i < TM; ++i) af[0][i] = *(const floatx4*)(st + a_off[0] + i * 32 * BK * 4);
-            bf[0] = *(const bfrag*)(st + b_off);
+            static_for<0, BF_AHEAD>([&](auto stc) { read_b(st, stc); });
             multiply(std::integral_constant<int, STEPS - 1>{});
-            __builtin_amdgcn_sched_group_barrier(0x100, TM + 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, TM + BF_AHEAD, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
             __builtin_amdgcn_sched_barrier(0);
-            // the stage that held slab s-1 is free: every wave passed the barrier after reading it
-            if (more) issue_loads(s + STAGES - 1);
+            // The stage that held slab s-1 is free: every wave passed the barrier after reading it.
+            const uint32_t nstage = (s + STAGES - 1) % STAGES;
+            const bool direct = s + STAGES - 1 < full_slabs;
+            if (more && !direct) issue_tail(nstage);
 
             static_for<0, STEPS - 1>([&](auto stc) {
                 constexpr int step = decltype(stc)::value;
                 constexpr int c = step / 4, e = step % 4;
                 constexpr bool next_a = (e == 1) && (c + 1 < CHUNKS);
-                constexpr int reads = 1 + (next_a ? TM : 0);
-                bf[(step + 1) & 1] = *(const bfrag*)(st + b_off + (8 * ((step + 1) / 4) + (step + 1) % 4) * BN * 4);
+                constexpr bool next_b = step + BF_AHEAD < STEPS;
+                constexpr int reads = (next_b ? 1 : 0) + (next_a ? TM : 0);
+                if constexpr (next_b) read_b(st, std::integral_constant<int, step + BF_AHEAD>{});
                 if constexpr (next_a) {
 #pragma unroll
                     for (int i = 0; i < TM; ++i) af[(c + 1) & 1][i] = *(const floatx4*)(st + a_off[c + 1] + i * 32 * BK * 4);
                 }
-                multiply(stc);
+                multiply_part(stc, std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, reads, 0);
-                if constexpr (TM * TN > 1) __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 1, 0);
+                if constexpr (reads > 0) __builtin_amdgcn_sched_group_barrier(0x100, reads, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (step < LOADS) {
+                    if (direct) issue_one(nstage, std::integral_constant<int, step>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                multiply_part(stc, std::integral_constant<int, 1>{}, std::integral_constant<int, TM * TN>{});
                 __builtin_amdgcn_sched_barrier(0);
             });
 
