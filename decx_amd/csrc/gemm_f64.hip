@@ -71,7 +71,8 @@ gemm_f64_dma_kernel(const GemmArgs g)
     block_to_tile(g, tile_m, tile_n);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
 
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);      // uniform: LDS destinations stay in scalar registers
     const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
     const int l16 = lane & 15, q = lane >> 4;
 
@@ -104,44 +105,47 @@ gemm_f64_dma_kernel(const GemmArgs g)
     const uint32_t full_slabs = g.K / BK, k_tail = g.K % BK;
     const uint32_t slabs = full_slabs + (k_tail ? 1u : 0u);
 
-    auto issue_loads = [&](uint32_t slab) {
-        const uint32_t stage = slab % STAGES;
-        if (slab < full_slabs) {
-            const uint32_t stage_off = lds_base + stage * STAGE_BYTES;
-#pragma unroll
-            for (int i = 0; i < A_LOADS; ++i) {
-                const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u);
-                const unsigned char* src = a_src[i] + (size_t)slab * RBYTES;
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
-            }
-#pragma unroll
-            for (int i = 0; i < B_LOADS; ++i) {
-                const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + A_STAGE_BYTES +
-                                                                    (uint32_t)(wave * B_LOADS + i) * 1024u);
-                const unsigned char* src = b_src[i] + (size_t)slab * BK * ldb_b;
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
-            }
+    // Slabs are issued in ascending order, so a_src / b_src simply run along K: each direct load
+    // leaves its pointer at the next slab.
+    const size_t b_step = (size_t)BK * ldb_b;
+    auto issue_one = [&](uint32_t stage, auto ic) {        // direct load ic of a full slab: A first, then B
+        constexpr int idx = decltype(ic)::value;
+        const uint32_t stage_off = lds_base + stage * STAGE_BYTES;
+        if constexpr (idx < A_LOADS) {
+            constexpr int i = idx;
+            const uint32_t dst = stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u;
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(a_src[i]) : "memory", "m0");
+            a_src[i] += RBYTES;
         } else {
-            // the partial last slab: through registers, zero beyond K
-            unsigned char* st = lds + stage * STAGE_BYTES;
-            const uint32_t k0 = full_slabs * BK;
-#pragma unroll
-            for (int i = 0; i < A_LOADS; ++i) {
-                const uint32_t k = k0 + a_chunk[i] * 2;
-                doublex2 v = doublex2{0.0, 0.0};
-                if (k < g.K) {
-                    v = *(const doublex2*)(a_src[i] + (size_t)k0 * 8);      // inside the pitch: lda is a multiple of 2
-                    if (k + 1 >= g.K) v[1] = 0.0;
-                }
-                *(doublex2*)(st + (wave * A_LOADS + i) * 1024 + lane * 16) = v;
-            }
-#pragma unroll
-            for (int i = 0; i < B_LOADS; ++i) {
-                doublex2 v = doublex2{0.0, 0.0};
-                if (k0 + b_krow[i] < g.K) v = *(const doublex2*)(b_src[i] + (size_t)k0 * ldb_b);
-                *(doublex2*)(st + A_STAGE_BYTES + (wave * B_LOADS + i) * 1024 + lane * 16) = v;
-            }
+            constexpr int i = idx - A_LOADS;
+            const uint32_t dst = stage_off + A_STAGE_BYTES + (uint32_t)(wave * B_LOADS + i) * 1024u;
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(b_src[i]) : "memory", "m0");
+            b_src[i] += b_step;
         }
+    };
+    auto issue_tail = [&](uint32_t stage) {                // the partial last slab: through registers, zero beyond K
+        unsigned char* st = lds + stage * STAGE_BYTES;
+        const uint32_t k0 = full_slabs * BK;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) {
+            const uint32_t k = k0 + a_chunk[i] * 2;
+            doublex2 v = doublex2{0.0, 0.0};
+            if (k < g.K) {
+                v = *(const doublex2*)a_src[i];            // inside the pitch: lda is even
+                if (k + 1 >= g.K) v[1] = 0.0;
+            }
+            *(doublex2*)(st + (wave * A_LOADS + i) * 1024 + lane * 16) = v;
+        }
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) {
+            doublex2 v = doublex2{0.0, 0.0};
+            if (k0 + b_krow[i] < g.K) v = *(const doublex2*)b_src[i];
+            *(doublex2*)(st + A_STAGE_BYTES + (wave * B_LOADS + i) * 1024 + lane * 16) = v;
+        }
+    };
+    auto issue_loads = [&](uint32_t slab) {                // a whole slab in one burst
+        if (slab < full_slabs) static_for<0, LOADS>([&](auto ic) { issue_one(slab % STAGES, ic); });
+        else issue_tail(slab % STAGES);
     };
 
     // ---- fragment addressing inside a stage
@@ -169,55 +173,72 @@ gemm_f64_dma_kernel(const GemmArgs g)
     // step ahead; the MFMAs of the last step of a slab are issued after the slab barrier, behind the first
     // fragment reads of the next slab (before the first slab they multiply zeros).
     doublex2 af[2][TM];
-    doublex2 bf[2][TP];
+    constexpr int BF_AHEAD = 2, BFM = 3;                   // B fragments are read 2 k steps ahead into a ring of 4
+    doublex2 bf[BFM + 1][TP];
 #pragma unroll
     for (int i = 0; i < TM; ++i) af[(GROUPS - 1) & 1][i] = doublex2{0.0, 0.0};
 #pragma unroll
-    for (int jj = 0; jj < TP; ++jj) bf[(STEPS - 1) & 1][jj] = doublex2{0.0, 0.0};
+    for (int jj = 0; jj < TP; ++jj) bf[(STEPS - 1) & BFM][jj] = doublex2{0.0, 0.0};
 
-    auto multiply = [&](auto stc) {
+    // MFMAs FIRST .. LAST-1 (in i-major order) of a k step
+    auto multiply_part = [&](auto stc, auto firstc, auto lastc) {
         constexpr int step = decltype(stc)::value;
         constexpr int tt = step / 2, e = step % 2;
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[tt & 1][i][e], bf[step & 1][j / 2][j % 2], acc[i][j], 0, 0, 0);
+        static_for<decltype(firstc)::value, decltype(lastc)::value>([&](auto nc) {
+            constexpr int i = decltype(nc)::value / TN, j = decltype(nc)::value % TN;
+            acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[tt & 1][i][e], bf[step & BFM][j / 2][j % 2], acc[i][j], 0, 0, 0);
+        });
+    };
+    auto multiply = [&](auto stc) {
+        multiply_part(stc, std::integral_constant<int, 0>{}, std::integral_constant<int, TM * TN>{});
     };
     auto read_b = [&](const unsigned char* st, auto stc) {
         constexpr int step = decltype(stc)::value;
 #pragma unroll
         for (int jj = 0; jj < TP; ++jj)
-            bf[step & 1][jj] = *(const doublex2*)(st + b_off + (8 * (step / 2) + step % 2) * BN * 8 + jj * 32 * 8);
+            bf[step & BFM][jj] = *(const doublex2*)(st + b_off + (8 * (step / 2) + step % 2) * BN * 8 + jj * 32 * 8);
     };
     auto read_a = [&](const unsigned char* st, auto tc) {
         constexpr int tt = decltype(tc)::value;
 #pragma unroll
         for (int i = 0; i < TM; ++i) af[tt & 1][i] = *(const doublex2*)(st + a_off[tt] + i * 16 * RBYTES);
     };
+    // the direct loads of a slab go out PER_STEP per k step, each group behind the first MFMA of its step
+    constexpr int PER_STEP = (LOADS + STEPS - 2) / (STEPS - 1);
 
     for (uint32_t s = 0; s < slabs; ++s) {
         const unsigned char* st = lds + (s % STAGES) * STAGE_BYTES;
         const bool more = s + STAGES - 1 < slabs;
 
         read_a(st, std::integral_constant<int, 0>{});
-        read_b(st, std::integral_constant<int, 0>{});
+        static_for<0, BF_AHEAD>([&](auto stc) { read_b(st, stc); });
         multiply(std::integral_constant<int, STEPS - 1>{});
-        __builtin_amdgcn_sched_group_barrier(0x100, TM + TP, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, TM + BF_AHEAD * TP, 0);
         __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
         __builtin_amdgcn_sched_barrier(0);
         // the stage that held slab s-1 is free: every wave passed the barrier after reading it
-        if (more) issue_loads(s + STAGES - 1);
+        const uint32_t nstage = (s + STAGES - 1) % STAGES;
+        const bool direct = s + STAGES - 1 < full_slabs;
+        if (more && !direct) issue_tail(nstage);
 
         static_for<0, STEPS - 1>([&](auto stc) {
             constexpr int step = decltype(stc)::value;
             constexpr bool next_a = (step % 2 == 1);                   // step + 1 opens the next k group
-            read_b(st, std::integral_constant<int, step + 1>{});
+            constexpr bool next_b = step + BF_AHEAD < STEPS;
+            constexpr int reads = (next_b ? TP : 0) + (next_a ? TM : 0);
+            if constexpr (next_b) read_b(st, std::integral_constant<int, step + BF_AHEAD>{});
             if constexpr (next_a) read_a(st, std::integral_constant<int, (step + 1) / 2>{});
-            multiply(stc);
+            multiply_part(stc, std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, TP + (next_a ? TM : 0), 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 1, 0);
+            if constexpr (reads > 0) __builtin_amdgcn_sched_group_barrier(0x100, reads, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (step * PER_STEP < LOADS) {
+                if (direct)
+                    static_for<step * PER_STEP, (step + 1) * PER_STEP < LOADS ? (step + 1) * PER_STEP : LOADS>(
+                        [&](auto ic) { issue_one(nstage, ic); });
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            multiply_part(stc, std::integral_constant<int, 1>{}, std::integral_constant<int, TM * TN>{});
             __builtin_amdgcn_sched_barrier(0);
         });
 
