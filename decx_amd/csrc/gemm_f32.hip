@@ -256,7 +256,7 @@ static int launch_shape(const GemmArgs& args, hipStream_t stream)
 
 int launch_gemm_f32(int shape, bool edge, const GemmArgs& args, hipStream_t stream)
 {
-    if (!edge && args.vec_ok && args.K > 0) return launch_gemm_f32_dma(shape, args, stream);
+    if (!edge && args.vec_ok && args.K > 0 && dma_offsets_fit(args, 4)) return launch_gemm_f32_dma(shape, args, stream);
     switch (shape) {
     case TILE_256x256: return launch_shape<256, 256, 16, 4, 2>(args, stream);
     case TILE_128x128: return launch_shape<128, 128, 16, 2, 2>(args, stream);

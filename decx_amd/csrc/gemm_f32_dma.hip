@@ -148,18 +148,34 @@ gemm_f32_dma_kernel(const GemmArgs g)
     const uint32_t full_slabs = g.K / BK, k_tail = g.K % BK;
     const uint32_t slabs = full_slabs + (k_tail ? 1u : 0u);
 
-    // Slabs are issued in ascending order, so a_src / b_src simply run along K: each direct load
-    // leaves its pointer at the next slab (CONV: hopping to the next image row at the end of a run).
+    // Slabs are issued in ascending order.  Plain GEMM: a direct load takes its address as a scalar base (the
+    // tile's first row of A / B's row k, running along K) plus a 32-bit lane offset that never changes, so
+    // that advancing to the next slab is scalar arithmetic.  CONV: the lanes' sources hop between image rows
+    // independently, so a_src / b_src are full per-lane pointers, each left at the next slab by its load.
     const size_t b_step = (size_t)BK * ldb_b;
+    uint32_t a_voff[CONV ? 1 : A_LOADS], b_voff[CONV ? 1 : B_LOADS];
+    const unsigned char* a_base = A + (size_t)m0 * lda_b;
+    const unsigned char* b_base = B;
+    if constexpr (!CONV) {
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) a_voff[i] = (uint32_t)(a_src[i] - a_base);       // < BM * lda_b: the launcher checks
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) b_voff[i] = (uint32_t)(b_src[i] - b_base);       // < BK * ldb_b
+    }
+    auto a_ptr = [&](int i) { if constexpr (CONV) return a_src[i]; else return a_base + a_voff[i]; };
+    auto b_ptr = [&](int i) { if constexpr (CONV) return b_src[i]; else return b_base + b_voff[i]; };
     auto issue_one = [&](uint32_t stage, auto ic) {        // direct load ic of a full slab: A first, then B
         constexpr int idx = decltype(ic)::value;
         const uint32_t stage_off = lds_base + stage * STAGE_BYTES;
         if constexpr (idx < A_LOADS) {
             constexpr int i = idx;
             const uint32_t dst = stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u;
-            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(a_src[i]) : "memory", "m0");
-            a_src[i] += BK * 4;
-            if constexpr (CONV) {
+            if constexpr (!CONV) {
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(a_voff[i]), "s"(a_base) : "memory", "m0");
+                if constexpr (i == A_LOADS - 1) a_base += BK * 4;
+            } else {
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(a_src[i]) : "memory", "m0");
+                a_src[i] += BK * 4;
                 a_seg[i] += BK * 4;
                 while (a_seg[i] >= g.conv_seg_bytes) {
                     a_seg[i] -= g.conv_seg_bytes;
@@ -169,8 +185,13 @@ gemm_f32_dma_kernel(const GemmArgs g)
         } else {
             constexpr int i = idx - A_LOADS;
             const uint32_t dst = stage_off + A_STAGE_BYTES + (uint32_t)(wave * B_LOADS + i) * 1024u;
-            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(b_src[i]) : "memory", "m0");
-            b_src[i] += b_step;
+            if constexpr (!CONV) {
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(b_voff[i]), "s"(b_base) : "memory", "m0");
+                if constexpr (i == B_LOADS - 1) b_base += b_step;
+            } else {
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(b_src[i]) : "memory", "m0");
+                b_src[i] += b_step;
+            }
         }
     };
     auto issue_tail = [&](uint32_t stage) {                // the partial last slab: through registers, zero beyond K
@@ -181,7 +202,7 @@ gemm_f32_dma_kernel(const GemmArgs g)
             const uint32_t k = k0 + a_chunk[i] * 4;
             floatx4 v = floatx4{0.f, 0.f, 0.f, 0.f};
             if (k < g.K) {
-                v = *(const floatx4*)a_src[i];             // inside the pitch: lda is a multiple of 4
+                v = *(const floatx4*)a_ptr(i);             // inside the pitch: lda is a multiple of 4
 #pragma unroll
                 for (int e = 1; e < 4; ++e) if (k + e >= g.K) v[e] = 0.f;
             }
@@ -190,7 +211,7 @@ gemm_f32_dma_kernel(const GemmArgs g)
 #pragma unroll
         for (int i = 0; i < B_LOADS; ++i) {
             floatx4 v = floatx4{0.f, 0.f, 0.f, 0.f};
-            if (k0 + b_krow[i] < g.K) v = *(const floatx4*)b_src[i];
+            if (k0 + b_krow[i] < g.K) v = *(const floatx4*)b_ptr(i);
             *(floatx4*)(st + A_STAGE_BYTES + (wave * B_LOADS + i) * 1024 + lane * 16) = v;
         }
     };
@@ -229,8 +250,8 @@ gemm_f32_dma_kernel(const GemmArgs g)
         // Large wave tiles: a k step is TM * TN MFMAs, long enough to hide an LDS read, so fragments
         // are fetched a few steps ahead, one or a few reads behind the first MFMA of each step (bursts
         // of reads, and reads only one step ahead, both measure slower: LDS reads are held up while
-        // direct loads land).  af[c & 1] holds chunk c of A (4 k per lane), read 3 steps before its
-        // first use; bf[step & 3] the B values of a k step, read 2 steps ahead.  The MFMAs of the last
+        // direct loads land).  af[c & 1] holds chunk c of A (4 k per lane), read during chunk c - 1, a
+        // quarter of it per step; bf[step & 3] the B values of a k step, read 2 steps ahead.  The MFMAs of the last
         // step of a slab are issued after the slab barrier, behind the first fragment reads of the next
         // slab (before the first slab they multiply zeros).
         floatx4 af[2][TM];
@@ -276,14 +297,14 @@ gemm_f32_dma_kernel(const GemmArgs g)
             static_for<0, STEPS - 1>([&](auto stc) {
                 constexpr int step = decltype(stc)::value;
                 constexpr int c = step / 4, e = step % 4;
-                constexpr bool next_a = (e == 1) && (c + 1 < CHUNKS);
                 constexpr bool next_b = step + BF_AHEAD < STEPS;
-                constexpr int reads = (next_b ? 1 : 0) + (next_a ? TM : 0);
+                constexpr int a_lo = (c + 1 < CHUNKS) ? (e * TM + 3) / 4 : 0, a_hi = (c + 1 < CHUNKS) ? ((e + 1) * TM + 3) / 4 : 0;
+                constexpr int reads = (next_b ? 1 : 0) + (a_hi - a_lo);
                 if constexpr (next_b) read_b(st, std::integral_constant<int, step + BF_AHEAD>{});
-                if constexpr (next_a) {
-#pragma unroll
-                    for (int i = 0; i < TM; ++i) af[(c + 1) & 1][i] = *(const floatx4*)(st + a_off[c + 1] + i * 32 * BK * 4);
-                }
+                static_for<a_lo, a_hi>([&](auto ic) {
+                    constexpr int i = decltype(ic)::value;
+                    af[(c + 1) & 1][i] = *(const floatx4*)(st + a_off[(c + 1) % CHUNKS] + i * 32 * BK * 4);
+                });
                 multiply_part(stc, std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 if constexpr (reads > 0) __builtin_amdgcn_sched_group_barrier(0x100, reads, 0);

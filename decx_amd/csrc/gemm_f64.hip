@@ -105,22 +105,30 @@ gemm_f64_dma_kernel(const GemmArgs g)
     const uint32_t full_slabs = g.K / BK, k_tail = g.K % BK;
     const uint32_t slabs = full_slabs + (k_tail ? 1u : 0u);
 
-    // Slabs are issued in ascending order, so a_src / b_src simply run along K: each direct load
-    // leaves its pointer at the next slab.
+    // Slabs are issued in ascending order.  A direct load takes its address as a scalar base (the tile's
+    // first row of A / B's row k, running along K) plus a 32-bit lane offset that never changes, so that
+    // advancing to the next slab is scalar arithmetic.
     const size_t b_step = (size_t)BK * ldb_b;
+    uint32_t a_voff[A_LOADS], b_voff[B_LOADS];
+    const unsigned char* a_base = A + (size_t)m0 * lda_b;
+    const unsigned char* b_base = B;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) a_voff[i] = (uint32_t)(a_src[i] - a_base);           // < BM * lda_b: the launcher checks
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) b_voff[i] = (uint32_t)(b_src[i] - b_base);           // < BK * ldb_b
     auto issue_one = [&](uint32_t stage, auto ic) {        // direct load ic of a full slab: A first, then B
         constexpr int idx = decltype(ic)::value;
         const uint32_t stage_off = lds_base + stage * STAGE_BYTES;
         if constexpr (idx < A_LOADS) {
             constexpr int i = idx;
             const uint32_t dst = stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u;
-            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(a_src[i]) : "memory", "m0");
-            a_src[i] += RBYTES;
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(a_voff[i]), "s"(a_base) : "memory", "m0");
+            if constexpr (i == A_LOADS - 1) a_base += RBYTES;
         } else {
             constexpr int i = idx - A_LOADS;
             const uint32_t dst = stage_off + A_STAGE_BYTES + (uint32_t)(wave * B_LOADS + i) * 1024u;
-            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(b_src[i]) : "memory", "m0");
-            b_src[i] += b_step;
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(b_voff[i]), "s"(b_base) : "memory", "m0");
+            if constexpr (i == B_LOADS - 1) b_base += b_step;
         }
     };
     auto issue_tail = [&](uint32_t stage) {                // the partial last slab: through registers, zero beyond K
@@ -131,7 +139,7 @@ gemm_f64_dma_kernel(const GemmArgs g)
             const uint32_t k = k0 + a_chunk[i] * 2;
             doublex2 v = doublex2{0.0, 0.0};
             if (k < g.K) {
-                v = *(const doublex2*)a_src[i];            // inside the pitch: lda is even
+                v = *(const doublex2*)(a_base + a_voff[i]);    // inside the pitch: lda is even
                 if (k + 1 >= g.K) v[1] = 0.0;
             }
             *(doublex2*)(st + (wave * A_LOADS + i) * 1024 + lane * 16) = v;
@@ -139,7 +147,7 @@ gemm_f64_dma_kernel(const GemmArgs g)
 #pragma unroll
         for (int i = 0; i < B_LOADS; ++i) {
             doublex2 v = doublex2{0.0, 0.0};
-            if (k0 + b_krow[i] < g.K) v = *(const doublex2*)b_src[i];
+            if (k0 + b_krow[i] < g.K) v = *(const doublex2*)(b_base + b_voff[i]);
             *(doublex2*)(st + A_STAGE_BYTES + (wave * B_LOADS + i) * 1024 + lane * 16) = v;
         }
     };
@@ -223,11 +231,15 @@ gemm_f64_dma_kernel(const GemmArgs g)
 
         static_for<0, STEPS - 1>([&](auto stc) {
             constexpr int step = decltype(stc)::value;
-            constexpr bool next_a = (step % 2 == 1);                   // step + 1 opens the next k group
+            constexpr int tt = step / 2, e = step % 2;                 // group tt + 1 of A is read during group tt, half per step
             constexpr bool next_b = step + BF_AHEAD < STEPS;
-            constexpr int reads = (next_b ? TP : 0) + (next_a ? TM : 0);
+            constexpr int a_lo = (tt + 1 < GROUPS) ? (e * TM + 1) / 2 : 0, a_hi = (tt + 1 < GROUPS) ? ((e + 1) * TM + 1) / 2 : 0;
+            constexpr int reads = (next_b ? TP : 0) + (a_hi - a_lo);
             if constexpr (next_b) read_b(st, std::integral_constant<int, step + BF_AHEAD>{});
-            if constexpr (next_a) read_a(st, std::integral_constant<int, (step + 1) / 2>{});
+            static_for<a_lo, a_hi>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                af[(tt + 1) & 1][i] = *(const doublex2*)(st + a_off[(tt + 1) % GROUPS] + i * 16 * RBYTES);
+            });
             multiply_part(stc, std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             if constexpr (reads > 0) __builtin_amdgcn_sched_group_barrier(0x100, reads, 0);
@@ -315,7 +327,7 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
 // shape: TILE_256x256 stands for the largest fp64 tile, 256 x 128 (eight wavefronts of 64 x 64).
 int launch_gemm_f64(int shape, bool plain, const GemmArgs& args, hipStream_t stream)
 {
-    if (plain || !args.vec_ok || args.K == 0) {
+    if (plain || !args.vec_ok || args.K == 0 || !dma_offsets_fit(args, 8)) {
         const dim3 grid((args.N + 15) / 16, (args.M + 15) / 16);
         hipLaunchKernelGGL(gemm_f64_plain_kernel, grid, dim3(256), 0, stream, args);
         return (int)hipGetLastError();
