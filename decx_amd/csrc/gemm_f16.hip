@@ -229,7 +229,7 @@ static int launch_shape(const GemmArgs& args, hipStream_t stream)
 
 int launch_gemm_f16(int shape, bool edge, const GemmArgs& args, hipStream_t stream)
 {
-    if (!edge && args.vec_ok && args.K > 0) return launch_gemm_f16_dma(shape, args, stream);
+    if (!edge && args.vec_ok && args.K > 0 && dma_offsets_fit(args, 2)) return launch_gemm_f16_dma(shape, args, stream);
     switch (shape) {
     case TILE_256x256: return launch_shape<256, 256, 64, 2, 2>(args, stream);
     case TILE_128x128: return launch_shape<128, 128, 64, 2, 1>(args, stream);

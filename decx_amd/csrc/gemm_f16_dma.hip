@@ -102,7 +102,8 @@ gemm_f16_dma_kernel(const GemmArgs g)
     block_to_tile(g, tile_m, tile_n);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
 
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);      // uniform: LDS destinations stay in scalar registers
     const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
     const int l32 = lane & 31, h = lane >> 5;
 
@@ -137,23 +138,33 @@ gemm_f16_dma_kernel(const GemmArgs g)
     const uint32_t full_slabs = g.K / BK, k_tail = g.K % BK;
     const uint32_t slabs = full_slabs + (k_tail ? 1u : 0u);
 
+    // Slabs are issued in ascending order.  A direct load takes its address as a scalar base (the tile's
+    // first row of A / B's row k, running along K) plus a 32-bit lane offset that never changes, so that
+    // advancing to the next slab is scalar arithmetic.
+    const size_t b_step = (size_t)BK * ldb_b;
+    uint32_t a_voff[A_LOADS], b_voff[B_LOADS];
+    const unsigned char* a_base = A + (size_t)m0 * lda_b;
+    const unsigned char* b_base = B;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) a_voff[i] = (uint32_t)(a_src[i] - a_base);           // < BM * lda_b: the launcher checks
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) b_voff[i] = (uint32_t)(b_src[i] - b_base);           // < BK * ldb_b
     auto issue_loads = [&](uint32_t slab) {
         const uint32_t stage = slab % STAGES;
         if (slab < full_slabs) {
             const uint32_t stage_off = lds_base + stage * STAGE_BYTES;
 #pragma unroll
             for (int i = 0; i < A_LOADS; ++i) {
-                const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u);
-                const unsigned char* src = a_src[i] + (size_t)slab * RB;
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
+                const uint32_t dst = stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u;
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(a_voff[i]), "s"(a_base) : "memory", "m0");
             }
+            a_base += RB;
 #pragma unroll
             for (int i = 0; i < B_LOADS; ++i) {
-                const uint32_t dst = __builtin_amdgcn_readfirstlane(stage_off + A_STAGE_BYTES +
-                                                                    (uint32_t)(wave * B_LOADS + i) * 1024u);
-                const unsigned char* src = b_src[i] + (size_t)slab * BK * ldb_b;
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory", "m0");
+                const uint32_t dst = stage_off + A_STAGE_BYTES + (uint32_t)(wave * B_LOADS + i) * 1024u;
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(b_voff[i]), "s"(b_base) : "memory", "m0");
             }
+            b_base += b_step;
         } else {
             // the partial last slab: through registers, zero beyond K
             unsigned char* st = lds + stage * STAGE_BYTES;
@@ -163,7 +174,7 @@ gemm_f16_dma_kernel(const GemmArgs g)
                 const uint32_t k = k0 + a_chunk[i] * 8;
                 halfx8 v = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
                 if (k < g.K) {
-                    v = *(const halfx8*)(a_src[i] + (size_t)k0 * 2);      // inside the pitch: lda is a multiple of 8
+                    v = *(const halfx8*)(a_base + a_voff[i]);             // inside the pitch: lda is a multiple of 8
 #pragma unroll
                     for (int e = 1; e < 8; ++e) if (k + e >= g.K) v[e] = (_Float16)0;
                 }
@@ -172,7 +183,7 @@ gemm_f16_dma_kernel(const GemmArgs g)
 #pragma unroll
             for (int i = 0; i < B_LOADS; ++i) {
                 halfx8 v = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
-                if (k0 + b_krow[i] < g.K) v = *(const halfx8*)(b_src[i] + (size_t)k0 * ldb_b);
+                if (k0 + b_krow[i] < g.K) v = *(const halfx8*)(b_base + b_voff[i]);
                 *(halfx8*)(st + A_STAGE_BYTES + (wave * B_LOADS + i) * 1024 + lane * 16) = v;
             }
         }
