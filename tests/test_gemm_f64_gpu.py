@@ -69,6 +69,15 @@ def test_every_k_remainder(hip, oracle, K, tile):
     assert rel_err(run(hip, A, B, tile=tile), oracle.gemm_f64(A, B), K) <= TOL
 
 
+def test_row_pitch_of_16_mib_takes_the_plain_kernel(hip, oracle):
+    """256 rows of a 16 MiB pitch overflow the 32-bit lane offsets of the direct-load kernels: such
+    operands run on the plain kernel, bit-exact to the oracle's chain."""
+    M, N, K = 3, 40, 72
+    A = synth.uniform_f64(M, K, 931); B = synth.uniform_f64(K, N, 932)
+    got = run(hip, A, B, pitches=((1 << 21) + 64, 48, 48, 48))
+    assert np.array_equal(got.view(np.uint64), oracle.gemm_f64(A, B).view(np.uint64))
+
+
 def test_plain_kernel_is_the_oracle_chain(hip, oracle):
     """Unaligned operands (and K == 0) take the one-thread-per-element kernel: the oracle's own k-ascending fma chain."""
     M, N, K = 70, 90, 50

@@ -231,6 +231,23 @@ def test_unaligned_pitches_and_bases(hip, oracle, dtype):
         assert rel_err(got, ref, K) <= tol
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_row_pitch_of_16_mib_takes_the_register_staged_kernels(hip, oracle, dtype):
+    """The direct-load kernels address a tile with 32-bit lane offsets, which 256 rows of a 16 MiB
+    pitch overflow: such operands must be routed to the kernels with full 64-bit addresses."""
+    M, N, K = 3, 40, 72
+    pitch_a = (1 << 24) // np.dtype(dtype).itemsize + 64
+    if dtype == np.float32:
+        A = synth.uniform_f32(M, K, 141); B = synth.uniform_f32(K, N, 142)
+        ref = oracle.gemm_f32(A, B); tol = TOL_F32
+    else:
+        A = synth.normal_half(M, K, 141); B = synth.normal_half(K, N, 142)
+        ref = oracle.gemm_f16(A, B); tol = TOL_F16
+    pn = device_pitch(N, dtype)
+    for tile in (0, 2):
+        assert rel_err(run(hip, A, B, tile=tile, pitches=(pitch_a, pn, pn, pn)), ref, K) <= tol
+
+
 @pytest.mark.parametrize("tile", [0, 1, 2])
 def test_forced_edge_variant_equals_fast_variant(hip, tile):
     """On tile-multiple shapes the predicated kernel and the unpredicated one run the same
