@@ -192,6 +192,25 @@ def cpu_baseline(name, A, B):
             "bit_equal_to_fma_chain": same}
 
 
+def api_wall_time(name, repeats=10):
+    """End-to-end wall time of de::blas::cuda::GEMM(GPU_Matrix x 3) (the reference's entry point,
+    srcs/modules/BLAS/GEMM/CUDA/GEMM_LS.cu:315-350) for the workload, stream set-up, launch and the
+    completion wait included, measured by the C++ driver of the de:: API in a process of its own."""
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "cpp", "de_api_test")
+    dtype, M, N, K = WORKLOADS[name][:4]
+    if not os.path.exists(exe) or dtype not in ("f32", "f16"):
+        return None
+    out = subprocess.run([exe, "gemmtime", dtype, str(M), str(N), str(K), str(repeats)], capture_output=True, text=True, timeout=300)
+    for l in out.stdout.splitlines():
+        if l.startswith("gemmtime"):
+            f = l.split()
+            med, best = float(f[2]), float(f[4])
+            return {"entry": "de::blas::cuda::GEMM(GPU_Matrix, GPU_Matrix, GPU_Matrix)", "median_ms": med, "min_ms": best,
+                    "calls": int(f[6]), "tflops_at_median": round(2.0 * M * N * K / med / 1e9, 2)}
+    return {"error": (out.stderr or out.stdout)[-200:]}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -203,6 +222,9 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this GEMM path runs on one GPU; --gpus %d is not supported (use --gpus 1)" % args.gpus)
+
+    # the de:: API's own wall time, before this process takes the GPU
+    api = api_wall_time(args.workload) if (args.workload in WORKLOADS and not args.no_extra) else None
 
     from decx_amd import hip
     hip.init(0)
@@ -242,6 +264,8 @@ def main():
         "wall_ms_per_step": main_out["wall_ms_per_step"],
         "roofline": main_out["roofline"],
     }
+    if api is not None:
+        line["api_wall"] = api
     if not args.no_extra:
         others = []
         for name in WORKLOADS:

@@ -470,7 +470,8 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
     }
     if (M == 1 && K > 0) {
         out->path = DECX_HIP_PATH_GEVM;
-        out->tile_m = 1; out->tile_n = f16 ? 64 : 32;
+        out->tile_m = 1; out->tile_n = f16 ? 64 : 32;               // 128 bytes of a row, or 64 when that leaves CUs idle
+        if ((N + out->tile_n - 1) / out->tile_n < 256u) out->tile_n /= 2;
         out->grid = (N + out->tile_n - 1) / out->tile_n;
         return DECX_HIP_OK;
     }

@@ -20,7 +20,8 @@
 // gevm: a workgroup owns 128 bytes of columns (32 fp32 / 64 fp16); 8 lanes cover those with
 //   one 128-bit load each, the other lane bits and the 16 wavefronts stride over k
 //   (128 rows per sweep); partial sums meet in a shuffle over the row lanes and in LDS over
-//   the wavefronts.
+//   the wavefronts.  When that gives fewer workgroups than CUs, a workgroup owns 64 bytes
+//   (4 lanes, 256 rows per sweep) and the two workgroups sharing a cache line share an XCD.
 #include "gemm_common.hpp"
 
 namespace decx_hip {
@@ -128,19 +129,25 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
     }
 }
 
-template <typename T, typename TO>
+// CL lanes of 16 bytes cover a workgroup's columns (8: 128 bytes of a row, 4: 64 bytes), 64 / CL rows per wavefront.
+template <typename T, typename TO, int CL>
 __global__ void __launch_bounds__(GEMV_THREADS)
 gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restrict__ c, TO* __restrict__ y,
             uint32_t K, uint32_t N, uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy,
             float alpha, float beta, uint32_t vec_ok)
 {
     constexpr int N16 = Per16<T>::n;
-    constexpr int CB = 8 * N16;                            // columns per workgroup (128 bytes of a row)
+    constexpr int CB = CL * N16;                           // columns per workgroup
+    constexpr int RL = 64 / CL;                            // rows per wavefront and sweep
     __shared__ __attribute__((aligned(16))) float xs[GEMV_KC];
     __shared__ float red[GEMV_WAVES][CB];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int col_lane = lane & 7, row_lane = lane >> 3;   // 8 column groups x 8 rows per wavefront
-    const uint32_t n0 = blockIdx.x * CB + col_lane * N16;
+    const int col_lane = lane % CL, row_lane = lane / CL;
+    // Half-line column groups: the two workgroups that share every 128-byte line of B should share an L2,
+    // so blocks b and b + 8 (dealt to the same XCD) take adjacent groups.
+    uint32_t group = blockIdx.x;
+    if (CL == 4 && gridDim.x % 16 == 0) group = (group / 16) * 16 + (group % 8) * 2 + (group / 8) % 2;
+    const uint32_t n0 = group * CB + col_lane * N16;
     const bool whole = vec_ok && (n0 + N16 <= N);
     float acc[N16];
 #pragma unroll
@@ -153,7 +160,7 @@ gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restric
         __syncthreads();
         if (n0 < N) {
 #pragma unroll 2
-            for (uint32_t k = wave * 8 + row_lane; k < len; k += GEMV_WAVES * 8) {
+            for (uint32_t k = wave * RL + row_lane; k < len; k += GEMV_WAVES * RL) {
                 const T* p = B + (size_t)(kc + k) * ldb + n0;
                 const float xv = xs[k];
                 if (whole) {
@@ -172,6 +179,7 @@ gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restric
 #pragma unroll
     for (int e = 0; e < N16; ++e) {
         float v = acc[e];
+        if (CL == 4) v += __shfl_xor(v, 4, 64);
         v += __shfl_xor(v, 8, 64);
         v += __shfl_xor(v, 16, 64);
         v += __shfl_xor(v, 32, 64);
@@ -179,7 +187,7 @@ gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restric
     }
     __syncthreads();
     if (t < CB) {
-        const uint32_t n = blockIdx.x * CB + t;
+        const uint32_t n = group * CB + t;
         if (n < N) {
             float o = 0.f;
 #pragma unroll
@@ -216,23 +224,32 @@ int launch_gemv(bool f16, bool out_f32, const void* A, const void* x, const void
     return (int)hipGetLastError();
 }
 
+namespace {
+
+template <typename T, typename TO>
+void launch_gevm_as(const void* x, const void* B, const void* c, void* y, uint32_t K, uint32_t N, uint32_t ldb,
+                    uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream)
+{
+    // 128-byte column groups unless they leave CUs without a workgroup (fp16 at N = 8192: 128 groups for
+    // 256 CUs); then 64-byte groups, two workgroups per cache line
+    const uint32_t cb8 = 8u * Per16<T>::n;
+    const uint32_t vec = rows_vectorisable<T>(B, ldb);
+    if ((N + cb8 - 1) / cb8 >= 256u)
+        hipLaunchKernelGGL((gevm_kernel<T, TO, 8>), dim3((N + cb8 - 1) / cb8), dim3(GEMV_THREADS), 0, stream, (const T*)x,
+                           (const T*)B, (const T*)c, (TO*)y, K, N, ldb, incx, incc, incy, alpha, beta, vec);
+    else
+        hipLaunchKernelGGL((gevm_kernel<T, TO, 4>), dim3((N + cb8 / 2 - 1) / (cb8 / 2)), dim3(GEMV_THREADS), 0, stream,
+                           (const T*)x, (const T*)B, (const T*)c, (TO*)y, K, N, ldb, incx, incc, incy, alpha, beta, vec);
+}
+
+}  // namespace
+
 int launch_gevm(bool f16, bool out_f32, const void* x, const void* B, const void* c, void* y, uint32_t K, uint32_t N,
                 uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream)
 {
-    const uint32_t cb = f16 ? 64u : 32u;
-    const dim3 grid((N + cb - 1) / cb), block(GEMV_THREADS);
-    if (!f16)
-        hipLaunchKernelGGL((gevm_kernel<float, float>), grid, block, 0, stream, (const float*)x, (const float*)B,
-                           (const float*)c, (float*)y, K, N, ldb, incx, incc, incy, alpha, beta,
-                           rows_vectorisable<float>(B, ldb));
-    else if (out_f32)
-        hipLaunchKernelGGL((gevm_kernel<_Float16, float>), grid, block, 0, stream, (const _Float16*)x,
-                           (const _Float16*)B, (const _Float16*)c, (float*)y, K, N, ldb, incx, incc, incy, alpha, beta,
-                           rows_vectorisable<_Float16>(B, ldb));
-    else
-        hipLaunchKernelGGL((gevm_kernel<_Float16, _Float16>), grid, block, 0, stream, (const _Float16*)x,
-                           (const _Float16*)B, (const _Float16*)c, (_Float16*)y, K, N, ldb, incx, incc, incy, alpha,
-                           beta, rows_vectorisable<_Float16>(B, ldb));
+    if (!f16) launch_gevm_as<float, float>(x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream);
+    else if (out_f32) launch_gevm_as<_Float16, float>(x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream);
+    else launch_gevm_as<_Float16, _Float16>(x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream);
     return (int)hipGetLastError();
 }
 

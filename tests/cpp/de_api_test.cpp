@@ -19,6 +19,7 @@
 //                                         vector forms of GEMM
 #include "DECX.h"
 
+#include <algorithm>
 #include <chrono>
 #include <cmath>
 #include <cstdlib>
@@ -570,6 +571,39 @@ template <typename T> static int hostgemm_files(const std::string& dir, de::_DAT
     return out ? 0 : 2;
 }
 
+template <typename T> static T from_float(float v) { return (T)v; }
+template <> de::Half from_float<de::Half>(float v) { return de::Float2Half(v); }
+
+// Wall time of de::blas::cuda::GEMM(GPU_Matrix x 3) as a caller sees it (the call returns when dst is complete).
+template <typename T> static int gemm_wall_time(de::_DATA_TYPES_FLAGS_ ty, uint32_t M, uint32_t N, uint32_t K, int repeats)
+{
+    de::InitCuda();
+    de::ResetLastError();
+    de::Matrix& A = de::CreateMatrixRef(ty, K, M);
+    de::Matrix& B = de::CreateMatrixRef(ty, N, K);
+    uint64_t state = 0x9E3779B97F4A7C15ull;                               // any non-constant data will do
+    auto next = [&]() { state = state * 6364136223846793005ull + 1442695040888963407ull; return (float)((state >> 40) & 0xFFFF) / 32768.f - 1.f; };
+    for (uint32_t i = 0; i < M; ++i) for (uint32_t k = 0; k < K; ++k) *A.ptr<T>(i, k) = from_float<T>(next());
+    for (uint32_t k = 0; k < K; ++k) for (uint32_t j = 0; j < N; ++j) *B.ptr<T>(k, j) = from_float<T>(next());
+    de::GPU_Matrix& dA = de::CreateGPUMatrixRef(ty, K, M);
+    de::GPU_Matrix& dB = de::CreateGPUMatrixRef(ty, N, K);
+    de::GPU_Matrix& dD = de::CreateGPUMatrixRef();
+    if (de::Memcpy(A, dA, de::Point2D(0, 0), de::Point2D(0, 0), de::Point2D(K, M), de::DECX_MEMCPY_H2D).error_type) return 3;
+    if (de::Memcpy(B, dB, de::Point2D(0, 0), de::Point2D(0, 0), de::Point2D(N, K), de::DECX_MEMCPY_H2D).error_type) return 3;
+    std::vector<double> ms;
+    const auto begin = std::chrono::steady_clock::now();
+    for (int r = 0; r < repeats + 3 || std::chrono::duration<double>(std::chrono::steady_clock::now() - begin).count() < 0.3; ++r) {
+        const auto t0 = std::chrono::steady_clock::now();
+        de::blas::cuda::GEMM(dA, dB, dD);
+        ms.push_back(std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count());
+        if (de::GetLastError()->error_type != 0) { std::cerr << de::GetLastError()->error_string << "\n"; return 3; }
+    }
+    std::vector<double> last(ms.end() - repeats, ms.end());               // what came before is warm-up
+    std::sort(last.begin(), last.end());
+    std::cout << "gemmtime median_ms " << last[last.size() / 2] << " min_ms " << last.front() << " calls " << last.size() << "\n";
+    return (dD.Width() == N && dD.Height() == M) ? 0 : 4;
+}
+
 int main(int argc, char** argv)
 {
     const std::string mode = argc > 1 ? argv[1] : "host";
@@ -584,6 +618,12 @@ int main(int argc, char** argv)
         rc = f16 ? hostgemm_files<de::Half>(argv[2], de::_FP16_, M, N, K, with_c, pinned, repeats)
                  : std::string(argv[3]) == "f64" ? hostgemm_files<double>(argv[2], de::_FP64_, M, N, K, with_c, pinned, repeats)
                  : hostgemm_files<float>(argv[2], de::_FP32_, M, N, K, with_c, pinned, repeats);
+    }
+    else if (mode == "gemmtime" && argc == 7) {
+        const uint32_t M = std::atoi(argv[3]), N = std::atoi(argv[4]), K = std::atoi(argv[5]);
+        const int repeats = std::max(1, std::atoi(argv[6]));
+        rc = std::string(argv[2]) == "f16" ? gemm_wall_time<de::Half>(de::_FP16_, M, N, K, repeats)
+                                           : gemm_wall_time<float>(de::_FP32_, M, N, K, repeats);
     }
     else if (mode == "tensor_host") rc = tensor_host_checks();
     else if (mode == "conv" && argc == 12)
@@ -607,7 +647,7 @@ int main(int argc, char** argv)
                  : gemm_files<float>(argv[2], de::_FP32_, M, N, K, with_c, alpha, beta);
     } else {
         std::cerr << "usage: de_api_test host | gpu | vector_host | vector_gpu | gemm <dir> <f32|f16> M N K withC alpha beta"
-                     " | vmm <dir> <f32|f16> <mv|vm> W H level\n";
+                     " | vmm <dir> <f32|f16> <mv|vm> W H level | gemmtime <f32|f16> M N K repeats\n";
         return 64;
     }
     std::cout << (rc == 0 ? "de_api_test: all checks passed" : "de_api_test: FAILED") << " (" << mode << ")\n";

@@ -76,7 +76,8 @@ def test_planner_choices():
         p = hip.plan(eb, 8192, 1, 8192)
         assert (p.path, p.grid) == (hip.PATH_GEMV, 8192 // 32)
         p = hip.plan(eb, 1, 8192, 8192)
-        assert (p.path, p.grid) == (hip.PATH_GEVM, 8192 // (128 // eb))
+        assert (p.path, p.grid) == (hip.PATH_GEVM, 256)    # 128-byte column groups in fp32, 64-byte ones in fp16: 256 either way
+    assert hip.plan(2, 1, 32768, 64).tile_n == 64 and hip.plan(4, 1, 4096, 64).tile_n == 16
     assert hip.plan(4, 0, 5, 5).grid == 0
     bad = hip.Plan()
     assert hip.lib().decx_hip_gemm_plan(3, 4, 4, 4, 1, ctypes.byref(bad)) == -1
