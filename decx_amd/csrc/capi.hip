@@ -22,9 +22,8 @@ inline hipStream_t as_stream(void* s) { return (hipStream_t)s; }
 
 inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
-// Picks the block tile: cost = (tiles the busiest CU runs) x (tile area) / (relative speed
-// of that shape).  Big tiles win once they fill the chip; small tiles win while the grid
-// would otherwise leave CUs idle.  Ties go to the larger tile.
+// Picks the block tile by the time estimate of tile_cost().  Big tiles win once they fill the chip;
+// small tiles win while the grid would otherwise leave CUs idle.  Ties go to the larger tile.
 int choose_tile_f64(uint32_t M, uint32_t N)
 {
     int best = TILE_64x64;
@@ -32,8 +31,7 @@ int choose_tile_f64(uint32_t M, uint32_t N)
     for (int s = TILE_COUNT - 1; s >= 0; --s) {
         const TileInfo ti = tile_info_f64(s);
         const uint64_t tiles = (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
-        const uint64_t per_cu = (tiles + g_dev.compute_units - 1) / g_dev.compute_units;
-        const double cost = (double)per_cu * ti.bm * ti.bn / ti.rel_speed;
+        const double cost = tile_cost(ti, tiles, g_dev.compute_units);
         if (cost <= best_cost) { best_cost = cost; best = s; }
     }
     return best;
@@ -46,8 +44,7 @@ int choose_tile(bool f16, uint32_t M, uint32_t N, bool aligned)
     for (int s = TILE_COUNT - 1; s >= 0; --s) {
         const TileInfo ti = f16 ? tile_info_f16(s, aligned) : tile_info_f32(s, aligned);
         const uint64_t tiles = (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
-        const uint64_t per_cu = (tiles + g_dev.compute_units - 1) / g_dev.compute_units;
-        const double cost = (double)per_cu * ti.bm * ti.bn / ti.rel_speed;
+        const double cost = tile_cost(ti, tiles, g_dev.compute_units);
         if (cost <= best_cost) { best_cost = cost; best = s; }
     }
     return best;

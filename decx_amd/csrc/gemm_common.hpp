@@ -71,38 +71,63 @@ enum TileShape : int {
     TILE_COUNT   = 3,
 };
 
-struct TileInfo { int bm, bn, threads; float rel_speed; };
+// per_cu: workgroups of the shape that share a CU.  full: throughput of a CU filled with them, alone: of a
+// workgroup that has its CU to itself (or, for the largest tile, of a chip no more than half occupied: fp16
+// runs under the power cap, so a CU does more when its neighbours idle), both relative to the largest tile on
+// a full chip.  Smaller tiles fetch more operand bytes per flop.
+struct TileInfo { int bm, bn, threads, per_cu; float full, alone; };
 
-// rel_speed: per-CU throughput of the shape relative to the largest one once the chip is
-// full (smaller tiles fetch more operand bytes per flop).  fp32, measured on MI355X at 2048^3 /
-// 3000^3: direct-to-LDS kernels 144 : 129 : 121 TFLOP/s, predicated register-staged kernels
-// (operands that are not 16-byte aligned) about 1 : 0.8 : 0.7.
+// Time (in units of tile area over rate) of `tiles` workgroups on `cus` CUs: whole rounds of cus * per_cu
+// workgroups at the full rate, then the remainder, which runs at the lone-workgroup rate when it leaves each
+// of its CUs one workgroup.
+__host__ inline double tile_cost(const TileInfo& ti, uint64_t tiles, uint32_t cus)
+{
+    const double area = (double)ti.bm * ti.bn;
+    const uint64_t slots = (uint64_t)cus * ti.per_cu;
+    const uint64_t rounds = tiles / slots, rest = tiles % slots;
+    double t = (double)rounds * ti.per_cu * area / ti.full;
+    if (rest > 0) {
+        if (rest <= cus) {
+            double rate = ti.alone;
+            if (ti.per_cu == 1 && rest > cus / 2)          // between half and all CUs busy: towards the full-chip rate
+                rate += (ti.full - ti.alone) * (double)(rest - cus / 2) / (double)(cus - cus / 2);
+            t += area / rate;
+        } else {
+            t += (double)((rest + cus - 1) / cus) * area / ti.full;
+        }
+    }
+    return t;
+}
+
+// fp32, measured on MI355X (TFLOP/s per CU, direct-to-LDS kernels): 256 x 256 0.578 alone or full; 128 x 128
+// 0.52 alone (2048^3), 0.575 two per CU (4096^3); 64 x 64 0.37 alone (1024^3), 0.51-0.53 full (2048^3, 4096^3).  The
+// predicated register-staged kernels (operands that are not 16-byte aligned) run at about 1 : 0.8 : 0.7 of that.
 __host__ inline TileInfo tile_info_f32(int shape, bool aligned = true)
 {
     switch (shape) {
-    case TILE_256x256: return {256, 256, 512, 1.00f};
-    case TILE_128x128: return {128, 128, 256, aligned ? 0.90f : 0.80f};
-    default:           return { 64,  64, 256, aligned ? 0.85f : 0.70f};
+    case TILE_256x256: return {256, 256, 512, 1, 1.00f, 1.00f};
+    case TILE_128x128: return {128, 128, 256, 2, aligned ? 0.99f : 0.80f, aligned ? 0.90f : 0.72f};
+    default:           return { 64,  64, 256, 2, aligned ? 0.90f : 0.70f, aligned ? 0.64f : 0.49f};
     }
 }
-// fp16, measured at 4096^3: direct-to-LDS kernels 1177 : 918 : 600 TFLOP/s; the predicated register-staged
-// kernels about 1 : 0.6 : 0.25.
+// fp16 (TFLOP/s per CU): 256 x 256 4.64 on a full chip, 6.4 with at most half the CUs busy; 128 x 128 3.1 alone,
+// 3.6 two per CU; 64 x 64 1.27 alone, 2.66 full.  Predicated register-staged kernels about 1 : 0.6 : 0.25.
 __host__ inline TileInfo tile_info_f16(int shape, bool aligned = true)
 {
     switch (shape) {
-    case TILE_256x256: return {256, 256, aligned ? 512 : 256, 1.00f};
-    case TILE_128x128: return {128, 128, aligned ? 256 : 128, aligned ? 0.78f : 0.60f};
-    default:           return { 64,  64, aligned ? 256 :  64, aligned ? 0.50f : 0.25f};
+    case TILE_256x256: return {256, 256, aligned ? 512 : 256, 1, 1.00f, aligned ? 1.38f : 1.00f};
+    case TILE_128x128: return {128, 128, aligned ? 256 : 128, 2, aligned ? 0.78f : 0.60f, aligned ? 0.67f : 0.50f};
+    default:           return { 64,  64, aligned ? 256 :  64, 2, aligned ? 0.57f : 0.25f, aligned ? 0.27f : 0.12f};
     }
 }
 
-// fp64, measured at 4096^3: 69.8 : 59.6 : 60.0 TFLOP/s.  TILE_256x256 stands for the largest fp64 tile, 256 x 128.
+// fp64, measured at 4096^3: 72.5 : 59.6 : 60.0 TFLOP/s.  TILE_256x256 stands for the largest fp64 tile, 256 x 128.
 __host__ inline TileInfo tile_info_f64(int shape)
 {
     switch (shape) {
-    case TILE_256x256: return {256, 128, 512, 1.00f};
-    case TILE_128x128: return {128, 128, 256, 0.85f};
-    default:           return { 64,  64, 256, 0.85f};
+    case TILE_256x256: return {256, 128, 512, 1, 1.00f, 1.00f};
+    case TILE_128x128: return {128, 128, 256, 2, 0.83f, 0.75f};
+    default:           return { 64,  64, 256, 2, 0.83f, 0.60f};
     }
 }
 
