@@ -71,15 +71,16 @@ enum TileShape : int {
     TILE_COUNT   = 3,
 };
 
-// per_cu: workgroups of the shape that share a CU.  full: throughput of a CU filled with them, alone: of a
-// workgroup that has its CU to itself (or, for the largest tile, of a chip no more than half occupied: fp16
+// per_cu: workgroups of the shape that fit a CU together.  full: throughput of a CU filled with them, alone: of
+// a workgroup that has its CU to itself (or, for the largest tile, of a chip no more than half occupied: fp16
 // runs under the power cap, so a CU does more when its neighbours idle), both relative to the largest tile on
-// a full chip.  Smaller tiles fetch more operand bytes per flop.
+// a full chip.  Smaller tiles fetch more operand bytes per flop and lean on co-resident workgroups to hide the
+// latency of their copies.
 struct TileInfo { int bm, bn, threads, per_cu; float full, alone; };
 
 // Time (in units of tile area over rate) of `tiles` workgroups on `cus` CUs: whole rounds of cus * per_cu
-// workgroups at the full rate, then the remainder, which runs at the lone-workgroup rate when it leaves each
-// of its CUs one workgroup.
+// workgroups at the full rate, then the remainder, whose busiest CU holds m workgroups and runs at a rate
+// between the lone-workgroup one (m = 1) and the full one (m = per_cu).
 __host__ inline double tile_cost(const TileInfo& ti, uint64_t tiles, uint32_t cus)
 {
     const double area = (double)ti.bm * ti.bn;
@@ -87,27 +88,26 @@ __host__ inline double tile_cost(const TileInfo& ti, uint64_t tiles, uint32_t cu
     const uint64_t rounds = tiles / slots, rest = tiles % slots;
     double t = (double)rounds * ti.per_cu * area / ti.full;
     if (rest > 0) {
-        if (rest <= cus) {
-            double rate = ti.alone;
-            if (ti.per_cu == 1 && rest > cus / 2)          // between half and all CUs busy: towards the full-chip rate
-                rate += (ti.full - ti.alone) * (double)(rest - cus / 2) / (double)(cus - cus / 2);
-            t += area / rate;
-        } else {
-            t += (double)((rest + cus - 1) / cus) * area / ti.full;
-        }
+        const uint64_t m = (rest + cus - 1) / cus;
+        double rate = ti.alone;
+        if (ti.per_cu > 1) rate += (ti.full - ti.alone) * (double)(m - 1) / (double)(ti.per_cu - 1);
+        else if (rest > cus / 2)                           // between half and all CUs busy: towards the full-chip rate
+            rate += (ti.full - ti.alone) * (double)(rest - cus / 2) / (double)(cus - cus / 2);
+        t += (double)m * area / rate;
     }
     return t;
 }
 
 // fp32, measured on MI355X (TFLOP/s per CU, direct-to-LDS kernels): 256 x 256 0.578 alone or full; 128 x 128
-// 0.52 alone (2048^3), 0.575 two per CU (4096^3); 64 x 64 0.37 alone (1024^3), 0.51-0.53 full (2048^3, 4096^3).  The
-// predicated register-staged kernels (operands that are not 16-byte aligned) run at about 1 : 0.8 : 0.7 of that.
+// 0.52 alone (2048^3), 0.58 four per CU (4096^3, 6144^3); 64 x 64 0.39 alone (1024^3), 0.54 five per CU (3072^3,
+// 4096^3).  The predicated register-staged kernels (operands that are not 16-byte aligned) run at about
+// 1 : 0.8 : 0.7 of the largest tile, two workgroups per CU.
 __host__ inline TileInfo tile_info_f32(int shape, bool aligned = true)
 {
     switch (shape) {
     case TILE_256x256: return {256, 256, 512, 1, 1.00f, 1.00f};
-    case TILE_128x128: return {128, 128, 256, 2, aligned ? 0.99f : 0.80f, aligned ? 0.90f : 0.72f};
-    default:           return { 64,  64, 256, 2, aligned ? 0.90f : 0.70f, aligned ? 0.64f : 0.49f};
+    case TILE_128x128: return {128, 128, 256, aligned ? 4 : 2, aligned ? 1.00f : 0.80f, aligned ? 0.895f : 0.72f};
+    default:           return { 64,  64, 256, aligned ? 5 : 2, aligned ? 0.94f : 0.70f, aligned ? 0.675f : 0.49f};
     }
 }
 // fp16 (TFLOP/s per CU): 256 x 256 4.64 on a full chip, 6.4 with at most half the CUs busy; 128 x 128 3.1 alone,

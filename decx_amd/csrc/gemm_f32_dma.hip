@@ -440,19 +440,20 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
 
 }  // namespace
 
-// M, N, K >= 1; 16-byte aligned bases and pitches (the caller checks).  Measured on MI355X: the
-// 64 x 64 tile runs best with 32-deep slabs in a 4-stage ring (two workgroups per CU) and
-// chunk-ahead fragments; deeper rings and a second accumulator chain changed nothing, its ceiling
-// is the L2 -> LDS rate (16 flop per byte fetched).  The 128 x 128 tile measures the same with 4 or
-// 8 wavefronts and 16- or 32-deep slabs.  The 256 x 256 tile: 8 wavefronts of 128 x 64 reach 144 TFLOP/s
-// at 8192^3; 64 x 128 wave tiles, 16 wavefronts, 32-deep slabs and rings of 3 to 5 stages all land
-// between 138 and 144.
+// M, N, K >= 1; 16-byte aligned bases and pitches (the caller checks).  Measured on MI355X:
+//   256 x 256: 8 wavefronts of 128 x 64, 16-deep slabs in a ring of 4 (one workgroup per CU): 148 TFLOP/s at 8192^3;
+//     64 x 128 wave tiles, 16 wavefronts, 32-deep slabs and rings of 3 to 5 stages land between 138 and 144.
+//   128 x 128 and 64 x 64: 4 wavefronts, chunk-ahead fragments, and a ring of only 2 stages (32 KB): what hides the
+//     copy latency for these is not a deep ring but several workgroups per CU (4 and 5 fit), e.g. 128 x 128 at
+//     6144^3 147 TFLOP/s against 130 with 4 stages, 64 x 64 at 3072^3 139 against 127; with a single workgroup per CU
+//     (1024^3) both rings measure the same.  Deeper rings, 64-deep slabs, a second accumulator chain and splitting K
+//     over two wavefront groups changed nothing or lost.
 int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
 {
     switch (shape) {
     case TILE_256x256: return launch_dma<256, 256, 2, 4, 16, 4, false>(args, stream);
-    case TILE_128x128: return launch_dma<128, 128, 2, 2, 16, 4, true>(args, stream);
-    case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 32, 4, true>(args, stream);
+    case TILE_128x128: return launch_dma<128, 128, 2, 2, 16, 2, true>(args, stream);
+    case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 32, 2, true>(args, stream);
     default:           return (int)hipErrorInvalidValue;
     }
 }
@@ -464,8 +465,8 @@ int launch_conv2d_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
 {
     switch (shape) {
     case TILE_256x256: return launch_dma<256, 256, 2, 4, 16, 4, false, true>(args, stream);
-    case TILE_128x128: return launch_dma<128, 128, 2, 2, 16, 4, true, true>(args, stream);
-    case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 32, 4, true, true>(args, stream);
+    case TILE_128x128: return launch_dma<128, 128, 2, 2, 16, 2, true, true>(args, stream);
+    case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 32, 2, true, true>(args, stream);
     default:           return (int)hipErrorInvalidValue;
     }
 }
