@@ -111,13 +111,13 @@ __host__ inline TileInfo tile_info_f32(int shape, bool aligned = true)
     }
 }
 // fp16 (TFLOP/s per CU): 256 x 256 4.64 on a full chip, 6.4 with at most half the CUs busy; 128 x 128 3.1 alone,
-// 3.6 two per CU; 64 x 64 1.27 alone, 2.66 full.  Predicated register-staged kernels about 1 : 0.6 : 0.25.
+// 3.9 two per CU; 64 x 64 1.27 alone, 2.4 four per CU.  Predicated register-staged kernels about 1 : 0.6 : 0.25.
 __host__ inline TileInfo tile_info_f16(int shape, bool aligned = true)
 {
     switch (shape) {
     case TILE_256x256: return {256, 256, aligned ? 512 : 256, 1, 1.00f, aligned ? 1.38f : 1.00f};
-    case TILE_128x128: return {128, 128, aligned ? 256 : 128, 2, aligned ? 0.78f : 0.60f, aligned ? 0.67f : 0.50f};
-    default:           return { 64,  64, aligned ? 256 :  64, 2, aligned ? 0.57f : 0.25f, aligned ? 0.27f : 0.12f};
+    case TILE_128x128: return {128, 128, aligned ? 256 : 128, 2, aligned ? 0.84f : 0.60f, aligned ? 0.67f : 0.50f};
+    default:           return { 64,  64, aligned ? 256 :  64, aligned ? 4 : 2, aligned ? 0.55f : 0.25f, aligned ? 0.27f : 0.12f};
     }
 }
 

@@ -356,9 +356,11 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
 //     8192^3); 4 wavefronts of 128 x 128 reach 1075-1124, 16 wavefronts 1144, 32-deep slabs 1100-1124.
 //     Two wavefronts per SIMD take turns on the matrix pipe while the other waits for LDS or the barrier.
 //     Spreading the direct loads over the k steps, or raising the wave priority around the MFMAs, is 3-4 % slower.
-//   128 x 128: 4 wavefronts of 64 x 64; 64-deep slabs in 4 stages when there is at most one workgroup
-//     per CU (751 TFLOP/s at 2048^3), else 32-deep so that two workgroups share a CU (640 at 3000^3).
-//   64 x 64: 4 wavefronts of 32 x 32, 64-deep slabs in 4 stages (287 TFLOP/s at 1024^3).
+//   128 x 128: 4 wavefronts of 64 x 64, 64-deep slabs; a ring of 4 stages when there is at most one workgroup
+//     per CU (741 TFLOP/s at 2048^3), else of 2 stages so that two workgroups share a CU (4096^3: 994 against
+//     940 with 32-deep slabs in 4 stages, 6144^3: 1035 against 960).
+//   64 x 64: 4 wavefronts of 32 x 32, 64-deep slabs in 4 stages (327 TFLOP/s at 1024^3), in 2 stages once more
+//     than two workgroups per CU are there to hide the copies (1536^3: 447 against 388).
 int launch_gemm_f16_dma(int shape, const GemmArgs& args, hipStream_t stream)
 {
     switch (shape) {
@@ -366,9 +368,13 @@ int launch_gemm_f16_dma(int shape, const GemmArgs& args, hipStream_t stream)
     case TILE_128x128: {
         const uint64_t blocks = (uint64_t)((args.M + 127) / 128) * ((args.N + 127) / 128);
         return blocks <= 256 ? launch_dma<128, 128, 2, 2, 64, 4>(args, stream)
-                             : launch_dma<128, 128, 2, 2, 32, 4>(args, stream);
+                             : launch_dma<128, 128, 2, 2, 64, 2>(args, stream);
     }
-    case TILE_64x64:   return launch_dma<64, 64, 2, 2, 64, 4>(args, stream);
+    case TILE_64x64: {
+        const uint64_t blocks = (uint64_t)((args.M + 63) / 64) * ((args.N + 63) / 64);
+        return blocks <= 512 ? launch_dma<64, 64, 2, 2, 64, 4>(args, stream)
+                             : launch_dma<64, 64, 2, 2, 64, 2>(args, stream);
+    }
     default:           return (int)hipErrorInvalidValue;
     }
 }

@@ -335,7 +335,7 @@ int launch_gemm_f64(int shape, bool plain, const GemmArgs& args, hipStream_t str
     switch (shape) {
     case TILE_256x256: return launch_dma<256, 128, 4, 2, 16, 3>(args, stream);
     case TILE_128x128: return launch_dma<128, 128, 2, 2, 16, 3>(args, stream);
-    case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 16, 4>(args, stream);
+    case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 16, 3>(args, stream);
     default:           return (int)hipErrorInvalidValue;
     }
 }
