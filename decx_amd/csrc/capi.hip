@@ -473,7 +473,7 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
         return DECX_HIP_OK;
     }
     const int shape = choose_tile(f16, M, N, aligned != 0);
-    const TileInfo ti = f16 ? tile_info_f16(shape) : tile_info_f32(shape);
+    const TileInfo ti = f16 ? tile_info_f16(shape, aligned != 0) : tile_info_f32(shape, aligned != 0);
     out->path = shape;
     out->tile_m = ti.bm; out->tile_n = ti.bn;
     out->grid = ((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);

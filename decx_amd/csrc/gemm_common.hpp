@@ -98,16 +98,17 @@ __host__ inline double tile_cost(const TileInfo& ti, uint64_t tiles, uint32_t cu
     return t;
 }
 
-// fp32, measured on MI355X (TFLOP/s per CU, direct-to-LDS kernels): 256 x 256 0.578 alone or full; 128 x 128
-// 0.52 alone (2048^3), 0.58 four per CU (4096^3, 6144^3); 64 x 64 0.39 alone (1024^3), 0.54 five per CU (3072^3,
+// fp32, measured on MI355X (TFLOP/s per CU, direct-to-LDS kernels): 256 x 128 (the largest tile; 256 x 256 in the
+// register-staged family) 0.56 alone, 0.586 two per CU; 128 x 128
+// 0.52 alone (2048^3), 0.586 four per CU (4096^3, 6144^3); 64 x 64 0.39 alone (1024^3), 0.56 five per CU (3072^3,
 // 4096^3).  The predicated register-staged kernels (operands that are not 16-byte aligned) run at about
 // 1 : 0.8 : 0.7 of the largest tile, two workgroups per CU.
 __host__ inline TileInfo tile_info_f32(int shape, bool aligned = true)
 {
     switch (shape) {
-    case TILE_256x256: return {256, 256, 512, 1, 1.00f, 1.00f};
-    case TILE_128x128: return {128, 128, 256, aligned ? 4 : 2, aligned ? 1.00f : 0.80f, aligned ? 0.895f : 0.72f};
-    default:           return { 64,  64, 256, aligned ? 5 : 2, aligned ? 0.94f : 0.70f, aligned ? 0.675f : 0.49f};
+    case TILE_256x256: return aligned ? TileInfo{256, 128, 256, 2, 1.00f, 0.95f} : TileInfo{256, 256, 512, 1, 1.00f, 1.00f};
+    case TILE_128x128: return {128, 128, 256, aligned ? 4 : 2, aligned ? 1.00f : 0.80f, aligned ? 0.88f : 0.72f};
+    default:           return { 64,  64, 256, aligned ? 5 : 2, aligned ? 0.96f : 0.70f, aligned ? 0.667f : 0.49f};
     }
 }
 // fp16 (TFLOP/s per CU): 256 x 256 4.64 on a full chip, 6.4 with at most half the CUs busy; 128 x 128 3.1 alone,

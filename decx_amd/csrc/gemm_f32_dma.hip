@@ -441,8 +441,11 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
 }  // namespace
 
 // M, N, K >= 1; 16-byte aligned bases and pitches (the caller checks).  Measured on MI355X:
-//   256 x 256: 8 wavefronts of 128 x 64, 16-deep slabs in a ring of 4 (one workgroup per CU): 148 TFLOP/s at 8192^3;
-//     64 x 128 wave tiles, 16 wavefronts, 32-deep slabs and rings of 3 to 5 stages land between 138 and 144.
+//   256 x 128 (TILE_256x256, the largest tile): 4 wavefronts of 128 x 64, 16-deep slabs in a ring of 2, two workgroups
+//     per CU, each with its own slab barrier: 149.3 TFLOP/s at 8192^3.  One 256 x 256 workgroup of 8 such wavefronts
+//     per CU (ring of 4) reaches 147.7-148.4 and leaves more of the chip idle on grids that are no multiple of the
+//     CU count (6144^3: 110 against 133); with 64 x 128 wave tiles, 16 wavefronts, 32-deep slabs or rings of 3 to
+//     5 stages it lands between 138 and 144.
 //   128 x 128 and 64 x 64: 4 wavefronts, chunk-ahead fragments, and a ring of only 2 stages (32 KB): what hides the
 //     copy latency for these is not a deep ring but several workgroups per CU (4 and 5 fit), e.g. 128 x 128 at
 //     6144^3 147 TFLOP/s against 130 with 4 stages, 64 x 64 at 3072^3 139 against 127; with a single workgroup per CU
@@ -451,7 +454,7 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
 int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
 {
     switch (shape) {
-    case TILE_256x256: return launch_dma<256, 256, 2, 4, 16, 4, false>(args, stream);
+    case TILE_256x256: return launch_dma<256, 128, 2, 2, 16, 2, false>(args, stream);
     case TILE_128x128: return launch_dma<128, 128, 2, 2, 16, 2, true>(args, stream);
     case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 32, 2, true>(args, stream);
     default:           return (int)hipErrorInvalidValue;
@@ -464,7 +467,7 @@ int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
 int launch_conv2d_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
 {
     switch (shape) {
-    case TILE_256x256: return launch_dma<256, 256, 2, 4, 16, 4, false, true>(args, stream);
+    case TILE_256x256: return launch_dma<256, 256, 2, 4, 16, 4, false, true>(args, stream);    // 134 TFLOP/s on the 3 x 3 x 112 workload; 256 x 128: 127
     case TILE_128x128: return launch_dma<128, 128, 2, 2, 16, 2, true, true>(args, stream);
     case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 32, 2, true, true>(args, stream);
     default:           return (int)hipErrorInvalidValue;

@@ -58,8 +58,10 @@ def test_planner_choices():
     # headline shapes take the big tile, the unpredicated variant
     for eb, (M, N, K) in [(4, (8192, 8192, 8192)), (2, (4096, 4096, 4096)), (4, (65536, 256, 1024))]:
         p = hip.plan(eb, M, N, K)
-        assert (p.path, p.edge, p.tile_m, p.tile_n) == (hip.TILE_256, 0, 256, 256)
-        assert p.grid == (M // 256) * (N // 256)
+        # the largest tile: 256 x 128 in fp32 (two workgroups per CU), 256 x 256 in fp16
+        assert (p.path, p.edge, p.tile_m, p.tile_n) == (hip.TILE_256, 0, 256, 128 if eb == 4 else 256)
+        assert p.grid == (M // p.tile_m) * (N // p.tile_n)
+    assert hip.plan(4, 8192, 8192, 8192, aligned=False).tile_n == 256     # the register-staged family keeps 256 x 256
     # small and ragged problems take smaller tiles so the chip fills; they stay on the direct-to-LDS
     # kernels as long as the operands are 16-byte aligned
     p = hip.plan(4, 1000, 1500, 777)
@@ -68,7 +70,8 @@ def test_planner_choices():
     assert hip.plan(2, 1000, 1500, 777).edge == 0 and hip.plan(2, 1000, 1500, 777).tile_m == 64
     assert hip.plan(2, 2048, 2048, 2048).tile_m == 128 and hip.plan(2, 1000, 1500, 777, aligned=False).edge == 1
     assert hip.plan(4, 1024, 1024, 1024).tile_m == 64
-    assert hip.plan(4, 2048, 2048, 2048).tile_m == 128
+    assert hip.plan(4, 2048, 2048, 2048).tile_m == 64      # 1024 small tiles, four or five to a CU, beat 256 lone 128 x 128 ones
+    assert hip.plan(4, 6144, 6144, 6144).tile_m == 128
     assert hip.plan(4, 3000, 3000, 3000).tile_m == 64
     assert hip.plan(4, 1024, 1024, 1024, aligned=False).edge == 1
     # N == 1 goes to the row-dot kernel and M == 1 to the column-sum kernel, in both element types
