@@ -47,7 +47,9 @@ typedef struct decx_hip_device_props {
     uint64_t global_mem_bytes;
 } decx_hip_device_props;
 
-/* Tile shapes the planner chooses between (block tile BM x BN). */
+/* Tile shapes the planner chooses between (block tile BM x BN).  DECX_HIP_TILE_256x256 is the largest tile of
+ * the element type: 256 x 256 in fp16, 256 x 128 in fp32 on 16-byte aligned operands (256 x 256 otherwise) and
+ * in fp64; decx_hip_gemm_plan reports the actual BM x BN. */
 enum {
     DECX_HIP_TILE_AUTO    = -1,
     DECX_HIP_TILE_256x256 = 0,
