@@ -15,16 +15,17 @@
 // alpha * acc) as the reference's F kernels do (GEMM_fp32_B128_kernels.cu:725-744).
 //
 // Data movement: `global_load_lds_dwordx4` writes LDS directly (no staging registers, no
-// ds_write), so the ring can be STAGES - 1 slabs deep and late loads are absorbed.  The direct
+// ds_write), so late loads are absorbed by the ring and by the other workgroups of the CU.  The direct
 // loads are inline assembly and the slab barrier is a bare `s_barrier` behind an explicit vmcnt
 // wait, because the compiler would otherwise wait for every outstanding load in front of each
 // LDS read and at each __syncthreads().  Fragment reads are pinned behind MFMAs with
 // `sched_group_barrier`; the MFMAs of the last k step of a slab are issued after the slab
 // barrier, behind the first fragment reads of the next slab.
-//   * tile shapes from 256 x 256 (eight wavefronts of 128 x 64) down to 64 x 64 (four
-//     wavefronts of 32 x 32), so that small problems still put a workgroup on every CU; wave
-//     tiles that small issue one MFMA per k step, less than an LDS read takes, so their
-//     fragments are fetched a whole 8-deep chunk ahead;
+//   * tile shapes from 256 x 128 (four wavefronts of 128 x 64, two workgroups per CU; the
+//     convolution keeps 256 x 256 with eight) down to 64 x 64 (four wavefronts of 32 x 32), so
+//     that small problems still put a workgroup on every CU; wave tiles that small issue one
+//     MFMA per k step, less than an LDS read takes, so their fragments are fetched a whole
+//     8-deep chunk ahead;
 //   * ragged M and N without predicated loads: a copy lane whose row or column chunk
 //     lies outside the matrix fetches the last valid row / chunk instead (always mapped
 //     memory); what it brings lands in accumulators of rows / columns that are never stored;
@@ -75,7 +76,7 @@ template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHU
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_f32_dma_kernel(const GemmArgs g)
 {
-    constexpr int WAVES = WAVES_M * WAVES_N, NT = WAVES * 64;
+    constexpr int WAVES = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
     constexpr int CPR = BK / 4, RP = 16 / CPR;                    // A chunks per row, rows per 256 bytes
     constexpr int CB = BN / 4, RB = 64 / CB;                      // B chunks per k row, k rows per direct load
