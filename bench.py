@@ -165,6 +165,44 @@ def run_conv(steps, warmup, settle_s=0.25):
     return out
 
 
+def run_complex(double, n, steps, warmup, settle_s=0.25):
+    """Complex GEMM D = A.B (interleaved re / im, n x n x n) through decx_hip_gemm_c32 / _c64 with a caller-held
+    workspace: one pass expanding B, then one real GEMM on the fp32 / fp64 matrix pipe.  8 real flops per complex
+    multiply-add; the expansion pass is inside the timed region."""
+    from decx_amd import hip, synth
+    L = hip.lib()
+    cdt, rb = (np.complex128, 8) if double else (np.complex64, 4)
+    draw = synth.uniform_f64 if double else synth.uniform_f32
+    a = (draw(n, n, 0xA008) + 1j * draw(n, n, 0xA009)).astype(cdt)
+    b = (draw(n, n, 0xB008) + 1j * draw(n, n, 0xB009)).astype(cdt)
+    dA = hip.DeviceMatrix(n, n, cdt, n, a); dB = hip.DeviceMatrix(n, n, cdt, n, b); dD = hip.DeviceMatrix(n, n, cdt, n)
+    need = L.decx_hip_gemm_complex_workspace(rb, n, n)
+    ws = hip.DeviceMatrix(1, need // 16, np.complex128)
+    fn = L.decx_hip_gemm_c64 if double else L.decx_hip_gemm_c32
+    call = lambda: hip.check(fn(dA.ptr, dB.ptr, None, dD.ptr, n, n, n, n, n, 0, n, 1.0, 0.0, 1.0, 0.0, ws.ptr, need, None))
+    for _ in range(warmup):
+        call()
+    hip.sync()
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < settle_s:
+        call()
+        hip.sync()
+    timer = hip.Timer(); timer.start()
+    for _ in range(steps):
+        call()
+    ms = timer.stop() / steps
+    tf = 8.0 * n ** 3 / (ms * 1e-3) / 1e12
+    peak = PEAK_F64_TFLOPS if double else PEAK_F32_TFLOPS
+    out = {"workload": "%s GEMM M=N=K=%d (real expansion of B + one %s GEMM), uniform[-1,1]" % (np.dtype(cdt).name, n, "fp64" if double else "fp32"),
+           "dtype": "c128" if double else "c64", "value": round(tf, 3), "unit": "TFLOP/s",
+           "hbm_gbs_algorithmic": round(3.0 * n * n * 2 * rb / (ms * 1e-3) / 1e9, 1), "kernel_ms": round(ms, 5),
+           "roofline": {"bound": "mfma", "achieved": round(tf, 3), "peak": peak, "unit": "TFLOP/s", "frac": round(tf / peak, 4),
+                        "traffic": None}}
+    for d in (dA, dB, dD, ws):
+        d.free()
+    return out
+
+
 def cpu_baseline(name, A, B):
     """Times the AVX2 restatement of the reference CPU GEMM once on this host and checks it
     bit-for-bit against the scalar fma chain on sampled rows."""
@@ -216,7 +254,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="fp32_8192", choices=sorted(WORKLOADS) + ["copy_1GiB", "conv2d"])
+    ap.add_argument("--workload", default="fp32_8192", choices=sorted(WORKLOADS) + ["copy_1GiB", "conv2d", "c64_4096", "c128_2048"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     args = ap.parse_args()
@@ -248,6 +286,9 @@ def main():
     if args.workload == "conv2d":
         print(json.dumps(run_conv(args.steps, args.warmup)))
         return
+    if args.workload in ("c64_4096", "c128_2048"):
+        print(json.dumps(run_complex(args.workload == "c128_2048", 4096 if args.workload == "c64_4096" else 2048, args.steps, args.warmup)))
+        return
 
     main_out, inputs = run_workload(args.workload, args.steps, args.warmup, keep_inputs=not args.no_cpu,
                                     settle_s=0.25 if args.workload != "fp32_8192" else 0.0)
@@ -273,6 +314,8 @@ def main():
                 small = WORKLOADS[name][1] * WORKLOADS[name][2] * WORKLOADS[name][3] < 2 ** 38
                 others.append(run_workload(name, 200 if small else args.steps, args.warmup, settle_s=0.25)[0])
         others.append(run_conv(200, args.warmup))
+        others.append(run_complex(False, 4096, args.steps, args.warmup))
+        others.append(run_complex(True, 2048, 50, args.warmup))
         line["other_workloads"] = others
     if not args.no_cpu:
         if main_out["dtype"] == "f32":
