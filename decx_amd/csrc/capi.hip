@@ -425,7 +425,7 @@ int decx_hip_conv2d_f32(const float* image, const float* kmat, float* dst, uint3
         dst_dpitch % 4 || kmat_pitch < out_c || dst_dpitch < out_c || dst_wpitch < out_w ||
         img_wpitch < (uint64_t)(out_w - 1) * stride_x + k_w || !aligned16(image) || !aligned16(kmat) || !aligned16(dst) ||
         (uint64_t)out_w * out_h > 0xffffffffull || (uint64_t)k_w * img_dpitch * 4 > 0xffffffffull ||
-        (uint64_t)k_h * k_w * img_dpitch > 0xffffffffull)
+        (uint64_t)k_h * k_w * img_dpitch > 0xffffffffull || (uint64_t)kmat_pitch * 256 >= (1ull << 31))
         return DECX_HIP_E_INVALID_ARG;
     GemmArgs g;
     std::memset(&g, 0, sizeof g);
@@ -440,6 +440,7 @@ int decx_hip_conv2d_f32(const float* image, const float* kmat, float* dst, uint3
     g.conv_dst_row = dst_wpitch * dst_dpitch;
     g.conv_seg_stride = (uint64_t)img_wpitch * img_dpitch * 4u;
     g.conv_py_bytes = (uint64_t)stride_y * img_wpitch * img_dpitch * 4u;
+    g.conv_image_bytes = ((uint64_t)(out_h - 1) * stride_y + k_h) * img_wpitch * img_dpitch * 4u;
     return launch_conv2d_f32_dma(choose_tile(false, g.M, g.N, true), g, as_stream(stream));
 }
 

@@ -39,6 +39,7 @@ struct GemmArgs {
     uint32_t conv_dst_row;       // floats per output image row
     uint64_t conv_seg_stride;
     uint64_t conv_py_bytes;      // bytes between patches of vertically adjacent output pixels
+    uint64_t conv_image_bytes;   // size of the image the patches lie in
 };
 
 constexpr int kXcds = 8;        // MI355X: 8 accelerator complex dies, blocks are dealt to them round-robin

@@ -72,7 +72,9 @@ template <int TN> __device__ __forceinline__ float lane_of(const typename BFrag<
 
 }  // namespace
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, bool CONV = false>
+// CONV: 0 plain GEMM; 1 convolution, every copy lane walks the image on its own; 2 convolution whose runs of
+// contiguous bytes are whole slabs, so that all lanes hop to the next image row in the same slab.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, int CONV = 0>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_f32_dma_kernel(const GemmArgs g)
 {
@@ -113,13 +115,15 @@ gemm_f32_dma_kernel(const GemmArgs g)
     // slot lane % CPR, fetching chunk slot ^ ((row / RP) % CPR).  B direct load I covers k rows RB I ..:
     // lane -> k row RB I + lane / CB, slot lane % CB, fetching column chunk slot ^ (B_SHIFT if k row & 4).
     // Rows beyond M and column chunks beyond N are replaced by the last valid ones.
-    // CONV: the A operand is gathered from an image.  a_src[i] then walks along the patch of the lane's output
-    // pixel: a_seg[i] is its byte position inside the current run of contiguous bytes (one kernel row), and
-    // every slab issued moves it on by BK floats, hopping to the next image row at the end of a run.
+    // CONV: the A operand is gathered from an image: the K elements of an output pixel are runs of conv_seg_bytes
+    // contiguous bytes (one kernel row), conv_seg_stride apart.  Mode 1: a_src[i] walks along the patch of the
+    // lane's pixel, a_seg[i] is its byte position inside the current run, and every slab issued moves it on by BK
+    // floats, hopping to the next image row at the end of a run.  Mode 2 (runs are whole slabs): the lanes hop
+    // together, so the walk is scalar, as in the plain GEMM.
     const unsigned char* a_src[A_LOADS];
-    const unsigned char* b_src[B_LOADS];
+    uint32_t b_voff[B_LOADS];
     int a_chunk[A_LOADS], b_krow[B_LOADS];
-    uint32_t a_seg[CONV ? A_LOADS : 1];
+    uint32_t a_seg[CONV == 1 ? A_LOADS : 1];
     const uint32_t last_row = g.M - 1, last_col_chunk = (g.N - 1) / 4;
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
@@ -127,12 +131,12 @@ gemm_f32_dma_kernel(const GemmArgs g)
         const int row = I * (64 / CPR) + lane / CPR;
         a_chunk[i] = (lane % CPR) ^ ((row / RP) % CPR);
         const uint32_t grow = (m0 + row) < last_row ? (m0 + row) : last_row;
-        if constexpr (CONV) {
+        if constexpr (CONV != 0) {
             const uint32_t py = grow / g.conv_wout, px = grow % g.conv_wout;
             const uint32_t k_bytes = a_chunk[i] * 16;
-            a_seg[i] = k_bytes % g.conv_seg_bytes;
+            if constexpr (CONV == 1) a_seg[i] = k_bytes % g.conv_seg_bytes;
             a_src[i] = A + (size_t)py * g.conv_py_bytes + (size_t)px * g.conv_px_bytes +
-                       (size_t)(k_bytes / g.conv_seg_bytes) * g.conv_seg_stride + a_seg[i];
+                       (size_t)(k_bytes / g.conv_seg_bytes) * g.conv_seg_stride + k_bytes % g.conv_seg_bytes;
         } else {
             a_src[i] = A + (size_t)grow * lda_b + a_chunk[i] * 16;
         }
@@ -143,37 +147,42 @@ gemm_f32_dma_kernel(const GemmArgs g)
         b_krow[i] = I * RB + lane / CB;
         const int chunk = (lane % CB) ^ ((b_krow[i] & 4) ? B_SHIFT : 0);
         const uint32_t gchunk = (n0 / 4 + chunk) < last_col_chunk ? (n0 / 4 + chunk) : last_col_chunk;
-        b_src[i] = B + (size_t)b_krow[i] * ldb_b + (size_t)gchunk * 16;
+        b_voff[i] = (uint32_t)((size_t)b_krow[i] * ldb_b + (size_t)gchunk * 16);           // < BK * ldb_b + 4 N: the launcher checks
     }
 
     const uint32_t full_slabs = g.K / BK, k_tail = g.K % BK;
     const uint32_t slabs = full_slabs + (k_tail ? 1u : 0u);
 
-    // Slabs are issued in ascending order.  Plain GEMM: a direct load takes its address as a scalar base (the
-    // tile's first row of A / B's row k, running along K) plus a 32-bit lane offset that never changes, so
-    // that advancing to the next slab is scalar arithmetic.  CONV: the lanes' sources hop between image rows
-    // independently, so a_src / b_src are full per-lane pointers, each left at the next slab by its load.
+    // Slabs are issued in ascending order.  A direct load takes its address as a scalar base (the tile's first
+    // row of A, or the image; B's row k; running along K) plus a 32-bit lane offset that never changes, so that
+    // advancing to the next slab is scalar arithmetic.  Only the per-lane image walk of CONV mode 1 keeps full
+    // per-lane pointers for A, each left at the next slab by its load.
     const size_t b_step = (size_t)BK * ldb_b;
-    uint32_t a_voff[CONV ? 1 : A_LOADS], b_voff[CONV ? 1 : B_LOADS];
-    const unsigned char* a_base = A + (size_t)m0 * lda_b;
+    uint32_t a_voff[CONV == 1 ? 1 : A_LOADS];
+    const unsigned char* a_base = CONV ? A : A + (size_t)m0 * lda_b;
     const unsigned char* b_base = B;
-    if constexpr (!CONV) {
+    uint32_t run_pos = 0;                                  // CONV mode 2: bytes of the current run already issued
+    if constexpr (CONV != 1) {
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) a_voff[i] = (uint32_t)(a_src[i] - a_base);       // < BM * lda_b: the launcher checks
-#pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) b_voff[i] = (uint32_t)(b_src[i] - b_base);       // < BK * ldb_b
+        for (int i = 0; i < A_LOADS; ++i) a_voff[i] = (uint32_t)(a_src[i] - a_base);       // < BM * lda_b / the image size: the launcher checks
     }
-    auto a_ptr = [&](int i) { if constexpr (CONV) return a_src[i]; else return a_base + a_voff[i]; };
-    auto b_ptr = [&](int i) { if constexpr (CONV) return b_src[i]; else return b_base + b_voff[i]; };
+    auto a_ptr = [&](int i) { if constexpr (CONV == 1) return a_src[i]; else return a_base + a_voff[i]; };
+    auto b_ptr = [&](int i) { return b_base + b_voff[i]; };
     auto issue_one = [&](uint32_t stage, auto ic) {        // direct load ic of a full slab: A first, then B
         constexpr int idx = decltype(ic)::value;
         const uint32_t stage_off = lds_base + stage * STAGE_BYTES;
         if constexpr (idx < A_LOADS) {
             constexpr int i = idx;
             const uint32_t dst = stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u;
-            if constexpr (!CONV) {
+            if constexpr (CONV != 1) {
                 asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(a_voff[i]), "s"(a_base) : "memory", "m0");
-                if constexpr (i == A_LOADS - 1) a_base += BK * 4;
+                if constexpr (i == A_LOADS - 1) {
+                    a_base += BK * 4;
+                    if constexpr (CONV == 2) {
+                        run_pos += BK * 4;
+                        if (run_pos == g.conv_seg_bytes) { run_pos = 0; a_base += g.conv_seg_stride - g.conv_seg_bytes; }
+                    }
+                }
             } else {
                 asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(a_src[i]) : "memory", "m0");
                 a_src[i] += BK * 4;
@@ -186,13 +195,8 @@ gemm_f32_dma_kernel(const GemmArgs g)
         } else {
             constexpr int i = idx - A_LOADS;
             const uint32_t dst = stage_off + A_STAGE_BYTES + (uint32_t)(wave * B_LOADS + i) * 1024u;
-            if constexpr (!CONV) {
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(b_voff[i]), "s"(b_base) : "memory", "m0");
-                if constexpr (i == B_LOADS - 1) b_base += b_step;
-            } else {
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(b_src[i]) : "memory", "m0");
-                b_src[i] += b_step;
-            }
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(b_voff[i]), "s"(b_base) : "memory", "m0");
+            if constexpr (i == B_LOADS - 1) b_base += b_step;
         }
     };
     auto issue_tail = [&](uint32_t stage) {                // the partial last slab: through registers, zero beyond K
@@ -392,7 +396,7 @@ gemm_f32_dma_kernel(const GemmArgs g)
         for (int r = 0; r < 16; ++r) {
             const uint32_t row = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * h + (r % 4);
             size_t d_row;                              // offset of the row's first element in D
-            if constexpr (CONV) d_row = (size_t)(row / g.conv_wout) * g.conv_dst_row + (size_t)(row % g.conv_wout) * g.ldd;
+            if constexpr (CONV != 0) d_row = (size_t)(row / g.conv_wout) * g.conv_dst_row + (size_t)(row % g.conv_wout) * g.ldd;
             else d_row = (size_t)row * g.ldd;
             float v[TN];
 #pragma unroll
@@ -426,7 +430,7 @@ gemm_f32_dma_kernel(const GemmArgs g)
 
 namespace {
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, bool CONV = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, int CONV = 0>
 int launch_dma(const GemmArgs& args, hipStream_t stream)
 {
     GemmArgs g = args;
@@ -467,10 +471,17 @@ int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
 // (srcs/modules/NN/convolution/CUDA/fp32/im2col_fp32.cu, im2col_GEMM_fp32.cu:40-106) and their im2col buffer.
 int launch_conv2d_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
 {
+    // runs that are a whole number of slabs (e.g. 3 x 112 channels: 21 slabs of 16 floats) let all copy lanes hop
+    // together; image_bytes bounds the lanes' 32-bit offsets
+    const uint32_t slab_bytes = (shape == TILE_64x64 ? 32u : 16u) * 4u;
+    const bool uniform = args.conv_seg_bytes % slab_bytes == 0 && args.conv_image_bytes < (1ull << 31);
     switch (shape) {
-    case TILE_256x256: return launch_dma<256, 256, 2, 4, 16, 4, false, true>(args, stream);    // 134 TFLOP/s on the 3 x 3 x 112 workload; 256 x 128: 127
-    case TILE_128x128: return launch_dma<128, 128, 2, 2, 16, 2, true, true>(args, stream);
-    case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 32, 2, true, true>(args, stream);
+    case TILE_256x256: return uniform ? launch_dma<256, 256, 2, 4, 16, 4, false, 2>(args, stream)     // 137 TFLOP/s on the 3 x 3 x 112 workload; 256 x 128: 136
+                                      : launch_dma<256, 256, 2, 4, 16, 4, false, 1>(args, stream);
+    case TILE_128x128: return uniform ? launch_dma<128, 128, 2, 2, 16, 2, true, 2>(args, stream)
+                                      : launch_dma<128, 128, 2, 2, 16, 2, true, 1>(args, stream);
+    case TILE_64x64:   return uniform ? launch_dma< 64,  64, 2, 2, 32, 2, true, 2>(args, stream)
+                                      : launch_dma< 64,  64, 2, 2, 32, 2, true, 1>(args, stream);
     default:           return (int)hipErrorInvalidValue;
     }
 }
