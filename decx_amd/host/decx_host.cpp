@@ -7,6 +7,7 @@
 #include <cstring>
 #include <new>
 #include <thread>
+#include <vector>
 
 namespace {
 
@@ -470,16 +471,104 @@ _DECX_API_ void de::blas::cuda::GEMM(de::GPU_Matrix& A, de::GPU_Matrix& B, de::G
 namespace {
 
 // Streams and events of the host-matrix form, created on first use and kept.
+// rows x width bytes from one pitched host buffer to another, on several host threads for large blocks
+void copy_rows_parallel(char* dst, size_t dpitch, const char* src, size_t spitch, size_t width, size_t rows)
+{
+    const size_t bytes = width * rows;
+    size_t workers = bytes / (2u << 20);                   // one thread per 2 MiB, at most 8 and what the host has
+    const size_t hw = std::thread::hardware_concurrency();
+    if (workers > 8) workers = 8;
+    if (hw && workers > hw) workers = hw;
+    auto part = [=](size_t r0, size_t r1) {
+        if (dpitch == width && spitch == width) std::memcpy(dst + r0 * width, src + r0 * width, (r1 - r0) * width);
+        else for (size_t r = r0; r < r1; ++r) std::memcpy(dst + r * dpitch, src + r * spitch, width);
+    };
+    if (workers <= 1 || rows < workers) { part(0, rows); return; }
+    std::vector<std::thread> team;
+    for (size_t w = 1; w < workers; ++w) team.emplace_back(part, rows * w / workers, rows * (w + 1) / workers);
+    part(0, rows / workers);
+    for (auto& t : team) t.join();
+}
+
+// Streams of the host-matrix pipeline, and the page-locked bounce buffers that pageable host memory travels
+// through: the runtime's own staging of pageable copies is synchronous and several times slower than filling a
+// page-locked buffer with host threads and copying that asynchronously.
 struct HostPipe {
+    static constexpr size_t kBuf = 16u << 20;              // bytes per bounce buffer
+    static constexpr int kRing = 3;                        // buffers per direction
     void* in = nullptr;        // host -> device copies
     void* out = nullptr;       // device -> host copies
     bool ok = false;
+    struct Slot { void* buf = nullptr; void* done = nullptr; bool busy = false; char* host = nullptr; size_t hpitch = 0, width = 0, rows = 0; };
+    Slot up[kRing], down[kRing];
+    int up_next = 0, down_next = 0;
+
+    // pageable host -> device on stream `in`
+    int upload(void* dev, size_t dpitch, const char* host, size_t hpitch, size_t width, size_t rows)
+    {
+        const size_t wpiece = width < kBuf ? width : kBuf;
+        const size_t rpiece = kBuf / wpiece ? kBuf / wpiece : 1;
+        for (size_t c0 = 0; c0 < width; c0 += wpiece) {
+            const size_t w = width - c0 < wpiece ? width - c0 : wpiece;
+            for (size_t r0 = 0; r0 < rows; r0 += rpiece) {
+                const size_t r = rows - r0 < rpiece ? rows - r0 : rpiece;
+                Slot& s = up[up_next]; up_next = (up_next + 1) % kRing;
+                int rc = s.busy ? decx_hip_event_sync(s.done) : DECX_HIP_OK;     // its previous copy has left the buffer
+                if (rc != DECX_HIP_OK) return rc;
+                copy_rows_parallel((char*)s.buf, w, host + r0 * hpitch + c0, hpitch, w, r);
+                rc = decx_hip_memcpy2d_async((char*)dev + r0 * dpitch + c0, dpitch, s.buf, w, w, r, 0, in);
+                if (rc == DECX_HIP_OK) rc = decx_hip_event_record(s.done, in);
+                if (rc != DECX_HIP_OK) return rc;
+                s.busy = true;
+            }
+        }
+        return DECX_HIP_OK;
+    }
+    int drain(Slot& s)                                     // a finished device -> host piece goes to its pageable home
+    {
+        if (!s.busy || !s.host) return DECX_HIP_OK;
+        const int rc = decx_hip_event_sync(s.done);
+        if (rc == DECX_HIP_OK) copy_rows_parallel(s.host, s.hpitch, (const char*)s.buf, s.width, s.width, s.rows);
+        s.busy = false; s.host = nullptr;
+        return rc;
+    }
+    // device -> pageable host on stream `out`; pieces land in their home when their buffer is needed again, or in flush()
+    int download(char* host, size_t hpitch, const void* dev, size_t dpitch, size_t width, size_t rows)
+    {
+        const size_t wpiece = width < kBuf ? width : kBuf;
+        const size_t rpiece = kBuf / wpiece ? kBuf / wpiece : 1;
+        for (size_t c0 = 0; c0 < width; c0 += wpiece) {
+            const size_t w = width - c0 < wpiece ? width - c0 : wpiece;
+            for (size_t r0 = 0; r0 < rows; r0 += rpiece) {
+                const size_t r = rows - r0 < rpiece ? rows - r0 : rpiece;
+                Slot& s = down[down_next]; down_next = (down_next + 1) % kRing;
+                int rc = drain(s);
+                if (rc == DECX_HIP_OK) rc = decx_hip_memcpy2d_async(s.buf, w, (const char*)dev + r0 * dpitch + c0, dpitch, w, r, 1, out);
+                if (rc == DECX_HIP_OK) rc = decx_hip_event_record(s.done, out);
+                if (rc != DECX_HIP_OK) return rc;
+                s.busy = true; s.host = host + r0 * hpitch + c0; s.hpitch = hpitch; s.width = w; s.rows = r;
+            }
+        }
+        return DECX_HIP_OK;
+    }
+    int flush()
+    {
+        int rc = DECX_HIP_OK;
+        for (int i = 0; i < kRing; ++i) {                  // oldest first
+            const int r = drain(down[(down_next + i) % kRing]);
+            if (rc == DECX_HIP_OK) rc = r;
+        }
+        return rc;
+    }
 };
 HostPipe& host_pipe()
 {
     static HostPipe p;
     if (!p.ok && decx::gpu_ready()) {
         p.ok = decx_hip_stream_create(&p.in) == DECX_HIP_OK && decx_hip_stream_create(&p.out) == DECX_HIP_OK;
+        for (int i = 0; i < HostPipe::kRing && p.ok; ++i)
+            p.ok = decx_hip_host_malloc(&p.up[i].buf, HostPipe::kBuf) == DECX_HIP_OK && decx_hip_event_create(&p.up[i].done) == DECX_HIP_OK &&
+                   decx_hip_host_malloc(&p.down[i].buf, HostPipe::kBuf) == DECX_HIP_OK && decx_hip_event_create(&p.down[i].done) == DECX_HIP_OK;
     }
     return p;
 }
@@ -494,8 +583,8 @@ struct EventList {
 // Host-matrix form.  The original declares these overloads (srcs/includes/DECX/BLAS/BLAS.h:69-70) and defines
 // them nowhere.  Here the operands are staged through device memory in row panels of A (and C): panel p + 1
 // travels host -> device while panel p is multiplied and panel p - 1 of the result travels back, on three
-// streams chained by events.  The copies are asynchronous when the host matrices are page-locked
-// (de::cuda::PinMemory); with pageable memory the runtime stages them and the overlap is partial.
+// streams chained by events.  Page-locked host matrices (de::cuda::PinMemory) are copied directly; pageable ones
+// travel through the pipeline's page-locked bounce buffers, which several host threads fill and empty.
 void gemm_host(de::Matrix& A, de::Matrix& B, de::Matrix* C, de::Matrix& dst)
 {
     de::DH* h = de::GetLastError();
@@ -539,19 +628,25 @@ void gemm_host(de::Matrix& A, de::Matrix& B, de::Matrix* C, de::Matrix& dst)
 
     EventList events;
     int rc = DECX_HIP_OK;
-    auto copy = [&](void* dp, size_t dpitch, const void* hp, size_t hpitch, size_t width, size_t rows, int kind, void* st) {
-        if (rc == DECX_HIP_OK && width && rows)
+    // kind 0: host -> device on pipe.in, 1: device -> host on pipe.out; pitches and width in elements
+    auto copy = [&](void* dp, size_t dpitch, const void* hp, size_t hpitch, size_t width, size_t rows, int kind, bool pinned) {
+        if (rc != DECX_HIP_OK || !width || !rows) return;
+        if (pinned)
             rc = decx_hip_memcpy2d_async(kind == 0 ? dp : const_cast<void*>(hp), (kind == 0 ? dpitch : hpitch) * es,
-                                         kind == 0 ? hp : dp, (kind == 0 ? hpitch : dpitch) * es, width * es, rows, kind, st);
+                                         kind == 0 ? hp : dp, (kind == 0 ? hpitch : dpitch) * es, width * es, rows, kind,
+                                         kind == 0 ? pipe.in : pipe.out);
+        else if (kind == 0) rc = pipe.upload(dp, dpitch * es, (const char*)hp, hpitch * es, width * es, rows);
+        else rc = pipe.download((char*)const_cast<void*>(hp), hpitch * es, dp, dpitch * es, width * es, rows);
     };
-    copy(dB.data(), dB.Pitch(), b->data(), b->Pitch(), N, K, 0, pipe.in);
+    const bool a_pinned = a->is_pinned(), b_pinned = b->is_pinned(), c_pinned = c && c->is_pinned(), d_pinned = d->is_pinned();
+    copy(dB.data(), dB.Pitch(), b->data(), b->Pitch(), N, K, 0, b_pinned);
     for (uint32_t p = 0; p < panels && rc == DECX_HIP_OK; ++p) {
         const uint32_t r0 = p * rows_per, rows = (M - r0) < rows_per ? (M - r0) : rows_per;
         char* a_dev = (char*)dA.data() + (size_t)r0 * dA.Pitch() * es;
         char* d_dev = (char*)dD.data() + (size_t)r0 * dD.Pitch() * es;
         char* c_dev = c ? (char*)dC.data() + (size_t)r0 * dC.Pitch() * es : nullptr;
-        copy(a_dev, dA.Pitch(), (const char*)a->data() + (size_t)r0 * a->Pitch() * es, a->Pitch(), K, rows, 0, pipe.in);
-        if (c) copy(c_dev, dC.Pitch(), c_host + (size_t)r0 * c_host_pitch * es, c_host_pitch, N, rows, 0, pipe.in);
+        copy(a_dev, dA.Pitch(), (const char*)a->data() + (size_t)r0 * a->Pitch() * es, a->Pitch(), K, rows, 0, a_pinned);
+        if (c) copy(c_dev, dC.Pitch(), c_host + (size_t)r0 * c_host_pitch * es, c_host_pitch, N, rows, 0, c_pinned);
         void* arrived = events.make();
         void* done = events.make();
         if (!arrived || !done) { rc = DECX_HIP_E_INVALID_ARG; break; }
@@ -569,8 +664,10 @@ void gemm_host(de::Matrix& A, de::Matrix& B, de::Matrix* C, de::Matrix& dst)
                                          dD.Pitch(), 1.f, 1.f, S);
         if (rc == DECX_HIP_OK) rc = decx_hip_event_record(done, S);
         if (rc == DECX_HIP_OK) rc = decx_hip_stream_wait_event(pipe.out, done);
-        copy(d_dev, dD.Pitch(), (char*)d->data() + (size_t)r0 * d->Pitch() * es, d->Pitch(), N, rows, 1, pipe.out);
+        copy(d_dev, dD.Pitch(), (char*)d->data() + (size_t)r0 * d->Pitch() * es, d->Pitch(), N, rows, 1, d_pinned);
     }
+    const int rf = pipe.flush();                           // the last pieces of a pageable dst
+    if (rc == DECX_HIP_OK) rc = rf;
     // drain all three streams whatever happened, so that nothing is in flight when the device twins die
     const int r1 = decx_hip_stream_sync(pipe.in), r2 = decx_hip_stream_sync(S), r3 = decx_hip_stream_sync(pipe.out);
     if (rc == DECX_HIP_OK) rc = r1 != DECX_HIP_OK ? r1 : (r2 != DECX_HIP_OK ? r2 : r3);

@@ -604,6 +604,33 @@ template <typename T> static int gemm_wall_time(de::_DATA_TYPES_FLAGS_ ty, uint3
     return (dD.Width() == N && dD.Height() == M) ? 0 : 4;
 }
 
+// Wall time of the host-matrix form de::blas::cuda::GEMM(Matrix x 3): staging in, multiply, staging out.
+template <typename T> static int hostgemm_wall_time(de::_DATA_TYPES_FLAGS_ ty, uint32_t M, uint32_t N, uint32_t K, int repeats, bool pinned)
+{
+    de::InitCuda();
+    de::ResetLastError();
+    de::Matrix& A = de::CreateMatrixRef(ty, K, M);
+    de::Matrix& B = de::CreateMatrixRef(ty, N, K);
+    de::Matrix& D = de::CreateMatrixRef(ty, N, M);
+    uint64_t state = 0x9E3779B97F4A7C15ull;
+    auto next = [&]() { state = state * 6364136223846793005ull + 1442695040888963407ull; return (float)((state >> 40) & 0xFFFF) / 32768.f - 1.f; };
+    for (uint32_t i = 0; i < M; ++i) for (uint32_t k = 0; k < K; ++k) *A.ptr<T>(i, k) = from_float<T>(next());
+    for (uint32_t k = 0; k < K; ++k) for (uint32_t j = 0; j < N; ++j) *B.ptr<T>(k, j) = from_float<T>(next());
+    if (pinned && (de::cuda::PinMemory(A).error_type || de::cuda::PinMemory(B).error_type || de::cuda::PinMemory(D).error_type)) return 5;
+    std::vector<double> ms;
+    for (int r = 0; r < repeats + 1; ++r) {
+        const auto t0 = std::chrono::steady_clock::now();
+        de::blas::cuda::GEMM(A, B, D);
+        ms.push_back(std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count());
+        if (de::GetLastError()->error_type != 0) { std::cerr << de::GetLastError()->error_string << "\n"; return 3; }
+    }
+    std::vector<double> last(ms.begin() + 1, ms.end());                   // the first call creates streams and buffers
+    std::sort(last.begin(), last.end());
+    std::cout << "hostgemmtime " << (pinned ? "pinned" : "pageable") << " median_ms " << last[last.size() / 2] << " min_ms " << last.front()
+              << " first_ms " << ms.front() << "\n";
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
     const std::string mode = argc > 1 ? argv[1] : "host";
@@ -624,6 +651,13 @@ int main(int argc, char** argv)
         const int repeats = std::max(1, std::atoi(argv[6]));
         rc = std::string(argv[2]) == "f16" ? gemm_wall_time<de::Half>(de::_FP16_, M, N, K, repeats)
                                            : gemm_wall_time<float>(de::_FP32_, M, N, K, repeats);
+    }
+    else if (mode == "hostgemmtime" && argc == 8) {
+        const uint32_t M = std::atoi(argv[3]), N = std::atoi(argv[4]), K = std::atoi(argv[5]);
+        const int repeats = std::max(1, std::atoi(argv[6]));
+        const bool pinned = std::atoi(argv[7]) != 0;
+        rc = std::string(argv[2]) == "f16" ? hostgemm_wall_time<de::Half>(de::_FP16_, M, N, K, repeats, pinned)
+                                           : hostgemm_wall_time<float>(de::_FP32_, M, N, K, repeats, pinned);
     }
     else if (mode == "tensor_host") rc = tensor_host_checks();
     else if (mode == "conv" && argc == 12)
@@ -647,7 +681,7 @@ int main(int argc, char** argv)
                  : gemm_files<float>(argv[2], de::_FP32_, M, N, K, with_c, alpha, beta);
     } else {
         std::cerr << "usage: de_api_test host | gpu | vector_host | vector_gpu | gemm <dir> <f32|f16> M N K withC alpha beta"
-                     " | vmm <dir> <f32|f16> <mv|vm> W H level | gemmtime <f32|f16> M N K repeats\n";
+                     " | vmm <dir> <f32|f16> <mv|vm> W H level | gemmtime <f32|f16> M N K repeats | hostgemmtime <f32|f16> M N K repeats pinned\n";
         return 64;
     }
     std::cout << (rc == 0 ? "de_api_test: all checks passed" : "de_api_test: FAILED") << " (" << mode << ")\n";
