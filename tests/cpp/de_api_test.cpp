@@ -588,8 +588,12 @@ template <typename T> static int gemm_wall_time(de::_DATA_TYPES_FLAGS_ ty, uint3
     de::GPU_Matrix& dA = de::CreateGPUMatrixRef(ty, K, M);
     de::GPU_Matrix& dB = de::CreateGPUMatrixRef(ty, N, K);
     de::GPU_Matrix& dD = de::CreateGPUMatrixRef();
+    auto now = [] { return std::chrono::steady_clock::now(); };
+    auto since = [&](std::chrono::steady_clock::time_point t0) { return std::chrono::duration<double, std::milli>(now() - t0).count(); };
     if (de::Memcpy(A, dA, de::Point2D(0, 0), de::Point2D(0, 0), de::Point2D(K, M), de::DECX_MEMCPY_H2D).error_type) return 3;
+    auto t_up = now();
     if (de::Memcpy(B, dB, de::Point2D(0, 0), de::Point2D(0, 0), de::Point2D(N, K), de::DECX_MEMCPY_H2D).error_type) return 3;
+    const double up_ms = since(t_up);
     std::vector<double> ms;
     const auto begin = std::chrono::steady_clock::now();
     for (int r = 0; r < repeats + 3 || std::chrono::duration<double>(std::chrono::steady_clock::now() - begin).count() < 0.3; ++r) {
@@ -601,6 +605,13 @@ template <typename T> static int gemm_wall_time(de::_DATA_TYPES_FLAGS_ ty, uint3
     std::vector<double> last(ms.end() - repeats, ms.end());               // what came before is warm-up
     std::sort(last.begin(), last.end());
     std::cout << "gemmtime median_ms " << last[last.size() / 2] << " min_ms " << last.front() << " calls " << last.size() << "\n";
+    de::Matrix& D = de::CreateMatrixRef(ty, N, M);
+    if (de::Memcpy(D, dD, de::Point2D(0, 0), de::Point2D(0, 0), de::Point2D(N, M), de::DECX_MEMCPY_D2H).error_type) return 3;   // touches D's pages
+    auto t_down = now();
+    if (de::Memcpy(D, dD, de::Point2D(0, 0), de::Point2D(0, 0), de::Point2D(N, M), de::DECX_MEMCPY_D2H).error_type) return 3;
+    const double down_ms = since(t_down);
+    std::cout << "memcpytime pageable h2d_ms " << up_ms << " (" << (double)K * N * sizeof(T) / up_ms / 1e6 << " GB/s) d2h_ms " << down_ms
+              << " (" << (double)M * N * sizeof(T) / down_ms / 1e6 << " GB/s)\n";
     return (dD.Width() == N && dD.Height() == M) ? 0 : 4;
 }
 
