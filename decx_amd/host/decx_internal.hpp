@@ -269,5 +269,11 @@ public:
 // (the original guards its cached planner with a plain flag).
 void* module_stream();
 std::mutex& module_mutex();
+// Host <-> device copies of pitched blocks (sizes in bytes) for callers that hold module_mutex().  Page-locked
+// host memory is copied directly; pageable memory goes through page-locked bounce buffers filled by host threads.
+// The copies are complete, and device -> host data in place, once stage_finish() has returned.
+int stage_h2d(void* dev, size_t dpitch, const void* host, size_t hpitch, size_t width, size_t rows, bool host_pinned);
+int stage_d2h(void* host, size_t hpitch, const void* dev, size_t dpitch, size_t width, size_t rows, bool host_pinned);
+int stage_finish();
 
 }  // namespace decx

@@ -272,15 +272,15 @@ _DECX_API_ de::DH de::Memcpy(de::Tensor& host, de::GPU_Tensor& device, const de:
     const size_t es = SL._single_element_size;
     const char* sp = (const char*)(h2d ? h->data() : d->data());
     char* dp = (char*)(h2d ? d->data() : h->data());
-    void* S = decx::module_stream();
+    std::lock_guard<std::mutex> guard(decx::module_mutex());
     int rc = DECX_HIP_OK;
     for (int32_t r = 0; r < size.z && rc == DECX_HIP_OK; ++r) {
         const char* s_row = sp + (((size_t)(start_src.z + r) * SL.wpitch + start_src.y) * SL.dpitch + start_src.x) * es;
         char* d_row = dp + (((size_t)(start_dst.z + r) * DL.wpitch + start_dst.y) * DL.dpitch + start_dst.x) * es;
-        rc = decx_hip_memcpy2d_async(d_row, (size_t)DL.dpitch * es, s_row, (size_t)SL.dpitch * es, (size_t)size.x * es,
-                                     (size_t)size.y, h2d ? 0 : 1, S);
+        rc = h2d ? decx::stage_h2d(d_row, (size_t)DL.dpitch * es, s_row, (size_t)SL.dpitch * es, (size_t)size.x * es, (size_t)size.y, false)
+                 : decx::stage_d2h(d_row, (size_t)DL.dpitch * es, s_row, (size_t)SL.dpitch * es, (size_t)size.x * es, (size_t)size.y, false);
     }
-    const int rs = decx_hip_stream_sync(S);
+    const int rs = decx::stage_finish();
     decx::err::from_hip(&handle, rc != DECX_HIP_OK ? rc : rs, "Memcpy");
     return handle;
 }
