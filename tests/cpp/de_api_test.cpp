@@ -122,6 +122,40 @@ static int gpu_checks()
         worst = std::fmax(worst, std::fabs((double)*D.ptr<float>(i, j) - 337853530.0) / 337853530.0);
     CHECK(worst < 4e-6);
 
+    // pageable host matrices travel through bounce buffers in pieces: sub-regions at offsets, rows wider than a
+    // piece (split by columns), page-locked storage (copied directly) and a round trip of each
+    {
+        const uint32_t WW = 5000011, HH = 3;                                   // 20 MB rows, 60 MB in all
+        de::Matrix& wide = de::CreateMatrixRef(de::_INT32_, WW, HH);
+        de::Matrix& back = de::CreateMatrixRef(de::_INT32_, WW, HH);
+        de::GPU_Matrix& dwide = de::CreateGPUMatrixRef(de::_INT32_, WW, HH);
+        for (uint32_t i = 0; i < HH; ++i) for (uint32_t j = 0; j < WW; ++j) *wide.ptr<int>(i, j) = (int)(i * 7919u + j * 31u);
+        CHECK(de::Memcpy(wide, dwide, O, O, de::Point2D(WW, HH), de::DECX_MEMCPY_H2D).error_type == 0);
+        CHECK(de::Memcpy(back, dwide, O, O, de::Point2D(WW, HH), de::DECX_MEMCPY_D2H).error_type == 0);
+        bool same = true;
+        for (uint32_t i = 0; i < HH && same; ++i) same = std::memcmp(wide.ptr<int>(i, 0), back.ptr<int>(i, 0), (size_t)WW * 4) == 0;
+        CHECK(same);
+        const uint32_t TW = 3001, TH = 2999;                                   // 36 MB, copied as an inner region
+        de::Matrix& tall = de::CreateMatrixRef(de::_FP32_, TW, TH);
+        de::Matrix& tall_back = de::CreateMatrixRef(de::_FP32_, TW, TH);
+        de::GPU_Matrix& dtall = de::CreateGPUMatrixRef(de::_FP32_, TW + 10, TH + 10);
+        fill<float>(tall, [](int i, int j) { return (float)(i * 3 + j); });
+        CHECK(de::Memcpy(tall, dtall, de::Point2D(5, 7), de::Point2D(9, 3), de::Point2D(TW - 5, TH - 7), de::DECX_MEMCPY_H2D).error_type == 0);
+        CHECK(de::Memcpy(tall_back, dtall, de::Point2D(9, 3), de::Point2D(5, 7), de::Point2D(TW - 5, TH - 7), de::DECX_MEMCPY_D2H).error_type == 0);
+        same = true;
+        for (uint32_t i = 7; i < TH && same; ++i) same = std::memcmp(tall.ptr<float>(i, 5), tall_back.ptr<float>(i, 5), (size_t)(TW - 5) * 4) == 0;
+        CHECK(same && *tall_back.ptr<float>(0, 0) == 0.f && *tall_back.ptr<float>(6, TW - 1) == 0.f && *tall_back.ptr<float>(TH - 1, 4) == 0.f);
+        CHECK(de::cuda::PinMemory(tall).error_type == 0);
+        de::Matrix& pinned_back = de::CreateMatrixRef(de::_FP32_, TW, TH);
+        CHECK(de::cuda::PinMemory(pinned_back).error_type == 0);
+        CHECK(de::Memcpy(tall, dtall, O, O, de::Point2D(TW, TH), de::DECX_MEMCPY_H2D).error_type == 0);
+        CHECK(de::Memcpy(pinned_back, dtall, O, O, de::Point2D(TW, TH), de::DECX_MEMCPY_D2H).error_type == 0);
+        same = true;
+        for (uint32_t i = 0; i < TH && same; ++i) same = std::memcmp(tall.ptr<float>(i, 0), pinned_back.ptr<float>(i, 0), (size_t)TW * 4) == 0;
+        CHECK(same);
+        wide.release(); back.release(); dwide.release(); tall.release(); tall_back.release(); dtall.release(); pinned_back.release();
+    }
+
     // four-matrix form, alpha = 2, beta = -1, C = ones: 2 * sum - 1; C aliasing dst
     de::GPU_Matrix& dC = de::CreateGPUMatrixRef(de::_FP32_, W, H);
     de::Matrix& C = de::CreateMatrixRef(de::_FP32_, W, H);
