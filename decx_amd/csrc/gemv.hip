@@ -144,9 +144,9 @@ gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restric
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int col_lane = lane % CL, row_lane = lane / CL;
     // Half-line column groups: the two workgroups that share every 128-byte line of B should share an L2,
-    // so blocks b and b + 8 (dealt to the same XCD) take adjacent groups.
+    // so blocks b and b + 8 (dealt to the same XCD) take adjacent groups (the last grid % 16 blocks stay as they are).
     uint32_t group = blockIdx.x;
-    if (CL == 4 && gridDim.x % 16 == 0) group = (group / 16) * 16 + (group % 8) * 2 + (group / 8) % 2;
+    if (CL == 4 && group < gridDim.x / 16 * 16) group = (group / 16) * 16 + (group % 8) * 2 + (group / 8) % 2;
     const uint32_t n0 = group * CB + col_lane * N16;
     const bool whole = vec_ok && (n0 + N16 <= N);
     float acc[N16];
