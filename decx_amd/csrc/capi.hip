@@ -59,10 +59,18 @@ int check_gemm(const void* A, const void* B, const void* C, const void* D, uint3
     return DECX_HIP_OK;
 }
 
+// Split K is planned for fp32 products on 16-byte aligned operands whose tiles would leave most CUs idle
+SplitPlan split_plan_f32(uint32_t M, uint32_t N, uint32_t K)
+{
+    if (M <= 1 || N <= 1) return {1, 0};                   // the vector corners have their own kernels
+    const TileInfo ti = tile_info_f32(choose_tile(false, M, N, true), true);
+    return plan_split_k((uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn), K, g_dev.compute_units);
+}
+
 template <bool F16>
 int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, uint32_t N, uint32_t K,
              uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha, float beta, void* stream,
-             int tile, int force_edge)
+             int tile, int force_edge, void* workspace = nullptr, size_t workspace_bytes = 0)
 {
     if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
     const int rc = check_gemm(A, B, C, D, M, N, K, lda, ldb, ldc, ldd);
@@ -86,6 +94,15 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
                 lda % per16 == 0 && ldb % per16 == 0 && ldd % per16 == 0 && (!C || ldc % per16 == 0)) ? 1u : 0u;
     const int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile(F16, M, N, g.vec_ok != 0) : tile;
     const bool edge = force_edge != 0 || K == 0;
+    if (!F16 && workspace && tile == DECX_HIP_TILE_AUTO && !edge && g.vec_ok && dma_offsets_fit(g, 4) && aligned16(workspace)) {
+        const SplitPlan sp = split_plan_f32(M, N, K);
+        const uint32_t ldw = (N + 3) / 4 * 4;
+        if (sp.splits > 1 && workspace_bytes >= (size_t)sp.splits * M * ldw * 4) {
+            g.split_len = sp.len; g.split_ldd = ldw; g.split_stride = (uint64_t)M * ldw; g.split_ws = (float*)workspace;
+            const int rl = launch_gemm_f32(shape, false, g, as_stream(stream));
+            return rl != 0 ? rl : launch_split_reduce_f32(g, sp.splits, as_stream(stream));
+        }
+    }
     return F16 ? launch_gemm_f16(shape, edge, g, as_stream(stream))
                : launch_gemm_f32(shape, edge, g, as_stream(stream));
 }
@@ -249,6 +266,21 @@ int decx_hip_gemm_f32(const float* A, const float* B, const float* C, float* D, 
                       uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha, float beta, void* stream)
 {
     return run_gemm<false>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0);
+}
+
+size_t decx_hip_gemm_f32_workspace(uint32_t M, uint32_t N, uint32_t K)
+{
+    if (!g_dev.ready || M == 0 || N == 0) return 0;
+    const SplitPlan sp = split_plan_f32(M, N, K);
+    return sp.splits > 1 ? (size_t)sp.splits * M * ((N + 3) / 4 * 4) * 4 : 0;
+}
+
+int decx_hip_gemm_f32_ws(const float* A, const float* B, const float* C, float* D, uint32_t M, uint32_t N, uint32_t K,
+                         uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha, float beta,
+                         void* workspace, size_t workspace_bytes, void* stream)
+{
+    return run_gemm<false>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0, workspace,
+                           workspace_bytes);
 }
 
 int decx_hip_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, uint32_t M, uint32_t N,

@@ -76,8 +76,18 @@ template <int TN> __device__ __forceinline__ float lane_of(const typename BFrag<
 // contiguous bytes are whole slabs, so that all lanes hop to the next image row in the same slab.
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, int CONV = 0>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
-gemm_f32_dma_kernel(const GemmArgs g)
+gemm_f32_dma_kernel(const GemmArgs g_in)
 {
+    GemmArgs g = g_in;
+    if (CONV == 0 && g.split_len) {                        // this workgroup's share of K and its partial product
+        const uint32_t k0 = blockIdx.y * g.split_len;
+        g.A = (const unsigned char*)g.A + (size_t)k0 * 4;
+        g.B = (const unsigned char*)g.B + (size_t)k0 * g.ldb * 4;
+        g.K = g.K - k0 < g.split_len ? g.K - k0 : g.split_len;
+        g.D = g.split_ws + (size_t)blockIdx.y * g.split_stride;
+        g.ldd = g.split_ldd;
+        g.C = nullptr;
+    }
     constexpr int WAVES = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
     constexpr int CPR = BK / 4, RP = 16 / CPR;                    // A chunks per row, rows per 256 bytes
@@ -430,6 +440,32 @@ gemm_f32_dma_kernel(const GemmArgs g)
 
 namespace {
 
+// one thread per four columns: D = sum of the partial products in split order (+ the C term)
+__global__ void __launch_bounds__(256) split_reduce_f32_kernel(const GemmArgs g, uint32_t splits)
+{
+    const uint32_t quads = g.split_ldd / 4;
+    const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (uint64_t)g.M * quads) return;
+    const uint32_t row = (uint32_t)(idx / quads), col = (uint32_t)(idx % quads) * 4;
+    const float* p = g.split_ws + (size_t)row * g.split_ldd + col;
+    floatx4 sum = *(const floatx4*)p;
+    for (uint32_t z = 1; z < splits; ++z) {
+        const floatx4 v = *(const floatx4*)(p + (size_t)z * g.split_stride);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sum[e] += v[e];
+    }
+    const float* C = (const float*)g.C;
+    float* D = (float*)g.D;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        if (col + e < g.N) {
+            float o = sum[e];
+            if (C) o = __builtin_fmaf(C[(size_t)row * g.ldc + col + e], g.beta, g.alpha * o);
+            D[(size_t)row * g.ldd + col + e] = o;
+        }
+    }
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, int CONV = 0>
 int launch_dma(const GemmArgs& args, hipStream_t stream)
 {
@@ -438,8 +474,9 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
     g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
-    hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD, CONV>), dim3(nb), dim3(WAVES_M * WAVES_N * 64),
-                       0, stream, g);
+    const uint32_t splits = (CONV == 0 && g.split_len) ? (g.K + g.split_len - 1) / g.split_len : 1u;
+    hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD, CONV>), dim3(nb, splits),
+                       dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
     return (int)hipGetLastError();
 }
 
@@ -464,6 +501,13 @@ int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
     case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 32, 2, true>(args, stream);
     default:           return (int)hipErrorInvalidValue;
     }
+}
+
+int launch_split_reduce_f32(const GemmArgs& args, uint32_t splits, hipStream_t stream)
+{
+    const uint64_t threads = (uint64_t)args.M * (args.split_ldd / 4);
+    hipLaunchKernelGGL(split_reduce_f32_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, args, splits);
+    return (int)hipGetLastError();
 }
 
 // 2-D convolution as an implicit GEMM: M = output pixels, N = output channels, K = kernel rows x (kernel columns x

@@ -52,6 +52,8 @@ SYMBOLS = {
     "decx_hip_event_elapsed_ms": (_int, [_vp, _vp, ctypes.POINTER(_f)]),
     "decx_hip_gemm_f32": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp]),
     "decx_hip_gemm_f16": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp]),
+    "decx_hip_gemm_f32_workspace": (ctypes.c_size_t, [_u32] * 3),
+    "decx_hip_gemm_f32_ws": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, ctypes.c_size_t, _vp]),
     "decx_hip_gemv_f32": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _vp]),
     "decx_hip_gemv_f16": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _int, _vp]),
     "decx_hip_gevm_f32": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _vp]),
@@ -177,8 +179,9 @@ class DeviceMatrix:
             pass
 
 
-def gemm(A, B, D, C=None, alpha=1.0, beta=1.0, stream=None, tile=TILE_AUTO, force_edge=False):
-    """D = A.B or fma(C, beta, alpha*A.B) on DeviceMatrix operands through the C ABI."""
+def gemm(A, B, D, C=None, alpha=1.0, beta=1.0, stream=None, tile=TILE_AUTO, force_edge=False, workspace=None):
+    """D = A.B or fma(C, beta, alpha*A.B) on DeviceMatrix operands through the C ABI.  workspace: a DeviceMatrix the
+    fp32 product may split K through (decx_hip_gemm_f32_ws)."""
     assert A.dtype == B.dtype == D.dtype
     M, K, N = A.rows, A.cols, B.cols
     assert B.rows == K and D.rows == M and D.cols == N
@@ -204,7 +207,9 @@ def gemm(A, B, D, C=None, alpha=1.0, beta=1.0, stream=None, tile=TILE_AUTO, forc
         else:
             check(L.decx_hip_gemm_f64_tile(*args, tile, 1 if force_edge else 0), "gemm")
         return
-    if tile == TILE_AUTO and not force_edge:
+    if workspace is not None and A.dtype == np.float32 and tile == TILE_AUTO and not force_edge:
+        rc = L.decx_hip_gemm_f32_ws(*args[:-1], workspace.ptr, workspace.rows * workspace.pitch * workspace.dtype.itemsize, stream)
+    elif tile == TILE_AUTO and not force_edge:
         rc = (L.decx_hip_gemm_f16 if f16 else L.decx_hip_gemm_f32)(*args)
     else:
         rc = (L.decx_hip_gemm_f16_tile if f16 else L.decx_hip_gemm_f32_tile)(*args, tile, 1 if force_edge else 0)

@@ -533,8 +533,22 @@ bool validate(const decx::_GPU_Matrix* A, const decx::_GPU_Matrix* B, const decx
     return true;
 }
 
-// workspace of the complex forms (the real expansion of B), kept between calls; guarded by the module mutex
+// device workspace kept between calls (the real expansion of B of the complex forms, the partial products of
+// a split K); grow-only, guarded by the module mutex
 std::shared_ptr<decx::DeviceBlock>& complex_workspace() { static std::shared_ptr<decx::DeviceBlock> w; return w; }
+bool ensure_workspace(size_t need, de::DH* h)
+{
+    std::shared_ptr<decx::DeviceBlock>& ws = complex_workspace();
+    if (ws && ws->bytes >= need) return true;
+    auto block = std::make_shared<decx::DeviceBlock>();
+    block->bytes = need ? need : 64;
+    if (decx_hip_malloc(&block->ptr, block->bytes) != DECX_HIP_OK) {
+        block->ptr = nullptr;
+        decx::err::set(h, decx::DECX_FAIL_CUDA_ALLOCATION, kDevAllocFail); return false;
+    }
+    ws = block;
+    return true;
+}
 
 struct Scalar { double re, im; };
 
@@ -552,16 +566,8 @@ bool gemm_device(decx::_GPU_Matrix* A, decx::_GPU_Matrix* B, decx::_GPU_Matrix* 
     if (A->Type() == de::_COMPLEX_F32_ || A->Type() == de::_COMPLEX_F64_) {
         const bool single = A->Type() == de::_COMPLEX_F32_;
         const size_t need = decx_hip_gemm_complex_workspace(single ? 4 : 8, B->Width(), A->Width());
+        if (!ensure_workspace(need, h)) return false;
         std::shared_ptr<decx::DeviceBlock>& ws = complex_workspace();
-        if (!ws || ws->bytes < need) {
-            auto block = std::make_shared<decx::DeviceBlock>();
-            block->bytes = need ? need : 64;
-            if (decx_hip_malloc(&block->ptr, block->bytes) != DECX_HIP_OK) {
-                block->ptr = nullptr;
-                decx::err::set(h, decx::DECX_FAIL_CUDA_ALLOCATION, kDevAllocFail); return false;
-            }
-            ws = block;
-        }
         rc = single ? decx_hip_gemm_c32((const float*)A->data(), (const float*)B->data(), (const float*)c_ptr, (float*)dst->data(),
                                         A->Height(), B->Width(), A->Width(), A->Pitch(), B->Pitch(), ldc, dst->Pitch(),
                                         (float)alpha_c.re, (float)alpha_c.im, (float)beta_c.re, (float)beta_c.im, ws->ptr, ws->bytes, S)
@@ -569,10 +575,15 @@ bool gemm_device(decx::_GPU_Matrix* A, decx::_GPU_Matrix* B, decx::_GPU_Matrix* 
                                         A->Height(), B->Width(), A->Width(), A->Pitch(), B->Pitch(), ldc, dst->Pitch(),
                                         alpha_c.re, alpha_c.im, beta_c.re, beta_c.im, ws->ptr, ws->bytes, S);
     }
-    else if (A->Type() == de::_FP32_)
-        rc = decx_hip_gemm_f32((const float*)A->data(), (const float*)B->data(), (const float*)c_ptr,
-                               (float*)dst->data(), A->Height(), B->Width(), A->Width(),
-                               A->Pitch(), B->Pitch(), ldc, dst->Pitch(), (float)alpha, (float)beta, S);
+    else if (A->Type() == de::_FP32_) {
+        // few output tiles and a long K: the product may split K through the module's workspace
+        const size_t need = decx_hip_gemm_f32_workspace(A->Height(), B->Width(), A->Width());
+        if (need && !ensure_workspace(need, h)) return false;
+        rc = decx_hip_gemm_f32_ws((const float*)A->data(), (const float*)B->data(), (const float*)c_ptr,
+                                  (float*)dst->data(), A->Height(), B->Width(), A->Width(),
+                                  A->Pitch(), B->Pitch(), ldc, dst->Pitch(), (float)alpha, (float)beta,
+                                  need ? complex_workspace()->ptr : nullptr, need ? complex_workspace()->bytes : 0, S);
+    }
     else if (A->Type() == de::_FP64_)
         rc = decx_hip_gemm_f64((const double*)A->data(), (const double*)B->data(), (const double*)c_ptr,
                                (double*)dst->data(), A->Height(), B->Width(), A->Width(),

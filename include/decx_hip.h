@@ -112,6 +112,20 @@ DECX_HIP_API int decx_hip_gemm_f32(const float* A, const float* B, const float* 
                                    uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
                                    float alpha, float beta, void* stream);
 
+/* The same product with a device workspace the library may use to split K: when the output has too few tiles to
+ * occupy the chip and K is long (e.g. 300 x 300 x 8192), several workgroups share a tile, each multiplying a
+ * range of K into a partial product in the workspace, and a second kernel adds the partial products in a fixed
+ * order (results do not vary from run to run).  decx_hip_gemm_f32_workspace returns the bytes that make the
+ * split possible for a shape (0: the plain kernel is used anyway); a smaller or null workspace is never an
+ * error.  The workspace must be 16-byte aligned and is free again when the call's work on `stream` is done.
+ * Plays the part of the scratch the reference's planner keeps for itself (cuda_GEMM_LS_planner: the transposed
+ * A, srcs/modules/BLAS/GEMM/CUDA/large_squares/common/cuda_GEMM_LS_planner.cu:95-160). */
+DECX_HIP_API size_t decx_hip_gemm_f32_workspace(uint32_t M, uint32_t N, uint32_t K);
+DECX_HIP_API int decx_hip_gemm_f32_ws(const float* A, const float* B, const float* C, float* D,
+                                      uint32_t M, uint32_t N, uint32_t K,
+                                      uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                                      float alpha, float beta, void* workspace, size_t workspace_bytes, void* stream);
+
 /* fp16 in, fp32 accumulate, one rounding to fp16 out.  Replaces the kernels launched by
  * cuda_GEMM_LS_planner<de::Half>::run (large_squares/fp16/GEMM_fp16_callers.cu:57-124). */
 DECX_HIP_API int decx_hip_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,

@@ -248,6 +248,52 @@ def test_row_pitch_of_16_mib_takes_the_register_staged_kernels(hip, oracle, dtyp
         assert rel_err(run(hip, A, B, tile=tile, pitches=(pitch_a, pn, pn, pn)), ref, K) <= tol
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 300, 8192), (64, 64, 4099), (130, 70, 2500), (512, 512, 1024), (33, 1000, 3000)])
+def test_f32_split_k_through_a_workspace(hip, oracle, M, N, K):
+    """Few output tiles and a long K: with a workspace the product is split along K and the partial products are added
+    in a fixed order.  Parity with the oracle, identical results from run to run, C / alpha / beta, untouched padding,
+    and a workspace that is too small simply means no split."""
+    A = synth.uniform_f32(M, K, 151); B = synth.uniform_f32(K, N, 152); C = synth.uniform_f32(M, N, 153)
+    need = hip.lib().decx_hip_gemm_f32_workspace(M, N, K)
+    assert need > 0 and need % 16 == 0
+    ws = hip.DeviceMatrix(1, need // 4, np.float32)
+    ws.upload_raw(np.full((1, ws.pitch), np.nan, np.float32))            # partial products never read what they did not write
+    pa, pn = device_pitch(K, np.float32), device_pitch(N, np.float32)
+
+    def product(c, alpha, beta, workspace):
+        dA = hip.DeviceMatrix(M, K, np.float32, pa, A, pad_value=np.nan); dB = hip.DeviceMatrix(K, N, np.float32, pn, B, pad_value=np.nan)
+        dC = hip.DeviceMatrix(M, N, np.float32, pn, c, pad_value=np.nan) if c is not None else None
+        dD = hip.DeviceMatrix(M, N, np.float32, pn)
+        dD.upload_raw(np.full((M, pn), -12345.0, np.float32))
+        hip.gemm(dA, dB, dD, dC, alpha, beta, workspace=workspace)
+        hip.sync()
+        raw = dD.download_raw()
+        for d in (dA, dB, dC, dD):
+            if d is not None:
+                d.free()
+        assert np.all(raw[:, N:] == np.float32(-12345.0))
+        return raw[:, :N].copy()
+
+    first = product(None, 1.0, 1.0, ws)
+    assert rel_err(first, oracle.gemm_f32(A, B), K) <= TOL_F32
+    assert np.array_equal(first, product(None, 1.0, 1.0, ws))             # fixed summation order
+    assert rel_err(product(C, 1.5, -0.5, ws), oracle.gemm_f32(A, B, C, 1.5, -0.5), K) <= TOL_F32
+    plain = product(None, 1.0, 1.0, None)
+    assert rel_err(plain, oracle.gemm_f32(A, B), K) <= TOL_F32
+    small = hip.DeviceMatrix(1, 64, np.float32)
+    assert np.array_equal(product(None, 1.0, 1.0, small), plain)          # too small: the plain kernel runs
+    for d in (ws, small):
+        d.free()
+
+
+def test_f32_split_k_is_planned_only_where_it_pays(hip):
+    L = hip.lib()
+    assert L.decx_hip_gemm_f32_workspace(8192, 8192, 8192) == 0           # enough tiles
+    assert L.decx_hip_gemm_f32_workspace(300, 300, 512) == 0              # K too short to cut
+    assert L.decx_hip_gemm_f32_workspace(8192, 1, 8192) == 0 and L.decx_hip_gemm_f32_workspace(1, 8192, 8192) == 0
+    assert L.decx_hip_gemm_f32_workspace(0, 5, 5000) == 0
+
+
 @pytest.mark.parametrize("tile", [0, 1, 2])
 def test_forced_edge_variant_equals_fast_variant(hip, tile):
     """On tile-multiple shapes the predicated kernel and the unpredicated one run the same
