@@ -74,20 +74,25 @@ template <int TN> __device__ __forceinline__ float lane_of(const typename BFrag<
 
 // CONV: 0 plain GEMM; 1 convolution, every copy lane walks the image on its own; 2 convolution whose runs of
 // contiguous bytes are whole slabs, so that all lanes hop to the next image row in the same slab.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, int CONV = 0>
+// SPLIT: grid.y workgroups share each tile, each with its own range of K (a separate instantiation, so that the
+// plain kernel keeps reading its arguments straight from the kernel-argument segment).
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, int CONV = 0, bool SPLIT = false>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_f32_dma_kernel(const GemmArgs g_in)
 {
-    GemmArgs g = g_in;
-    if (CONV == 0 && g.split_len) {                        // this workgroup's share of K and its partial product
-        const uint32_t k0 = blockIdx.y * g.split_len;
-        g.A = (const unsigned char*)g.A + (size_t)k0 * 4;
-        g.B = (const unsigned char*)g.B + (size_t)k0 * g.ldb * 4;
-        g.K = g.K - k0 < g.split_len ? g.K - k0 : g.split_len;
-        g.D = g.split_ws + (size_t)blockIdx.y * g.split_stride;
-        g.ldd = g.split_ldd;
-        g.C = nullptr;
+    struct Nothing {};
+    std::conditional_t<SPLIT, GemmArgs, Nothing> g_split;
+    if constexpr (SPLIT) {                                 // this workgroup's share of K and its partial product
+        g_split = g_in;
+        const uint32_t k0 = blockIdx.y * g_in.split_len;
+        g_split.A = (const unsigned char*)g_in.A + (size_t)k0 * 4;
+        g_split.B = (const unsigned char*)g_in.B + (size_t)k0 * g_in.ldb * 4;
+        g_split.K = g_in.K - k0 < g_in.split_len ? g_in.K - k0 : g_in.split_len;
+        g_split.D = g_in.split_ws + (size_t)blockIdx.y * g_in.split_stride;
+        g_split.ldd = g_in.split_ldd;
+        g_split.C = nullptr;
     }
+    const GemmArgs& g = [&]() -> const GemmArgs& { if constexpr (SPLIT) return g_split; else return g_in; }();
     constexpr int WAVES = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
     constexpr int CPR = BK / 4, RP = 16 / CPR;                    // A chunks per row, rows per 256 bytes
@@ -474,8 +479,15 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
     g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
-    const uint32_t splits = (CONV == 0 && g.split_len) ? (g.K + g.split_len - 1) / g.split_len : 1u;
-    hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD, CONV>), dim3(nb, splits),
+    if constexpr (CONV == 0) {
+        if (g.split_len) {
+            const uint32_t splits = (g.K + g.split_len - 1) / g.split_len;
+            hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD, 0, true>), dim3(nb, splits),
+                               dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
+            return (int)hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD, CONV>), dim3(nb),
                        dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
     return (int)hipGetLastError();
 }
