@@ -122,7 +122,7 @@ CONV = {"W": 256, "H": 256, "C": 112, "OC": 256, "KW": 3, "KH": 3}     # 64 516 
 
 def run_conv(steps, warmup, settle_s=0.25):
     """fp32 3 x 3 convolution of a 256 x 256 x 112 image with 256 kernels through decx_hip_conv2d_f32 (implicit GEMM,
-    operands resident): the workload BASELINE's tall-skinny GEMM shape stands for."""
+    operands resident): the workload the tall-skinny GEMM shape 65536 x 256 x 1024 stands for."""
     from decx_amd import hip, synth
     c = CONV
     L = hip.lib()

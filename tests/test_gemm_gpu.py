@@ -90,7 +90,7 @@ def test_golden_f16(hip, path):
         assert rel_err(got, g["D"].view(np.float16), K) <= TOL_F16, (path, tile)
 
 
-# ------------------------------------------------------------------ BASELINE configs, full or sampled
+# ------------------------------------------------------------------ the benchmark configurations, full or sampled
 
 def sample_rows(M, count, seed):
     rng = np.random.default_rng(seed)
