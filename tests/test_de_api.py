@@ -144,6 +144,7 @@ def test_vector_forms_through_the_objects_match_oracle(oracle, dt, form, W, H, l
     ("f32", 1000, 1500, 777, 2, 1),        # C is dst
     ("f32", 5000, 300, 260, 2, 0),         # 10 panels of 512 rows, the last one ragged
     ("f32", 100, 70, 33, 1, 0),            # a single panel
+    ("f32", 4100, 2300, 4700, 1, 0),       # pageable operands larger than the ring of bounce buffers (B: 43 MB)
     ("f16", 1300, 520, 515, 0, 1),
     ("f16", 1300, 520, 515, 2, 0),
     ("f64", 700, 300, 129, 1, 1),
