@@ -130,13 +130,15 @@ __host__ inline TileInfo tile_info_f16(int shape, bool aligned = true)
     }
 }
 
-// fp64, measured at 4096^3: 72.5 : 59.6 : 60.0 TFLOP/s.  TILE_256x256 stands for the largest fp64 tile, 256 x 128.
+// fp64 (TFLOP/s per CU): 256 x 128 (what TILE_256x256 stands for) 0.283 alone or full; 128 x 128 0.27 alone or two per
+// CU; 64 x 64 0.22 alone (1024^3), 0.27 two per CU (3072^3).  All three run 8 wavefronts per workgroup: with 4, the
+// two smaller tiles reach 0.24 (their accumulators leave no room for the four workgroups per CU that the fp32 tiles use).
 __host__ inline TileInfo tile_info_f64(int shape)
 {
     switch (shape) {
     case TILE_256x256: return {256, 128, 512, 1, 1.00f, 1.00f};
-    case TILE_128x128: return {128, 128, 256, 2, 0.83f, 0.75f};
-    default:           return { 64,  64, 256, 2, 0.83f, 0.60f};
+    case TILE_128x128: return {128, 128, 512, 2, 0.96f, 0.96f};
+    default:           return { 64,  64, 512, 2, 0.95f, 0.77f};
     }
 }
 
