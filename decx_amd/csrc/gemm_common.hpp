@@ -125,7 +125,7 @@ __host__ inline TileInfo tile_info_f16(int shape, bool aligned = true)
 {
     switch (shape) {
     case TILE_256x256: return {256, 256, aligned ? 512 : 256, 1, 1.00f, aligned ? 1.38f : 1.00f};
-    case TILE_128x128: return {128, 128, aligned ? 256 : 128, 2, aligned ? 0.84f : 0.60f, aligned ? 0.67f : 0.50f};
+    case TILE_128x128: return {128, 128, aligned ? 512 : 128, 2, aligned ? 0.84f : 0.60f, aligned ? 0.70f : 0.50f};
     default:           return { 64,  64, aligned ? 256 :  64, aligned ? 4 : 2, aligned ? 0.55f : 0.25f, aligned ? 0.27f : 0.12f};
     }
 }

@@ -356,9 +356,10 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
 //     8192^3); 4 wavefronts of 128 x 128 reach 1075-1124, 16 wavefronts 1144, 32-deep slabs 1100-1124.
 //     Two wavefronts per SIMD take turns on the matrix pipe while the other waits for LDS or the barrier.
 //     Spreading the direct loads over the k steps, or raising the wave priority around the MFMAs, is 3-4 % slower.
-//   128 x 128: 4 wavefronts of 64 x 64, 64-deep slabs; a ring of 4 stages when there is at most one workgroup
-//     per CU (741 TFLOP/s at 2048^3), else of 2 stages so that two workgroups share a CU (4096^3: 994 against
-//     940 with 32-deep slabs in 4 stages, 6144^3: 1035 against 960).
+//   128 x 128: 8 wavefronts of 64 x 32 (1536^3: 526 TFLOP/s against 453 with 4 of 64 x 64; the same from 2560^3 up),
+//     64-deep slabs; a ring of 4 stages when there is at most one workgroup per CU (784 TFLOP/s at 2048^3), else of
+//     2 stages so that two workgroups share a CU (4096^3: 994 against 940 with 32-deep slabs in 4 stages, 6144^3:
+//     1035 against 960).
 //   64 x 64: 4 wavefronts of 32 x 32, 64-deep slabs in 4 stages (327 TFLOP/s at 1024^3), in 2 stages once more
 //     than two workgroups per CU are there to hide the copies (1536^3: 447 against 388).
 int launch_gemm_f16_dma(int shape, const GemmArgs& args, hipStream_t stream)
@@ -367,8 +368,8 @@ int launch_gemm_f16_dma(int shape, const GemmArgs& args, hipStream_t stream)
     case TILE_256x256: return launch_dma<256, 256, 2, 4, 64, 2>(args, stream);
     case TILE_128x128: {
         const uint64_t blocks = (uint64_t)((args.M + 127) / 128) * ((args.N + 127) / 128);
-        return blocks <= 256 ? launch_dma<128, 128, 2, 2, 64, 4>(args, stream)
-                             : launch_dma<128, 128, 2, 2, 64, 2>(args, stream);
+        return blocks <= 256 ? launch_dma<128, 128, 2, 4, 64, 4>(args, stream)
+                             : launch_dma<128, 128, 2, 4, 64, 2>(args, stream);
     }
     case TILE_64x64: {
         const uint64_t blocks = (uint64_t)((args.M + 63) / 64) * ((args.N + 63) / 64);
