@@ -59,12 +59,28 @@ int check_gemm(const void* A, const void* B, const void* C, const void* D, uint3
     return DECX_HIP_OK;
 }
 
-// Split K is planned for fp32 products on 16-byte aligned operands whose tiles would leave most CUs idle
-SplitPlan split_plan_f32(uint32_t M, uint32_t N, uint32_t K)
+// Split K is planned for products on 16-byte aligned operands whose tiles would leave most CUs idle.
+// elem_bytes: 2, 4 or 8.
+SplitPlan split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
 {
-    if (M <= 1 || N <= 1) return {1, 0};                   // the vector corners have their own kernels
-    const TileInfo ti = tile_info_f32(choose_tile(false, M, N, true), true);
+    if (M == 0 || N == 0) return {1, 0};
+    if (elem_bytes != 8 && (M == 1 || N == 1)) return {1, 0};      // the vector corners have their own kernels
+    const TileInfo ti = elem_bytes == 8 ? tile_info_f64(choose_tile_f64(M, N))
+                                        : elem_bytes == 2 ? tile_info_f16(choose_tile(true, M, N, true), true)
+                                                          : tile_info_f32(choose_tile(false, M, N, true), true);
     return plan_split_k((uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn), K, g_dev.compute_units);
+}
+
+// Fills the split fields of g when the plan says so and the workspace is large enough; returns the number of splits.
+uint32_t arm_split(GemmArgs& g, int elem_bytes, void* workspace, size_t workspace_bytes)
+{
+    if (!workspace || !aligned16(workspace)) return 1;
+    const SplitPlan sp = split_plan(elem_bytes, g.M, g.N, g.K);
+    const uint32_t ldw = (g.N + 3) / 4 * 4;
+    const size_t part = (size_t)(elem_bytes == 8 ? 8 : 4);
+    if (sp.splits <= 1 || workspace_bytes < (size_t)sp.splits * g.M * ldw * part) return 1;
+    g.split_len = sp.len; g.split_ldd = ldw; g.split_stride = (uint64_t)g.M * ldw; g.split_ws = workspace;
+    return sp.splits;
 }
 
 template <bool F16>
@@ -94,13 +110,11 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
                 lda % per16 == 0 && ldb % per16 == 0 && ldd % per16 == 0 && (!C || ldc % per16 == 0)) ? 1u : 0u;
     const int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile(F16, M, N, g.vec_ok != 0) : tile;
     const bool edge = force_edge != 0 || K == 0;
-    if (!F16 && workspace && tile == DECX_HIP_TILE_AUTO && !edge && g.vec_ok && dma_offsets_fit(g, 4) && aligned16(workspace)) {
-        const SplitPlan sp = split_plan_f32(M, N, K);
-        const uint32_t ldw = (N + 3) / 4 * 4;
-        if (sp.splits > 1 && workspace_bytes >= (size_t)sp.splits * M * ldw * 4) {
-            g.split_len = sp.len; g.split_ldd = ldw; g.split_stride = (uint64_t)M * ldw; g.split_ws = (float*)workspace;
-            const int rl = launch_gemm_f32(shape, false, g, as_stream(stream));
-            return rl != 0 ? rl : launch_split_reduce_f32(g, sp.splits, as_stream(stream));
+    if (workspace && tile == DECX_HIP_TILE_AUTO && !edge && g.vec_ok && dma_offsets_fit(g, F16 ? 2 : 4)) {
+        const uint32_t splits = arm_split(g, F16 ? 2 : 4, workspace, workspace_bytes);
+        if (splits > 1) {
+            const int rl = F16 ? launch_gemm_f16(shape, false, g, as_stream(stream)) : launch_gemm_f32(shape, false, g, as_stream(stream));
+            return rl != 0 ? rl : launch_split_reduce(F16 ? 2 : 4, g, splits, as_stream(stream));
         }
     }
     return F16 ? launch_gemm_f16(shape, edge, g, as_stream(stream))
@@ -268,12 +282,14 @@ int decx_hip_gemm_f32(const float* A, const float* B, const float* C, float* D, 
     return run_gemm<false>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0);
 }
 
-size_t decx_hip_gemm_f32_workspace(uint32_t M, uint32_t N, uint32_t K)
+size_t decx_hip_gemm_workspace(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
 {
-    if (!g_dev.ready || M == 0 || N == 0) return 0;
-    const SplitPlan sp = split_plan_f32(M, N, K);
-    return sp.splits > 1 ? (size_t)sp.splits * M * ((N + 3) / 4 * 4) * 4 : 0;
+    if (!g_dev.ready || (elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8)) return 0;
+    const SplitPlan sp = split_plan(elem_bytes, M, N, K);
+    return sp.splits > 1 ? (size_t)sp.splits * M * ((N + 3) / 4 * 4) * (elem_bytes == 8 ? 8 : 4) : 0;
 }
+
+size_t decx_hip_gemm_f32_workspace(uint32_t M, uint32_t N, uint32_t K) { return decx_hip_gemm_workspace(4, M, N, K); }
 
 int decx_hip_gemm_f32_ws(const float* A, const float* B, const float* C, float* D, uint32_t M, uint32_t N, uint32_t K,
                          uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha, float beta,
@@ -281,6 +297,14 @@ int decx_hip_gemm_f32_ws(const float* A, const float* B, const float* C, float* 
 {
     return run_gemm<false>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0, workspace,
                            workspace_bytes);
+}
+
+int decx_hip_gemm_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, uint32_t M, uint32_t N,
+                         uint32_t K, uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha, float beta,
+                         void* workspace, size_t workspace_bytes, void* stream)
+{
+    return run_gemm<true>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0, workspace,
+                          workspace_bytes);
 }
 
 int decx_hip_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, uint32_t M, uint32_t N,
@@ -292,7 +316,7 @@ int decx_hip_gemm_f16(const uint16_t* A, const uint16_t* B, const uint16_t* C, u
 
 static int run_gemm_f64(const double* A, const double* B, const double* C, double* D, uint32_t M, uint32_t N, uint32_t K,
                         uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, double alpha, double beta, void* stream,
-                        int tile, int force_plain)
+                        int tile, int force_plain, void* workspace = nullptr, size_t workspace_bytes = 0)
 {
     if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
     const int rc = check_gemm(A, B, C, D, M, N, K, lda, ldb, ldc, ldd);
@@ -308,6 +332,13 @@ static int run_gemm_f64(const double* A, const double* B, const double* C, doubl
     g.vec_ok = (aligned16(A) && aligned16(B) && aligned16(D) && (!C || aligned16(C)) &&
                 lda % 2 == 0 && ldb % 2 == 0 && ldd % 2 == 0 && (!C || ldc % 2 == 0)) ? 1u : 0u;
     const int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile_f64(M, N) : tile;
+    if (workspace && tile == DECX_HIP_TILE_AUTO && !force_plain && K > 0 && g.vec_ok && dma_offsets_fit(g, 8)) {
+        const uint32_t splits = arm_split(g, 8, workspace, workspace_bytes);
+        if (splits > 1) {
+            const int rl = launch_gemm_f64(shape, false, g, as_stream(stream));
+            return rl != 0 ? rl : launch_split_reduce(8, g, splits, as_stream(stream));
+        }
+    }
     return launch_gemm_f64(shape, force_plain != 0, g, as_stream(stream));
 }
 
@@ -315,6 +346,14 @@ int decx_hip_gemm_f64(const double* A, const double* B, const double* C, double*
                       uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, double alpha, double beta, void* stream)
 {
     return run_gemm_f64(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0);
+}
+
+int decx_hip_gemm_f64_ws(const double* A, const double* B, const double* C, double* D, uint32_t M, uint32_t N, uint32_t K,
+                         uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, double alpha, double beta,
+                         void* workspace, size_t workspace_bytes, void* stream)
+{
+    return run_gemm_f64(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0, workspace,
+                        workspace_bytes);
 }
 
 int decx_hip_gemm_f64_tile(const double* A, const double* B, const double* C, double* D, uint32_t M, uint32_t N,

@@ -29,13 +29,14 @@ struct GemmArgs {
     uint32_t tiles_m, tiles_n;   // number of block tiles along M and N
     uint32_t xcd_remap;          // 1: grid size is a multiple of 8, use the per-XCD ordering
     uint32_t vec_ok;             // 1: every base pointer is 16-byte aligned and every pitch a multiple of 16 bytes
-    // Split K (fp32 direct-load kernels, grid.y = number of splits): split z multiplies k in [z * split_len,
-    // min(K, (z + 1) * split_len)) and writes its M x N partial product, pitch split_ldd, to
-    // split_ws + z * split_stride floats; a second kernel adds the partial products in split order.
+    // Split K (direct-load kernels, grid.y = number of splits): split z multiplies k in [z * split_len,
+    // min(K, (z + 1) * split_len)) and writes its M x N partial product (fp32 for fp32 and fp16 operands, fp64
+    // for fp64), pitch split_ldd, to split_ws + z * split_stride elements; a second kernel adds the partial
+    // products in split order.
     uint32_t split_len;          // 0: no split
     uint32_t split_ldd;
     uint64_t split_stride;
-    float*   split_ws;
+    void*    split_ws;
     // Convolution as an implicit GEMM (used by the CONV instantiations only): row p of the A operand is the
     // patch under output pixel (p / conv_wout, p % conv_wout) of an image stored [row][column][channel]; its K
     // elements are KH runs of conv_seg_bytes contiguous bytes (KW columns x channel pitch), conv_seg_stride bytes
@@ -154,8 +155,9 @@ inline bool dma_offsets_fit(const GemmArgs& g, uint32_t elem_bytes)
 int launch_gemm_f64(int shape, bool plain, const GemmArgs& args, hipStream_t stream);
 // direct-to-LDS fp32 kernel for any M, N, K >= 1 on 16-byte aligned bases and pitches, in the three tile shapes
 int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream);
-// D = sum over splits of the partial products (in split order), then fma(C, beta, alpha * sum) when C is given
-int launch_split_reduce_f32(const GemmArgs& args, uint32_t splits, hipStream_t stream);
+// D = sum over splits of the partial products (in split order), then fma(C, beta, alpha * sum) when C is given;
+// elem_bytes 2 (fp32 partial products, fp16 C and D), 4 or 8
+int launch_split_reduce(int elem_bytes, const GemmArgs& args, uint32_t splits, hipStream_t stream);
 
 // Split K pays when the tiles alone would leave most CUs without work and K is long enough to cut: aim at two
 // workgroups per CU, pieces of at least 256 and a multiple of 32 (the deepest slab).

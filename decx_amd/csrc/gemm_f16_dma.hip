@@ -78,10 +78,21 @@ template <int MFMAS, int READS> __device__ __forceinline__ void interleave()
 
 }  // namespace
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES>
+// SPLIT: grid.y workgroups share each tile, each with its own range of K, writing its partial product in fp32.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool SPLIT = false>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
-gemm_f16_dma_kernel(const GemmArgs g)
+gemm_f16_dma_kernel(const GemmArgs g_in)
 {
+    struct Nothing {};
+    std::conditional_t<SPLIT, GemmArgs, Nothing> g_split;
+    if constexpr (SPLIT) {
+        g_split = g_in;
+        const uint32_t k0 = blockIdx.y * g_in.split_len;
+        g_split.A = (const unsigned char*)g_in.A + (size_t)k0 * 2;
+        g_split.B = (const unsigned char*)g_in.B + (size_t)k0 * g_in.ldb * 2;
+        g_split.K = g_in.K - k0 < g_in.split_len ? g_in.K - k0 : g_in.split_len;
+    }
+    const GemmArgs& g = [&]() -> const GemmArgs& { if constexpr (SPLIT) return g_split; else return g_in; }();
     constexpr int WAVES = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
     constexpr int RB = BK * 2, CPR = RB / 16, RPB = 16 / CPR;         // A row bytes, chunks per row, rows per 256 bytes
@@ -279,6 +290,26 @@ gemm_f16_dma_kernel(const GemmArgs g)
     // Epilogue.  Lane (l32, h) holds output row l32 of the m tile; register 4 q + e is column
     // 8 q + 4 h + e of the n tile.  Interior tiles: `v_permlane32_swap` trades the halves of an even
     // and an odd 8-column group between lane l and lane l + 32, after which each lane stores 16 bytes.
+    if constexpr (SPLIT) {                                 // the fp32 partial product of this range of K
+        float* __restrict__ P = (float*)g.split_ws + (size_t)blockIdx.y * g.split_stride;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const uint32_t row = m0 + wm0 + 32 * i + l32;
+            if (row < g.M) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const uint32_t col = n0 + wn0 + 32 * j + 8 * q + 4 * h;
+                        // split_ldd is a multiple of 4 and col a multiple of 4: whole 16-byte pieces lie inside the pitch
+                        if (col < g.split_ldd)
+                            *(floatx4*)(P + (size_t)row * g.split_ldd + col) =
+                                floatx4{accT[j][i][4 * q], accT[j][i][4 * q + 1], accT[j][i][4 * q + 2], accT[j][i][4 * q + 3]};
+                    }
+            }
+        }
+        return;
+    }
     const _Float16* __restrict__ C = (const _Float16*)g.C;
     _Float16* __restrict__ D = (_Float16*)g.D;
     auto pack2 = [](float lo, float hi) -> uint32_t {
@@ -344,6 +375,12 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
     g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
+    if (g.split_len) {
+        const uint32_t splits = (g.K + g.split_len - 1) / g.split_len;
+        hipLaunchKernelGGL((gemm_f16_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, true>), dim3(nb, splits),
+                           dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
+        return (int)hipGetLastError();
+    }
     hipLaunchKernelGGL((gemm_f16_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES>), dim3(nb), dim3(WAVES_M * WAVES_N * 64),
                        0, stream, g);
     return (int)hipGetLastError();

@@ -88,7 +88,7 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
         g_split.A = (const unsigned char*)g_in.A + (size_t)k0 * 4;
         g_split.B = (const unsigned char*)g_in.B + (size_t)k0 * g_in.ldb * 4;
         g_split.K = g_in.K - k0 < g_in.split_len ? g_in.K - k0 : g_in.split_len;
-        g_split.D = g_in.split_ws + (size_t)blockIdx.y * g_in.split_stride;
+        g_split.D = (float*)g_in.split_ws + (size_t)blockIdx.y * g_in.split_stride;
         g_split.ldd = g_in.split_ldd;
         g_split.C = nullptr;
     }
@@ -445,28 +445,32 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
 
 namespace {
 
-// one thread per four columns: D = sum of the partial products in split order (+ the C term)
-__global__ void __launch_bounds__(256) split_reduce_f32_kernel(const GemmArgs g, uint32_t splits)
+// one thread per four columns: D = sum of the partial products in split order (+ the C term).  TA: type of the
+// partial products and of the arithmetic, TO: type of C and D.
+template <typename TA, typename TO>
+__global__ void __launch_bounds__(256) split_reduce_kernel(const GemmArgs g, uint32_t splits, TA alpha, TA beta)
 {
     const uint32_t quads = g.split_ldd / 4;
     const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (uint64_t)g.M * quads) return;
     const uint32_t row = (uint32_t)(idx / quads), col = (uint32_t)(idx % quads) * 4;
-    const float* p = g.split_ws + (size_t)row * g.split_ldd + col;
-    floatx4 sum = *(const floatx4*)p;
-    for (uint32_t z = 1; z < splits; ++z) {
-        const floatx4 v = *(const floatx4*)(p + (size_t)z * g.split_stride);
+    const TA* p = (const TA*)g.split_ws + (size_t)row * g.split_ldd + col;
+    TA sum[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) sum[e] += v[e];
+    for (int e = 0; e < 4; ++e) sum[e] = p[e];
+    for (uint32_t z = 1; z < splits; ++z) {
+        const TA* q = p + (size_t)z * g.split_stride;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sum[e] += q[e];
     }
-    const float* C = (const float*)g.C;
-    float* D = (float*)g.D;
+    const TO* C = (const TO*)g.C;
+    TO* D = (TO*)g.D;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         if (col + e < g.N) {
-            float o = sum[e];
-            if (C) o = __builtin_fmaf(C[(size_t)row * g.ldc + col + e], g.beta, g.alpha * o);
-            D[(size_t)row * g.ldd + col + e] = o;
+            TA o = sum[e];
+            if (C) o = __builtin_fma((TA)C[(size_t)row * g.ldc + col + e], beta, alpha * o);
+            D[(size_t)row * g.ldd + col + e] = (TO)o;
         }
     }
 }
@@ -515,10 +519,16 @@ int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
     }
 }
 
-int launch_split_reduce_f32(const GemmArgs& args, uint32_t splits, hipStream_t stream)
+int launch_split_reduce(int elem_bytes, const GemmArgs& args, uint32_t splits, hipStream_t stream)
 {
     const uint64_t threads = (uint64_t)args.M * (args.split_ldd / 4);
-    hipLaunchKernelGGL(split_reduce_f32_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, args, splits);
+    const dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+    if (elem_bytes == 8)
+        hipLaunchKernelGGL((split_reduce_kernel<double, double>), grid, block, 0, stream, args, splits, args.alpha64, args.beta64);
+    else if (elem_bytes == 2)
+        hipLaunchKernelGGL((split_reduce_kernel<float, _Float16>), grid, block, 0, stream, args, splits, args.alpha, args.beta);
+    else
+        hipLaunchKernelGGL((split_reduce_kernel<float, float>), grid, block, 0, stream, args, splits, args.alpha, args.beta);
     return (int)hipGetLastError();
 }
 

@@ -45,10 +45,24 @@ template <int N> __device__ __forceinline__ void wait_loads_and_barrier()
 
 }  // namespace
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES>
+// SPLIT: grid.y workgroups share each tile, each with its own range of K, writing a partial product.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool SPLIT = false>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
-gemm_f64_dma_kernel(const GemmArgs g)
+gemm_f64_dma_kernel(const GemmArgs g_in)
 {
+    struct Nothing {};
+    std::conditional_t<SPLIT, GemmArgs, Nothing> g_split;
+    if constexpr (SPLIT) {
+        g_split = g_in;
+        const uint32_t k0 = blockIdx.y * g_in.split_len;
+        g_split.A = (const unsigned char*)g_in.A + (size_t)k0 * 8;
+        g_split.B = (const unsigned char*)g_in.B + (size_t)k0 * g_in.ldb * 8;
+        g_split.K = g_in.K - k0 < g_in.split_len ? g_in.K - k0 : g_in.split_len;
+        g_split.D = (double*)g_in.split_ws + (size_t)blockIdx.y * g_in.split_stride;
+        g_split.ldd = g_in.split_ldd;
+        g_split.C = nullptr;
+    }
+    const GemmArgs& g = [&]() -> const GemmArgs& { if constexpr (SPLIT) return g_split; else return g_in; }();
     constexpr int WAVES = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 16, TN = WN / 16, TP = TN / 2;
     constexpr int RBYTES = BK * 8, CPR = RBYTES / 16, RP = 16 / CPR;       // A row bytes, chunks per row, rows per 256 bytes
@@ -317,6 +331,12 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
     g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
+    if (g.split_len) {
+        const uint32_t splits = (g.K + g.split_len - 1) / g.split_len;
+        hipLaunchKernelGGL((gemm_f64_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, true>), dim3(nb, splits),
+                           dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
+        return (int)hipGetLastError();
+    }
     hipLaunchKernelGGL((gemm_f64_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES>), dim3(nb), dim3(WAVES_M * WAVES_N * 64),
                        0, stream, g);
     return (int)hipGetLastError();

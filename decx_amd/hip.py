@@ -54,6 +54,9 @@ SYMBOLS = {
     "decx_hip_gemm_f16": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp]),
     "decx_hip_gemm_f32_workspace": (ctypes.c_size_t, [_u32] * 3),
     "decx_hip_gemm_f32_ws": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, ctypes.c_size_t, _vp]),
+    "decx_hip_gemm_workspace": (ctypes.c_size_t, [_int] + [_u32] * 3),
+    "decx_hip_gemm_f16_ws": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, ctypes.c_size_t, _vp]),
+    "decx_hip_gemm_f64_ws": (_int, [_vp] * 4 + [_u32] * 7 + [ctypes.c_double, ctypes.c_double, _vp, ctypes.c_size_t, _vp]),
     "decx_hip_gemv_f32": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _vp]),
     "decx_hip_gemv_f16": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _int, _vp]),
     "decx_hip_gevm_f32": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _vp]),
@@ -202,13 +205,16 @@ def gemm(A, B, D, C=None, alpha=1.0, beta=1.0, stream=None, tile=TILE_AUTO, forc
         check(rc, "gemm")
         return
     if A.dtype == np.float64:
-        if tile == TILE_AUTO and not force_edge:
+        if workspace is not None and tile == TILE_AUTO and not force_edge:
+            check(L.decx_hip_gemm_f64_ws(*args[:-1], workspace.ptr, workspace.rows * workspace.pitch * workspace.dtype.itemsize, stream), "gemm")
+        elif tile == TILE_AUTO and not force_edge:
             check(L.decx_hip_gemm_f64(*args), "gemm")
         else:
             check(L.decx_hip_gemm_f64_tile(*args, tile, 1 if force_edge else 0), "gemm")
         return
-    if workspace is not None and A.dtype == np.float32 and tile == TILE_AUTO and not force_edge:
-        rc = L.decx_hip_gemm_f32_ws(*args[:-1], workspace.ptr, workspace.rows * workspace.pitch * workspace.dtype.itemsize, stream)
+    if workspace is not None and tile == TILE_AUTO and not force_edge:
+        fn = L.decx_hip_gemm_f16_ws if f16 else L.decx_hip_gemm_f32_ws
+        rc = fn(*args[:-1], workspace.ptr, workspace.rows * workspace.pitch * workspace.dtype.itemsize, stream)
     elif tile == TILE_AUTO and not force_edge:
         rc = (L.decx_hip_gemm_f16 if f16 else L.decx_hip_gemm_f32)(*args)
     else:

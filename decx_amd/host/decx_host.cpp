@@ -575,23 +575,26 @@ bool gemm_device(decx::_GPU_Matrix* A, decx::_GPU_Matrix* B, decx::_GPU_Matrix* 
                                         A->Height(), B->Width(), A->Width(), A->Pitch(), B->Pitch(), ldc, dst->Pitch(),
                                         alpha_c.re, alpha_c.im, beta_c.re, beta_c.im, ws->ptr, ws->bytes, S);
     }
-    else if (A->Type() == de::_FP32_) {
+    else {
         // few output tiles and a long K: the product may split K through the module's workspace
-        const size_t need = decx_hip_gemm_f32_workspace(A->Height(), B->Width(), A->Width());
+        const int eb = A->Type() == de::_FP32_ ? 4 : (A->Type() == de::_FP64_ ? 8 : 2);
+        const size_t need = decx_hip_gemm_workspace(eb, A->Height(), B->Width(), A->Width());
         if (need && !ensure_workspace(need, h)) return false;
-        rc = decx_hip_gemm_f32_ws((const float*)A->data(), (const float*)B->data(), (const float*)c_ptr,
-                                  (float*)dst->data(), A->Height(), B->Width(), A->Width(),
-                                  A->Pitch(), B->Pitch(), ldc, dst->Pitch(), (float)alpha, (float)beta,
-                                  need ? complex_workspace()->ptr : nullptr, need ? complex_workspace()->bytes : 0, S);
+        void* ws = need ? complex_workspace()->ptr : nullptr;
+        const size_t ws_bytes = need ? complex_workspace()->bytes : 0;
+        if (eb == 4)
+            rc = decx_hip_gemm_f32_ws((const float*)A->data(), (const float*)B->data(), (const float*)c_ptr,
+                                      (float*)dst->data(), A->Height(), B->Width(), A->Width(),
+                                      A->Pitch(), B->Pitch(), ldc, dst->Pitch(), (float)alpha, (float)beta, ws, ws_bytes, S);
+        else if (eb == 8)
+            rc = decx_hip_gemm_f64_ws((const double*)A->data(), (const double*)B->data(), (const double*)c_ptr,
+                                      (double*)dst->data(), A->Height(), B->Width(), A->Width(),
+                                      A->Pitch(), B->Pitch(), ldc, dst->Pitch(), alpha, beta, ws, ws_bytes, S);
+        else
+            rc = decx_hip_gemm_f16_ws((const uint16_t*)A->data(), (const uint16_t*)B->data(), (const uint16_t*)c_ptr,
+                                      (uint16_t*)dst->data(), A->Height(), B->Width(), A->Width(),
+                                      A->Pitch(), B->Pitch(), ldc, dst->Pitch(), (float)alpha, (float)beta, ws, ws_bytes, S);
     }
-    else if (A->Type() == de::_FP64_)
-        rc = decx_hip_gemm_f64((const double*)A->data(), (const double*)B->data(), (const double*)c_ptr,
-                               (double*)dst->data(), A->Height(), B->Width(), A->Width(),
-                               A->Pitch(), B->Pitch(), ldc, dst->Pitch(), alpha, beta, S);
-    else
-        rc = decx_hip_gemm_f16((const uint16_t*)A->data(), (const uint16_t*)B->data(), (const uint16_t*)c_ptr,
-                               (uint16_t*)dst->data(), A->Height(), B->Width(), A->Width(),
-                               A->Pitch(), B->Pitch(), ldc, dst->Pitch(), (float)alpha, (float)beta, S);
     if (rc == DECX_HIP_OK) rc = decx_hip_stream_sync(S);                     // result complete on return
     return !decx::err::from_hip(h, rc, "GEMM");
 }

@@ -125,6 +125,17 @@ DECX_HIP_API int decx_hip_gemm_f32_ws(const float* A, const float* B, const floa
                                       uint32_t M, uint32_t N, uint32_t K,
                                       uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
                                       float alpha, float beta, void* workspace, size_t workspace_bytes, void* stream);
+/* The same for the other two real types (elem_bytes 2, 4 or 8 in the query).  fp16 products keep their partial
+ * products in fp32 and round once, after the sum. */
+DECX_HIP_API size_t decx_hip_gemm_workspace(int elem_bytes, uint32_t M, uint32_t N, uint32_t K);
+DECX_HIP_API int decx_hip_gemm_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D,
+                                      uint32_t M, uint32_t N, uint32_t K,
+                                      uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                                      float alpha, float beta, void* workspace, size_t workspace_bytes, void* stream);
+DECX_HIP_API int decx_hip_gemm_f64_ws(const double* A, const double* B, const double* C, double* D,
+                                      uint32_t M, uint32_t N, uint32_t K,
+                                      uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                                      double alpha, double beta, void* workspace, size_t workspace_bytes, void* stream);
 
 /* fp16 in, fp32 accumulate, one rounding to fp16 out.  Replaces the kernels launched by
  * cuda_GEMM_LS_planner<de::Half>::run (large_squares/fp16/GEMM_fp16_callers.cu:57-124). */

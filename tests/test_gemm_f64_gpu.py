@@ -78,6 +78,37 @@ def test_row_pitch_of_16_mib_takes_the_plain_kernel(hip, oracle):
     assert np.array_equal(got.view(np.uint64), oracle.gemm_f64(A, B).view(np.uint64))
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 300, 8192), (70, 130, 4099)])
+def test_split_k_through_a_workspace(hip, oracle, M, N, K):
+    """Few output tiles and a long K: partial products in double, added in a fixed order."""
+    A = synth.uniform_f64(M, K, 941); B = synth.uniform_f64(K, N, 942); C = synth.uniform_f64(M, N, 943)
+    need = hip.lib().decx_hip_gemm_workspace(8, M, N, K)
+    assert need > 0
+    ws = hip.DeviceMatrix(1, need // 8, np.float64)
+    ws.upload_raw(np.full((1, ws.pitch), np.nan, np.float64))
+    r16 = lambda v: (v + 15) // 16 * 16                       # the device pitch rule: 128 bytes
+
+    def product(c, alpha, beta, workspace):
+        dA = hip.DeviceMatrix(M, K, np.float64, r16(K), A, pad_value=np.nan); dB = hip.DeviceMatrix(K, N, np.float64, r16(N), B, pad_value=np.nan)
+        dC = hip.DeviceMatrix(M, N, np.float64, r16(N), c, pad_value=np.nan) if c is not None else None
+        dD = hip.DeviceMatrix(M, N, np.float64, r16(N))
+        dD.upload_raw(np.full((M, r16(N)), -12345.0))
+        hip.gemm(dA, dB, dD, dC, alpha, beta, workspace=workspace)
+        hip.sync()
+        raw = dD.download_raw()
+        for d in (dA, dB, dC, dD):
+            if d is not None:
+                d.free()
+        assert np.all(raw[:, N:] == -12345.0)
+        return raw[:, :N].copy()
+
+    first = product(None, 1.0, 1.0, ws)
+    assert rel_err(first, oracle.gemm_f64(A, B), K) <= TOL
+    assert np.array_equal(first, product(None, 1.0, 1.0, ws))
+    assert rel_err(product(C, 1.5, -0.5, ws), oracle.gemm_f64(A, B, C, 1.5, -0.5), K) <= TOL
+    ws.free()
+
+
 def test_plain_kernel_is_the_oracle_chain(hip, oracle):
     """Unaligned operands (and K == 0) take the one-thread-per-element kernel: the oracle's own k-ascending fma chain."""
     M, N, K = 70, 90, 50

@@ -286,6 +286,38 @@ def test_f32_split_k_through_a_workspace(hip, oracle, M, N, K):
         d.free()
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 300, 8192), (70, 130, 4099), (512, 384, 2048)])
+def test_f16_split_k_through_a_workspace(hip, oracle, M, N, K):
+    """fp16 products keep their partial products in fp32 and round once after the sum."""
+    A = synth.normal_half(M, K, 161); B = synth.normal_half(K, N, 162); C = synth.normal_half(M, N, 163)
+    need = hip.lib().decx_hip_gemm_workspace(2, M, N, K)
+    assert need > 0
+    ws = hip.DeviceMatrix(1, need // 4, np.float32)
+    ws.upload_raw(np.full((1, ws.pitch), np.nan, np.float32))
+    pa, pn = device_pitch(K, np.float16), device_pitch(N, np.float16)
+
+    def product(c, alpha, beta, workspace):
+        dA = hip.DeviceMatrix(M, K, np.float16, pa, A, pad_value=np.nan); dB = hip.DeviceMatrix(K, N, np.float16, pn, B, pad_value=np.nan)
+        dC = hip.DeviceMatrix(M, N, np.float16, pn, c, pad_value=np.nan) if c is not None else None
+        dD = hip.DeviceMatrix(M, N, np.float16, pn)
+        dD.upload_raw(np.full((M, pn), -12345.0, np.float16))
+        hip.gemm(dA, dB, dD, dC, alpha, beta, workspace=workspace)
+        hip.sync()
+        raw = dD.download_raw()
+        for d in (dA, dB, dC, dD):
+            if d is not None:
+                d.free()
+        assert np.all(raw[:, N:] == np.float16(-12345.0))
+        return raw[:, :N].copy()
+
+    first = product(None, 1.0, 1.0, ws)
+    assert rel_err(first, oracle.gemm_f16(A, B), K) <= TOL_F16
+    assert np.array_equal(first.view(np.uint16), product(None, 1.0, 1.0, ws).view(np.uint16))
+    assert rel_err(product(C, 1.5, -0.5, ws), oracle.gemm_f16(A, B, C, 1.5, -0.5), K) <= TOL_F16
+    assert rel_err(product(None, 1.0, 1.0, None), oracle.gemm_f16(A, B), K) <= TOL_F16
+    ws.free()
+
+
 def test_f32_split_k_is_planned_only_where_it_pays(hip):
     L = hip.lib()
     assert L.decx_hip_gemm_f32_workspace(8192, 8192, 8192) == 0           # enough tiles
