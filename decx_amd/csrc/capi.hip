@@ -519,6 +519,7 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
 {
     if (!out || (elem_bytes != 4 && elem_bytes != 2 && elem_bytes != 8)) return DECX_HIP_E_INVALID_ARG;
     std::memset(out, 0, sizeof *out);
+    out->k_splits = 1;
     if (M == 0 || N == 0) return DECX_HIP_OK;
     if (elem_bytes == 8) {                      // fp64 has no vector-corner kernels: N == 1 / M == 1 run as thin GEMMs
         const int shape = choose_tile_f64(M, N);
@@ -528,6 +529,7 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
         out->grid = ((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
         out->edge = (K == 0 || !aligned) ? 1 : 0;
         if (out->edge) { out->tile_m = out->tile_n = 16; out->grid = ((M + 15) / 16) * ((N + 15) / 16); }
+        else { out->k_splits = split_plan(8, M, N, K).splits; out->grid *= out->k_splits; }
         return DECX_HIP_OK;
     }
     const bool f16 = elem_bytes == 2;
@@ -552,6 +554,7 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
     out->grid = ((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
     // the direct-to-LDS kernels take every aligned shape
     out->edge = (K == 0 || !aligned) ? 1 : 0;
+    if (!out->edge) { out->k_splits = split_plan(elem_bytes, M, N, K).splits; out->grid *= out->k_splits; }
     return DECX_HIP_OK;
 }
 

@@ -64,7 +64,8 @@ typedef struct decx_hip_plan {
     int32_t  edge;                 /* 1: the predicated register-staged kernel runs (operands not 16-byte
                                       aligned, or K == 0); 0: a direct-to-LDS kernel */
     uint32_t tile_m, tile_n;       /* block tile */
-    uint32_t grid;                 /* workgroups launched */
+    uint32_t grid;                 /* workgroups launched (tiles x k_splits) */
+    uint32_t k_splits;             /* ranges K is cut into when the *_ws entry point gets its workspace; 1: no split */
 } decx_hip_plan;
 
 /* ---- device, memory, streams, events --------------------------------------------------

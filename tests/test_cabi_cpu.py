@@ -82,6 +82,10 @@ def test_planner_choices():
         assert (p.path, p.grid) == (hip.PATH_GEVM, 256)    # 128-byte column groups in fp32, 64-byte ones in fp16: 256 either way
     assert hip.plan(2, 1, 32768, 64).tile_n == 64 and hip.plan(4, 1, 4096, 64).tile_n == 16
     assert hip.plan(4, 0, 5, 5).grid == 0
+    # few tiles and a long K: the plan reports the split a workspace makes possible
+    p = hip.plan(4, 300, 300, 8192)
+    assert p.k_splits > 1 and p.grid == 25 * p.k_splits and hip.plan(4, 8192, 8192, 8192).k_splits == 1
+    assert hip.plan(4, 300, 300, 512).k_splits == 1 and hip.plan(2, 256, 256, 65536).k_splits > 1
     bad = hip.Plan()
     assert hip.lib().decx_hip_gemm_plan(3, 4, 4, 4, 1, ctypes.byref(bad)) == -1
 

@@ -78,7 +78,7 @@ def test_row_pitch_of_16_mib_takes_the_plain_kernel(hip, oracle):
     assert np.array_equal(got.view(np.uint64), oracle.gemm_f64(A, B).view(np.uint64))
 
 
-@pytest.mark.parametrize("M,N,K", [(300, 300, 8192), (70, 130, 4099)])
+@pytest.mark.parametrize("M,N,K", [(300, 300, 8192), (70, 130, 4099), (4096, 1, 8192), (1, 3000, 4096)])
 def test_split_k_through_a_workspace(hip, oracle, M, N, K):
     """Few output tiles and a long K: partial products in double, added in a fixed order."""
     A = synth.uniform_f64(M, K, 941); B = synth.uniform_f64(K, N, 942); C = synth.uniform_f64(M, N, 943)
