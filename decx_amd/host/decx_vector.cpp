@@ -226,12 +226,13 @@ _DECX_API_ de::DH de::Memcpy(de::Vector& host, de::GPU_Vector& device, const uin
     const size_t es = h->element_bytes();
     char* hptr = (char*)h->data() + (h2d ? start_src : start_dst) * es;
     char* dptr = (char*)d->data() + (h2d ? start_dst : start_src) * es;
-    void* S = decx::module_stream();
     int rc = DECX_HIP_OK;
     if (len) {
-        rc = h2d ? decx_hip_memcpy2d_async(dptr, len * es, hptr, len * es, len * es, 1, 0, S)
-                 : decx_hip_memcpy2d_async(hptr, len * es, dptr, len * es, len * es, 1, 1, S);
-        if (rc == DECX_HIP_OK) rc = decx_hip_stream_sync(S);
+        std::lock_guard<std::mutex> guard(decx::module_mutex());
+        rc = h2d ? decx::stage_h2d(dptr, len * es, hptr, len * es, len * es, 1, h->is_pinned())
+                 : decx::stage_d2h(hptr, len * es, dptr, len * es, len * es, 1, h->is_pinned());
+        const int rf = decx::stage_finish();
+        if (rc == DECX_HIP_OK) rc = rf;
     }
     decx::err::from_hip(&handle, rc, "Memcpy");
     return handle;
