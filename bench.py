@@ -12,6 +12,7 @@ once on the host cores on the same workload and checked bit-for-bit against the 
 fma chain on sampled rows.
 """
 import argparse
+import math
 import json
 import os
 import sys
@@ -111,7 +112,7 @@ def run_workload(name, steps, warmup, keep_inputs=False, settle_s=0.0):
            "hbm_gbs_algorithmic": round(gbs, 1), "kernel_ms": round(kernel_ms, 5), "wall_ms_per_step": round(wall_ms, 5),
            "plan": {"path": int(p.path), "tile": [int(p.tile_m), int(p.tile_n)], "grid": int(p.grid), "edge": int(p.edge)},
            "roofline": roof}
-    result = (out, (A, B) if keep_inputs else None)
+    result = (out, (A, B, dD.download()) if keep_inputs else None)    # the result goes to the CPU leg's comparison
     for d in (dA, dB, dD):
         d.free()
     return result
@@ -203,9 +204,9 @@ def run_complex(double, n, steps, warmup, settle_s=0.25):
     return out
 
 
-def cpu_baseline(name, A, B):
-    """Times the AVX2 restatement of the reference CPU GEMM once on this host and checks it
-    bit-for-bit against the scalar fma chain on sampled rows."""
+def cpu_baseline(name, A, B, D_gpu):
+    """Times the AVX2 restatement of the reference CPU GEMM once on this host, checks it bit-for-bit
+    against the scalar fma chain on sampled rows, and compares the GPU's whole result with it."""
     from oracle import binding as oracle
     import ctypes
     _, M, N, K, _, _, desc = WORKLOADS[name]
@@ -225,9 +226,13 @@ def cpu_baseline(name, A, B):
     rows = np.unique(np.random.default_rng(0).integers(0, M, 16)).astype(np.uint32)
     chain = oracle.gemm_f32(A, B, rows=rows)
     same = bool(np.array_equal(d[rows, :N].view(np.uint32), chain.view(np.uint32)))
+    ref_max = float(np.max(np.abs(d[:, :N])))
+    gpu_err = float(np.max(np.abs(D_gpu - d[:, :N]))) / (ref_max * math.sqrt(K))
     return {"value": round(2.0 * M * N * K / secs / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
             "sample": "one full call of the same workload (%s), %.2f s wall" % (desc.split(",")[0], secs),
-            "bit_equal_to_fma_chain": same}
+            "bit_equal_to_fma_chain": same,
+            "gpu_parity": {"rel_err": float("%.3g" % gpu_err), "bar": 1e-5, "elements": int(M) * int(N),
+                           "measure": "max|gpu - cpu| / (max|cpu| sqrt(K)) over the whole output"}}
 
 
 def api_wall_time(name, repeats=10):
