@@ -13,8 +13,10 @@
 // 8-byte segment s % 4) and lane i receives column i of it, 4 consecutive k of one n; two such
 // reads give the 8 k a lane needs.  So neither a transpose pass nor a register shuffle is needed.
 // The MFMA is issued with its operands swapped (B fragment first): it then produces the transposed
-// 32 x 32 tile, in which a lane owns adjacent columns of one output row, and the epilogue stores
-// 16 bytes per lane after one `v_permlane32_swap`.
+// 32 x 32 tile, in which a lane owns adjacent columns of one output row: after one
+// `v_permlane32_swap` a lane holds 16-byte pieces of its row, which a wave turns around through
+// LDS so that it stores whole rows of its tile (128 contiguous bytes per row instead of 32:
+// 1.1 us less per launch at 4096 x 4096 outputs).
 //
 // Slabs reach LDS by `global_load_lds_dwordx4` (no VGPRs, no ds_write).  These are inline assembly
 // and the slab barrier is a bare `s_barrier` behind an explicit vmcnt wait, because the compiler
@@ -289,7 +291,7 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
 
     // Epilogue.  Lane (l32, h) holds output row l32 of the m tile; register 4 q + e is column
     // 8 q + 4 h + e of the n tile.  Interior tiles: `v_permlane32_swap` trades the halves of an even
-    // and an odd 8-column group between lane l and lane l + 32, after which each lane stores 16 bytes.
+    // and an odd 8-column group between lane l and lane l + 32, after which each lane holds 16-byte pieces.
     if constexpr (SPLIT) {                                 // the fp32 partial product of this range of K
         float* __restrict__ P = (float*)g.split_ws + (size_t)blockIdx.y * g.split_stride;
 #pragma unroll
@@ -318,9 +320,22 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
         return w.u;
     };
     const bool interior = (m0 + BM <= g.M) && (n0 + BN <= g.N);
+    // Interior tiles go through LDS once more (the ring is free: every wave has passed the last slab
+    // barrier): a lane holds 16-byte pieces of ONE row, two lanes a row, so storing from the
+    // accumulator layout would touch 32 bytes of 32 different rows per instruction.  Each wave turns
+    // 32 rows x WN columns around in a private buffer (two of them, taking turns) and stores whole
+    // rows: WN * 2 contiguous bytes per row, 64 / PPR rows per instruction.
+    constexpr int ROW_BYTES = WN * 2, PPR = WN / 8, ROWS_PER_STORE = 64 / PPR, STORES = 32 / ROWS_PER_STORE;
+    static_assert(WAVES * 2 * 32 * ROW_BYTES <= STAGES * STAGE_BYTES, "staging rows must fit in the ring");
+    auto wave_sync = [] {                                  // LDS traffic of one wave is in order; this is for the compiler
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const uint32_t row = m0 + wm0 + 32 * i + l32;
+        unsigned char* stage_rows = lds + (wave * 2 + (i & 1)) * (32 * ROW_BYTES);
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             if (interior) {
@@ -345,8 +360,10 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
                     const auto s0 = __builtin_amdgcn_permlane32_swap(w[0][0], w[1][0], false, false);
                     const auto s1 = __builtin_amdgcn_permlane32_swap(w[0][1], w[1][1], false, false);
                     const uintx4 out = {s0[0], s1[0], s0[1], s1[1]};
-                    const uint32_t col = n0 + wn0 + 32 * j + 8 * (2 * qp + h);
-                    *(uintx4*)(D + (size_t)row * g.ldd + col) = out;
+                    // into this wave's staging rows: piece p of row l32, pieces XOR-permuted so that any 8
+                    // consecutive lanes hit 8 different 16-byte bank groups on the way in and on the way out
+                    const int p = 4 * j + 2 * qp + h;
+                    *(uintx4*)(stage_rows + l32 * ROW_BYTES + ((p ^ ((l32 / (8 / PPR)) % PPR)) * 16)) = out;
                 }
             } else if (row < g.M) {
 #pragma unroll
@@ -361,6 +378,16 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
                         }
                     }
             }
+        }
+        if (interior) {
+            wave_sync();
+#pragma unroll
+            for (int t = 0; t < STORES; ++t) {
+                const int r = ROWS_PER_STORE * t + lane / PPR, pc = lane % PPR;
+                const uintx4 v = *(const uintx4*)(stage_rows + r * ROW_BYTES + ((pc ^ ((r / (8 / PPR)) % PPR)) * 16));
+                *(uintx4*)(D + (size_t)(m0 + wm0 + 32 * i + r) * g.ldd + n0 + wn0 + 8 * pc) = v;
+            }
+            wave_sync();
         }
     }
 }
