@@ -94,8 +94,14 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
     if (tile != DECX_HIP_TILE_AUTO && (tile < 0 || tile >= TILE_COUNT)) return DECX_HIP_E_INVALID_ARG;
 
     // the two vector corners are bandwidth-bound and have kernels of their own
-    if (N == 1 && tile == DECX_HIP_TILE_AUTO && K > 0)
+    if (N == 1 && tile == DECX_HIP_TILE_AUTO && K > 0) {
+        // x is the single column of a pitched K x 1 matrix: with a workspace it is gathered once into a dense vector
+        if (workspace && workspace_bytes >= (size_t)K * (F16 ? 2 : 4) && gemv_gather_pays(M, K, ldb)) {
+            const int rg = launch_gather(F16, B, workspace, K, ldb, as_stream(stream));
+            return rg != 0 ? rg : launch_gemv(F16, false, A, workspace, C, D, M, K, lda, 1, ldc, ldd, alpha, beta, as_stream(stream));
+        }
         return launch_gemv(F16, false, A, B, C, D, M, K, lda, ldb, ldc, ldd, alpha, beta, as_stream(stream));
+    }
     if (M == 1 && tile == DECX_HIP_TILE_AUTO && K > 0)
         return launch_gevm(F16, false, A, B, C, D, K, N, ldb, 1, 1, 1, alpha, beta, as_stream(stream));
 
@@ -285,6 +291,8 @@ int decx_hip_gemm_f32(const float* A, const float* B, const float* C, float* D, 
 size_t decx_hip_gemm_workspace(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
 {
     if (!g_dev.ready || (elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8)) return 0;
+    if (elem_bytes != 8 && N == 1 && M > 0)                        // room for a dense copy of x
+        return gemv_gather_pays(M, K, 2) ? ((size_t)K * elem_bytes + 15) / 16 * 16 : 0;
     const SplitPlan sp = split_plan(elem_bytes, M, N, K);
     return sp.splits > 1 ? (size_t)sp.splits * M * ((N + 3) / 4 * 4) * (elem_bytes == 8 ? 8 : 4) : 0;
 }

@@ -322,8 +322,52 @@ def test_f32_split_k_is_planned_only_where_it_pays(hip):
     L = hip.lib()
     assert L.decx_hip_gemm_f32_workspace(8192, 8192, 8192) == 0           # enough tiles
     assert L.decx_hip_gemm_f32_workspace(300, 300, 512) == 0              # K too short to cut
-    assert L.decx_hip_gemm_f32_workspace(8192, 1, 8192) == 0 and L.decx_hip_gemm_f32_workspace(1, 8192, 8192) == 0
+    assert L.decx_hip_gemm_f32_workspace(1, 8192, 8192) == 0              # a row vector is dense already
     assert L.decx_hip_gemm_f32_workspace(0, 5, 5000) == 0
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("M,K", [(2048, 4096), (1030, 8200), (5, 16390)])
+def test_column_operand_gathered_through_a_workspace(hip, oracle, dtype, M, K):
+    """N = 1: B is the single column of a pitched K x 1 matrix.  With a workspace it is copied once into a dense
+    vector in front of the matrix-vector kernel; the result is the one the strided path gives, bit for bit (same
+    kernel, same order), and a workspace that is too small means the strided path."""
+    f16 = dtype == np.float16
+    A = synth.normal_half(M, K, 171) if f16 else synth.uniform_f32(M, K, 171)
+    B = synth.normal_half(K, 1, 172) if f16 else synth.uniform_f32(K, 1, 172)
+    C = synth.normal_half(M, 1, 173) if f16 else synth.uniform_f32(M, 1, 173)
+    need = hip.lib().decx_hip_gemm_workspace(dtype().itemsize, M, 1, K)
+    assert need >= K * dtype().itemsize and need % 16 == 0
+    assert hip.lib().decx_hip_gemm_workspace(dtype().itemsize, 512, 1, 1024) == 0      # too small to pay
+    ws = hip.DeviceMatrix(1, need // 4, np.float32)
+    ws.upload_raw(np.full((1, ws.pitch), np.nan, np.float32))
+    pa, p1 = device_pitch(K, dtype), device_pitch(1, dtype)
+    ref = oracle.gemm_f16 if f16 else oracle.gemm_f32
+    tol = TOL_F16 if f16 else TOL_F32
+
+    def product(c, alpha, beta, workspace):
+        dA = hip.DeviceMatrix(M, K, dtype, pa, A, pad_value=np.nan); dB = hip.DeviceMatrix(K, 1, dtype, p1, B, pad_value=np.nan)
+        dC = hip.DeviceMatrix(M, 1, dtype, p1, c, pad_value=np.nan) if c is not None else None
+        dD = hip.DeviceMatrix(M, 1, dtype, p1)
+        dD.upload_raw(np.full((M, p1), -12345.0, dtype))
+        hip.gemm(dA, dB, dD, dC, alpha, beta, workspace=workspace)
+        hip.sync()
+        raw = dD.download_raw()
+        for d in (dA, dB, dC, dD):
+            if d is not None:
+                d.free()
+        assert np.all(raw[:, 1:] == dtype(-12345.0))
+        return raw[:, :1].copy()
+
+    gathered = product(None, 1.0, 1.0, ws)
+    assert rel_err(gathered, ref(A, B), K) <= tol
+    strided = product(None, 1.0, 1.0, None)
+    assert np.array_equal(gathered.view(np.uint8), strided.view(np.uint8))
+    assert rel_err(product(C, 1.5, -0.5, ws), ref(A, B, C, 1.5, -0.5), K) <= tol
+    small = hip.DeviceMatrix(1, 64, np.float32)
+    assert np.array_equal(product(None, 1.0, 1.0, small).view(np.uint8), strided.view(np.uint8))
+    for d in (ws, small):
+        d.free()
 
 
 @pytest.mark.parametrize("tile", [0, 1, 2])
