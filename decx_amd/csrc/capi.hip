@@ -543,7 +543,7 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
     const bool f16 = elem_bytes == 2;
     if (N == 1 && K > 0) {
         out->path = DECX_HIP_PATH_GEMV;
-        out->tile_m = (M + 31) / 32 >= 256u ? 32 : 16;         // two rows per wavefront, or one while that leaves CUs idle
+        out->tile_m = gemv_rows_per_block(M);                  // 32 (two rows per wavefront) down to 1 (16 wavefronts per row)
         out->tile_n = 1;
         out->grid = (M + out->tile_m - 1) / out->tile_m;
         return DECX_HIP_OK;

@@ -185,6 +185,7 @@ int launch_complex_scale(const T* C, T* D, uint32_t M, uint32_t N, uint32_t ldc,
 
 // y = alpha * A.x (+ beta * c) and y = alpha * x.B (+ beta * c); f16 inputs accumulate in fp32 and write
 // fp32 (out_f32) or fp16.  inc* are element strides.
+uint32_t gemv_rows_per_block(uint32_t M);
 bool gemv_gather_pays(uint32_t M, uint32_t K, uint32_t incx);
 int launch_gather(bool f16, const void* x, void* dst, uint32_t K, uint32_t inc, hipStream_t stream);
 int launch_gemv(bool f16, bool out_f32, const void* A, const void* x, const void* c, void* y, uint32_t M, uint32_t K,

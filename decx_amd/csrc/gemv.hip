@@ -13,7 +13,9 @@
 //
 // gemv: 16 wavefronts per workgroup, two rows per wavefront (32 rows per workgroup: 8192
 //   rows give one workgroup per CU with 64 KB of A in flight), one row per wavefront for
-//   matrices of fewer than 8192 rows (2048 x 8192: 24.3 -> 22.2 us); x is staged in LDS once per
+//   matrices of fewer than 8192 rows, and below 4096 rows 2, 4, 8 or all 16 wavefronts share a row
+//   (they deal the steps of K among themselves), always the fewest that still give every CU a
+//   workgroup (2048 x 8192: 24.3 -> 16.1 us with a dense x, 512 x 32768: 60.9 -> 23.8); x is staged in LDS once per
 //   workgroup, as fp32, in chunks of 4096 -- x may be strided (the single column of a
 //   pitched K x 1 matrix puts every element in its own cache line), so staging it once per
 //   32 rows keeps that gather small; A is read with 128-bit loads; per lane an fp32 fma
@@ -60,8 +62,10 @@ __device__ __forceinline__ float wave_sum(float v)
     return v;
 }
 
-// RPW rows per wavefront: 2, or 1 when two would leave CUs without a workgroup.
-template <typename T, typename TO, int RPW>
+// RPW rows per wavefront: 2, or 1 when two would leave CUs without a workgroup.  WPR wavefronts per
+// row (RPW == 1 only): for matrices of few rows the wavefronts of a row deal the steps of K among
+// themselves and their sums meet in LDS, in wavefront order, so that a workgroup holds 16 / WPR rows.
+template <typename T, typename TO, int RPW, int WPR>
 __global__ void __launch_bounds__(GEMV_THREADS)
 gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restrict__ c, TO* __restrict__ y,
             uint32_t M, uint32_t K, uint32_t lda, uint32_t incx, uint32_t incc, uint32_t incy,
@@ -70,7 +74,10 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
     constexpr int N16 = Per16<T>::n;
     __shared__ __attribute__((aligned(16))) float xs[GEMV_KC];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const uint32_t row0 = blockIdx.x * (RPW * GEMV_WAVES) + wave * RPW;
+    static_assert(WPR == 1 || RPW == 1, "rows are split over wavefronts only one at a time");
+    __shared__ float wave_sums[GEMV_WAVES];
+    const int sub = wave % WPR;                            // which share of the steps of K this wavefront takes
+    const uint32_t row0 = blockIdx.x * (RPW * GEMV_WAVES / WPR) + (wave / WPR) * RPW;
     const bool has0 = row0 < M, has1 = RPW == 2 && row0 + 1 < M;
     const T* a0 = A + (size_t)(has0 ? row0 : 0) * lda;
     const T* a1 = A + (size_t)(has1 ? row0 + 1 : 0) * lda;
@@ -92,9 +99,9 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
         if (has0) {
             constexpr uint32_t STEP = 64 * N16;
             const uint32_t steps = (lenv + STEP - 1) / STEP;
-            const uint32_t step0 = steps ? ((blockIdx.x * GEMV_WAVES + wave) * 5u) % steps : 0u;
+            const uint32_t step0 = steps ? ((blockIdx.x * GEMV_WAVES + wave - sub) * 5u) % steps : 0u;   // one start per row
 #pragma unroll 4
-            for (uint32_t i = 0; i < steps; ++i) {
+            for (uint32_t i = sub; i < steps; i += WPR) {
                 const uint32_t step = step0 + i < steps ? step0 + i : step0 + i - steps;
                 const uint32_t k = step * STEP + lane * N16;
                 if (k < lenv) {
@@ -109,7 +116,7 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
                     }
                 }
             }
-            for (uint32_t k = lenv + lane; k < len; k += 64) {
+            for (uint32_t k = lenv + lane + (sub ? len : 0u); k < len; k += 64) {   // the first wavefront of a row takes the tail
                 s0 = __builtin_fmaf(to_float(a0[kc + k]), xs[k], s0);
                 if (has1) s1 = __builtin_fmaf(to_float(a1[kc + k]), xs[k], s1);
             }
@@ -117,6 +124,13 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
     }
     s0 = wave_sum(s0);
     s1 = wave_sum(s1);
+    if constexpr (WPR > 1) {
+        if (lane == 0) wave_sums[wave] = s0;
+        __syncthreads();
+        if (sub != 0) return;
+#pragma unroll
+        for (int w = 1; w < WPR; ++w) s0 += wave_sums[wave + w];
+    }
     if (lane == 0) {
         if (has0) {
             float o = s0;
@@ -214,12 +228,21 @@ void launch_gemv_as(const void* A, const void* x, const void* c, void* y, uint32
                     uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream)
 {
     const uint32_t vec = rows_vectorisable<T>(A, lda);
-    if ((M + GEMV_ROWS_PER_BLOCK - 1) / GEMV_ROWS_PER_BLOCK >= 256u)
-        hipLaunchKernelGGL((gemv_kernel<T, TO, 2>), dim3((M + GEMV_ROWS_PER_BLOCK - 1) / GEMV_ROWS_PER_BLOCK), dim3(GEMV_THREADS), 0,
-                           stream, (const T*)A, (const T*)x, (const T*)c, (TO*)y, M, K, lda, incx, incc, incy, alpha, beta, vec);
-    else
-        hipLaunchKernelGGL((gemv_kernel<T, TO, 1>), dim3((M + GEMV_WAVES - 1) / GEMV_WAVES), dim3(GEMV_THREADS), 0,
-                           stream, (const T*)A, (const T*)x, (const T*)c, (TO*)y, M, K, lda, incx, incc, incy, alpha, beta, vec);
+    auto launch = [&](auto rpw_c, auto wpr_c) {
+        constexpr int RPW = decltype(rpw_c)::value, WPR = decltype(wpr_c)::value;
+        constexpr uint32_t ROWS = RPW * GEMV_WAVES / WPR;
+        hipLaunchKernelGGL((gemv_kernel<T, TO, RPW, WPR>), dim3((M + ROWS - 1) / ROWS), dim3(GEMV_THREADS), 0, stream,
+                           (const T*)A, (const T*)x, (const T*)c, (TO*)y, M, K, lda, incx, incc, incy, alpha, beta, vec);
+    };
+    using std::integral_constant;
+    switch (gemv_rows_per_block(M)) {
+    case 32: launch(integral_constant<int, 2>{}, integral_constant<int, 1>{}); break;
+    case 16: launch(integral_constant<int, 1>{}, integral_constant<int, 1>{}); break;
+    case 8:  launch(integral_constant<int, 1>{}, integral_constant<int, 2>{}); break;
+    case 4:  launch(integral_constant<int, 1>{}, integral_constant<int, 4>{}); break;
+    case 2:  launch(integral_constant<int, 1>{}, integral_constant<int, 8>{}); break;
+    default: launch(integral_constant<int, 1>{}, integral_constant<int, 16>{}); break;
+    }
 }
 
 // dst[i] = x[i * inc]: the dense copy of a strided vector
@@ -232,12 +255,25 @@ __global__ void __launch_bounds__(256) gather_kernel(const T* __restrict__ x, T*
 
 }  // namespace
 
+// Rows per workgroup of gemv: 32 (two per wavefront) while that gives every CU a workgroup, else the largest
+// power of two down to 1 (all 16 wavefronts on one row) that still does.
+uint32_t gemv_rows_per_block(uint32_t M)
+{
+    uint32_t rows = 32;
+    while (rows > 1 && (M + rows - 1) / rows < 256u) rows /= 2;
+    return rows;
+}
+
 // A strided x (the single column of a pitched K x 1 matrix) costs every workgroup of gemv one cache
 // line request per element; gathered once into a dense buffer it costs one per 32 (fp32) or 64.
-// That pays once enough workgroups would repeat the gather (8192 x 8192: 46.7 -> 42 us).
+// The copy is a launch of its own (about 4.5 us with its loads, all L2 misses): it pays from the sizes
+// below (8192 x 8192: 46.7 -> 43.9 us, 512 x 32768: 44.7 -> 23.8, 256 x 8192: 10.8 -> 7.2, 4096 x 2048: 7.7 -> 7.9).
 bool gemv_gather_pays(uint32_t M, uint32_t K, uint32_t incx)
 {
-    return incx > 1 && (K >= 16384 || (K >= 8192 && M >= 1024) || (K >= 4096 && M >= 2048));
+    if (incx <= 1) return false;
+    if (K >= 8192) return M >= 64;
+    if (K >= 4096) return M >= 1024;
+    return K >= 3072 && M >= 3072;
 }
 
 int launch_gather(bool f16, const void* x, void* dst, uint32_t K, uint32_t inc, hipStream_t stream)

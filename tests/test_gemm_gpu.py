@@ -327,7 +327,7 @@ def test_f32_split_k_is_planned_only_where_it_pays(hip):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
-@pytest.mark.parametrize("M,K", [(2048, 4096), (1030, 8200), (5, 16390)])
+@pytest.mark.parametrize("M,K", [(2048, 4096), (1030, 8200), (70, 16390), (3100, 3080)])
 def test_column_operand_gathered_through_a_workspace(hip, oracle, dtype, M, K):
     """N = 1: B is the single column of a pitched K x 1 matrix.  With a workspace it is copied once into a dense
     vector in front of the matrix-vector kernel; the result is the one the strided path gives, bit for bit (same

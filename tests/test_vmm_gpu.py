@@ -76,7 +76,9 @@ CASES = [  # (in dtype, out dtype, tolerance)
     (np.float16, np.float32, TOL_F32),
     (np.float16, np.float16, TOL_F16),
 ]
-MV_SHAPES = [(1, 1), (3, 5), (33, 63), (64, 256), (65, 257), (1000, 1), (257, 8200), (2, 20000), (700, 1030)]
+MV_SHAPES = [(1, 1), (3, 5), (33, 63), (64, 256), (65, 257), (1000, 1), (257, 8200), (2, 20000), (700, 1030),
+             # one shape per number of wavefronts that share a row (8, 4, 2, 1) and for two rows per wavefront
+             (600, 300), (1100, 9001), (2100, 4100), (4100, 40), (8200, 33)]
 
 
 @pytest.mark.parametrize("tin,tout,tol", CASES)
