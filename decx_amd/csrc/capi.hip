@@ -102,8 +102,23 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
         }
         return launch_gemv(F16, false, A, B, C, D, M, K, lda, ldb, ldc, ldd, alpha, beta, as_stream(stream));
     }
-    if (M == 1 && tile == DECX_HIP_TILE_AUTO && K > 0)
+    if (M == 1 && tile == DECX_HIP_TILE_AUTO && K > 0) {
+        // few columns and a long K: with a workspace, ranges of K go to workgroups of their own and a second kernel
+        // adds their partial sums in range order
+        const SplitPlan sp = plan_gevm_split(F16, N, K, g_dev.compute_units);
+        const uint32_t ldw = (N + 3) / 4 * 4;
+        if (sp.splits > 1 && workspace && aligned16(workspace) && workspace_bytes >= (size_t)sp.splits * ldw * 4) {
+            const int rv = launch_gevm(F16, false, A, B, nullptr, D, K, N, ldb, 1, 1, 1, 1.f, 1.f, as_stream(stream), sp.len,
+                                       (float*)workspace, ldw);
+            if (rv != 0) return rv;
+            GemmArgs r;
+            std::memset(&r, 0, sizeof r);
+            r.C = C; r.D = D; r.M = 1; r.N = N; r.ldc = ldc; r.ldd = ldd; r.alpha = alpha; r.beta = beta;
+            r.split_ws = workspace; r.split_ldd = ldw; r.split_stride = ldw;
+            return launch_split_reduce(F16 ? 2 : 4, r, sp.splits, as_stream(stream));
+        }
         return launch_gevm(F16, false, A, B, C, D, K, N, ldb, 1, 1, 1, alpha, beta, as_stream(stream));
+    }
 
     constexpr uint32_t per16 = F16 ? 8u : 4u;          // elements per 16 bytes
     GemmArgs g;
@@ -293,6 +308,10 @@ size_t decx_hip_gemm_workspace(int elem_bytes, uint32_t M, uint32_t N, uint32_t 
     if (!g_dev.ready || (elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8)) return 0;
     if (elem_bytes != 8 && N == 1 && M > 0)                        // room for a dense copy of x
         return gemv_gather_pays(M, K, 2) ? ((size_t)K * elem_bytes + 15) / 16 * 16 : 0;
+    if (elem_bytes != 8 && M == 1 && N > 0) {                      // room for the partial sums of ranges of K
+        const SplitPlan sp = plan_gevm_split(elem_bytes == 2, N, K, g_dev.compute_units);
+        return sp.splits > 1 ? (size_t)sp.splits * ((N + 3) / 4 * 4) * 4 : 0;
+    }
     const SplitPlan sp = split_plan(elem_bytes, M, N, K);
     return sp.splits > 1 ? (size_t)sp.splits * M * ((N + 3) / 4 * 4) * (elem_bytes == 8 ? 8 : 4) : 0;
 }
@@ -551,6 +570,12 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
     if (M == 1 && K > 0) {
         out->path = DECX_HIP_PATH_GEVM;
         out->tile_m = 1; out->tile_n = f16 ? 64 : 32;               // 128 bytes of a row, or 64 when that leaves CUs idle
+        const SplitPlan sp = plan_gevm_split(f16, N, K, g_dev.ready ? g_dev.compute_units : 256);
+        if (sp.splits > 1) {                                        // with a workspace: whole lines, several ranges of K
+            out->k_splits = sp.splits;
+            out->grid = (N + out->tile_n - 1) / out->tile_n * sp.splits;
+            return DECX_HIP_OK;
+        }
         if ((N + out->tile_n - 1) / out->tile_n < 256u) out->tile_n /= 2;
         out->grid = (N + out->tile_n - 1) / out->tile_n;
         return DECX_HIP_OK;

@@ -191,6 +191,8 @@ int launch_gather(bool f16, const void* x, void* dst, uint32_t K, uint32_t inc, 
 int launch_gemv(bool f16, bool out_f32, const void* A, const void* x, const void* c, void* y, uint32_t M, uint32_t K,
                 uint32_t lda, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream);
 int launch_gevm(bool f16, bool out_f32, const void* x, const void* B, const void* c, void* y, uint32_t K, uint32_t N,
-                uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream);
+                uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream,
+                uint32_t split_len = 0, float* partial = nullptr, uint32_t partial_stride = 0);
+SplitPlan plan_gevm_split(bool f16, uint32_t N, uint32_t K, uint32_t cus);
 
 }  // namespace decx_hip

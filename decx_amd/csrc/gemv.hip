@@ -150,10 +150,16 @@ template <typename T, typename TO, int CL>
 __global__ void __launch_bounds__(GEMV_THREADS)
 gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restrict__ c, TO* __restrict__ y,
             uint32_t K, uint32_t N, uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy,
-            float alpha, float beta, uint32_t vec_ok)
+            float alpha, float beta, uint32_t vec_ok, uint32_t split_len, float* __restrict__ partial, uint32_t partial_stride)
 {
     constexpr int N16 = Per16<T>::n;
     constexpr int CB = CL * N16;                           // columns per workgroup
+    if (split_len) {                                       // blockIdx.y takes a range of K; its sums go to `partial`
+        const uint32_t k0 = blockIdx.y * split_len;
+        x += (size_t)k0 * incx;
+        B += (size_t)k0 * ldb;
+        K = K - k0 < split_len ? K - k0 : split_len;
+    }
     constexpr int RL = 64 / CL;                            // rows per wavefront and sweep
     __shared__ __attribute__((aligned(16))) float xs[GEMV_KC];
     __shared__ float red[GEMV_WAVES][CB];
@@ -208,6 +214,7 @@ gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restric
             float o = 0.f;
 #pragma unroll
             for (int w = 0; w < GEMV_WAVES; ++w) o += red[w][t];
+            if (split_len) { partial[(size_t)blockIdx.y * partial_stride + n] = o; return; }
             if (c) o = __builtin_fmaf(to_float(c[(size_t)n * incc]), beta, alpha * o);
             y[(size_t)n * incy] = (TO)o;
         }
@@ -298,28 +305,53 @@ namespace {
 
 template <typename T, typename TO>
 void launch_gevm_as(const void* x, const void* B, const void* c, void* y, uint32_t K, uint32_t N, uint32_t ldb,
-                    uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream)
+                    uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream,
+                    uint32_t split_len, float* partial, uint32_t partial_stride)
 {
     // 128-byte column groups unless they leave CUs without a workgroup (fp16 at N = 8192: 128 groups for
-    // 256 CUs); then 64-byte groups, two workgroups per cache line
+    // 256 CUs); then 64-byte groups, two workgroups per cache line -- or, with a workspace for partial sums,
+    // 128-byte groups and several workgroups per group, each on a range of K (split_len != 0)
     const uint32_t cb8 = 8u * Per16<T>::n;
     const uint32_t vec = rows_vectorisable<T>(B, ldb);
-    if ((N + cb8 - 1) / cb8 >= 256u)
-        hipLaunchKernelGGL((gevm_kernel<T, TO, 8>), dim3((N + cb8 - 1) / cb8), dim3(GEMV_THREADS), 0, stream, (const T*)x,
-                           (const T*)B, (const T*)c, (TO*)y, K, N, ldb, incx, incc, incy, alpha, beta, vec);
+    const uint32_t splits = split_len ? (K + split_len - 1) / split_len : 1u;
+    if (split_len || (N + cb8 - 1) / cb8 >= 256u)
+        hipLaunchKernelGGL((gevm_kernel<T, TO, 8>), dim3((N + cb8 - 1) / cb8, splits), dim3(GEMV_THREADS), 0, stream, (const T*)x,
+                           (const T*)B, (const T*)c, (TO*)y, K, N, ldb, incx, incc, incy, alpha, beta, vec, split_len, partial,
+                           partial_stride);
     else
         hipLaunchKernelGGL((gevm_kernel<T, TO, 4>), dim3((N + cb8 / 2 - 1) / (cb8 / 2)), dim3(GEMV_THREADS), 0, stream,
-                           (const T*)x, (const T*)B, (const T*)c, (TO*)y, K, N, ldb, incx, incc, incy, alpha, beta, vec);
+                           (const T*)x, (const T*)B, (const T*)c, (TO*)y, K, N, ldb, incx, incc, incy, alpha, beta, vec, 0u,
+                           (float*)nullptr, 0u);
 }
 
 }  // namespace
 
-int launch_gevm(bool f16, bool out_f32, const void* x, const void* B, const void* c, void* y, uint32_t K, uint32_t N,
-                uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream)
+// Few columns and a long K: 128-byte column groups alone would leave CUs without a workgroup.  With room for
+// partial sums the groups are multiplied by ranges of K, aiming at two workgroups per CU.  The second kernel
+// that adds the partial sums costs a launch, so this is for matrices that keep the first one busy long enough:
+// 1 x 2048 x 8192 19.5 -> 16.5 us, 1 x 512 x 32768 69 -> 23, 1 x 64 x 65536 116 -> 23 (1 x 512 x 8192 would go from
+// 9 to 14 and stays whole).  A range is a multiple of the 128 rows a workgroup sweeps at a time, at least 256 long.
+SplitPlan plan_gevm_split(bool f16, uint32_t N, uint32_t K, uint32_t cus)
 {
-    if (!f16) launch_gevm_as<float, float>(x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream);
-    else if (out_f32) launch_gevm_as<_Float16, float>(x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream);
-    else launch_gevm_as<_Float16, _Float16>(x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream);
+    const uint32_t cb8 = f16 ? 64u : 32u;
+    const uint32_t groups = (N + cb8 - 1) / cb8;
+    const uint64_t bytes = (uint64_t)K * N * (f16 ? 2 : 4);
+    if (groups == 0 || groups * 4 > cus || (K < 16384 && bytes < (32ull << 20))) return {1, 0};
+    uint32_t splits = (2 * cus + groups - 1) / groups;
+    if (splits > K / 256) splits = K / 256;
+    if (splits > 64) splits = 64;
+    if (splits < 2) return {1, 0};
+    const uint32_t len = ((K + splits - 1) / splits + 127) / 128 * 128;
+    return {(K + len - 1) / len, len};
+}
+
+int launch_gevm(bool f16, bool out_f32, const void* x, const void* B, const void* c, void* y, uint32_t K, uint32_t N,
+                uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream,
+                uint32_t split_len, float* partial, uint32_t partial_stride)
+{
+    if (!f16) launch_gevm_as<float, float>(x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream, split_len, partial, partial_stride);
+    else if (out_f32) launch_gevm_as<_Float16, float>(x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream, split_len, partial, partial_stride);
+    else launch_gevm_as<_Float16, _Float16>(x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream, split_len, partial, partial_stride);
     return (int)hipGetLastError();
 }
 

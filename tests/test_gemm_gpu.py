@@ -370,6 +370,53 @@ def test_column_operand_gathered_through_a_workspace(hip, oracle, dtype, M, K):
         d.free()
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("K,N", [(8192, 2048), (20000, 70), (16500, 7), (33000, 513)])
+def test_row_operand_few_columns_split_through_a_workspace(hip, oracle, dtype, K, N):
+    """M = 1 with few columns and a long K: with a workspace, ranges of K go to workgroups of their own and their
+    partial sums are added in range order by a second kernel.  Parity, identical results from run to run,
+    C / alpha / beta, untouched padding; a workspace that is too small means the single-kernel path."""
+    f16 = dtype == np.float16
+    A = synth.normal_half(1, K, 181) if f16 else synth.uniform_f32(1, K, 181)
+    B = synth.normal_half(K, N, 182) if f16 else synth.uniform_f32(K, N, 182)
+    C = synth.normal_half(1, N, 183) if f16 else synth.uniform_f32(1, N, 183)
+    need = hip.lib().decx_hip_gemm_workspace(dtype().itemsize, 1, N, K)
+    assert need > 0 and need % 16 == 0
+    assert hip.plan(dtype().itemsize, 1, N, K).k_splits > 1
+    assert hip.lib().decx_hip_gemm_workspace(dtype().itemsize, 1, 512, 8192) == 0       # too short to pay for a second kernel
+    assert hip.lib().decx_hip_gemm_workspace(dtype().itemsize, 1, 8192, 8192) == 0      # enough column groups
+    ws = hip.DeviceMatrix(1, need // 4, np.float32)
+    ws.upload_raw(np.full((1, ws.pitch), np.nan, np.float32))
+    pk, pn = device_pitch(K, dtype), device_pitch(N, dtype)
+    ref = oracle.gemm_f16 if f16 else oracle.gemm_f32
+    tol = TOL_F16 if f16 else TOL_F32
+
+    def product(c, alpha, beta, workspace):
+        dA = hip.DeviceMatrix(1, K, dtype, pk, A, pad_value=np.nan); dB = hip.DeviceMatrix(K, N, dtype, pn, B, pad_value=np.nan)
+        dC = hip.DeviceMatrix(1, N, dtype, pn, c, pad_value=np.nan) if c is not None else None
+        dD = hip.DeviceMatrix(1, N, dtype, pn)
+        dD.upload_raw(np.full((1, pn), -12345.0, dtype))
+        hip.gemm(dA, dB, dD, dC, alpha, beta, workspace=workspace)
+        hip.sync()
+        raw = dD.download_raw()
+        for d in (dA, dB, dC, dD):
+            if d is not None:
+                d.free()
+        assert np.all(raw[:, N:] == dtype(-12345.0))
+        return raw[:, :N].copy()
+
+    first = product(None, 1.0, 1.0, ws)
+    assert rel_err(first, ref(A, B), K) <= tol
+    assert np.array_equal(first.view(np.uint8), product(None, 1.0, 1.0, ws).view(np.uint8))      # fixed summation order
+    assert rel_err(product(C, 1.5, -0.5, ws), ref(A, B, C, 1.5, -0.5), K) <= tol
+    plain = product(None, 1.0, 1.0, None)
+    assert rel_err(plain, ref(A, B), K) <= tol
+    small = hip.DeviceMatrix(1, 64, np.float32)
+    assert np.array_equal(product(None, 1.0, 1.0, small).view(np.uint8), plain.view(np.uint8))
+    for d in (ws, small):
+        d.free()
+
+
 @pytest.mark.parametrize("tile", [0, 1, 2])
 def test_forced_edge_variant_equals_fast_variant(hip, tile):
     """On tile-multiple shapes the predicated kernel and the unpredicated one run the same
