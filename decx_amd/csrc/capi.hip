@@ -83,6 +83,28 @@ uint32_t arm_split(GemmArgs& g, int elem_bytes, void* workspace, size_t workspac
     return sp.splits;
 }
 
+// y = alpha * x.B (+ beta * c).  Few columns and a long K: with a workspace, ranges of K go to workgroups of their
+// own and a second kernel adds their partial sums in range order; that kernel writes a dense y and reads c in y's type.
+int gevm_maybe_split(bool f16, bool out_f32, const void* x, const void* B, const void* c, void* y, uint32_t K, uint32_t N,
+                     uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, void* workspace,
+                     size_t workspace_bytes, hipStream_t stream)
+{
+    const SplitPlan sp = plan_gevm_split(f16, N, K, g_dev.compute_units);
+    const uint32_t ldw = (N + 3) / 4 * 4;
+    const bool reducible = incy == 1 && (!c || (incc == 1 && !(f16 && out_f32)));
+    if (sp.splits > 1 && reducible && workspace && aligned16(workspace) && workspace_bytes >= (size_t)sp.splits * ldw * 4) {
+        const int rv = launch_gevm(f16, out_f32, x, B, nullptr, y, K, N, ldb, incx, 1, 1, 1.f, 1.f, stream, sp.len,
+                                   (float*)workspace, ldw);
+        if (rv != 0) return rv;
+        GemmArgs r;
+        std::memset(&r, 0, sizeof r);
+        r.C = c; r.D = y; r.M = 1; r.N = N; r.ldc = N; r.ldd = N; r.alpha = alpha; r.beta = beta;
+        r.split_ws = workspace; r.split_ldd = ldw; r.split_stride = ldw;
+        return launch_split_reduce(f16 && !out_f32 ? 2 : 4, r, sp.splits, stream);
+    }
+    return launch_gevm(f16, out_f32, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream);
+}
+
 template <bool F16>
 int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, uint32_t N, uint32_t K,
              uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha, float beta, void* stream,
@@ -102,23 +124,9 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
         }
         return launch_gemv(F16, false, A, B, C, D, M, K, lda, ldb, ldc, ldd, alpha, beta, as_stream(stream));
     }
-    if (M == 1 && tile == DECX_HIP_TILE_AUTO && K > 0) {
-        // few columns and a long K: with a workspace, ranges of K go to workgroups of their own and a second kernel
-        // adds their partial sums in range order
-        const SplitPlan sp = plan_gevm_split(F16, N, K, g_dev.compute_units);
-        const uint32_t ldw = (N + 3) / 4 * 4;
-        if (sp.splits > 1 && workspace && aligned16(workspace) && workspace_bytes >= (size_t)sp.splits * ldw * 4) {
-            const int rv = launch_gevm(F16, false, A, B, nullptr, D, K, N, ldb, 1, 1, 1, 1.f, 1.f, as_stream(stream), sp.len,
-                                       (float*)workspace, ldw);
-            if (rv != 0) return rv;
-            GemmArgs r;
-            std::memset(&r, 0, sizeof r);
-            r.C = C; r.D = D; r.M = 1; r.N = N; r.ldc = ldc; r.ldd = ldd; r.alpha = alpha; r.beta = beta;
-            r.split_ws = workspace; r.split_ldd = ldw; r.split_stride = ldw;
-            return launch_split_reduce(F16 ? 2 : 4, r, sp.splits, as_stream(stream));
-        }
-        return launch_gevm(F16, false, A, B, C, D, K, N, ldb, 1, 1, 1, alpha, beta, as_stream(stream));
-    }
+    if (M == 1 && tile == DECX_HIP_TILE_AUTO && K > 0)
+        return gevm_maybe_split(F16, false, A, B, C, D, K, N, ldb, 1, 1, 1, alpha, beta, workspace, workspace_bytes,
+                                as_stream(stream));
 
     constexpr uint32_t per16 = F16 ? 8u : 4u;          // elements per 16 bytes
     GemmArgs g;
@@ -467,12 +475,13 @@ static int run_gemv(bool f16, bool out_f32, const void* A, const void* x, const 
 
 static int run_gevm(bool f16, bool out_f32, const void* x, const void* B, const void* c, void* y, uint32_t K,
                     uint32_t N, uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta,
-                    void* stream)
+                    void* stream, void* workspace = nullptr, size_t workspace_bytes = 0)
 {
     if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
     if (N == 0) return DECX_HIP_OK;
     if (!x || !B || !y || ldb < N || incx == 0 || incy == 0 || (c && incc == 0)) return DECX_HIP_E_INVALID_ARG;
-    return launch_gevm(f16, out_f32, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, as_stream(stream));
+    return gevm_maybe_split(f16, out_f32, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, workspace, workspace_bytes,
+                            as_stream(stream));
 }
 
 int decx_hip_gemv_f32(const float* A, const float* x, const float* c, float* y, uint32_t M, uint32_t K, uint32_t lda,
@@ -496,6 +505,20 @@ int decx_hip_gevm_f16(const uint16_t* x, const uint16_t* B, const uint16_t* c, v
                       void* stream)
 {
     return run_gevm(true, y_is_f32 != 0, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream);
+}
+
+int decx_hip_gevm_f32_ws(const float* x, const float* B, const float* c, float* y, uint32_t K, uint32_t N, uint32_t ldb,
+                         uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, void* workspace,
+                         size_t workspace_bytes, void* stream)
+{
+    return run_gevm(false, true, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream, workspace, workspace_bytes);
+}
+int decx_hip_gevm_f16_ws(const uint16_t* x, const uint16_t* B, const uint16_t* c, void* y, uint32_t K, uint32_t N,
+                         uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, int y_is_f32,
+                         void* workspace, size_t workspace_bytes, void* stream)
+{
+    return run_gevm(true, y_is_f32 != 0, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream, workspace,
+                    workspace_bytes);
 }
 
 int decx_hip_conv2d_pack_kernels_f32(const float* kernels, float* kmat, uint32_t k_w, uint32_t k_h, uint32_t depth,

@@ -61,6 +61,8 @@ SYMBOLS = {
     "decx_hip_gemv_f16": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _int, _vp]),
     "decx_hip_gevm_f32": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _vp]),
     "decx_hip_gevm_f16": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _int, _vp]),
+    "decx_hip_gevm_f32_ws": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _vp, _sz, _vp]),
+    "decx_hip_gevm_f16_ws": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _int, _vp, _sz, _vp]),
     "decx_hip_conv2d_pack_kernels_f32": (_int, [_vp, _vp] + [_u32] * 5 + [ctypes.c_uint64] + [_u32] * 3 + [_vp]),
     "decx_hip_conv2d_f32": (_int, [_vp] * 3 + [_u32] * 12 + [_vp]),
     "decx_hip_gemm_f64": (_int, [_vp] * 4 + [_u32] * 7 + [ctypes.c_double, ctypes.c_double, _vp]),
@@ -247,19 +249,22 @@ def gemv(A, x, y, c=None, alpha=1.0, beta=1.0, stream=None):
     check(rc, "gemv")
 
 
-def gevm(x, B, y, c=None, alpha=1.0, beta=1.0, stream=None):
-    """y (N) = alpha * x (K) . B (K x N) + beta * c through decx_hip_gevm_f32 / _f16."""
+def gevm(x, B, y, c=None, alpha=1.0, beta=1.0, stream=None, workspace=None):
+    """y (N) = alpha * x (K) . B (K x N) + beta * c through decx_hip_gevm_f32 / _f16, or their _ws forms when a
+    workspace (a DeviceMatrix) is given."""
     K, N = B.rows, B.cols
     (xp, incx), (yp, incy) = _as_vector(x, K), _as_vector(y, N)
     cp, incc = _as_vector(c, N) if c is not None else (None, 0)
     L = lib()
+    ws = () if workspace is None else (workspace.ptr, workspace.rows * workspace.pitch * workspace.dtype.itemsize)
     if B.dtype == np.float16:
         assert x.dtype == np.float16 and y.dtype in (np.float16, np.float32)
-        rc = L.decx_hip_gevm_f16(xp, B.ptr, cp, yp, K, N, B.pitch, incx, incc, incy, alpha, beta,
-                                 1 if y.dtype == np.float32 else 0, stream)
+        fn = L.decx_hip_gevm_f16 if workspace is None else L.decx_hip_gevm_f16_ws
+        rc = fn(xp, B.ptr, cp, yp, K, N, B.pitch, incx, incc, incy, alpha, beta, 1 if y.dtype == np.float32 else 0, *ws, stream)
     else:
         assert x.dtype == y.dtype == np.float32
-        rc = L.decx_hip_gevm_f32(xp, B.ptr, cp, yp, K, N, B.pitch, incx, incc, incy, alpha, beta, stream)
+        fn = L.decx_hip_gevm_f32 if workspace is None else L.decx_hip_gevm_f32_ws
+        rc = fn(xp, B.ptr, cp, yp, K, N, B.pitch, incx, incc, incy, alpha, beta, *ws, stream)
     check(rc, "gevm")
 
 

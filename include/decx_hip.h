@@ -200,6 +200,21 @@ DECX_HIP_API int decx_hip_gevm_f16(const uint16_t* x, const uint16_t* B, const u
                                    uint32_t K, uint32_t N, uint32_t ldb,
                                    uint32_t incx, uint32_t incc, uint32_t incy,
                                    float alpha, float beta, int y_is_f32, void* stream);
+/* Vector x matrix with a device workspace (decx_hip_gemm_workspace(elem_bytes, 1, N, K) bytes, 16-byte aligned): when
+ * the matrix has few columns and a long K, ranges of K go to workgroups of their own and a second kernel adds their
+ * partial sums in a fixed order -- the part of the reference's second pass reduce_sum2D_v_fp32_Async behind
+ * cu_vec_m_mat_fp32 (srcs/modules/BLAS/GEMM/CUDA/extreme_shapes/VMM_callers.cuh:67-202), taken only where one
+ * kernel would leave most CUs idle.  Needs incy == 1 (and incc == 1, c of y's type); otherwise, or with a smaller or
+ * null workspace, the single-kernel path runs. */
+DECX_HIP_API int decx_hip_gevm_f32_ws(const float* x, const float* B, const float* c, float* y,
+                                      uint32_t K, uint32_t N, uint32_t ldb,
+                                      uint32_t incx, uint32_t incc, uint32_t incy,
+                                      float alpha, float beta, void* workspace, size_t workspace_bytes, void* stream);
+DECX_HIP_API int decx_hip_gevm_f16_ws(const uint16_t* x, const uint16_t* B, const uint16_t* c, void* y,
+                                      uint32_t K, uint32_t N, uint32_t ldb,
+                                      uint32_t incx, uint32_t incc, uint32_t incy,
+                                      float alpha, float beta, int y_is_f32,
+                                      void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- 2-D convolution as an implicit GEMM ---------------------------------------------------
  * Replaces the planner, the im2col kernels, the im2col buffer and cu_im2col_GEMM_fp32 behind

@@ -116,6 +116,31 @@ def test_gevm_against_oracle(hip, oracle, tin, tout, tol, K, N, strided):
         assert rel_err(read_vec(dy), oracle_vm(oracle, x, B, c, 0.5, -2.0, tout), K) <= tol
 
 
+@pytest.mark.parametrize("tin,tout,tol", CASES)
+@pytest.mark.parametrize("K,N", [(8192, 2048), (33000, 100)])
+def test_gevm_split_over_k_through_a_workspace(hip, oracle, tin, tout, tol, K, N):
+    """Few columns and a long K through decx_hip_gevm_*_ws: ranges of K on workgroups of their own, partial sums added
+    in range order.  Strided x is fine; a strided y, or a c the second kernel cannot read, take the single kernel."""
+    esz = np.dtype(tin).itemsize
+    B = inputs(tin, K, N, 221); x = inputs(tin, 1, K, 222).reshape(-1); c = inputs(tin, 1, N, 223).reshape(-1)
+    need = hip.lib().decx_hip_gemm_workspace(esz, 1, N, K)
+    assert need > 0
+    ws = hip.DeviceMatrix(1, need // 4, np.float32)
+    ws.upload_raw(np.full((1, ws.pitch), np.nan, np.float32))
+    per = 16 // esz
+    dB = hip.DeviceMatrix(K, N, tin, (N + per - 1) // per * per, B, pad_value=np.nan)
+    for strided_x, strided_y in ((False, False), (True, False), (False, True)):
+        dx = vec(hip, x, strided_x); dc = vec(hip, c, strided_y)
+        dy = out_vec(hip, N, tout, strided_y)
+        hip.gevm(dx, dB, dy, workspace=ws); hip.sync()
+        first = read_vec(dy)
+        assert rel_err(first, oracle_vm(oracle, x, B, None, 1, 1, tout), K) <= tol
+        hip.gevm(dx, dB, dy, workspace=ws); hip.sync()
+        assert np.array_equal(read_vec(dy).view(np.uint8), first.view(np.uint8))
+        hip.gevm(dx, dB, dy, dc, 0.5, -2.0, workspace=ws); hip.sync()
+        assert rel_err(read_vec(dy), oracle_vm(oracle, x, B, c, 0.5, -2.0, tout), K) <= tol
+
+
 @pytest.mark.parametrize("tin,tout", [(np.float32, np.float32), (np.float16, np.float32), (np.float16, np.float16)])
 def test_exact_small_integer_sums(hip, tin, tout):
     """Small integers: every partial sum is an integer below 2^11, exact in any order and in fp16."""
