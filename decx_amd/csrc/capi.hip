@@ -64,7 +64,7 @@ int check_gemm(const void* A, const void* B, const void* C, const void* D, uint3
 SplitPlan split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
 {
     if (M == 0 || N == 0) return {1, 0};
-    if (elem_bytes != 8 && (M == 1 || N == 1)) return {1, 0};      // the vector corners have their own kernels
+    if (M == 1 || N == 1) return {1, 0};                            // the vector corners have their own kernels
     const TileInfo ti = elem_bytes == 8 ? tile_info_f64(choose_tile_f64(M, N))
                                         : elem_bytes == 2 ? tile_info_f16(choose_tile(true, M, N, true), true)
                                                           : tile_info_f32(choose_tile(false, M, N, true), true);
@@ -89,7 +89,7 @@ int gevm_maybe_split(bool f16, bool out_f32, const void* x, const void* B, const
                      uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, void* workspace,
                      size_t workspace_bytes, hipStream_t stream)
 {
-    const SplitPlan sp = plan_gevm_split(f16, N, K, g_dev.compute_units);
+    const SplitPlan sp = plan_gevm_split(f16 ? 2 : 4, N, K, g_dev.compute_units);
     const uint32_t ldw = (N + 3) / 4 * 4;
     const bool reducible = incy == 1 && (!c || (incc == 1 && !(f16 && out_f32)));
     if (sp.splits > 1 && reducible && workspace && aligned16(workspace) && workspace_bytes >= (size_t)sp.splits * ldw * 4) {
@@ -119,7 +119,7 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
     if (N == 1 && tile == DECX_HIP_TILE_AUTO && K > 0) {
         // x is the single column of a pitched K x 1 matrix: with a workspace it is gathered once into a dense vector
         if (workspace && workspace_bytes >= (size_t)K * (F16 ? 2 : 4) && gemv_gather_pays(M, K, ldb)) {
-            const int rg = launch_gather(F16, B, workspace, K, ldb, as_stream(stream));
+            const int rg = launch_gather(F16 ? 2 : 4, B, workspace, K, ldb, as_stream(stream));
             return rg != 0 ? rg : launch_gemv(F16, false, A, workspace, C, D, M, K, lda, 1, ldc, ldd, alpha, beta, as_stream(stream));
         }
         return launch_gemv(F16, false, A, B, C, D, M, K, lda, ldb, ldc, ldd, alpha, beta, as_stream(stream));
@@ -314,11 +314,11 @@ int decx_hip_gemm_f32(const float* A, const float* B, const float* C, float* D, 
 size_t decx_hip_gemm_workspace(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
 {
     if (!g_dev.ready || (elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8)) return 0;
-    if (elem_bytes != 8 && N == 1 && M > 0)                        // room for a dense copy of x
+    if (N == 1 && M > 0)                                           // room for a dense copy of x
         return gemv_gather_pays(M, K, 2) ? ((size_t)K * elem_bytes + 15) / 16 * 16 : 0;
-    if (elem_bytes != 8 && M == 1 && N > 0) {                      // room for the partial sums of ranges of K
-        const SplitPlan sp = plan_gevm_split(elem_bytes == 2, N, K, g_dev.compute_units);
-        return sp.splits > 1 ? (size_t)sp.splits * ((N + 3) / 4 * 4) * 4 : 0;
+    if (M == 1 && N > 0) {                                         // room for the partial sums of ranges of K
+        const SplitPlan sp = plan_gevm_split(elem_bytes, N, K, g_dev.compute_units);
+        return sp.splits > 1 ? (size_t)sp.splits * ((N + 3) / 4 * 4) * (elem_bytes == 8 ? 8 : 4) : 0;
     }
     const SplitPlan sp = split_plan(elem_bytes, M, N, K);
     return sp.splits > 1 ? (size_t)sp.splits * M * ((N + 3) / 4 * 4) * (elem_bytes == 8 ? 8 : 4) : 0;
@@ -357,6 +357,31 @@ static int run_gemm_f64(const double* A, const double* B, const double* C, doubl
     const int rc = check_gemm(A, B, C, D, M, N, K, lda, ldb, ldc, ldd);
     if (rc != DECX_HIP_OK || M == 0 || N == 0) return rc;
     if (tile != DECX_HIP_TILE_AUTO && (tile < 0 || tile >= TILE_COUNT)) return DECX_HIP_E_INVALID_ARG;
+
+    // the two vector corners: the bandwidth-bound kernels, as for the other real types
+    if (N == 1 && tile == DECX_HIP_TILE_AUTO && !force_plain && K > 0) {
+        if (workspace && workspace_bytes >= (size_t)K * 8 && gemv_gather_pays(M, K, ldb)) {
+            const int rg = launch_gather(8, B, workspace, K, ldb, as_stream(stream));
+            return rg != 0 ? rg : launch_gemv_f64(A, (const double*)workspace, C, D, M, K, lda, 1, ldc, ldd, alpha, beta, as_stream(stream));
+        }
+        return launch_gemv_f64(A, B, C, D, M, K, lda, ldb, ldc, ldd, alpha, beta, as_stream(stream));
+    }
+    if (M == 1 && tile == DECX_HIP_TILE_AUTO && !force_plain && K > 0) {
+        const SplitPlan sp = plan_gevm_split(8, N, K, g_dev.compute_units);
+        const uint32_t ldw = (N + 3) / 4 * 4;
+        if (sp.splits > 1 && workspace && aligned16(workspace) && workspace_bytes >= (size_t)sp.splits * ldw * 8) {
+            const int rv = launch_gevm_f64(A, B, nullptr, D, K, N, ldb, 1, 1, 1, 1.0, 1.0, as_stream(stream), sp.len,
+                                           (double*)workspace, ldw);
+            if (rv != 0) return rv;
+            GemmArgs r;
+            std::memset(&r, 0, sizeof r);
+            r.C = C; r.D = D; r.M = 1; r.N = N; r.ldc = ldc; r.ldd = ldd; r.alpha64 = alpha; r.beta64 = beta;
+            r.split_ws = workspace; r.split_ldd = ldw; r.split_stride = ldw;
+            return launch_split_reduce(8, r, sp.splits, as_stream(stream));
+        }
+        return launch_gevm_f64(A, B, C, D, K, N, ldb, 1, 1, 1, alpha, beta, as_stream(stream));
+    }
+
     GemmArgs g;
     std::memset(&g, 0, sizeof g);
     g.A = A; g.B = B; g.C = C; g.D = D;
@@ -571,7 +596,7 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
     std::memset(out, 0, sizeof *out);
     out->k_splits = 1;
     if (M == 0 || N == 0) return DECX_HIP_OK;
-    if (elem_bytes == 8) {                      // fp64 has no vector-corner kernels: N == 1 / M == 1 run as thin GEMMs
+    if (elem_bytes == 8 && !((N == 1 || M == 1) && K > 0)) {
         const int shape = choose_tile_f64(M, N);
         const TileInfo ti = tile_info_f64(shape);
         out->path = shape;
@@ -592,8 +617,8 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
     }
     if (M == 1 && K > 0) {
         out->path = DECX_HIP_PATH_GEVM;
-        out->tile_m = 1; out->tile_n = f16 ? 64 : 32;               // 128 bytes of a row, or 64 when that leaves CUs idle
-        const SplitPlan sp = plan_gevm_split(f16, N, K, g_dev.ready ? g_dev.compute_units : 256);
+        out->tile_m = 1; out->tile_n = 128u / (uint32_t)elem_bytes; // 128 bytes of a row, or 64 when that leaves CUs idle
+        const SplitPlan sp = plan_gevm_split(elem_bytes, N, K, g_dev.compute_units);
         if (sp.splits > 1) {                                        // with a workspace: whole lines, several ranges of K
             out->k_splits = sp.splits;
             out->grid = (N + out->tile_n - 1) / out->tile_n * sp.splits;

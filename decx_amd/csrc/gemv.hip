@@ -9,7 +9,8 @@
 // VMM_fp32.cu:35-146, VMM_fp16.cu, VMM_callers.cuh:67-202): here a workgroup finishes its
 // outputs itself, so there are no partial sums to reduce in another kernel.  fp16 inputs
 // are always accumulated in fp32 (the reference's level 1); the result is written as fp32
-// or rounded once to fp16, whichever the caller asks for.
+// or rounded once to fp16, whichever the caller asks for.  fp64 matrices (the reference's cu_mat_m_vec_fp64 /
+// cu_vec_m_mat_fp64, VMM_fp64.cu) run on the same kernels with sums in double.
 //
 // gemv: 16 wavefronts per workgroup, two rows per wavefront (32 rows per workgroup: 8192
 //   rows give one workgroup per CU with 64 KB of A in flight), one row per wavefront for
@@ -34,17 +35,29 @@ namespace {
 constexpr int GEMV_THREADS = 1024;
 constexpr int GEMV_WAVES = GEMV_THREADS / 64;
 constexpr int GEMV_ROWS_PER_BLOCK = 2 * GEMV_WAVES;
-constexpr int GEMV_KC = 4096;            // floats of x staged per chunk (16 KB of LDS)
+constexpr int GEMV_KC = 4096;            // elements of x staged per chunk (16 KB of LDS, 32 KB for fp64)
+
+typedef double doublex2 __attribute__((ext_vector_type(2)));
 
 template <typename T> struct Per16 { static constexpr int n = 16 / sizeof(T); };
 
-__device__ __forceinline__ float to_float(float v) { return v; }
-__device__ __forceinline__ float to_float(_Float16 v) { return (float)v; }
+// the type sums are kept in: fp32 for fp32 and fp16 inputs, fp64 for fp64
+template <typename T> struct Acc { typedef float type; };
+template <> struct Acc<double> { typedef double type; };
 
-// 16 bytes of T at p, widened to float
-template <typename T> __device__ __forceinline__ void load16(const T* p, float (&out)[Per16<T>::n])
+__device__ __forceinline__ float to_acc(float v) { return v; }
+__device__ __forceinline__ float to_acc(_Float16 v) { return (float)v; }
+__device__ __forceinline__ double to_acc(double v) { return v; }
+__device__ __forceinline__ float fma_acc(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double fma_acc(double a, double b, double c) { return __builtin_fma(a, b, c); }
+
+// 16 bytes of T at p, widened to the accumulation type
+template <typename T> __device__ __forceinline__ void load16(const T* p, typename Acc<T>::type (&out)[Per16<T>::n])
 {
-    if constexpr (sizeof(T) == 4) {
+    if constexpr (sizeof(T) == 8) {
+        const doublex2 v = *(const doublex2*)p;
+        out[0] = v[0]; out[1] = v[1];
+    } else if constexpr (sizeof(T) == 4) {
         const floatx4 v = *(const floatx4*)p;
 #pragma unroll
         for (int e = 0; e < 4; ++e) out[e] = v[e];
@@ -55,7 +68,7 @@ template <typename T> __device__ __forceinline__ void load16(const T* p, float (
     }
 }
 
-__device__ __forceinline__ float wave_sum(float v)
+template <typename A> __device__ __forceinline__ A wave_sum(A v)
 {
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
@@ -69,19 +82,20 @@ template <typename T, typename TO, int RPW, int WPR>
 __global__ void __launch_bounds__(GEMV_THREADS)
 gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restrict__ c, TO* __restrict__ y,
             uint32_t M, uint32_t K, uint32_t lda, uint32_t incx, uint32_t incc, uint32_t incy,
-            float alpha, float beta, uint32_t vec_ok)
+            typename Acc<T>::type alpha, typename Acc<T>::type beta, uint32_t vec_ok)
 {
+    typedef typename Acc<T>::type A_t;
     constexpr int N16 = Per16<T>::n;
-    __shared__ __attribute__((aligned(16))) float xs[GEMV_KC];
+    __shared__ __attribute__((aligned(16))) A_t xs[GEMV_KC];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     static_assert(WPR == 1 || RPW == 1, "rows are split over wavefronts only one at a time");
-    __shared__ float wave_sums[GEMV_WAVES];
+    __shared__ A_t wave_sums[GEMV_WAVES];
     const int sub = wave % WPR;                            // which share of the steps of K this wavefront takes
     const uint32_t row0 = blockIdx.x * (RPW * GEMV_WAVES / WPR) + (wave / WPR) * RPW;
     const bool has0 = row0 < M, has1 = RPW == 2 && row0 + 1 < M;
     const T* a0 = A + (size_t)(has0 ? row0 : 0) * lda;
     const T* a1 = A + (size_t)(has1 ? row0 + 1 : 0) * lda;
-    float s0 = 0.f, s1 = 0.f;
+    A_t s0 = 0, s1 = 0;
 
     // Every workgroup walks the same K range of rows that lie a whole number of pitches apart; started
     // together at k = 0 they would all pull on the same memory channels at the same time.  So each
@@ -93,7 +107,7 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
         const uint32_t kc = chunk * GEMV_KC;
         const uint32_t len = (K - kc) < (uint32_t)GEMV_KC ? (K - kc) : (uint32_t)GEMV_KC;
         __syncthreads();                                   // previous chunk fully consumed
-        for (uint32_t i = t; i < len; i += GEMV_THREADS) xs[i] = to_float(x[(size_t)(kc + i) * incx]);
+        for (uint32_t i = t; i < len; i += GEMV_THREADS) xs[i] = to_acc(x[(size_t)(kc + i) * incx]);
         __syncthreads();
         const uint32_t lenv = vec_ok ? (len / N16) * N16 : 0u;   // part done with 128-bit loads
         if (has0) {
@@ -105,20 +119,20 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
                 const uint32_t step = step0 + i < steps ? step0 + i : step0 + i - steps;
                 const uint32_t k = step * STEP + lane * N16;
                 if (k < lenv) {
-                    float av[N16], bv[N16];
+                    A_t av[N16], bv[N16];
                     load16<T>(a0 + kc + k, av);
                     if (has1) load16<T>(a1 + kc + k, bv);
 #pragma unroll
                     for (int e = 0; e < N16; ++e) {
-                        const float xv = xs[k + e];
-                        s0 = __builtin_fmaf(av[e], xv, s0);
-                        if (has1) s1 = __builtin_fmaf(bv[e], xv, s1);
+                        const A_t xv = xs[k + e];
+                        s0 = fma_acc(av[e], xv, s0);
+                        if (has1) s1 = fma_acc(bv[e], xv, s1);
                     }
                 }
             }
             for (uint32_t k = lenv + lane + (sub ? len : 0u); k < len; k += 64) {   // the first wavefront of a row takes the tail
-                s0 = __builtin_fmaf(to_float(a0[kc + k]), xs[k], s0);
-                if (has1) s1 = __builtin_fmaf(to_float(a1[kc + k]), xs[k], s1);
+                s0 = fma_acc(to_acc(a0[kc + k]), xs[k], s0);
+                if (has1) s1 = fma_acc(to_acc(a1[kc + k]), xs[k], s1);
             }
         }
     }
@@ -133,13 +147,13 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
     }
     if (lane == 0) {
         if (has0) {
-            float o = s0;
-            if (c) o = __builtin_fmaf(to_float(c[(size_t)row0 * incc]), beta, alpha * o);
+            A_t o = s0;
+            if (c) o = fma_acc(to_acc(c[(size_t)row0 * incc]), beta, alpha * o);
             y[(size_t)row0 * incy] = (TO)o;
         }
         if (has1) {
-            float o = s1;
-            if (c) o = __builtin_fmaf(to_float(c[(size_t)(row0 + 1) * incc]), beta, alpha * o);
+            A_t o = s1;
+            if (c) o = fma_acc(to_acc(c[(size_t)(row0 + 1) * incc]), beta, alpha * o);
             y[(size_t)(row0 + 1) * incy] = (TO)o;
         }
     }
@@ -150,8 +164,10 @@ template <typename T, typename TO, int CL>
 __global__ void __launch_bounds__(GEMV_THREADS)
 gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restrict__ c, TO* __restrict__ y,
             uint32_t K, uint32_t N, uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy,
-            float alpha, float beta, uint32_t vec_ok, uint32_t split_len, float* __restrict__ partial, uint32_t partial_stride)
+            typename Acc<T>::type alpha, typename Acc<T>::type beta, uint32_t vec_ok, uint32_t split_len,
+            typename Acc<T>::type* __restrict__ partial, uint32_t partial_stride)
 {
+    typedef typename Acc<T>::type A_t;
     constexpr int N16 = Per16<T>::n;
     constexpr int CB = CL * N16;                           // columns per workgroup
     if (split_len) {                                       // blockIdx.y takes a range of K; its sums go to `partial`
@@ -161,8 +177,8 @@ gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restric
         K = K - k0 < split_len ? K - k0 : split_len;
     }
     constexpr int RL = 64 / CL;                            // rows per wavefront and sweep
-    __shared__ __attribute__((aligned(16))) float xs[GEMV_KC];
-    __shared__ float red[GEMV_WAVES][CB];
+    __shared__ __attribute__((aligned(16))) A_t xs[GEMV_KC];
+    __shared__ A_t red[GEMV_WAVES][CB];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int col_lane = lane % CL, row_lane = lane / CL;
     // Half-line column groups: the two workgroups that share every 128-byte line of B should share an L2,
@@ -171,36 +187,36 @@ gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restric
     if (CL == 4 && group < gridDim.x / 16 * 16) group = (group / 16) * 16 + (group % 8) * 2 + (group / 8) % 2;
     const uint32_t n0 = group * CB + col_lane * N16;
     const bool whole = vec_ok && (n0 + N16 <= N);
-    float acc[N16];
+    A_t acc[N16];
 #pragma unroll
-    for (int e = 0; e < N16; ++e) acc[e] = 0.f;
+    for (int e = 0; e < N16; ++e) acc[e] = 0;
 
     for (uint32_t kc = 0; kc < K; kc += GEMV_KC) {
         const uint32_t len = (K - kc) < (uint32_t)GEMV_KC ? (K - kc) : (uint32_t)GEMV_KC;
         __syncthreads();
-        for (uint32_t i = t; i < len; i += GEMV_THREADS) xs[i] = to_float(x[(size_t)(kc + i) * incx]);
+        for (uint32_t i = t; i < len; i += GEMV_THREADS) xs[i] = to_acc(x[(size_t)(kc + i) * incx]);
         __syncthreads();
         if (n0 < N) {
 #pragma unroll 2
             for (uint32_t k = wave * RL + row_lane; k < len; k += GEMV_WAVES * RL) {
                 const T* p = B + (size_t)(kc + k) * ldb + n0;
-                const float xv = xs[k];
+                const A_t xv = xs[k];
                 if (whole) {
-                    float bv[N16];
+                    A_t bv[N16];
                     load16<T>(p, bv);
 #pragma unroll
-                    for (int e = 0; e < N16; ++e) acc[e] = __builtin_fmaf(xv, bv[e], acc[e]);
+                    for (int e = 0; e < N16; ++e) acc[e] = fma_acc(xv, bv[e], acc[e]);
                 } else {
 #pragma unroll
                     for (int e = 0; e < N16; ++e)
-                        if (n0 + e < N) acc[e] = __builtin_fmaf(xv, to_float(p[e]), acc[e]);
+                        if (n0 + e < N) acc[e] = fma_acc(xv, to_acc(p[e]), acc[e]);
                 }
             }
         }
     }
 #pragma unroll
     for (int e = 0; e < N16; ++e) {
-        float v = acc[e];
+        A_t v = acc[e];
         if (CL == 4) v += __shfl_xor(v, 4, 64);
         v += __shfl_xor(v, 8, 64);
         v += __shfl_xor(v, 16, 64);
@@ -211,11 +227,11 @@ gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restric
     if (t < CB) {
         const uint32_t n = group * CB + t;
         if (n < N) {
-            float o = 0.f;
+            A_t o = 0;
 #pragma unroll
             for (int w = 0; w < GEMV_WAVES; ++w) o += red[w][t];
             if (split_len) { partial[(size_t)blockIdx.y * partial_stride + n] = o; return; }
-            if (c) o = __builtin_fmaf(to_float(c[(size_t)n * incc]), beta, alpha * o);
+            if (c) o = fma_acc(to_acc(c[(size_t)n * incc]), beta, alpha * o);
             y[(size_t)n * incy] = (TO)o;
         }
     }
@@ -232,7 +248,8 @@ namespace {
 
 template <typename T, typename TO>
 void launch_gemv_as(const void* A, const void* x, const void* c, void* y, uint32_t M, uint32_t K, uint32_t lda,
-                    uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream)
+                    uint32_t incx, uint32_t incc, uint32_t incy, typename Acc<T>::type alpha, typename Acc<T>::type beta,
+                    hipStream_t stream)
 {
     const uint32_t vec = rows_vectorisable<T>(A, lda);
     auto launch = [&](auto rpw_c, auto wpr_c) {
@@ -283,12 +300,20 @@ bool gemv_gather_pays(uint32_t M, uint32_t K, uint32_t incx)
     return K >= 3072 && M >= 3072;
 }
 
-int launch_gather(bool f16, const void* x, void* dst, uint32_t K, uint32_t inc, hipStream_t stream)
+int launch_gather(int elem_bytes, const void* x, void* dst, uint32_t K, uint32_t inc, hipStream_t stream)
 {
     if (K == 0) return 0;
     const dim3 grid((K + 255) / 256);
-    if (f16) hipLaunchKernelGGL(gather_kernel<_Float16>, grid, dim3(256), 0, stream, (const _Float16*)x, (_Float16*)dst, K, inc);
+    if (elem_bytes == 2) hipLaunchKernelGGL(gather_kernel<_Float16>, grid, dim3(256), 0, stream, (const _Float16*)x, (_Float16*)dst, K, inc);
+    else if (elem_bytes == 8) hipLaunchKernelGGL(gather_kernel<double>, grid, dim3(256), 0, stream, (const double*)x, (double*)dst, K, inc);
     else hipLaunchKernelGGL(gather_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, (float*)dst, K, inc);
+    return (int)hipGetLastError();
+}
+
+int launch_gemv_f64(const double* A, const double* x, const double* c, double* y, uint32_t M, uint32_t K, uint32_t lda,
+                    uint32_t incx, uint32_t incc, uint32_t incy, double alpha, double beta, hipStream_t stream)
+{
+    launch_gemv_as<double, double>(A, x, c, y, M, K, lda, incx, incc, incy, alpha, beta, stream);
     return (int)hipGetLastError();
 }
 
@@ -305,8 +330,8 @@ namespace {
 
 template <typename T, typename TO>
 void launch_gevm_as(const void* x, const void* B, const void* c, void* y, uint32_t K, uint32_t N, uint32_t ldb,
-                    uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream,
-                    uint32_t split_len, float* partial, uint32_t partial_stride)
+                    uint32_t incx, uint32_t incc, uint32_t incy, typename Acc<T>::type alpha, typename Acc<T>::type beta,
+                    hipStream_t stream, uint32_t split_len, typename Acc<T>::type* partial, uint32_t partial_stride)
 {
     // 128-byte column groups unless they leave CUs without a workgroup (fp16 at N = 8192: 128 groups for
     // 256 CUs); then 64-byte groups, two workgroups per cache line -- or, with a workspace for partial sums,
@@ -321,7 +346,7 @@ void launch_gevm_as(const void* x, const void* B, const void* c, void* y, uint32
     else
         hipLaunchKernelGGL((gevm_kernel<T, TO, 4>), dim3((N + cb8 / 2 - 1) / (cb8 / 2)), dim3(GEMV_THREADS), 0, stream,
                            (const T*)x, (const T*)B, (const T*)c, (TO*)y, K, N, ldb, incx, incc, incy, alpha, beta, vec, 0u,
-                           (float*)nullptr, 0u);
+                           (typename Acc<T>::type*)nullptr, 0u);
 }
 
 }  // namespace
@@ -331,11 +356,11 @@ void launch_gevm_as(const void* x, const void* B, const void* c, void* y, uint32
 // that adds the partial sums costs a launch, so this is for matrices that keep the first one busy long enough:
 // 1 x 2048 x 8192 19.5 -> 16.5 us, 1 x 512 x 32768 69 -> 23, 1 x 64 x 65536 116 -> 23 (1 x 512 x 8192 would go from
 // 9 to 14 and stays whole).  A range is a multiple of the 128 rows a workgroup sweeps at a time, at least 256 long.
-SplitPlan plan_gevm_split(bool f16, uint32_t N, uint32_t K, uint32_t cus)
+SplitPlan plan_gevm_split(int elem_bytes, uint32_t N, uint32_t K, uint32_t cus)
 {
-    const uint32_t cb8 = f16 ? 64u : 32u;
+    const uint32_t cb8 = 128u / (uint32_t)elem_bytes;
     const uint32_t groups = (N + cb8 - 1) / cb8;
-    const uint64_t bytes = (uint64_t)K * N * (f16 ? 2 : 4);
+    const uint64_t bytes = (uint64_t)K * N * (uint32_t)elem_bytes;
     if (groups == 0 || groups * 4 > cus || (K < 16384 && bytes < (32ull << 20))) return {1, 0};
     uint32_t splits = (2 * cus + groups - 1) / groups;
     if (splits > K / 256) splits = K / 256;
@@ -352,6 +377,14 @@ int launch_gevm(bool f16, bool out_f32, const void* x, const void* B, const void
     if (!f16) launch_gevm_as<float, float>(x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream, split_len, partial, partial_stride);
     else if (out_f32) launch_gevm_as<_Float16, float>(x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream, split_len, partial, partial_stride);
     else launch_gevm_as<_Float16, _Float16>(x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream, split_len, partial, partial_stride);
+    return (int)hipGetLastError();
+}
+
+int launch_gevm_f64(const double* x, const double* B, const double* c, double* y, uint32_t K, uint32_t N, uint32_t ldb,
+                    uint32_t incx, uint32_t incc, uint32_t incy, double alpha, double beta, hipStream_t stream,
+                    uint32_t split_len, double* partial, uint32_t partial_stride)
+{
+    launch_gevm_as<double, double>(x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream, split_len, partial, partial_stride);
     return (int)hipGetLastError();
 }
 
