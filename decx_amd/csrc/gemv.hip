@@ -9,8 +9,8 @@
 // VMM_fp32.cu:35-146, VMM_fp16.cu, VMM_callers.cuh:67-202): here a workgroup finishes its
 // outputs itself, so there are no partial sums to reduce in another kernel.  fp16 inputs
 // are always accumulated in fp32 (the reference's level 1); the result is written as fp32
-// or rounded once to fp16, whichever the caller asks for.  fp64 matrices (the reference's cu_mat_m_vec_fp64 /
-// cu_vec_m_mat_fp64, VMM_fp64.cu) run on the same kernels with sums in double.
+// or rounded once to fp16, whichever the caller asks for.  fp64 matrices run on the same kernels
+// with sums in double (the reference has no fp64 form of these: its VMM_fp64.cu is empty).
 //
 // gemv: 16 wavefronts per workgroup, two rows per wavefront (32 rows per workgroup: 8192
 //   rows give one workgroup per CU with 64 KB of A in flight), one row per wavefront for

@@ -154,8 +154,8 @@ DECX_HIP_API int decx_hip_gemm_f16(const uint16_t* A, const uint16_t* B, const u
  * Replaces the body of decx::blas::GEMM_fp64 (srcs/modules/BLAS/GEMM/CUDA/GEMM_LS.cu:164-211) and
  * cu_GEMM_fp64_*_16_64_64 (large_squares/GEMM_kernels.cuh:182-189).  Operands that are not 16-byte
  * aligned (base or pitch), and K == 0, take a plain one-thread-per-element kernel.  N == 1 and M == 1 run on the
- * bandwidth-bound vector kernels with sums in double (the reference's cu_mat_m_vec_fp64 / cu_vec_m_mat_fp64,
- * srcs/modules/BLAS/GEMM/CUDA/extreme_shapes/VMM_fp64.cu). */
+ * bandwidth-bound vector kernels with sums in double (the reference has none for fp64: its
+ * srcs/modules/BLAS/GEMM/CUDA/extreme_shapes/VMM_fp64.cu is empty and such shapes go through GEMM_fp64). */
 DECX_HIP_API int decx_hip_gemm_f64(const double* A, const double* B, const double* C, double* D,
                                    uint32_t M, uint32_t N, uint32_t K,
                                    uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
