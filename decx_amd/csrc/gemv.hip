@@ -130,7 +130,7 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
                     }
                 }
             }
-            for (uint32_t k = lenv + lane + (sub ? len : 0u); k < len; k += 64) {   // the first wavefront of a row takes the tail
+            for (uint32_t k = lenv + lane + 64u * sub; k < len; k += 64u * WPR) {   // the tail, or a whole unaligned row
                 s0 = fma_acc(to_acc(a0[kc + k]), xs[k], s0);
                 if (has1) s1 = fma_acc(to_acc(a1[kc + k]), xs[k], s1);
             }
