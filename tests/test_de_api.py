@@ -72,6 +72,14 @@ def test_gpu_side_closed_forms_and_error_paths():
     ("f16", 257, 130, 515, True, 1.5, -0.5),
     ("f64", 1000, 700, 333, False, 1.0, 1.0),
     ("f64", 1000, 700, 333, True, -0.5, 2.0),
+    # the vector corners with the module's workspace: column operand copied into a dense vector, K of a row
+    # operand split over workgroups, fp64 on the vector kernels
+    ("f32", 1100, 1, 8200, True, 1.5, -0.5),
+    ("f16", 2100, 1, 4100, False, 1.0, 1.0),
+    ("f32", 1, 70, 20000, True, 1.5, -0.5),
+    ("f16", 1, 513, 33000, False, 1.0, 1.0),
+    ("f64", 2100, 1, 4100, True, -0.5, 2.0),
+    ("f64", 1, 100, 33000, False, 1.0, 1.0),
 ])
 def test_gemm_through_the_objects_matches_oracle(oracle, dt, M, N, K, with_c, alpha, beta):
     if dt == "f32":
