@@ -59,27 +59,73 @@ int check_gemm(const void* A, const void* B, const void* C, const void* D, uint3
     return DECX_HIP_OK;
 }
 
-// Split K is planned for products on 16-byte aligned operands whose tiles would leave most CUs idle.
-// elem_bytes: 2, 4 or 8.
-SplitPlan split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
+// Split K is planned for products on 16-byte aligned operands whose tiles would leave CUs idle or unevenly loaded.
+// elem_bytes: 2, 4 or 8.  `shape` is the tile the split runs on (it may differ from the one the whole product takes).
+struct SplitChoice { int shape; uint32_t splits, len; };
+SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
 {
-    if (M == 0 || N == 0) return {1, 0};
-    if (M == 1 || N == 1) return {1, 0};                            // the vector corners have their own kernels
-    const TileInfo ti = elem_bytes == 8 ? tile_info_f64(choose_tile_f64(M, N))
-                                        : elem_bytes == 2 ? tile_info_f16(choose_tile(true, M, N, true), true)
-                                                          : tile_info_f32(choose_tile(false, M, N, true), true);
-    return plan_split_k((uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn), K, g_dev.compute_units);
+    if (M == 0 || N == 0) return {0, 1, 0};
+    if (M == 1 || N == 1) return {0, 1, 0};                         // the vector corners have their own kernels
+    const uint32_t cus = g_dev.compute_units;
+    const int shape = elem_bytes == 8 ? choose_tile_f64(M, N) : choose_tile(elem_bytes == 2, M, N, true);
+    const TileInfo ti = elem_bytes == 8 ? tile_info_f64(shape)
+                                        : elem_bytes == 2 ? tile_info_f16(shape, true) : tile_info_f32(shape, true);
+    // outputs of at most half as many tiles as there are CUs: up to two workgroups per CU
+    const SplitPlan sp = plan_split_k((uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn), K, cus);
+    if (sp.splits > 1) return {shape, sp.splits, sp.len};
+    // Outputs of a few hundred small tiles and a long K: one or two workgroups per CU run well below the rate of a
+    // full CU, and 1.5 per CU leave half the chip waiting for the other half.  Measured: fp32 1280 x 1024 x 8192
+    // 259 -> 186 us with 64 x 64 tiles on 3 ranges, 768 x 768 x 16384 292 -> 165 (7 ranges); fp16 1536 x 1024 x 8192
+    // 57 -> 43 us with 128 x 128 tiles on 2 ranges, 768 x 768 x 16384 61 -> 37 (4 ranges); 2048 x 2048 x 8192 and
+    // 1024 x 2048 x 4096 gain nothing and stay whole.
+    const auto tiles_of = [&](uint32_t b) { return (uint64_t)((M + b - 1) / b) * ((N + b - 1) / b); };
+    if (elem_bytes == 4 && K >= 4096) {
+        // 64 x 64 tiles, up to five workgroups per CU.  score = (workgroups on the busiest CU / the average) x what a
+        // CU loses with m workgroups against a full one; the ranges p that make t * p an even three to five per CU win.
+        const uint64_t t = tiles_of(64);
+        const auto score = [&](uint32_t p) {
+            const uint64_t wgs = t * p, m = (wgs + cus - 1) / cus;
+            static const double loss[6] = {1.0, 1.35, 1.10, 1.03, 1.0, 1.0};
+            return (double)(m * cus) / (double)wgs * (m <= 5 ? loss[m] : 1.0) + 0.01 * p;
+        };
+        if (t <= 3ull * cus) {
+            uint32_t best = 1;
+            double best_score = score(1) / 1.15;                    // the second kernel must be worth it
+            for (uint32_t p2 = 2; p2 <= 8 && K / p2 >= 1024 && t * p2 <= 5ull * cus; ++p2)
+                if (score(p2) < best_score) { best_score = score(p2); best = p2; }
+            if (best > 1) {
+                const uint32_t len = ((K + best - 1) / best + 31) / 32 * 32;
+                return {TILE_64x64, (K + len - 1) / len, len};
+            }
+        }
+    }
+    if (elem_bytes == 2 && K >= 6144) {
+        // 128 x 128 tiles towards one workgroup per CU, a power of two of ranges at least 2048 long, and only when
+        // that occupies more than half the chip (1024 x 1024 x 6144 on 2 ranges: 26.6 -> 28.9 us)
+        const uint64_t t = tiles_of(128);
+        if (t * 2 < cus) {
+            uint32_t p2 = 1;
+            while (p2 * 2 * t <= cus && p2 < 8 && K / (p2 * 2) >= 2048) p2 *= 2;
+            if (p2 > 1 && t * p2 * 20 >= 11ull * cus) {
+                const uint32_t len = ((K + p2 - 1) / p2 + 31) / 32 * 32;
+                return {TILE_128x128, (K + len - 1) / len, len};
+            }
+        }
+    }
+    return {shape, 1, 0};
 }
 
-// Fills the split fields of g when the plan says so and the workspace is large enough; returns the number of splits.
-uint32_t arm_split(GemmArgs& g, int elem_bytes, void* workspace, size_t workspace_bytes)
+// Fills the split fields of g when the plan says so and the workspace is large enough; returns the number of splits
+// and, with more than one, the tile shape they run on.
+uint32_t arm_split(GemmArgs& g, int elem_bytes, void* workspace, size_t workspace_bytes, int& shape)
 {
     if (!workspace || !aligned16(workspace)) return 1;
-    const SplitPlan sp = split_plan(elem_bytes, g.M, g.N, g.K);
+    const SplitChoice sp = split_plan(elem_bytes, g.M, g.N, g.K);
     const uint32_t ldw = (g.N + 3) / 4 * 4;
     const size_t part = (size_t)(elem_bytes == 8 ? 8 : 4);
     if (sp.splits <= 1 || workspace_bytes < (size_t)sp.splits * g.M * ldw * part) return 1;
     g.split_len = sp.len; g.split_ldd = ldw; g.split_stride = (uint64_t)g.M * ldw; g.split_ws = workspace;
+    shape = sp.shape;
     return sp.splits;
 }
 
@@ -137,10 +183,10 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
     g.alpha = alpha; g.beta = beta;
     g.vec_ok = (aligned16(A) && aligned16(B) && aligned16(D) && (!C || aligned16(C)) &&
                 lda % per16 == 0 && ldb % per16 == 0 && ldd % per16 == 0 && (!C || ldc % per16 == 0)) ? 1u : 0u;
-    const int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile(F16, M, N, g.vec_ok != 0) : tile;
+    int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile(F16, M, N, g.vec_ok != 0) : tile;
     const bool edge = force_edge != 0 || K == 0;
     if (workspace && tile == DECX_HIP_TILE_AUTO && !edge && g.vec_ok && dma_offsets_fit(g, F16 ? 2 : 4)) {
-        const uint32_t splits = arm_split(g, F16 ? 2 : 4, workspace, workspace_bytes);
+        const uint32_t splits = arm_split(g, F16 ? 2 : 4, workspace, workspace_bytes, shape);
         if (splits > 1) {
             const int rl = F16 ? launch_gemm_f16(shape, false, g, as_stream(stream)) : launch_gemm_f32(shape, false, g, as_stream(stream));
             return rl != 0 ? rl : launch_split_reduce(F16 ? 2 : 4, g, splits, as_stream(stream));
@@ -320,7 +366,7 @@ size_t decx_hip_gemm_workspace(int elem_bytes, uint32_t M, uint32_t N, uint32_t 
         const SplitPlan sp = plan_gevm_split(elem_bytes, N, K, g_dev.compute_units);
         return sp.splits > 1 ? (size_t)sp.splits * ((N + 3) / 4 * 4) * (elem_bytes == 8 ? 8 : 4) : 0;
     }
-    const SplitPlan sp = split_plan(elem_bytes, M, N, K);
+    const SplitChoice sp = split_plan(elem_bytes, M, N, K);
     return sp.splits > 1 ? (size_t)sp.splits * M * ((N + 3) / 4 * 4) * (elem_bytes == 8 ? 8 : 4) : 0;
 }
 
@@ -391,9 +437,9 @@ static int run_gemm_f64(const double* A, const double* B, const double* C, doubl
     g.alpha64 = alpha; g.beta64 = beta;
     g.vec_ok = (aligned16(A) && aligned16(B) && aligned16(D) && (!C || aligned16(C)) &&
                 lda % 2 == 0 && ldb % 2 == 0 && ldd % 2 == 0 && (!C || ldc % 2 == 0)) ? 1u : 0u;
-    const int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile_f64(M, N) : tile;
+    int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile_f64(M, N) : tile;
     if (workspace && tile == DECX_HIP_TILE_AUTO && !force_plain && K > 0 && g.vec_ok && dma_offsets_fit(g, 8)) {
-        const uint32_t splits = arm_split(g, 8, workspace, workspace_bytes);
+        const uint32_t splits = arm_split(g, 8, workspace, workspace_bytes, shape);
         if (splits > 1) {
             const int rl = launch_gemm_f64(shape, false, g, as_stream(stream));
             return rl != 0 ? rl : launch_split_reduce(8, g, splits, as_stream(stream));
@@ -604,7 +650,10 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
         out->grid = ((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
         out->edge = (K == 0 || !aligned) ? 1 : 0;
         if (out->edge) { out->tile_m = out->tile_n = 16; out->grid = ((M + 15) / 16) * ((N + 15) / 16); }
-        else { out->k_splits = split_plan(8, M, N, K).splits; out->grid *= out->k_splits; }
+        else {
+            const SplitChoice sc = split_plan(8, M, N, K);
+            out->k_splits = sc.splits; out->grid *= out->k_splits;
+        }
         return DECX_HIP_OK;
     }
     const bool f16 = elem_bytes == 2;
@@ -635,7 +684,15 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
     out->grid = ((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
     // the direct-to-LDS kernels take every aligned shape
     out->edge = (K == 0 || !aligned) ? 1 : 0;
-    if (!out->edge) { out->k_splits = split_plan(elem_bytes, M, N, K).splits; out->grid *= out->k_splits; }
+    if (!out->edge) {
+        const SplitChoice sc = split_plan(elem_bytes, M, N, K);
+        if (sc.splits > 1 && sc.shape != shape) {                   // the split runs on another tile than the whole product
+            const TileInfo ts = f16 ? tile_info_f16(sc.shape, true) : tile_info_f32(sc.shape, true);
+            out->path = sc.shape; out->tile_m = ts.bm; out->tile_n = ts.bn;
+            out->grid = ((M + ts.bm - 1) / ts.bm) * ((N + ts.bn - 1) / ts.bn);
+        }
+        out->k_splits = sc.splits; out->grid *= out->k_splits;
+    }
     return DECX_HIP_OK;
 }
 

@@ -65,7 +65,9 @@ typedef struct decx_hip_plan {
                                       aligned, or K == 0); 0: a direct-to-LDS kernel */
     uint32_t tile_m, tile_n;       /* block tile */
     uint32_t grid;                 /* workgroups launched (tiles x k_splits) */
-    uint32_t k_splits;             /* ranges K is cut into when the *_ws entry point gets its workspace; 1: no split */
+    uint32_t k_splits;             /* ranges K is cut into when the *_ws entry point gets its workspace; 1: no split.
+                                      With more than one, path / tile are those of the split (it may run on a smaller
+                                      tile than the whole product takes without a workspace) */
 } decx_hip_plan;
 
 /* ---- device, memory, streams, events --------------------------------------------------

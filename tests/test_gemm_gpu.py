@@ -318,6 +318,51 @@ def test_f16_split_k_through_a_workspace(hip, oracle, M, N, K):
     ws.free()
 
 
+@pytest.mark.parametrize("dtype,M,N,K,tile,splits", [
+    (np.float32, 1280, 1024, 4096, 64, 4),          # 320 tiles of 64 x 64: 1.25 per CU, on 4 ranges five per CU
+    (np.float32, 900, 700, 4100, 64, 3),            # ragged output, K not a multiple of the range
+    (np.float16, 1280, 1024, 6144, 128, 2),         # 80 tiles of 128 x 128 on 2 ranges
+    (np.float16, 768, 768, 8200, 128, 4),
+])
+def test_split_k_for_a_few_hundred_tiles(hip, oracle, dtype, M, N, K, tile, splits):
+    """Outputs of a few hundred small tiles and a long K: with a workspace the product runs on the tile shape that
+    splits best, on the planned number of ranges.  Parity on sampled rows, a column checksum over the whole output
+    against the product without a workspace, identical results from run to run, untouched padding."""
+    f16 = dtype == np.float16
+    A = synth.normal_half(M, K, 191) if f16 else synth.uniform_f32(M, K, 191)
+    B = synth.normal_half(K, N, 192) if f16 else synth.uniform_f32(K, N, 192)
+    esz = dtype().itemsize
+    plan = hip.plan(esz, M, N, K)
+    assert (plan.tile_m, plan.tile_n, plan.k_splits) == (tile, tile, splits)
+    need = hip.lib().decx_hip_gemm_workspace(esz, M, N, K)
+    assert need >= splits * M * N * 4
+    ws = hip.DeviceMatrix(1, need // 4, np.float32)
+    ws.upload_raw(np.full((1, ws.pitch), np.nan, np.float32))
+    pa, pn = device_pitch(K, dtype), device_pitch(N, dtype)
+    dA = hip.DeviceMatrix(M, K, dtype, pa, A, pad_value=np.nan); dB = hip.DeviceMatrix(K, N, dtype, pn, B, pad_value=np.nan)
+
+    def product(workspace):
+        dD = hip.DeviceMatrix(M, N, dtype, pn)
+        dD.upload_raw(np.full((M, pn), -12345.0, dtype))
+        hip.gemm(dA, dB, dD, workspace=workspace)
+        hip.sync()
+        raw = dD.download_raw()
+        dD.free()
+        assert np.all(raw[:, N:] == dtype(-12345.0))
+        return raw[:, :N].copy()
+
+    split = product(ws)
+    rows = sample_rows(M, 48, 9)
+    ref = (oracle.gemm_f16 if f16 else oracle.gemm_f32)(A, B, rows=rows)
+    assert rel_err(split[rows], ref, K) <= (TOL_F16 if f16 else TOL_F32)
+    assert np.array_equal(split.view(np.uint8), product(ws).view(np.uint8))
+    whole = product(None)
+    col_a = split.astype(np.float64).sum(axis=0); col_b = whole.astype(np.float64).sum(axis=0)
+    assert np.max(np.abs(col_a - col_b)) <= (2e-2 if f16 else 1e-4) * np.max(np.abs(col_b))
+    for d in (dA, dB, ws):
+        d.free()
+
+
 def test_f32_split_k_is_planned_only_where_it_pays(hip):
     L = hip.lib()
     assert L.decx_hip_gemm_f32_workspace(8192, 8192, 8192) == 0           # enough tiles
