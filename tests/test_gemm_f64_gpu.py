@@ -109,6 +109,40 @@ def test_split_k_through_a_workspace(hip, oracle, M, N, K):
     ws.free()
 
 
+def test_split_k_for_a_few_hundred_tiles(hip, oracle):
+    """320 tiles of 64 x 64 (1.25 per CU) and a long K: with a workspace the planner cuts K so that whole rounds of
+    workgroups result.  Parity on sampled rows, the same result from run to run, untouched padding."""
+    M, N, K = 1280, 1024, 4100
+    A = synth.uniform_f64(M, K, 961); B = synth.uniform_f64(K, N, 962)
+    plan = hip.plan(8, M, N, K)
+    assert plan.k_splits > 1 and plan.tile_m == 64
+    need = hip.lib().decx_hip_gemm_workspace(8, M, N, K)
+    assert need >= plan.k_splits * M * N * 8
+    ws = hip.DeviceMatrix(1, need // 8, np.float64)
+    ws.upload_raw(np.full((1, ws.pitch), np.nan, np.float64))
+    r16 = lambda v: (v + 15) // 16 * 16
+    dA = hip.DeviceMatrix(M, K, np.float64, r16(K), A, pad_value=np.nan); dB = hip.DeviceMatrix(K, N, np.float64, r16(N), B, pad_value=np.nan)
+
+    def product(workspace):
+        dD = hip.DeviceMatrix(M, N, np.float64, r16(N) + 16)
+        dD.upload_raw(np.full((M, r16(N) + 16), -12345.0))
+        hip.gemm(dA, dB, dD, workspace=workspace)
+        hip.sync()
+        raw = dD.download_raw()
+        dD.free()
+        assert np.all(raw[:, N:] == -12345.0)
+        return raw[:, :N].copy()
+
+    split = product(ws)
+    rows = np.array([0, 1, 63, 64, 640, 1000, 1279], np.uint32)
+    assert rel_err(split[rows], oracle.gemm_f64(A, B, rows=rows), K) <= TOL
+    assert np.array_equal(split, product(ws))
+    whole = product(None)
+    assert np.max(np.abs(split - whole)) <= 1e-12 * np.sqrt(K)
+    for d in (dA, dB, ws):
+        d.free()
+
+
 @pytest.mark.parametrize("M,N,K", [(4096, 1, 8192), (700, 1, 1030), (8200, 1, 33), (2100, 1, 4100), (33, 1, 257), (1, 1, 5),
                                    (1, 3000, 4096), (1, 100, 33000), (1, 9, 70), (1, 5000, 300), (1, 513, 16390)])
 def test_vector_corners(hip, oracle, M, N, K):
