@@ -86,6 +86,25 @@ def test_planner_choices():
     p = hip.plan(4, 300, 300, 8192)
     assert p.k_splits > 1 and p.grid == 25 * p.k_splits and hip.plan(4, 8192, 8192, 8192).k_splits == 1
     assert hip.plan(4, 300, 300, 512).k_splits == 1 and hip.plan(2, 256, 256, 65536).k_splits > 1
+    # a few hundred tiles that do not divide among 256 CUs and a long K: even rounds of workgroups on the small tile
+    p = hip.plan(4, 1280, 1024, 8192)                      # 320 tiles of 64 x 64 on 4 ranges: five per CU
+    assert (p.tile_m, p.k_splits, p.grid) == (64, 4, 320 * 4)
+    p = hip.plan(4, 1536, 1024, 8192)                      # 384 tiles on 2 ranges: three per CU
+    assert (p.tile_m, p.k_splits) == (64, 2)
+    assert hip.plan(4, 2048, 2048, 8192).k_splits == 1 and hip.plan(4, 1280, 1024, 2048).k_splits == 1
+    p = hip.plan(2, 1536, 1024, 8192)                      # fp16: 96 tiles of 128 x 128 on 2 ranges
+    assert (p.tile_m, p.k_splits) == (128, 2)
+    assert hip.plan(2, 1024, 1024, 6144).k_splits == 1     # 64 tiles on 2 ranges would leave half the chip idle
+    assert hip.plan(2, 768, 768, 16384).k_splits == 4 and hip.plan(2, 2048, 2048, 8192).k_splits == 1
+    p = hip.plan(8, 1280, 1024, 8192)
+    assert p.tile_m == 64 and p.k_splits > 1 and hip.plan(8, 4096, 4096, 4096).k_splits == 1
+    # the vector corners: rows per workgroup of the row-dot kernel, ranges of K for few columns, fp64 on the same kernels
+    assert [hip.plan(4, M, 1, 4096).tile_m for M in (9000, 5000, 3000, 1500, 600, 100)] == [32, 16, 8, 4, 2, 1]
+    p = hip.plan(4, 1, 512, 32768)
+    assert (p.path, p.tile_n) == (hip.PATH_GEVM, 32) and p.k_splits > 1 and p.grid == 16 * p.k_splits
+    assert hip.plan(4, 1, 512, 8192).k_splits == 1 and hip.plan(2, 1, 8192, 8192).k_splits == 1
+    assert hip.plan(8, 8192, 1, 8192).path == hip.PATH_GEMV and hip.plan(8, 1, 8192, 8192).path == hip.PATH_GEVM
+    assert hip.plan(8, 1, 8192, 8192).tile_n == 16
     bad = hip.Plan()
     assert hip.lib().decx_hip_gemm_plan(3, 4, 4, 4, 1, ctypes.byref(bad)) == -1
 
