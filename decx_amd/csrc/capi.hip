@@ -42,7 +42,7 @@ int choose_tile(bool f16, uint32_t M, uint32_t N, bool aligned)
     int best = TILE_64x64;
     double best_cost = 1e300;
     for (int s = TILE_COUNT - 1; s >= 0; --s) {
-        const TileInfo ti = f16 ? tile_info_f16(s, aligned) : tile_info_f32(s, aligned);
+        const TileInfo ti = f16 ? tile_info_f16(s, aligned) : tile_info_f32(s, aligned, N);
         const uint64_t tiles = (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
         const double cost = tile_cost(ti, tiles, g_dev.compute_units);
         if (cost <= best_cost) { best_cost = cost; best = s; }
@@ -69,7 +69,7 @@ SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
     const uint32_t cus = g_dev.compute_units;
     const int shape = elem_bytes == 8 ? choose_tile_f64(M, N) : choose_tile(elem_bytes == 2, M, N, true);
     const TileInfo ti = elem_bytes == 8 ? tile_info_f64(shape)
-                                        : elem_bytes == 2 ? tile_info_f16(shape, true) : tile_info_f32(shape, true);
+                                        : elem_bytes == 2 ? tile_info_f16(shape, true) : tile_info_f32(shape, true, N);
     // outputs of at most half as many tiles as there are CUs: up to two workgroups per CU
     const SplitPlan sp = plan_split_k((uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn), K, cus);
     if (sp.splits > 1) return {shape, sp.splits, sp.len};
@@ -82,7 +82,8 @@ SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
     if (elem_bytes == 4 && K >= 4096) {
         // 64 x 64 tiles, up to five workgroups per CU.  score = (workgroups on the busiest CU / the average) x what a
         // CU loses with m workgroups against a full one; the ranges p that make t * p an even three to five per CU win.
-        const uint64_t t = tiles_of(64);
+        const TileInfo small = tile_info_f32(TILE_64x64, true, N);
+        const uint64_t t = (uint64_t)((M + small.bm - 1) / small.bm) * ((N + small.bn - 1) / small.bn);
         const auto score = [&](uint32_t p) {
             const uint64_t wgs = t * p, m = (wgs + cus - 1) / cus;
             static const double loss[6] = {1.0, 1.35, 1.10, 1.03, 1.0, 1.0};
@@ -91,7 +92,7 @@ SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
         if (t <= 3ull * cus) {
             uint32_t best = 1;
             double best_score = score(1) / 1.15;                    // the second kernel must be worth it
-            for (uint32_t p2 = 2; p2 <= 8 && K / p2 >= 1024 && t * p2 <= 5ull * cus; ++p2)
+            for (uint32_t p2 = 2; p2 <= 8 && K / p2 >= 1024 && t * p2 <= (uint64_t)small.per_cu * cus; ++p2)
                 if (score(p2) < best_score) { best_score = score(p2); best = p2; }
             if (best > 1) {
                 const uint32_t len = ((K + best - 1) / best + 31) / 32 * 32;
@@ -698,7 +699,7 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
         return DECX_HIP_OK;
     }
     const int shape = choose_tile(f16, M, N, aligned != 0);
-    const TileInfo ti = f16 ? tile_info_f16(shape, aligned != 0) : tile_info_f32(shape, aligned != 0);
+    const TileInfo ti = f16 ? tile_info_f16(shape, aligned != 0) : tile_info_f32(shape, aligned != 0, N);
     out->path = shape;
     out->tile_m = ti.bm; out->tile_n = ti.bn;
     out->grid = ((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
@@ -707,7 +708,7 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
     if (!out->edge) {
         const SplitChoice sc = split_plan(elem_bytes, M, N, K);
         if (sc.splits > 1 && sc.shape != shape) {                   // the split runs on another tile than the whole product
-            const TileInfo ts = f16 ? tile_info_f16(sc.shape, true) : tile_info_f32(sc.shape, true);
+            const TileInfo ts = f16 ? tile_info_f16(sc.shape, true) : tile_info_f32(sc.shape, true, N);
             out->path = sc.shape; out->tile_m = ts.bm; out->tile_n = ts.bn;
             out->grid = ((M + ts.bm - 1) / ts.bm) * ((N + ts.bn - 1) / ts.bn);
         }

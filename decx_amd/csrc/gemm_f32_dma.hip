@@ -99,7 +99,13 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
     constexpr int CB = BN / 4, RB = 64 / CB;                      // B chunks per k row, k rows per direct load
     constexpr int A_STAGE_BYTES = BM * BK * 4, B_STAGE_BYTES = BK * BN * 4, STAGE_BYTES = A_STAGE_BYTES + B_STAGE_BYTES;
     constexpr int A_LOADS = A_STAGE_BYTES / 1024 / WAVES, B_LOADS = B_STAGE_BYTES / 1024 / WAVES, LOADS = A_LOADS + B_LOADS;
-    constexpr int B_SHIFT = (TN == 1) ? 8 : 0;                    // chunk shift of k rows with bit 2 set
+    // The two half-waves read k rows r and r + 4 of B at the same time.  In rows of 256 bytes or more those hit the
+    // same banks unless rows with bit 2 set are shifted by 8 chunks (only TN == 1 reads as little as 128 bytes per
+    // half-wave); 128-byte rows (BN == 32) have no room for that shift and are stored in the order 0 4 1 5 2 6 3 7
+    // instead, so that r and r + 4 lie side by side.
+    constexpr bool B_PAIRED_ROWS = BN == 32;
+    constexpr int B_SHIFT = (TN == 1 && !B_PAIRED_ROWS) ? 8 : 0;  // chunk shift of k rows with bit 2 set
+    static_assert(!B_PAIRED_ROWS || CHUNK_AHEAD, "paired rows are read by the small-tile loop only");
     static_assert(TM >= 1 && (TN == 1 || TN == 2 || TN == 4), "wave tile");
     static_assert(BK == 16 || BK == 32, "slab depth");     // an even number of 8-deep chunks: the fragments of a slab's last
                                                             // chunk and of the next slab's first one sit in different registers
@@ -128,7 +134,8 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
 
     // ---- copy plan.  A direct load I covers rows (64 / CPR) I ..: lane -> row I * 64 / CPR + lane / CPR,
     // slot lane % CPR, fetching chunk slot ^ ((row / RP) % CPR).  B direct load I covers k rows RB I ..:
-    // lane -> k row RB I + lane / CB, slot lane % CB, fetching column chunk slot ^ (B_SHIFT if k row & 4).
+    // lane -> row position RB I + lane / CB (= the k row, except for paired rows), slot lane % CB, fetching column
+    // chunk slot ^ (B_SHIFT if k row & 4).
     // Rows beyond M and column chunks beyond N are replaced by the last valid ones.
     // CONV: the A operand is gathered from an image: the K elements of an output pixel are runs of conv_seg_bytes
     // contiguous bytes (one kernel row), conv_seg_stride apart.  Mode 1: a_src[i] walks along the patch of the
@@ -159,7 +166,8 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
 #pragma unroll
     for (int i = 0; i < B_LOADS; ++i) {
         const int I = wave * B_LOADS + i;
-        b_krow[i] = I * RB + lane / CB;
+        const int pos = I * RB + lane / CB;                // row position inside the stage
+        b_krow[i] = B_PAIRED_ROWS ? (pos & ~7) + ((pos & 7) >> 1) + 4 * (pos & 1) : pos;
         const int chunk = (lane % CB) ^ ((b_krow[i] & 4) ? B_SHIFT : 0);
         const uint32_t gchunk = (n0 / 4 + chunk) < last_col_chunk ? (n0 / 4 + chunk) : last_col_chunk;
         b_voff[i] = (uint32_t)((size_t)b_krow[i] * ldb_b + (size_t)gchunk * 16);           // < BK * ldb_b + 4 N: the launcher checks
@@ -247,7 +255,8 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
 #pragma unroll
     for (int c = 0; c < BK / 8; ++c) a_off[c] = a_row * (BK * 4) + (((2 * c + h) ^ a_sw) * 16);
     const int b_col = wn0 + TN * l32;
-    const int b_off = A_STAGE_BYTES + (4 * h) * BN * 4 + (((b_col / 4) ^ (h ? B_SHIFT : 0)) * 16) + (b_col % 4) * 4;
+    const int b_off = A_STAGE_BYTES + (B_PAIRED_ROWS ? h : 4 * h) * BN * 4 + (((b_col / 4) ^ (h ? B_SHIFT : 0)) * 16) + (b_col % 4) * 4;
+    constexpr int B_ROW_STEP = (B_PAIRED_ROWS ? 2 : 1) * BN * 4;  // from k row r to r + 1 (r % 8 < 3) inside a stage
 
     floatx16 acc[TM][TN];
 #pragma unroll
@@ -359,7 +368,7 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
 #pragma unroll
             for (int i = 0; i < TM; ++i) fa[c & 1][i] = *(const floatx4*)(st + a_off[c] + i * 32 * BK * 4);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) fb[c & 1][e] = *(const bfrag*)(st + b_off + (8 * c + e) * BN * 4);
+            for (int e = 0; e < 4; ++e) fb[c & 1][e] = *(const bfrag*)(st + b_off + 8 * c * BN * 4 + e * B_ROW_STEP);
         };
         auto multiply_chunk = [&](auto cc) {
             constexpr int c = decltype(cc)::value;
@@ -514,7 +523,9 @@ int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
     switch (shape) {
     case TILE_256x256: return launch_dma<256, 128, 2, 2, 16, 2, false>(args, stream);
     case TILE_128x128: return launch_dma<128, 128, 2, 2, 16, 2, true>(args, stream);
-    case TILE_64x64:   return launch_dma< 64,  64, 2, 2, 32, 2, true>(args, stream);
+    case TILE_64x64:                                           // outputs of at most 32 columns: 128 x 32 tiles, no idle half
+        return args.N <= kNarrowN ? launch_dma<128, 32, 4, 1, 32, 2, true>(args, stream)
+                                  : launch_dma< 64, 64, 2, 2, 32, 2, true>(args, stream);
     default:           return (int)hipErrorInvalidValue;
     }
 }
@@ -546,8 +557,12 @@ int launch_conv2d_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
                                       : launch_dma<256, 256, 2, 4, 16, 4, false, 1>(args, stream);
     case TILE_128x128: return uniform ? launch_dma<128, 128, 2, 2, 16, 2, true, 2>(args, stream)
                                       : launch_dma<128, 128, 2, 2, 16, 2, true, 1>(args, stream);
-    case TILE_64x64:   return uniform ? launch_dma< 64,  64, 2, 2, 32, 2, true, 2>(args, stream)
-                                      : launch_dma< 64,  64, 2, 2, 32, 2, true, 1>(args, stream);
+    case TILE_64x64:
+        if (args.N <= kNarrowN)                                // at most 32 kernels, all the reference's own path takes
+            return uniform ? launch_dma<128, 32, 4, 1, 32, 2, true, 2>(args, stream)
+                           : launch_dma<128, 32, 4, 1, 32, 2, true, 1>(args, stream);
+        return uniform ? launch_dma< 64,  64, 2, 2, 32, 2, true, 2>(args, stream)
+                       : launch_dma< 64,  64, 2, 2, 32, 2, true, 1>(args, stream);
     default:           return (int)hipErrorInvalidValue;
     }
 }

@@ -49,7 +49,8 @@ typedef struct decx_hip_device_props {
 
 /* Tile shapes the planner chooses between (block tile BM x BN).  DECX_HIP_TILE_256x256 is the largest tile of
  * the element type: 256 x 256 in fp16, 256 x 128 in fp32 on 16-byte aligned operands (256 x 256 otherwise) and
- * in fp64; decx_hip_gemm_plan reports the actual BM x BN. */
+ * in fp64.  DECX_HIP_TILE_64x64 is the smallest: 64 x 64, or 128 x 32 for aligned fp32 outputs of at most 32
+ * columns (all the kernel counts the reference's convolution takes).  decx_hip_gemm_plan reports the actual BM x BN. */
 enum {
     DECX_HIP_TILE_AUTO    = -1,
     DECX_HIP_TILE_256x256 = 0,

@@ -196,6 +196,19 @@ def test_f32_every_k_remainder(hip, oracle, K, tile):
     assert rel_err(run(hip, A, B, C, -1.0, 0.5, tile=tile), oracle.gemm_f32(A, B, C, -1.0, 0.5), K) <= TOL_F32
 
 
+@pytest.mark.parametrize("M,N", [(70, 5), (300, 20), (1000, 32), (129, 31), (4100, 24)])
+@pytest.mark.parametrize("K", [1, 31, 32, 33, 64, 100, 777])
+def test_f32_outputs_of_at_most_32_columns(hip, oracle, M, N, K):
+    """At most 32 columns: the smallest tile class runs as 128 x 32 (B rows of 128 bytes, k rows r and r + 4 stored
+    side by side).  Planner's choice and the forced smallest class, every K remainder around the slab depth."""
+    A = synth.uniform_f32(M, K, 211); B = synth.uniform_f32(K, N, 212); C = synth.uniform_f32(M, N, 213)
+    plan = hip.plan(4, M, N, K)
+    assert (plan.tile_m, plan.tile_n) == (128, 32)
+    for tile in (-1, 2):
+        assert rel_err(run(hip, A, B, tile=tile), oracle.gemm_f32(A, B), K) <= TOL_F32
+        assert rel_err(run(hip, A, B, C, 1.5, -0.5, tile=tile), oracle.gemm_f32(A, B, C, 1.5, -0.5), K) <= TOL_F32
+
+
 def test_f32_large_ragged_sampled(hip, oracle):
     """A ragged problem large enough for several rounds of workgroups per CU, planner's choice of tile."""
     M, N, K = 3001, 2903, 3107
