@@ -23,7 +23,7 @@ HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibilit
              # packed-fp32 VALU forms are kept out of the generated code on purpose
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              "-Wno-unused-command-line-argument"]
-HIP_SOURCES = ["gemm_f32.hip", "gemm_f32_dma.hip", "gemm_f16.hip", "gemm_f16_dma.hip", "gemm_f64.hip", "gemm_complex.hip", "gemv.hip", "capi.hip"]
+HIP_SOURCES = ["gemm_f32.hip", "gemm_f32_dma.hip", "gemm_f16.hip", "gemm_f16_dma.hip", "gemm_f64.hip", "gemm_complex.hip", "gemv.hip", "conv_direct.hip", "capi.hip"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wextra",
               "-I" + os.path.join(ROOT, "include")]
 

@@ -654,6 +654,7 @@ int decx_hip_conv2d_f32(const float* image, const float* kmat, float* dst, uint3
     g.conv_seg_stride = (uint64_t)img_wpitch * img_dpitch * 4u;
     g.conv_py_bytes = (uint64_t)stride_y * img_wpitch * img_dpitch * 4u;
     g.conv_image_bytes = ((uint64_t)(out_h - 1) * stride_y + k_h) * img_wpitch * img_dpitch * 4u;
+    if (conv2d_direct_pays(g.N, g.K, img_dpitch)) return launch_conv2d_direct_f32(g, as_stream(stream));
     return launch_conv2d_f32_dma(choose_tile(false, g.M, g.N, true), g, as_stream(stream));
 }
 

@@ -1,0 +1,109 @@
+// Direct 2-D convolution for shallow patches and few kernels (fp32), gfx950.
+//
+// The implicit GEMM of gemm_f32_dma.hip pays a workgroup's prologue, two slab barriers and an epilogue per
+// 128 output pixels; with a patch of a few dozen values and at most 32 kernels (a 3 x 3 filter bank over an
+// RGB image: K = 36) that is nearly all it does.  Here a lane owns one output pixel: it walks the KH runs of
+// KW x channel-pitch contiguous floats of its patch with 128-bit loads (neighbouring lanes read neighbouring
+// pixels, so the loads coalesce) and multiplies every value into one accumulator per kernel.  The weights of
+// a patch element are the same for all lanes, so they come through scalar loads and cost no vector
+// instruction; the vector pipe does one fma per (pixel, patch element, kernel), which is the arithmetic itself.
+//
+// Same operands and layouts as the GEMM form (image [row][column][channel pitch], kernels packed
+// [patch element][kernel] with zero rows for padded channels, destination [row][column][channel pitch]), same
+// k-ascending fma chain per output as the CPU oracle.  Replaces, for these sizes, the same reference path:
+// cu_im2col_*_fp32 + cu_im2col_GEMM_fp32 (srcs/modules/NN/convolution/CUDA/fp32/im2col_fp32.cu,
+// im2col_GEMM_fp32.cu:40-106).
+#include "gemm_common.hpp"
+
+namespace decx_hip {
+
+namespace {
+
+// NACC: accumulators per pixel = kernels rounded up to a multiple of 4 (never beyond the pitch of the packed kernels).
+template <int NACC>
+__global__ void __launch_bounds__(256)
+conv2d_direct_kernel(const float* __restrict__ image, const float* __restrict__ kmat, float* __restrict__ dst,
+                     uint32_t out_w, uint32_t pixels, uint32_t out_c, uint32_t k_h, uint32_t seg_floats,
+                     uint64_t row_floats, uint32_t px_floats, uint64_t py_floats, uint32_t kmat_pitch,
+                     uint32_t dst_dpitch, uint32_t dst_wpitch)
+{
+    const uint32_t p = blockIdx.x * 256 + threadIdx.x;
+    const bool live = p < pixels;
+    const uint32_t q = live ? p : pixels - 1;              // idle lanes of the last workgroup repeat the last pixel
+    const uint32_t oy = q / out_w, ox = q % out_w;
+    const float* patch = image + (size_t)oy * py_floats + (size_t)ox * px_floats;
+    float acc[NACC];
+#pragma unroll
+    for (int o = 0; o < NACC; ++o) acc[o] = 0.f;
+
+    const float* w = kmat;                                 // row k of the packed kernels: the same for every lane
+    for (uint32_t kh = 0; kh < k_h; ++kh) {
+        const float* run = patch + (size_t)kh * row_floats;
+        for (uint32_t e = 0; e < seg_floats; e += 4) {
+            const floatx4 v = *(const floatx4*)(run + e);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const float* wr = w + (size_t)c * kmat_pitch;
+#pragma unroll
+                for (int o = 0; o < NACC; ++o) acc[o] = __builtin_fmaf(v[c], wr[o], acc[o]);
+            }
+            w += (size_t)4 * kmat_pitch;
+        }
+    }
+    if (!live) return;
+    float* out = dst + ((size_t)oy * dst_wpitch + ox) * dst_dpitch;
+#pragma unroll
+    for (int o = 0; o < NACC; o += 4) {
+        if ((uint32_t)o + 4 <= out_c) {
+            *(floatx4*)(out + o) = floatx4{acc[o], acc[o + 1], acc[o + 2], acc[o + 3]};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if ((uint32_t)(o + e) < out_c) out[o + e] = acc[o + e];      // padding channels stay untouched
+        }
+    }
+}
+
+template <int NACC>
+int launch_direct(const GemmArgs& g, uint32_t k_h, hipStream_t stream)
+{
+    const uint32_t pixels = g.M;
+    hipLaunchKernelGGL((conv2d_direct_kernel<NACC>), dim3((pixels + 255) / 256), dim3(256), 0, stream,
+                       (const float*)g.A, (const float*)g.B, (float*)g.D, g.conv_wout, pixels, g.N, k_h,
+                       g.conv_seg_bytes / 4u, g.conv_seg_stride / 4u, g.conv_px_bytes / 4u, g.conv_py_bytes / 4u, g.ldb, g.ldd,
+                       g.conv_dst_row / g.ldd);
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
+// One fma per (pixel, patch element, kernel) on the vector pipe against the implicit GEMM's fixed cost per 128
+// pixels.  Measured on MI355X, picoseconds per output pixel: direct about 8 + 0.037 x patch elements x accumulators
+// (640 x 480 x 3 image, 16 kernels of 3 x 3: 43, against 91 for the GEMM form; 1920 x 1080 x 3, 4 kernels: 10 against 73),
+// the GEMM form about 70 + 0.55 x patch elements for any number of kernels up to 32.  The direct form also wants a
+// short channel pitch: a lane reads 16 bytes per load, channel pitch x 4 bytes away from its neighbour's.
+bool conv2d_direct_pays(uint32_t out_c, uint64_t patch_floats, uint32_t channel_pitch)
+{
+    if (out_c > 32 || channel_pitch > 8) return false;
+    const double k = (double)patch_floats, nacc = (double)((out_c + 3) / 4 * 4);
+    return 8.0 + 0.037 * k * nacc < 0.9 * (70.0 + 0.55 * k);
+}
+
+// g: the arguments of the GEMM form (M = pixels, N = kernels, conv_* set, ldb = pitch of the packed kernels).
+int launch_conv2d_direct_f32(const GemmArgs& g, hipStream_t stream)
+{
+    const uint32_t k_h = g.K / (g.conv_seg_bytes / 4u);
+    switch ((g.N + 3) / 4) {
+    case 1: return launch_direct<4>(g, k_h, stream);
+    case 2: return launch_direct<8>(g, k_h, stream);
+    case 3: return launch_direct<12>(g, k_h, stream);
+    case 4: return launch_direct<16>(g, k_h, stream);
+    case 5: return launch_direct<20>(g, k_h, stream);
+    case 6: return launch_direct<24>(g, k_h, stream);
+    case 7: return launch_direct<28>(g, k_h, stream);
+    case 8: return launch_direct<32>(g, k_h, stream);
+    default: return (int)hipErrorInvalidValue;
+    }
+}
+
+}  // namespace decx_hip

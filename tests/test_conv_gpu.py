@@ -32,6 +32,8 @@ CASES = [  # W, H, C, OC, KW, KH, sx, sy
     (31, 29, 1, 1, 7, 7, 3, 2), (8, 8, 16, 33, 1, 1, 1, 1), (10, 11, 2, 4, 3, 3, 2, 2),
     (64, 48, 16, 64, 3, 3, 1, 1), (57, 43, 13, 70, 3, 3, 1, 1), (130, 70, 32, 96, 5, 5, 2, 2), (40, 40, 64, 300, 3, 3, 1, 1),
     (33, 9, 24, 16, 11, 1, 1, 1), (12, 40, 12, 16, 1, 9, 1, 3),
+    # shallow patches, few kernels, a short channel pitch: the lane-per-pixel kernel (several workgroups, a partial last one)
+    (640, 480, 3, 16, 3, 3, 1, 1), (200, 150, 4, 32, 5, 5, 2, 1), (333, 77, 7, 5, 2, 3, 1, 2), (1030, 9, 1, 29, 3, 3, 1, 1),
 ]
 
 
