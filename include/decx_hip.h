@@ -234,7 +234,9 @@ DECX_HIP_API int decx_hip_gevm_f16_ws(const uint16_t* x, const uint16_t* B, cons
  * kernel element (0, 0) of output pixel (0, 0): for zero-extended borders pass a zero-padded copy.
  * The kernel set comes packed as kmat[(kh * k_w + kw) * img_dpitch + ic][oc] (row pitch kmat_pitch,
  * zero rows for ic >= depth); decx_hip_conv2d_pack_kernels_f32 builds it from out_c kernels stored
- * like images, tensor_stride floats apart. */
+ * like images, tensor_stride floats apart.  Shallow patches with at most 32 kernels and a channel pitch of
+ * 4 or 8 (a 3 x 3 filter bank over an RGB image) run a lane per output pixel on the vector pipe instead of the
+ * matrix cores; same operands, same result. */
 DECX_HIP_API int decx_hip_conv2d_pack_kernels_f32(const float* kernels, float* kmat, uint32_t k_w, uint32_t k_h,
                                                   uint32_t depth, uint32_t k_dpitch, uint32_t k_wpitch,
                                                   uint64_t tensor_stride, uint32_t out_c, uint32_t kmat_pitch,
