@@ -46,6 +46,7 @@ WORKLOADS = {
     "fp32_1024": ("f32", 1024, 1024, 1024, "mfma", 1, "fp32 GEMM M=N=K=1024, uniform[-1,1]"),
     "fp32_ragged": ("f32", 1000, 1500, 777, "mfma", 2, "fp32 GEMM M=1000 N=1500 K=777, uniform[-1,1]"),
     "fp32_tall_skinny": ("f32", 65536, 256, 1024, "mfma", 5, "fp32 GEMM M=65536 N=256 K=1024, uniform[-1,1]"),
+    "fp32_mid_long_k": ("f32", 1280, 1024, 8192, "mfma", 8, "fp32 GEMM M=1280 N=1024 K=8192 (320 small tiles, split along K through the workspace), uniform[-1,1]"),
     "fp32_gemv": ("f32", 8192, 1, 8192, "hbm", 6, "fp32 GEMM M=8192 N=1 K=8192 (GEMV-like), uniform[-1,1]"),
     "fp32_gevm": ("f32", 1, 8192, 8192, "hbm", 6, "fp32 GEMM M=1 N=8192 K=8192 (vector x matrix), uniform[-1,1]"),
     "fp16_gemv": ("f16", 8192, 1, 8192, "hbm", 6, "fp16 GEMM M=8192 N=1 K=8192 (fp32 accumulate), normal(0,0.5)"),
@@ -125,13 +126,15 @@ def run_workload(name, steps, warmup, keep_inputs=False, settle_s=0.0):
 
 
 CONV = {"W": 256, "H": 256, "C": 112, "OC": 256, "KW": 3, "KH": 3}     # 64 516 pixels x 256 channels x 1008 taps
+CONV_RGB = {"W": 1920, "H": 1080, "C": 3, "OC": 8, "KW": 3, "KH": 3}    # a filter bank over an RGB frame: 36 taps, bound by HBM
 
 
-def run_conv(steps, warmup, settle_s=0.25):
+def run_conv(steps, warmup, settle_s=0.25, c=None):
     """fp32 3 x 3 convolution of a 256 x 256 x 112 image with 256 kernels through decx_hip_conv2d_f32 (implicit GEMM,
-    operands resident): the workload the tall-skinny GEMM shape 65536 x 256 x 1024 stands for."""
+    operands resident): the workload the tall-skinny GEMM shape 65536 x 256 x 1024 stands for.  c: another
+    configuration (CONV_RGB: a shallow patch and few kernels, which the library runs a lane per output pixel)."""
     from decx_amd import hip, synth
-    c = CONV
+    c = c or CONV
     L = hip.lib()
     dp, wp = (c["C"] + 3) // 4 * 4, (c["W"] + 7) // 8 * 8
     img = np.zeros((c["H"], wp, dp), np.float32)
@@ -161,12 +164,18 @@ def run_conv(steps, warmup, settle_s=0.25):
     flops = 2.0 * ow * oh * c["OC"] * c["KH"] * c["KW"] * c["C"]
     abytes = 4.0 * (c["H"] * c["W"] * c["C"] + c["KH"] * c["KW"] * c["C"] * c["OC"] + ow * oh * c["OC"])
     tf = flops / (ms * 1e-3) / 1e12
-    out = {"workload": "fp32 conv2D 3x3, image 256x256x112, 256 kernels (implicit GEMM 64516 x 256 x 1008), uniform[-1,1]",
-           "dtype": "f32", "value": round(tf, 3), "unit": "TFLOP/s", "hbm_gbs_algorithmic": round(abytes / (ms * 1e-3) / 1e9, 1),
-           "kernel_ms": round(ms, 5),
-           "roofline": {"bound": "mfma", "achieved": round(tf, 3), "peak": PEAK_F32_TFLOPS, "unit": "TFLOP/s",
-                        "frac": round(tf / PEAK_F32_TFLOPS, 4),
-                        "traffic": 1.80e8}}      # FETCH_SIZE 55 474 x 2.0 KiB + WRITE_SIZE 64 516 KiB
+    gbs = abytes / (ms * 1e-3) / 1e9
+    desc = "fp32 conv2D %dx%d, image %dx%dx%d, %d kernels (%d x %d x %d as a GEMM), uniform[-1,1]" % (
+        c["KW"], c["KH"], c["W"], c["H"], c["C"], c["OC"], ow * oh, c["OC"], K)
+    if c is CONV:
+        roof = {"bound": "mfma", "achieved": round(tf, 3), "peak": PEAK_F32_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(tf / PEAK_F32_TFLOPS, 4),
+                "traffic": 1.80e8}               # FETCH_SIZE 55 474 x 2.0 KiB + WRITE_SIZE 64 516 KiB
+    else:                                        # 16 flop per byte: the memory system bounds it
+        roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}
+    out = {"workload": desc, "dtype": "f32", "value": round(tf, 3), "unit": "TFLOP/s", "hbm_gbs_algorithmic": round(gbs, 1),
+           "kernel_ms": round(ms, 5), "roofline": roof}
     for d in (d_img, d_kmat, d_out):
         d.free()
     return out
@@ -265,7 +274,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="fp32_8192", choices=sorted(WORKLOADS) + ["copy_1GiB", "conv2d", "c64_4096", "c128_2048"])
+    ap.add_argument("--workload", default="fp32_8192", choices=sorted(WORKLOADS) + ["copy_1GiB", "conv2d", "conv2d_rgb", "c64_4096", "c128_2048"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     args = ap.parse_args()
@@ -294,8 +303,8 @@ def main():
         print(json.dumps({"workload": "calibration copy 1 GiB", "kernel_ms": ms, "GB/s_read_plus_write": 2 * n / ms / 1e6}))
         return
 
-    if args.workload == "conv2d":
-        print(json.dumps(run_conv(args.steps, args.warmup)))
+    if args.workload in ("conv2d", "conv2d_rgb"):
+        print(json.dumps(run_conv(args.steps, args.warmup, c=CONV if args.workload == "conv2d" else CONV_RGB)))
         return
     if args.workload in ("c64_4096", "c128_2048"):
         print(json.dumps(run_complex(args.workload == "c128_2048", 4096 if args.workload == "c64_4096" else 2048, args.steps, args.warmup)))
@@ -325,6 +334,7 @@ def main():
                 small = WORKLOADS[name][1] * WORKLOADS[name][2] * WORKLOADS[name][3] < 2 ** 38
                 others.append(run_workload(name, 200 if small else args.steps, args.warmup, settle_s=0.25)[0])
         others.append(run_conv(200, args.warmup))
+        others.append(run_conv(200, args.warmup, c=CONV_RGB))
         others.append(run_complex(False, 4096, args.steps, args.warmup))
         others.append(run_complex(True, 2048, 50, args.warmup))
         line["other_workloads"] = others
