@@ -261,7 +261,7 @@ def test_row_pitch_of_16_mib_takes_the_register_staged_kernels(hip, oracle, dtyp
         assert rel_err(run(hip, A, B, tile=tile, pitches=(pitch_a, pn, pn, pn)), ref, K) <= tol
 
 
-@pytest.mark.parametrize("M,N,K", [(300, 300, 8192), (64, 64, 4099), (130, 70, 2500), (512, 512, 1024), (33, 1000, 3000)])
+@pytest.mark.parametrize("M,N,K", [(300, 300, 8192), (64, 64, 4099), (130, 70, 2500), (512, 512, 1024), (33, 1000, 3000), (4100, 20, 4099)])
 def test_f32_split_k_through_a_workspace(hip, oracle, M, N, K):
     """Few output tiles and a long K: with a workspace the product is split along K and the partial products are added
     in a fixed order.  Parity with the oracle, identical results from run to run, C / alpha / beta, untouched padding,
