@@ -129,6 +129,21 @@ def test_compute_entry_points_refuse_to_run_uninitialised():
     subprocess.run([sys.executable, "-c", code], check=True, timeout=120)
 
 
+def test_missing_library_is_an_error_not_a_fallback():
+    """Without the built HIP library the Python layer raises; there is no CPU path behind it."""
+    import subprocess
+    import sys
+    code = ("from decx_amd import hip\n"
+            "hip.LIB_PATH = '/nonexistent/libdecx_hip.so'\n"
+            "try:\n"
+            "    hip.lib()\n"
+            "except hip.HipError as e:\n"
+            "    assert 'native library missing' in str(e); print('raised')\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=root, timeout=120)
+    assert out.returncode == 0 and out.stdout.strip() == "raised", out.stderr
+
+
 def test_error_strings():
     L = hip.lib()
     assert L.decx_hip_error_string(0) == b"success"
