@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by a
 # copy kernel of known size; None until measured for that workload.
 MEASURED_TRAFFIC = {
-    "fp32_8192": 7.71e9,     # FETCH_SIZE 3.6317e6 x 2.0 KiB + WRITE_SIZE 2.621e5 KiB (5.45e9 in another run)
+    "fp32_8192": 5.71e9,     # FETCH_SIZE 2.6574e6 x 2.0 KiB + WRITE_SIZE 2.621e5 KiB
     "fp16_4096": 2.35e8,     # FETCH_SIZE 98 461 x 2.0 KiB + WRITE_SIZE 32 793 KiB
     "fp32_gemv": 2.70e8,     # FETCH_SIZE (131 228 + 522) x 2.0 KiB + WRITE_SIZE (256 + 32) KiB: matrix-vector kernel + the copy of x
     "fp32_gevm": 2.69e8,     # FETCH_SIZE 131 224 x 2.0 KiB + WRITE_SIZE 32 KiB

@@ -33,6 +33,7 @@ struct GemmArgs {
     // min(K, (z + 1) * split_len)) and writes its M x N partial product (fp32 for fp32 and fp16 operands, fp64
     // for fp64), pitch split_ldd, to split_ws + z * split_stride elements; a second kernel adds the partial
     // products in split order.
+    uint32_t group_m;            // tile-rows per L2 patch of the block -> tile map (0: the default, kGroupM)
     uint32_t split_len;          // 0: no split
     uint32_t split_ldd;
     uint64_t split_stride;
@@ -63,10 +64,11 @@ __device__ __forceinline__ void block_to_tile(const GemmArgs& g, uint32_t& tile_
     const uint32_t nb = g.tiles_m * g.tiles_n;
     uint32_t id = blockIdx.x;
     if (g.xcd_remap) id = (id % kXcds) * (nb / kXcds) + id / kXcds;
-    const uint32_t per_group = kGroupM * g.tiles_n;
+    const uint32_t group_m = g.group_m ? g.group_m : (uint32_t)kGroupM;
+    const uint32_t per_group = group_m * g.tiles_n;
     const uint32_t group = id / per_group;
-    const uint32_t first_m = group * kGroupM;
-    const uint32_t rows = (g.tiles_m - first_m) < (uint32_t)kGroupM ? (g.tiles_m - first_m) : (uint32_t)kGroupM;
+    const uint32_t first_m = group * group_m;
+    const uint32_t rows = (g.tiles_m - first_m) < group_m ? (g.tiles_m - first_m) : group_m;
     const uint32_t in_group = id % per_group;
     tile_m = first_m + in_group % rows;
     tile_n = in_group / rows;
