@@ -130,7 +130,7 @@ CONV_RGB = {"W": 1920, "H": 1080, "C": 3, "OC": 8, "KW": 3, "KH": 3}    # a filt
 
 
 def run_conv(steps, warmup, settle_s=0.25, c=None):
-    """fp32 3 x 3 convolution of a 256 x 256 x 112 image with 256 kernels through decx_hip_conv2d_f32 (implicit GEMM,
+    """fp32 3 x 3 convolution of a 256 x 256 x 112 image with 256 kernels through decx_hip_conv2d_f32_depth (implicit GEMM,
     operands resident): the workload the tall-skinny GEMM shape 65536 x 256 x 1024 stands for.  c: another
     configuration (CONV_RGB: a shallow patch and few kernels, which the library runs a lane per output pixel)."""
     from decx_amd import hip, synth
@@ -147,7 +147,7 @@ def run_conv(steps, warmup, settle_s=0.25, c=None):
     ow, oh = c["W"] - c["KW"] + 1, c["H"] - c["KH"] + 1
     owp = (ow + 7) // 8 * 8
     d_out = hip.DeviceMatrix(oh, owp * c["OC"], np.float32)
-    call = lambda: hip.check(L.decx_hip_conv2d_f32(d_img.ptr, d_kmat.ptr, d_out.ptr, ow, oh, c["OC"], c["KW"], c["KH"], dp, wp,
+    call = lambda: hip.check(L.decx_hip_conv2d_f32_depth(d_img.ptr, d_kmat.ptr, d_out.ptr, ow, oh, c["OC"], c["KW"], c["KH"], c["C"], dp, wp,
                                                    1, 1, c["OC"], c["OC"], owp, None))
     for _ in range(warmup):
         call()

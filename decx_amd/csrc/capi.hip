@@ -632,9 +632,19 @@ int decx_hip_conv2d_f32(const float* image, const float* kmat, float* dst, uint3
                         uint32_t k_w, uint32_t k_h, uint32_t img_dpitch, uint32_t img_wpitch, uint32_t stride_x,
                         uint32_t stride_y, uint32_t kmat_pitch, uint32_t dst_dpitch, uint32_t dst_wpitch, void* stream)
 {
+    return decx_hip_conv2d_f32_depth(image, kmat, dst, out_w, out_h, out_c, k_w, k_h, img_dpitch, img_dpitch, img_wpitch, stride_x,
+                                     stride_y, kmat_pitch, dst_dpitch, dst_wpitch, stream);
+}
+
+int decx_hip_conv2d_f32_depth(const float* image, const float* kmat, float* dst, uint32_t out_w, uint32_t out_h, uint32_t out_c,
+                              uint32_t k_w, uint32_t k_h, uint32_t depth, uint32_t img_dpitch, uint32_t img_wpitch,
+                              uint32_t stride_x, uint32_t stride_y, uint32_t kmat_pitch, uint32_t dst_dpitch, uint32_t dst_wpitch,
+                              void* stream)
+{
     if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
     if (!out_w || !out_h || !out_c) return DECX_HIP_OK;
     if (!image || !kmat || !dst || !k_w || !k_h || !stride_x || !stride_y || !img_dpitch || img_dpitch % 4 || kmat_pitch % 4 ||
+        !depth || depth > img_dpitch ||
         dst_dpitch % 4 || kmat_pitch < out_c || dst_dpitch < out_c || dst_wpitch < out_w ||
         img_wpitch < (uint64_t)(out_w - 1) * stride_x + k_w || !aligned16(image) || !aligned16(kmat) || !aligned16(dst) ||
         (uint64_t)out_w * out_h > 0xffffffffull || (uint64_t)k_w * img_dpitch * 4 > 0xffffffffull ||
@@ -654,7 +664,7 @@ int decx_hip_conv2d_f32(const float* image, const float* kmat, float* dst, uint3
     g.conv_seg_stride = (uint64_t)img_wpitch * img_dpitch * 4u;
     g.conv_py_bytes = (uint64_t)stride_y * img_wpitch * img_dpitch * 4u;
     g.conv_image_bytes = ((uint64_t)(out_h - 1) * stride_y + k_h) * img_wpitch * img_dpitch * 4u;
-    if (conv2d_direct_pays(g.N, g.K, img_dpitch)) return launch_conv2d_direct_f32(g, as_stream(stream));
+    if (conv2d_direct_pays(g.N, g.K, img_dpitch, depth)) return launch_conv2d_direct_f32(g, img_dpitch, depth, as_stream(stream));
     return launch_conv2d_f32_dma(choose_tile(false, g.M, g.N, true), g, as_stream(stream));
 }
 

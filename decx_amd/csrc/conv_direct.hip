@@ -20,7 +20,9 @@ namespace decx_hip {
 namespace {
 
 // NACC: accumulators per pixel = kernels rounded up to a multiple of 4 (never beyond the pitch of the packed kernels).
-template <int NACC>
+// REAL: channels of a 16-byte group that exist; below 4 only for a channel pitch of 4 with 1 to 3 channels (grey, RGB),
+// whose padding channel meets zero weights and is left out of the arithmetic.
+template <int NACC, int REAL>
 __global__ void __launch_bounds__(256)
 conv2d_direct_kernel(const float* __restrict__ image, const float* __restrict__ kmat, float* __restrict__ dst,
                      uint32_t out_w, uint32_t pixels, uint32_t out_c, uint32_t k_h, uint32_t seg_floats,
@@ -42,7 +44,7 @@ conv2d_direct_kernel(const float* __restrict__ image, const float* __restrict__ 
         for (uint32_t e = 0; e < seg_floats; e += 4) {
             const floatx4 v = *(const floatx4*)(run + e);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
+            for (int c = 0; c < REAL; ++c) {
                 const float* wr = w + (size_t)c * kmat_pitch;
 #pragma unroll
                 for (int o = 0; o < NACC; ++o) acc[o] = __builtin_fmaf(v[c], wr[o], acc[o]);
@@ -64,15 +66,26 @@ conv2d_direct_kernel(const float* __restrict__ image, const float* __restrict__ 
     }
 }
 
-template <int NACC>
+template <int NACC, int REAL>
 int launch_direct(const GemmArgs& g, uint32_t k_h, hipStream_t stream)
 {
     const uint32_t pixels = g.M;
-    hipLaunchKernelGGL((conv2d_direct_kernel<NACC>), dim3((pixels + 255) / 256), dim3(256), 0, stream,
+    hipLaunchKernelGGL((conv2d_direct_kernel<NACC, REAL>), dim3((pixels + 255) / 256), dim3(256), 0, stream,
                        (const float*)g.A, (const float*)g.B, (float*)g.D, g.conv_wout, pixels, g.N, k_h,
                        g.conv_seg_bytes / 4u, g.conv_seg_stride / 4u, g.conv_px_bytes / 4u, g.conv_py_bytes / 4u, g.ldb, g.ldd,
                        g.conv_dst_row / g.ldd);
     return (int)hipGetLastError();
+}
+
+template <int NACC>
+int launch_direct_real(const GemmArgs& g, uint32_t k_h, uint32_t real, hipStream_t stream)
+{
+    switch (real) {
+    case 1:  return launch_direct<NACC, 1>(g, k_h, stream);
+    case 2:  return launch_direct<NACC, 2>(g, k_h, stream);
+    case 3:  return launch_direct<NACC, 3>(g, k_h, stream);
+    default: return launch_direct<NACC, 4>(g, k_h, stream);
+    }
 }
 
 }  // namespace
@@ -82,26 +95,29 @@ int launch_direct(const GemmArgs& g, uint32_t k_h, hipStream_t stream)
 // (640 x 480 x 3 image, 16 kernels of 3 x 3: 43, against 91 for the GEMM form; 1920 x 1080 x 3, 4 kernels: 10 against 73),
 // the GEMM form about 70 + 0.55 x patch elements for any number of kernels up to 32.  The direct form also wants a
 // short channel pitch: a lane reads 16 bytes per load, channel pitch x 4 bytes away from its neighbour's.
-bool conv2d_direct_pays(uint32_t out_c, uint64_t patch_floats, uint32_t channel_pitch)
+bool conv2d_direct_pays(uint32_t out_c, uint64_t patch_floats, uint32_t channel_pitch, uint32_t depth)
 {
     if (out_c > 32 || channel_pitch > 8) return false;
+    const double real = channel_pitch == 4 && depth < 4 ? depth / 4.0 : 1.0;      // share of the patch that is multiplied
     const double k = (double)patch_floats, nacc = (double)((out_c + 3) / 4 * 4);
-    return 8.0 + 0.037 * k * nacc < 0.9 * (70.0 + 0.55 * k);
+    return 8.0 + 0.037 * k * real * nacc < 0.9 * (70.0 + 0.55 * k);
 }
 
-// g: the arguments of the GEMM form (M = pixels, N = kernels, conv_* set, ldb = pitch of the packed kernels).
-int launch_conv2d_direct_f32(const GemmArgs& g, hipStream_t stream)
+// g: the arguments of the GEMM form (M = pixels, N = kernels, conv_* set, ldb = pitch of the packed kernels);
+// depth: channels that exist (<= the channel pitch).
+int launch_conv2d_direct_f32(const GemmArgs& g, uint32_t channel_pitch, uint32_t depth, hipStream_t stream)
 {
     const uint32_t k_h = g.K / (g.conv_seg_bytes / 4u);
+    const uint32_t real = channel_pitch == 4 && depth >= 1 && depth < 4 ? depth : 4;
     switch ((g.N + 3) / 4) {
-    case 1: return launch_direct<4>(g, k_h, stream);
-    case 2: return launch_direct<8>(g, k_h, stream);
-    case 3: return launch_direct<12>(g, k_h, stream);
-    case 4: return launch_direct<16>(g, k_h, stream);
-    case 5: return launch_direct<20>(g, k_h, stream);
-    case 6: return launch_direct<24>(g, k_h, stream);
-    case 7: return launch_direct<28>(g, k_h, stream);
-    case 8: return launch_direct<32>(g, k_h, stream);
+    case 1: return launch_direct_real<4>(g, k_h, real, stream);
+    case 2: return launch_direct_real<8>(g, k_h, real, stream);
+    case 3: return launch_direct_real<12>(g, k_h, real, stream);
+    case 4: return launch_direct_real<16>(g, k_h, real, stream);
+    case 5: return launch_direct_real<20>(g, k_h, real, stream);
+    case 6: return launch_direct_real<24>(g, k_h, real, stream);
+    case 7: return launch_direct_real<28>(g, k_h, real, stream);
+    case 8: return launch_direct_real<32>(g, k_h, real, stream);
     default: return (int)hipErrorInvalidValue;
     }
 }

@@ -182,8 +182,8 @@ __host__ inline SplitPlan plan_split_k(uint64_t tiles, uint32_t K, uint32_t cus)
 // the same kernels with the A operand gathered from an image (GemmArgs::conv_*): 2-D convolution without an im2col buffer
 int launch_conv2d_f32_dma(int shape, const GemmArgs& args, hipStream_t stream);
 // shallow patches and at most 32 kernels: a lane per output pixel on the vector pipe (conv_direct.hip)
-bool conv2d_direct_pays(uint32_t out_c, uint64_t patch_floats, uint32_t channel_pitch);
-int launch_conv2d_direct_f32(const GemmArgs& args, hipStream_t stream);
+bool conv2d_direct_pays(uint32_t out_c, uint64_t patch_floats, uint32_t channel_pitch, uint32_t depth);
+int launch_conv2d_direct_f32(const GemmArgs& args, uint32_t channel_pitch, uint32_t depth, hipStream_t stream);
 int launch_gemm_f16(int shape, bool edge, const GemmArgs& args, hipStream_t stream);
 // direct-to-LDS fp16 kernel for any M, N, K >= 1 on 16-byte aligned bases and pitches, in the three tile shapes
 int launch_gemm_f16_dma(int shape, const GemmArgs& args, hipStream_t stream);

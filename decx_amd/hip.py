@@ -65,6 +65,7 @@ SYMBOLS = {
     "decx_hip_gevm_f16_ws": (_int, [_vp] * 4 + [_u32] * 6 + [_f, _f, _int, _vp, _sz, _vp]),
     "decx_hip_conv2d_pack_kernels_f32": (_int, [_vp, _vp] + [_u32] * 5 + [ctypes.c_uint64] + [_u32] * 3 + [_vp]),
     "decx_hip_conv2d_f32": (_int, [_vp] * 3 + [_u32] * 12 + [_vp]),
+    "decx_hip_conv2d_f32_depth": (_int, [_vp] * 3 + [_u32] * 13 + [_vp]),
     "decx_hip_gemm_f64": (_int, [_vp] * 4 + [_u32] * 7 + [ctypes.c_double, ctypes.c_double, _vp]),
     "decx_hip_gemm_f64_tile": (_int, [_vp] * 4 + [_u32] * 7 + [ctypes.c_double, ctypes.c_double, _vp, _int, _int]),
     "decx_hip_gemm_complex_workspace": (ctypes.c_size_t, [_int, _u32, _u32]),
@@ -273,7 +274,7 @@ def _align(v, a):
 
 
 def conv2d(image, kernels, stride_x=1, stride_y=1, extend=False, stream=None, pad_value=np.nan):
-    """dst[oy][ox][oc] = sum image[oy*sy+kh][ox*sx+kw][ic] * kernels[oc][kh][kw][ic] through decx_hip_conv2d_f32.
+    """dst[oy][ox][oc] = sum image[oy*sy+kh][ox*sx+kw][ic] * kernels[oc][kh][kw][ic] through decx_hip_conv2d_f32_depth.
     image [H][W][C], kernels [OC][KH][KW][C] (numpy fp32).  Device layouts follow the original's device tensors:
     channel pitch = C rounded up to 4, row pitch = W rounded up to 8 columns; unused columns hold `pad_value`,
     unused channels zero.  extend: zero-extended borders, output W/sx x H/sy."""
@@ -308,8 +309,8 @@ def conv2d(image, kernels, stride_x=1, stride_y=1, extend=False, stream=None, pa
     odp, owp = _align(OC, 4), _align(max(ow, 1), 8)
     d_out = DeviceMatrix(max(oh, 1), owp * odp, np.float32)
     d_out.upload_raw(np.full((max(oh, 1), owp * odp), -555.0, np.float32))
-    check(L.decx_hip_conv2d_f32(d_img.ptr, d_kmat.ptr, d_out.ptr, ow, oh, OC, KW, KH, dp, wp, stride_x, stride_y, kp, odp, owp,
-                                stream), "conv2d")
+    check(L.decx_hip_conv2d_f32_depth(d_img.ptr, d_kmat.ptr, d_out.ptr, ow, oh, OC, KW, KH, C, dp, wp, stride_x, stride_y, kp, odp,
+                                      owp, stream), "conv2d")
     check(L.decx_hip_stream_sync(stream))
     out_raw = d_out.download_raw().reshape(max(oh, 1), owp, odp)
     for d in (d_img, d_ker, d_kmat, d_out):

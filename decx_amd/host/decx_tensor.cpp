@@ -363,8 +363,8 @@ _DECX_API_ de::DH de::nn::cuda::Conv2D(de::GPU_Tensor& src, de::GPU_TensorArray&
         image = (const float*)scratch.padded->ptr;
     }
     if (rc == DECX_HIP_OK)
-        rc = decx_hip_conv2d_f32(image, (const float*)scratch.kmat->ptr, (float*)d->data(), OW, OH, OC, KW, KH, SL.dpitch,
-                                 img_wpitch, sx, sy, kmat_pitch, DL.dpitch, DL.wpitch, S);
+        rc = decx_hip_conv2d_f32_depth(image, (const float*)scratch.kmat->ptr, (float*)d->data(), OW, OH, OC, KW, KH, SL.depth,
+                                       SL.dpitch, img_wpitch, sx, sy, kmat_pitch, DL.dpitch, DL.wpitch, S);
     const int rs = decx_hip_stream_sync(S);
     decx::err::from_hip(&handle, rc != DECX_HIP_OK ? rc : rs, "Conv2D");
     return handle;

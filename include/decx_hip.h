@@ -245,6 +245,14 @@ DECX_HIP_API int decx_hip_conv2d_f32(const float* image, const float* kmat, floa
                                      uint32_t out_w, uint32_t out_h, uint32_t out_c, uint32_t k_w, uint32_t k_h,
                                      uint32_t img_dpitch, uint32_t img_wpitch, uint32_t stride_x, uint32_t stride_y,
                                      uint32_t kmat_pitch, uint32_t dst_dpitch, uint32_t dst_wpitch, void* stream);
+/* The same with the number of channels that exist (1 <= depth <= img_dpitch; the rest of the pitch is padding that
+ * meets zero rows of kmat): the lane-per-pixel kernel then leaves the padding channel of grey and RGB images
+ * (channel pitch 4) out of its arithmetic.  decx_hip_conv2d_f32 is this call with depth = img_dpitch. */
+DECX_HIP_API int decx_hip_conv2d_f32_depth(const float* image, const float* kmat, float* dst,
+                                           uint32_t out_w, uint32_t out_h, uint32_t out_c, uint32_t k_w, uint32_t k_h,
+                                           uint32_t depth, uint32_t img_dpitch, uint32_t img_wpitch,
+                                           uint32_t stride_x, uint32_t stride_y,
+                                           uint32_t kmat_pitch, uint32_t dst_dpitch, uint32_t dst_wpitch, void* stream);
 
 /* Same as decx_hip_gemm_f32 / _f16 with the planner's choice overridden (`tile` = one of
  * DECX_HIP_TILE_*; AUTO = planner) and, with force_edge != 0, the predicated kernel
