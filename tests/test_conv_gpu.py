@@ -90,3 +90,6 @@ def test_conv2d_invalid_arguments(hip):
         args = list(ok); args[idx] = bad
         assert L.decx_hip_conv2d_f32(*args) == -1, idx
     assert L.decx_hip_conv2d_f32(d.ptr, d.ptr, d.ptr, 0, 2, 4, 3, 3, 4, 8, 1, 1, 4, 4, 8, None) == 0      # empty output
+    # the same call with the number of channels that exist: 1 .. the channel pitch
+    withdepth = lambda depth: L.decx_hip_conv2d_f32_depth(d.ptr, d.ptr, d.ptr, 2, 2, 4, 3, 3, depth, 4, 8, 1, 1, 4, 4, 8, None)
+    assert withdepth(3) == 0 and withdepth(4) == 0 and withdepth(0) == -1 and withdepth(5) == -1
