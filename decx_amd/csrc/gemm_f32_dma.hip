@@ -454,6 +454,9 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
 
 namespace {
 
+__device__ __forceinline__ float  fma_as(float a, float b, float c)    { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double fma_as(double a, double b, double c) { return __builtin_fma(a, b, c); }
+
 // one thread per four columns: D = sum of the partial products in split order (+ the C term).  TA: type of the
 // partial products and of the arithmetic, TO: type of C and D.
 template <typename TA, typename TO>
@@ -478,7 +481,7 @@ __global__ void __launch_bounds__(256) split_reduce_kernel(const GemmArgs g, uin
     for (int e = 0; e < 4; ++e) {
         if (col + e < g.N) {
             TA o = sum[e];
-            if (C) o = __builtin_fma((TA)C[(size_t)row * g.ldc + col + e], beta, alpha * o);
+            if (C) o = fma_as((TA)C[(size_t)row * g.ldc + col + e], beta, alpha * o);   // one fma in TA, as the unsplit epilogue
             D[(size_t)row * g.ldd + col + e] = (TO)o;
         }
     }
