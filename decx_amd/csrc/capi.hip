@@ -17,6 +17,15 @@ struct DeviceState {
 };
 DeviceState g_dev;
 
+// Workspace of decx_hip_gemm_f32_static: a device array that exists from the moment the code object is loaded, so the
+// entry point never allocates.  Each GPU holds its own copy at its own address; g_scratch[d] is the address on device d,
+// looked up once by decx_hip_init(d).  The array's name is only a host-side handle: kernels, copies and fills get the
+// looked-up pointer.
+constexpr size_t kScratchBytes = (size_t)DECX_HIP_STATIC_WORKSPACE_BYTES;
+constexpr int kMaxDevices = 16;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+void* g_scratch[kMaxDevices] = {};
+
 inline int hip_rc(hipError_t e) { return (int)e; }
 inline hipStream_t as_stream(void* s) { return (hipStream_t)s; }
 
@@ -265,6 +274,11 @@ int decx_hip_init(int device)
     if (count <= 0 || device < 0 || device >= count) return DECX_HIP_E_NO_DEVICE;
     if ((e = hipSetDevice(device)) != hipSuccess) return hip_rc(e);
     if ((e = hipGetDeviceProperties(&g_dev.prop, device)) != hipSuccess) return hip_rc(e);
+    if (device < kMaxDevices && !g_scratch[device]) {              // this device's copy of the static workspace
+        void* p = nullptr;
+        if ((e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) != hipSuccess) return hip_rc(e);
+        g_scratch[device] = p;
+    }
     g_dev.device = device;
     g_dev.compute_units = g_dev.prop.multiProcessorCount > 0 ? g_dev.prop.multiProcessorCount : 256;
     g_dev.ready = true;
@@ -295,6 +309,7 @@ const char* decx_hip_error_string(int code)
     case DECX_HIP_E_INVALID_ARG: return "invalid argument (null pointer, pitch smaller than width, or unknown enum)";
     case DECX_HIP_E_NOT_INIT:    return "decx_hip_init() has not been called";
     case DECX_HIP_E_NO_DEVICE:   return "no usable GPU";
+    case DECX_HIP_E_TOO_LARGE:   return "the product needs more workspace than the static one holds";
     default:                     return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
     }
 }
@@ -399,6 +414,16 @@ int decx_hip_gemm_f32_ws(const float* A, const float* B, const float* C, float* 
 {
     return run_gemm<false>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0, workspace,
                            workspace_bytes);
+}
+
+int decx_hip_gemm_f32_static(const float* A, const float* B, const float* C, float* D, uint32_t M, uint32_t N, uint32_t K,
+                             uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha, float beta, void* stream)
+{
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    void* const ws = g_dev.device < kMaxDevices ? g_scratch[g_dev.device] : nullptr;
+    if (!ws) return DECX_HIP_E_NOT_INIT;
+    if (decx_hip_gemm_workspace(4, M, N, K) > kScratchBytes) return DECX_HIP_E_TOO_LARGE;
+    return run_gemm<false>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0, ws, kScratchBytes);
 }
 
 int decx_hip_gemm_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, uint32_t M, uint32_t N,

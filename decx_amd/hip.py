@@ -54,6 +54,7 @@ SYMBOLS = {
     "decx_hip_gemm_f16": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp]),
     "decx_hip_gemm_f32_workspace": (ctypes.c_size_t, [_u32] * 3),
     "decx_hip_gemm_f32_ws": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, ctypes.c_size_t, _vp]),
+    "decx_hip_gemm_f32_static": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp]),
     "decx_hip_gemm_workspace": (ctypes.c_size_t, [_int] + [_u32] * 3),
     "decx_hip_gemm_f16_ws": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, ctypes.c_size_t, _vp]),
     "decx_hip_gemm_f64_ws": (_int, [_vp] * 4 + [_u32] * 7 + [ctypes.c_double, ctypes.c_double, _vp, ctypes.c_size_t, _vp]),

@@ -32,7 +32,8 @@ enum {
     DECX_HIP_OK            = 0,
     DECX_HIP_E_INVALID_ARG = -1,   /* null pointer, pitch smaller than width, unknown enum */
     DECX_HIP_E_NOT_INIT    = -2,   /* decx_hip_init() has not succeeded yet */
-    DECX_HIP_E_NO_DEVICE   = -3    /* no usable GPU */
+    DECX_HIP_E_NO_DEVICE   = -3,   /* no usable GPU */
+    DECX_HIP_E_TOO_LARGE   = -4    /* decx_hip_gemm_f32_static: the shape wants more workspace than the static one */
 };
 
 typedef struct decx_hip_device_props {
@@ -134,6 +135,21 @@ DECX_HIP_API int decx_hip_gemm_f32_ws(const float* A, const float* B, const floa
                                       uint32_t M, uint32_t N, uint32_t K,
                                       uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
                                       float alpha, float beta, void* workspace, size_t workspace_bytes, void* stream);
+/* decx_hip_gemm_f32_ws without the workspace arguments and without any allocation, by this call or by the library
+ * on its behalf: the workspace is a device array of DECX_HIP_STATIC_WORKSPACE_BYTES that is part of the library's
+ * code object (every GPU the library runs on holds its copy until the process ends; its address on a device is
+ * looked up by decx_hip_init for that device).  It has no counterpart in the reference: it is for callers that
+ * cannot allocate -- code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same
+ * results as decx_hip_gemm_f32_ws with a workspace of decx_hip_gemm_f32_workspace(M, N, K) bytes, bit for bit.
+ * Shapes whose workspace query exceeds DECX_HIP_STATIC_WORKSPACE_BYTES return DECX_HIP_E_TOO_LARGE and launch
+ * nothing (decx_hip_gemm_f32 still takes them, unsplit).  All calls on one GPU share the one array, which keeps
+ * the last call's contents (every call writes what it reads, nothing needs clearing): calls that overlap on one
+ * GPU -- two streams, two threads -- race; serialise them. */
+#define DECX_HIP_STATIC_WORKSPACE_BYTES (16u << 20)
+DECX_HIP_API int decx_hip_gemm_f32_static(const float* A, const float* B, const float* C, float* D,
+                                          uint32_t M, uint32_t N, uint32_t K,
+                                          uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
+                                          float alpha, float beta, void* stream);
 /* The same for the other two real types (elem_bytes 2, 4 or 8 in the query).  fp16 products keep their partial
  * products in fp32 and round once, after the sum. */
 DECX_HIP_API size_t decx_hip_gemm_workspace(int elem_bytes, uint32_t M, uint32_t N, uint32_t K);
