@@ -1,5 +1,5 @@
 // fp16 GEMM for gfx950: half inputs, fp32 accumulation on the matrix cores
-// (v_mfma_f32_32x32x16_f16), one round-to-nearest-even conversion to half at the end.  This is
+// (v_mfma_f32_16x16x32_f16, the same instruction and k order as the direct-to-LDS kernels), one round-to-nearest-even conversion to half at the end.  This is
 // the register-staged, fully predicated kernel for operands of any alignment and K == 0;
 // 16-byte aligned operands go to the direct-to-LDS kernels (launch_gemm_f16 below routes).
 //
@@ -10,13 +10,13 @@
 //
 // Structure of one workgroup (BM x BN tile, WAVES_M x WAVES_N wavefronts, slab depth BK):
 //   * Both operands sit in LDS k-contiguous: As[BM][BK + 8], Bs[BN][BK + 8] halves, because a
-//     32x32x16 MFMA wants 8 consecutive k per lane for both A and B.  A is row-major already.
+//     16x16x32 MFMA wants 8 consecutive k per lane for both A and B.  A is row-major already.
 //     B (row-major K x N) is transposed on the way in: a thread fetches an 8(k) x 8(n) block
 //     with eight 128-bit loads, transposes it in registers with byte permutes, and writes
 //     eight 128-bit rows.  The +8-half pad puts 16 consecutive rows in 16 distinct 4-bank
 //     groups, so the 128-bit fragment reads are conflict-free.
 //   * The wave's TN column tiles are interleaved (lane j owns columns TN*j .. TN*j+TN-1): the
-//     transposing store places column TN*j + t of a wave's strip in LDS row 32*t + j, so
+//     transposing store places column TN*j + t of a wave's strip in LDS row 16*t + j, so
 //     the fragment reads stay unit-stride over lanes while the epilogue stores TN
 //     contiguous halves per lane.
 //   * Slab s+1 travels global -> registers while slab s is multiplied; two LDS stages, one
@@ -40,13 +40,13 @@ gemm_f16_kernel(const GemmArgs g)
 {
     constexpr int NT = WAVES_M * WAVES_N * 64;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
-    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int TM = WM / 16, TN = WN / 16;
     constexpr int STRIDE = BK + 8;                       // halves
     constexpr int A_STAGE = BM * STRIDE, B_STAGE = BN * STRIDE;
     constexpr int A_PER = BM * BK / 8 / NT;              // 16-byte chunks of A per thread
     constexpr int B_PER = (BK / 8) * (BN / 8) / NT;      // 8x8 blocks of B per thread
     static_assert(A_PER >= 1 && B_PER >= 1, "tile too small for the workgroup");
-    static_assert(BK % 16 == 0 && WM % 32 == 0 && WN % 32 == 0, "shape");
+    static_assert(BK % 32 == 0 && WM % 16 == 0 && WN % 16 == 0 && (TN == 4 || TN == 8), "shape");
 
     __shared__ __attribute__((aligned(16))) _Float16 lds[2 * (A_STAGE + B_STAGE)];
     _Float16* const As = lds;
@@ -58,7 +58,7 @@ gemm_f16_kernel(const GemmArgs g)
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
-    const int l32 = lane & 31, h = lane >> 5;
+    const int l16 = lane & 15, kg = lane >> 4;          // row / column inside a 16 x 16 tile, group of 8 k
 
     const uint16_t* __restrict__ A = (const uint16_t*)g.A;
     const uint16_t* __restrict__ B = (const uint16_t*)g.B;
@@ -132,19 +132,19 @@ gemm_f16_kernel(const GemmArgs g)
                                      : pack_lo(rb[i][2 * w][c / 2], rb[i][2 * w + 1][c / 2]);
                 const int n = n8 * 8 + c;                 // column inside the block tile
                 const int cw = n % WN;                    // column inside its wave strip
-                const int row = (n / WN) * WN + 32 * (cw % TN) + cw / TN;
+                const int row = (n / WN) * WN + 16 * (cw % TN) + cw / TN;
                 *(uintx4*)&Bs[buf * B_STAGE + row * STRIDE + k8 * 8] = col;
             }
         }
     };
 
-    floatx16 acc[TM][TN];
+    floatx4 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
     const uint32_t slabs = (g.K + BK - 1) / BK;
     load_slab(0);
@@ -155,41 +155,41 @@ gemm_f16_kernel(const GemmArgs g)
         const int buf = s & 1;
         if (s + 1 < slabs) load_slab((s + 1) * BK);
 
-        const _Float16* a_base = As + buf * A_STAGE + (wm0 + l32) * STRIDE + 8 * h;
-        const _Float16* b_base = Bs + buf * B_STAGE + (wn0 + l32) * STRIDE + 8 * h;
+        const _Float16* a_base = As + buf * A_STAGE + (wm0 + l16) * STRIDE + 8 * kg;
+        const _Float16* b_base = Bs + buf * B_STAGE + (wn0 + l16) * STRIDE + 8 * kg;
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
+        for (int ks = 0; ks < BK / 32; ++ks) {
             halfx8 af[TM], bf[TN];
 #pragma unroll
-            for (int i = 0; i < TM; ++i) af[i] = *(const halfx8*)(a_base + i * 32 * STRIDE + 16 * ks);
+            for (int i = 0; i < TM; ++i) af[i] = *(const halfx8*)(a_base + i * 16 * STRIDE + 32 * ks);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) bf[j] = *(const halfx8*)(b_base + j * 32 * STRIDE + 16 * ks);
+            for (int j = 0; j < TN; ++j) bf[j] = *(const halfx8*)(b_base + j * 16 * STRIDE + 32 * ks);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
         }
 
         if (s + 1 < slabs) store_slab(buf ^ 1);
         __syncthreads();
     }
 
-    // Epilogue: register r of lane (l32, h) is row 8*(r/4) + 4*h + r%4 of a 32x32 tile;
+    // Epilogue: register r of lane (kg, l16) is row 4 * kg + r, column l16 of a 16 x 16 tile;
     // the lane's TN tiles are TN adjacent columns.
     const _Float16* __restrict__ C = (const _Float16*)g.C;
     _Float16* __restrict__ D = (_Float16*)g.D;
-    const uint32_t col0 = n0 + wn0 + TN * l32;
-    typedef _Float16 hvec __attribute__((ext_vector_type(TN == 1 ? 2 : TN)));   // TN == 1 handled scalar
+    const uint32_t col0 = n0 + wn0 + TN * l16;
+    typedef _Float16 hvec __attribute__((ext_vector_type(TN)));
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const uint32_t row = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t row = m0 + wm0 + i * 16 + 4 * kg + r;
             float v[TN];
 #pragma unroll
             for (int j = 0; j < TN; ++j) v[j] = acc[i][j][r];
-            if (TN > 1 && (rows_inside && cols_inside)) {
+            if (rows_inside && cols_inside) {
                 if (C) {
                     const hvec cv = *(const hvec*)(C + (size_t)row * g.ldc + col0);
 #pragma unroll

@@ -6,17 +6,21 @@
 // its "_T" kernels (srcs/modules/BLAS/GEMM/CUDA/large_squares/fp16/, srcs/common/Basic_process/
 // transpose/CUDA/transpose_kernels.cuh:204-236).
 //
-// v_mfma_f32_32x32x16_f16 takes 8 consecutive k per lane for BOTH operands.  A (row-major M x K)
-// has them contiguous: A fragments are 128-bit LDS reads.  B (row-major K x N) does not; its
-// fragments come from the transposing read `ds_read_b64_tr_b16` straight out of the row-major B
-// slab: a group of 16 lanes hands in the addresses of a 4 (k) x 16 (n) block (lane s: row s / 4,
-// 8-byte segment s % 4) and lane i receives column i of it, 4 consecutive k of one n; two such
-// reads give the 8 k a lane needs.  So neither a transpose pass nor a register shuffle is needed.
+// The matrix instruction is v_mfma_f32_16x16x32_f16, not the 32x32x16 form: fp16 products of this size run
+// under the board's power cap, and per flop the 16x16x32 form moves a fifth less through the register file
+// (half the accumulator traffic per flop).  A register-only loop on random operands sustains 1 900 TFLOP/s
+// with it against 1 680 with 32x32x16; this kernel gained 12 % from the change.
+//
+// The instruction takes 8 consecutive k per lane for BOTH operands: lane (kg = lane / 16, l16 = lane % 16)
+// supplies row / column l16 and k = 8 kg .. 8 kg + 7 of a 32-deep step.  A (row-major M x K) has them
+// contiguous: A fragments are 128-bit LDS reads.  B (row-major K x N) does not; its fragments come from the
+// transposing read `ds_read_b64_tr_b16` straight out of the row-major B slab: a group of 16 lanes hands in
+// the addresses of a 4 (k) x 16 (n) block (lane s: row s / 4, 8-byte segment s % 4) and lane i receives
+// column i of it, 4 consecutive k of one n; two such reads give the 8 k a lane needs.  So neither a
+// transpose pass nor a register shuffle is needed.
 // The MFMA is issued with its operands swapped (B fragment first): it then produces the transposed
-// 32 x 32 tile, in which a lane owns adjacent columns of one output row: after one
-// `v_permlane32_swap` a lane holds 16-byte pieces of its row, which a wave turns around through
-// LDS so that it stores whole rows of its tile (128 contiguous bytes per row instead of 32:
-// 1.1 us less per launch at 4096 x 4096 outputs).
+// 16 x 16 tile, in which a lane owns 4 adjacent columns of one output row.  A wave turns 16 rows of its
+// tile around through LDS so that it stores whole rows (WN * 2 contiguous bytes per row instead of 8).
 //
 // Slabs reach LDS by `global_load_lds_dwordx4` (no VGPRs, no ds_write).  These are inline assembly
 // and the slab barrier is a bare `s_barrier` behind an explicit vmcnt wait, because the compiler
@@ -29,10 +33,11 @@
 //   * ragged K: the partial last slab goes through registers, zero-filled beyond K.
 //
 // LDS layout of a stage.  A: [BM rows][CPR chunks of 16 bytes], chunk c of row r in slot
-// c ^ ((r / RPB) % CPR).  B: [BK k rows][BN / 8 chunks], chunk c of row k in slot c ^ key(k),
-// key(k) = 4 (k & 3) for rows of 256 bytes or more and 4 ((k >> 1) & 1) for 128-byte rows, so
-// that the 4 k rows x 64 bytes a half-wave reads through the transposing read cover all banks
-// once.  Both permutations are applied on the global side of the copy.
+// c ^ ((r / RPB) % CPR): the 16 lanes of a read phase (16 consecutive rows, one chunk) cover all banks.
+// B: [BK k rows][BN / 8 chunks], chunk c of row k in slot c ^ key(k), key(k) = 4 (k & 3) ^ 2 ((k >> 3) & 1)
+// for rows of 256 bytes or more and 4 ((k >> 1) & 1) ^ 2 ((k >> 3) & 1) for 128-byte rows: a half-wave
+// of the transposing read takes 4 k rows x 32 bytes from each of two k groups 8 rows apart, and the 16
+// pieces land in 16 different bank groups.  Both permutations are applied on the global side of the copy.
 #include "gemm_common.hpp"
 #include <type_traits>
 
@@ -96,19 +101,22 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     }
     const GemmArgs& g = [&]() -> const GemmArgs& { if constexpr (SPLIT) return g_split; else return g_in; }();
     constexpr int WAVES = WAVES_M * WAVES_N;
-    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 16, TN = WN / 16;
+    constexpr int HALVES = TM >= 8 ? 2 : 1, TMH = TM / HALVES;        // the A fragments of a k step come in this many parts
     constexpr int RB = BK * 2, CPR = RB / 16, RPB = 16 / CPR;         // A row bytes, chunks per row, rows per 256 bytes
     constexpr int BRB = BN * 2, CBR = BRB / 16, BROWS = 1024 / BRB;   // B row bytes, chunks per row, k rows per direct load
     constexpr int A_STAGE_BYTES = BM * RB, B_STAGE_BYTES = BK * BRB, STAGE_BYTES = A_STAGE_BYTES + B_STAGE_BYTES;
     constexpr int A_LOADS = A_STAGE_BYTES / 1024 / WAVES, B_LOADS = B_STAGE_BYTES / 1024 / WAVES, LOADS = A_LOADS + B_LOADS;
-    constexpr int KS = BK / 16;                                       // MFMA k steps per slab
-    static_assert(TM >= 1 && TN >= 1 && (BK == 32 || BK == 64) && KS % 2 == 0, "shape");
+    constexpr int KS = BK / 32;                                       // MFMA k steps per slab
+    constexpr int UNITS = KS * HALVES;
+    static_assert(TM >= 1 && TN >= 1 && BK == 64 && UNITS % 2 == 0, "shape");
     static_assert(BN == 64 || BN == 128 || BN == 256, "B row must be 128, 256 or 512 bytes");
     static_assert(A_LOADS >= 1 && B_LOADS >= 1 && A_LOADS * WAVES * 1024 == A_STAGE_BYTES &&
                   B_LOADS * WAVES * 1024 == B_STAGE_BYTES, "copy plan must divide evenly");
-    static_assert(STAGES >= 2 && STAGES * STAGE_BYTES <= 160 * 1024, "LDS budget");
+    constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+    static_assert(STAGES >= 2 && LDS_BYTES <= 160 * 1024, "LDS budget");
     static_assert(LOADS * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[LDS_BYTES];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)lds;
 
     uint32_t tile_m, tile_n;
@@ -116,17 +124,18 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
 
     const int t = threadIdx.x, lane = t & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);      // uniform: LDS destinations stay in scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
-    const int l32 = lane & 31, h = lane >> 5;
+    const int l16 = lane & 15, kg = lane >> 4;                 // row / column inside a 16 x 16 tile, group of 8 k
 
     const unsigned char* __restrict__ A = (const unsigned char*)g.A;
     const unsigned char* __restrict__ B = (const unsigned char*)g.B;
     const size_t lda_b = (size_t)g.lda * 2, ldb_b = (size_t)g.ldb * 2;
 
-    auto b_key = [](int k) { return BN >= 128 ? 4 * (k & 3) : 4 * ((k >> 1) & 1); };
+    // chunk permutation of B row k: the transposing read of a half-wave takes 4 k rows from each of two groups of
+    // 8 k (rows 8 apart), 32 bytes each: all 16 pieces must fall into different 16-byte bank groups
+    auto b_key = [](int k) { return (BN >= 128 ? 4 * (k & 3) : 4 * ((k >> 1) & 1)) ^ (2 * ((k >> 3) & 1)); };
 
-    // ---- copy plan (rows beyond M and column chunks beyond N are replaced by the last valid ones)
     const unsigned char* a_src[A_LOADS];
     const unsigned char* b_src[B_LOADS];
     int a_chunk[A_LOADS], b_krow[B_LOADS];
@@ -151,17 +160,17 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     const uint32_t full_slabs = g.K / BK, k_tail = g.K % BK;
     const uint32_t slabs = full_slabs + (k_tail ? 1u : 0u);
 
-    // Slabs are issued in ascending order.  A direct load takes its address as a scalar base (the tile's
-    // first row of A / B's row k, running along K) plus a 32-bit lane offset that never changes, so that
-    // advancing to the next slab is scalar arithmetic.
     const size_t b_step = (size_t)BK * ldb_b;
     uint32_t a_voff[A_LOADS], b_voff[B_LOADS];
     const unsigned char* a_base = A + (size_t)m0 * lda_b;
     const unsigned char* b_base = B;
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) a_voff[i] = (uint32_t)(a_src[i] - a_base);           // < BM * lda_b: the launcher checks
+    for (int i = 0; i < A_LOADS; ++i) a_voff[i] = (uint32_t)(a_src[i] - a_base);
 #pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) b_voff[i] = (uint32_t)(b_src[i] - b_base);           // < BK * ldb_b
+    for (int i = 0; i < B_LOADS; ++i) b_voff[i] = (uint32_t)(b_src[i] - b_base);
+    // Slabs are issued in ascending order.  A direct load takes its address as a scalar base (the tile's
+    // first row of A / B's row k, running along K) plus a 32-bit lane offset that never changes, so that
+    // advancing to the next slab is scalar arithmetic.
     auto issue_loads = [&](uint32_t slab) {
         const uint32_t stage = slab % STAGES;
         if (slab < full_slabs) {
@@ -203,53 +212,62 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     };
 
     // ---- fragment addressing (byte offsets inside a stage)
-    // A fragment (tile i, k step ks): row = wm0 + 32 i + l32, chunk = 2 ks + h.
-    const int a_row = wm0 + l32;
-    const int a_sw = (a_row / RPB) % CPR;
+    // A fragment (tile i, k step ks): lane (kg, l16) takes row wm0 + 16 i + l16, k = 32 ks + 8 kg .. + 7: chunk 4 ks + kg.
+    const int a_row = wm0 + l16;
+    const int a_sw = (a_row / RPB) % CPR;                  // wm0 + 16 i leaves it unchanged (multiples of 16 rows)
     const int a_off = a_row * RB;
-    // B fragment (tile j, k step ks, half r): a 16-lane group handles the n half (lane >> 4) & 1;
-    // lane s = lane & 15 supplies k = 16 ks + 8 h + 4 r + s / 4 and the 8-byte segment s % 4 of the
-    // 16 columns starting at wn0 + 32 j + 16 * nhalf.
-    const int s16 = lane & 15;
-    const int bk_row = 8 * h + (s16 >> 2);
-    const int bk_col = wn0 + 16 * ((lane >> 4) & 1) + 4 * (s16 & 3);
-    const int bk_sw = b_key(bk_row);                       // unchanged by + 16 ks + 4 r
+    // B fragment (tile j, k step ks, half r): the 16 lanes of group kg hand in the 4 k rows 32 ks + 8 kg + 4 r + (0..3),
+    // lane s = l16 the row s / 4 and the 8-byte segment s % 4 of the 16 columns from wn0 + 16 j; lane l16 receives
+    // column l16, 4 consecutive k.
+    const int bk_row = 8 * kg + (l16 >> 2);
+    const int bk_col = wn0 + 4 * (l16 & 3);
+    const int bk_sw = b_key(bk_row);                       // unchanged by + 32 ks + 4 r
     int b_off[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-        const int col = bk_col + 32 * j;
+        const int col = bk_col + 16 * j;
         b_off[j] = A_STAGE_BYTES + bk_row * BRB + (((col >> 3) ^ bk_sw) * 16) + (col & 7) * 2;
     }
 
-    struct Frags { halfx8 a[TM], b[TN]; };
-    auto read_frags = [&](Frags& f, const unsigned char* st, int ks) {
+    struct FragA { halfx8 a[TMH]; };
+    struct FragB { halfx8 b[TN]; };
+    FragA fa[2];
+    FragB fb[2];
+    // unit u = (k step ks = u / HALVES, part u % HALVES of the A rows)
+    auto read_unit = [&](const unsigned char* st, auto uc) {
+        constexpr int u = decltype(uc)::value, ks = u / HALVES, part = u % HALVES;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) f.a[i] = *(const halfx8*)(st + a_off + i * 32 * RB + (((2 * ks + h) ^ a_sw) * 16));
+        for (int i = 0; i < TMH; ++i)
+            fa[u & 1].a[i] = *(const halfx8*)(st + a_off + (part * TMH + i) * 16 * RB + (((4 * ks + kg) ^ a_sw) * 16));
+        if constexpr (part == 0) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const unsigned char* p0 = st + b_off[j] + ks * 16 * BRB;
-            const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)p0);
-            const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(p0 + 4 * BRB));
-            f.b[j] = join(lo, hi);
+            for (int j = 0; j < TN; ++j) {
+                const unsigned char* p0 = st + b_off[j] + ks * 32 * BRB;
+                const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)p0);
+                const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4*)(p0 + 4 * BRB));
+                fb[ks & 1].b[j] = join(lo, hi);
+            }
         }
     };
 
-    floatx16 accT[TN][TM];                                 // n tile j, m tile i, transposed
+    floatx4 accT[TN][TM];                                  // n tile j, m tile i, transposed
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) accT[j][i][r] = 0.f;
+            for (int r = 0; r < 4; ++r) accT[j][i][r] = 0.f;
 
-    auto multiply = [&](const Frags& f) {
+    auto multiply_unit = [&](auto uc) {
+        constexpr int u = decltype(uc)::value, ks = u / HALVES, part = u % HALVES;
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int i = 0; i < TMH; ++i)
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
-                accT[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.b[j], f.a[i], accT[j][i], 0, 0, 0);
+            for (int j = 0; j < TN; ++j)
+                accT[j][part * TMH + i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[ks & 1].b[j], fa[u & 1].a[i], accT[j][part * TMH + i], 0, 0, 0);
     };
-    constexpr int MFMAS = TM * TN, READS = TM + 2 * TN;
+    constexpr int MFMAS = TMH * TN;
+    constexpr int READS_FIRST = TMH + 2 * TN, READS_NEXT = TMH;      // a unit that opens a k step also reads the B fragments
 
 #pragma unroll
     for (int p = 0; p < STAGES - 1; ++p)
@@ -257,57 +275,48 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     if (slabs >= (uint32_t)(STAGES - 1)) wait_loads_and_barrier<LOADS * (STAGES - 2)>();
     else wait_loads_and_barrier<0>();
 
-    // fr[ks & 1] holds the fragments of k step ks.  The last step of a slab is multiplied after
-    // the slab barrier, behind the fragment reads of the next slab's first step (before the first
-    // slab it multiplies zeros).
-    Frags fr[2];
+    // The last unit of a slab is multiplied after the slab barrier, behind the fragment reads of the next slab's
+    // first unit (before the first slab it multiplies zeros).
 #pragma unroll
-    for (int i = 0; i < TM; ++i) fr[(KS - 1) & 1].a[i] = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
+    for (int i = 0; i < TMH; ++i) fa[(UNITS - 1) & 1].a[i] = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int j = 0; j < TN; ++j) fr[(KS - 1) & 1].b[j] = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
+    for (int j = 0; j < TN; ++j) fb[(KS - 1) & 1].b[j] = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
 
     for (uint32_t s = 0; s < slabs; ++s) {
         const unsigned char* st = lds + (s % STAGES) * STAGE_BYTES;
         const bool more = s + STAGES - 1 < slabs;
 
-        read_frags(fr[0], st, 0);
-        multiply(fr[(KS - 1) & 1]);
-        interleave<MFMAS, READS>();
+        read_unit(st, std::integral_constant<int, 0>{});
+        multiply_unit(std::integral_constant<int, UNITS - 1>{});
+        interleave<MFMAS, READS_FIRST>();
         __builtin_amdgcn_sched_barrier(0);
         // the stage that held slab s-1 is free: every wave passed the barrier after reading it
         if (more) issue_loads(s + STAGES - 1);
 
-        static_for<0, KS - 1>([&](auto kc) {
-            constexpr int ks = decltype(kc)::value;
-            read_frags(fr[(ks + 1) & 1], st, ks + 1);
-            multiply(fr[ks & 1]);
-            interleave<MFMAS, READS>();
+        static_for<0, UNITS - 1>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            read_unit(st, std::integral_constant<int, u + 1>{});
+            multiply_unit(uc);
+            interleave<MFMAS, ((u + 1) % HALVES == 0) ? READS_FIRST : READS_NEXT>();
             __builtin_amdgcn_sched_barrier(0);
         });
 
         if (more) wait_loads_and_barrier<LOADS * (STAGES - 2)>(); else wait_loads_and_barrier<0>();
     }
-    multiply(fr[(KS - 1) & 1]);
+    multiply_unit(std::integral_constant<int, UNITS - 1>{});
 
-    // Epilogue.  Lane (l32, h) holds output row l32 of the m tile; register 4 q + e is column
-    // 8 q + 4 h + e of the n tile.  Interior tiles: `v_permlane32_swap` trades the halves of an even
-    // and an odd 8-column group between lane l and lane l + 32, after which each lane holds 16-byte pieces.
-    if constexpr (SPLIT) {                                 // the fp32 partial product of this range of K
+    // Epilogue.  Lane (kg, l16) holds, of the 16 x 16 tile (i, j), row l16 and the 4 adjacent columns 4 kg .. 4 kg + 3.
+    if constexpr (SPLIT) {
         float* __restrict__ P = (float*)g.split_ws + (size_t)blockIdx.y * g.split_stride;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            const uint32_t row = m0 + wm0 + 32 * i + l32;
+            const uint32_t row = m0 + wm0 + 16 * i + l16;
             if (row < g.M) {
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const uint32_t col = n0 + wn0 + 32 * j + 8 * q + 4 * h;
-                        // split_ldd is a multiple of 4 and col a multiple of 4: whole 16-byte pieces lie inside the pitch
-                        if (col < g.split_ldd)
-                            *(floatx4*)(P + (size_t)row * g.split_ldd + col) =
-                                floatx4{accT[j][i][4 * q], accT[j][i][4 * q + 1], accT[j][i][4 * q + 2], accT[j][i][4 * q + 3]};
-                    }
+                for (int j = 0; j < TN; ++j) {
+                    const uint32_t col = n0 + wn0 + 16 * j + 4 * kg;
+                    if (col < g.split_ldd) *(floatx4*)(P + (size_t)row * g.split_ldd + col) = accT[j][i];
+                }
             }
         }
         return;
@@ -320,74 +329,59 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
         return w.u;
     };
     const bool interior = (m0 + BM <= g.M) && (n0 + BN <= g.N);
-    // Interior tiles go through LDS once more (the ring is free: every wave has passed the last slab
-    // barrier): a lane holds 16-byte pieces of ONE row, two lanes a row, so storing from the
-    // accumulator layout would touch 32 bytes of 32 different rows per instruction.  Each wave turns
-    // 32 rows x WN columns around in a private buffer (two of them, taking turns) and stores whole
-    // rows: WN * 2 contiguous bytes per row, 64 / PPR rows per instruction.
-    constexpr int ROW_BYTES = WN * 2, PPR = WN / 8, ROWS_PER_STORE = 64 / PPR, STORES = 32 / ROWS_PER_STORE;
-    static_assert(WAVES * 2 * 32 * ROW_BYTES <= STAGES * STAGE_BYTES, "staging rows must fit in the ring");
-    auto wave_sync = [] {                                  // LDS traffic of one wave is in order; this is for the compiler
+    // Interior tiles go through LDS once more (the ring is free: every wave has passed the last slab barrier): a lane
+    // holds 8 bytes of a row, 4 lanes 32 contiguous bytes.  Each wave turns 16 rows x WN columns around in a private
+    // buffer (two of them, taking turns) and stores whole rows: WN * 2 contiguous bytes per row.
+    constexpr int ROW_BYTES = WN * 2, PPR = WN / 8, RPG = 256 / ROW_BYTES, ROWS_PER_STORE = 64 / PPR, STORES = 16 / ROWS_PER_STORE;
+    static_assert(PPR == 4 || PPR == 8 || PPR == 16, "staging rows of 64, 128 or 256 bytes");
+    static_assert(WAVES * 2 * 16 * ROW_BYTES <= LDS_BYTES, "staging rows must fit in the ring");
+    auto wave_sync = [] {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     };
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-        const uint32_t row = m0 + wm0 + 32 * i + l32;
-        unsigned char* stage_rows = lds + (wave * 2 + (i & 1)) * (32 * ROW_BYTES);
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            if (interior) {
-#pragma unroll
-                for (int qp = 0; qp < 2; ++qp) {
-                    uint32_t w[2][2];                      // [even / odd group][dword]
-#pragma unroll
-                    for (int o = 0; o < 2; ++o) {
-                        const int q = 2 * qp + o;
-                        float v[4];
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = accT[j][i][4 * q + e];
-                        if (C) {
-                            const uint32_t col = n0 + wn0 + 32 * j + 8 * q + 4 * h;
-                            const halfx4 cv = *(const halfx4*)(C + (size_t)row * g.ldc + col);
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf((float)cv[e], g.beta, g.alpha * v[e]);
-                        }
-                        w[o][0] = pack2(v[0], v[1]);
-                        w[o][1] = pack2(v[2], v[3]);
-                    }
-                    const auto s0 = __builtin_amdgcn_permlane32_swap(w[0][0], w[1][0], false, false);
-                    const auto s1 = __builtin_amdgcn_permlane32_swap(w[0][1], w[1][1], false, false);
-                    const uintx4 out = {s0[0], s1[0], s0[1], s1[1]};
-                    // into this wave's staging rows: piece p of row l32, pieces XOR-permuted so that any 8
-                    // consecutive lanes hit 8 different 16-byte bank groups on the way in and on the way out
-                    const int p = 4 * j + 2 * qp + h;
-                    *(uintx4*)(stage_rows + l32 * ROW_BYTES + ((p ^ ((l32 / (8 / PPR)) % PPR)) * 16)) = out;
-                }
-            } else if (row < g.M) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint32_t col = n0 + wn0 + 32 * j + 8 * q + 4 * h + e;
-                        if (col < g.N) {
-                            float v = accT[j][i][4 * q + e];
-                            if (C) v = __builtin_fmaf((float)C[(size_t)row * g.ldc + col], g.beta, g.alpha * v);
-                            D[(size_t)row * g.ldd + col] = (_Float16)v;
-                        }
-                    }
-            }
-        }
+        const uint32_t row = m0 + wm0 + 16 * i + l16;
+        unsigned char* stage_rows = lds + (wave * 2 + (i & 1)) * (16 * ROW_BYTES);
         if (interior) {
-            wave_sync();
 #pragma unroll
-            for (int t = 0; t < STORES; ++t) {
-                const int r = ROWS_PER_STORE * t + lane / PPR, pc = lane % PPR;
-                const uintx4 v = *(const uintx4*)(stage_rows + r * ROW_BYTES + ((pc ^ ((r / (8 / PPR)) % PPR)) * 16));
-                *(uintx4*)(D + (size_t)(m0 + wm0 + 32 * i + r) * g.ldd + n0 + wn0 + 8 * pc) = v;
+            for (int j = 0; j < TN; ++j) {
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = accT[j][i][e];
+                if (C) {
+                    const uint32_t col = n0 + wn0 + 16 * j + 4 * kg;
+                    const halfx4 cv = *(const halfx4*)(C + (size_t)row * g.ldc + col);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf((float)cv[e], g.beta, g.alpha * v[e]);
+                }
+                const uintx2 out = {pack2(v[0], v[1]), pack2(v[2], v[3])};
+                // piece p (16 bytes) of row l16, half kg & 1 of it; pieces XOR-permuted so that the 32 lanes of a write
+                // and the 16 lanes of a read-back each cover all banks once
+                const int p = 2 * j + (kg >> 1);
+                *(uintx2*)(stage_rows + l16 * ROW_BYTES + ((p ^ ((l16 / RPG) % PPR)) * 16) + (kg & 1) * 8) = out;
             }
             wave_sync();
+#pragma unroll
+            for (int t2 = 0; t2 < STORES; ++t2) {
+                const int r = ROWS_PER_STORE * t2 + lane / PPR, pc = lane % PPR;
+                const uintx4 v = *(const uintx4*)(stage_rows + r * ROW_BYTES + ((pc ^ ((r / RPG) % PPR)) * 16));
+                *(uintx4*)(D + (size_t)(m0 + wm0 + 16 * i + r) * g.ldd + n0 + wn0 + 8 * pc) = v;
+            }
+            wave_sync();
+        } else if (row < g.M) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t col = n0 + wn0 + 16 * j + 4 * kg + e;
+                    if (col < g.N) {
+                        float v = accT[j][i][e];
+                        if (C) v = __builtin_fmaf((float)C[(size_t)row * g.ldc + col], g.beta, g.alpha * v);
+                        D[(size_t)row * g.ldd + col] = (_Float16)v;
+                    }
+                }
         }
     }
 }
