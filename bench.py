@@ -8,8 +8,11 @@ fp32 M=N=K=8192 product (dense fp32 MFMA roof); the same JSON line carries the f
 product (dense fp16 MFMA roof) and the bandwidth-bound shapes under "other_workloads".
 The kernel time is measured with HIP events recorded on the launch stream.  The CPU
 baseline is the in-repo AVX2 restatement of the reference's multithreaded CPU GEMM, timed
-once on the host cores on the same workload and checked bit-for-bit against the scalar
-fma chain on sampled rows.
+on the host cores on the same workload (every fp32 workload of the baseline's configurations
+carries its own: thread count stated, best of a few calls for the short ones) and checked
+bit-for-bit against the scalar fma chain on sampled rows; every GEMM workload also carries
+the GPU result's error against the CPU result or, where the reference has no CPU form, against
+the chain on sampled rows ("gpu_parity").
 """
 import argparse
 import math
@@ -28,15 +31,49 @@ PEAK_F16_TFLOPS = 2500.0     # MI355X dense fp16 matrix
 PEAK_F64_TFLOPS = 78.6       # MI355X dense fp64 matrix
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by a
-# copy kernel of known size; None until measured for that workload.
+# Bytes per launch that crossed the L2 <-> fabric boundary (HBM or the memory-side cache behind it), recorded from
+# rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE in KiB per dispatch, scaled by what the same counters read for a copy
+# kernel of known size) of this same file's workloads.  Each figure names the profile that holds it and the source
+# file of the kernel it was measured on with that file's SHA-256 at the time: when the kernel source has changed
+# since, the figure is withheld ("traffic": null, "traffic_stale": true) until the workload is profiled again.
 MEASURED_TRAFFIC = {
-    "fp32_8192": 5.71e9,     # FETCH_SIZE 2.6574e6 x 2.0 KiB + WRITE_SIZE 2.621e5 KiB
-    "fp16_4096": 2.35e8,     # FETCH_SIZE 98 461 x 2.0 KiB + WRITE_SIZE 32 793 KiB
-    "fp32_gemv": 2.70e8,     # FETCH_SIZE (131 228 + 522) x 2.0 KiB + WRITE_SIZE (256 + 32) KiB: matrix-vector kernel + the copy of x
-    "fp32_gevm": 2.69e8,     # FETCH_SIZE 131 224 x 2.0 KiB + WRITE_SIZE 32 KiB
-    "fp64_4096": 1.21e9,     # FETCH_SIZE 524 415 x 2.0 KiB + WRITE_SIZE 131 072 KiB
+    "fp32_8192": {"bytes": 5.71e9, "counters": "FETCH_SIZE 2.6574e6 x 2.0 KiB + WRITE_SIZE 2.621e5 KiB",
+                  "kernel": "gemm_f32_dma_kernel<256, 128, 2, 2, 16, 2, false, 0, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
+                  "source_sha256": "", "profile": "profiles/gemm_f32_dma_fp32_8192cubed.md"},
+    "fp16_4096": {"bytes": 2.35e8, "counters": "FETCH_SIZE 98 461 x 2.0 KiB + WRITE_SIZE 32 793 KiB",
+                  "kernel": "gemm_f16_dma_kernel<256, 256, 2, 4, 64, 2, false>", "source": "decx_amd/csrc/gemm_f16_dma.hip",
+                  "source_sha256": "", "profile": "profiles/gemm_f16_dma_fp16_4096cubed.md"},
+    "fp32_gemv": {"bytes": 2.70e8, "counters": "FETCH_SIZE (131 228 + 522) x 2.0 KiB + WRITE_SIZE (256 + 32) KiB: matrix-vector kernel + the copy of x",
+                  "kernel": "gemv_kernel<float, float>", "source": "decx_amd/csrc/gemv.hip",
+                  "source_sha256": "", "profile": "profiles/gemv_gevm_8192x8192.md"},
+    "fp32_gevm": {"bytes": 2.69e8, "counters": "FETCH_SIZE 131 224 x 2.0 KiB + WRITE_SIZE 32 KiB",
+                  "kernel": "gevm_kernel<float, float>", "source": "decx_amd/csrc/gemv.hip",
+                  "source_sha256": "", "profile": "profiles/gemv_gevm_8192x8192.md"},
+    "fp64_4096": {"bytes": 1.21e9, "counters": "FETCH_SIZE 524 415 x 2.0 KiB + WRITE_SIZE 131 072 KiB",
+                  "kernel": "gemm_f64_dma_kernel<256, 128, 4, 2, 16, 3>", "source": "decx_amd/csrc/gemm_f64.hip",
+                  "source_sha256": "", "profile": "profiles/gemm_f64_dma_fp64_4096cubed.md"},
+    "conv2d": {"bytes": 1.80e8, "counters": "FETCH_SIZE 55 474 x 2.0 KiB + WRITE_SIZE 64 516 KiB",
+               "kernel": "gemm_f32_dma_kernel<256, 256, 2, 4, 16, 4, false, 2, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
+               "source_sha256": "", "profile": "profiles/conv2d_implicit_gemm_256x256x112_3x3x256.md"},
 }
+
+
+def traffic_fields(name):
+    """{"traffic": bytes or None, "traffic_measured_at": ...} for a roofline object."""
+    rec = MEASURED_TRAFFIC.get(name)
+    if rec is None:
+        return {"traffic": None}
+    import hashlib
+    try:
+        now = hashlib.sha256(open(os.path.join(ROOT, rec["source"]), "rb").read()).hexdigest()
+    except OSError:
+        now = None
+    at = {"kernel": rec["kernel"], "source": rec["source"], "source_sha256": rec["source_sha256"][:16],
+          "profile": rec["profile"], "counters": rec["counters"]}
+    if now is None or now != rec["source_sha256"]:
+        return {"traffic": None, "traffic_stale": True, "traffic_measured_at": at}
+    return {"traffic": rec["bytes"], "traffic_measured_at": at}
+
 
 WORKLOADS = {
     # name: (dtype, M, N, K, bound, config number for seeds, description)
@@ -45,6 +82,7 @@ WORKLOADS = {
     "fp64_4096": ("f64", 4096, 4096, 4096, "mfma", 7, "fp64 GEMM M=N=K=4096, uniform[-1,1]"),
     "fp32_1024": ("f32", 1024, 1024, 1024, "mfma", 1, "fp32 GEMM M=N=K=1024, uniform[-1,1]"),
     "fp32_ragged": ("f32", 1000, 1500, 777, "mfma", 2, "fp32 GEMM M=1000 N=1500 K=777, uniform[-1,1]"),
+    "fp32_ragged_abc": ("f32", 1000, 1500, 777, "mfma", 2, "fp32 GEMM D=A.B+C M=1000 N=1500 K=777 (four-matrix entry, alpha=beta=1), uniform[-1,1]"),
     "fp32_tall_skinny": ("f32", 65536, 256, 1024, "mfma", 5, "fp32 GEMM M=65536 N=256 K=1024, uniform[-1,1]"),
     "fp32_mid_long_k": ("f32", 1280, 1024, 8192, "mfma", 8, "fp32 GEMM M=1280 N=1024 K=8192 (320 small tiles, split along K through the workspace), uniform[-1,1]"),
     "fp32_gemv": ("f32", 8192, 1, 8192, "hbm", 6, "fp32 GEMM M=8192 N=1 K=8192 (GEMV-like), uniform[-1,1]"),
@@ -71,55 +109,59 @@ def device_pitch(cols, itemsize):
 
 
 def run_workload(name, steps, warmup, keep_inputs=False, settle_s=0.0):
-    from decx_amd import hip
-    dt, M, N, K, bound, _, desc = WORKLOADS[name]
+    from decx_amd import hip, synth
+    dt, M, N, K, bound, cfg, desc = WORKLOADS[name]
     npdt = {"f32": np.float32, "f16": np.float16, "f64": np.float64}[dt]
     A, B = make_inputs(name)
+    C = synth.uniform_f32(M, N, synth.seeds(cfg)[2]) if name.endswith("_abc") else None
     isz = np.dtype(npdt).itemsize
     dA = hip.DeviceMatrix(M, K, npdt, device_pitch(K, isz), A)
     dB = hip.DeviceMatrix(K, N, npdt, device_pitch(N, isz), B)
+    dC = hip.DeviceMatrix(M, N, npdt, device_pitch(N, isz), C) if C is not None else None
     dD = hip.DeviceMatrix(M, N, npdt, device_pitch(N, isz))
     # the workspace the library asks for (split K, the dense copy of a column operand), held by the caller as the
     # de:: layer holds it; none for most shapes
     need = int(hip.lib().decx_hip_gemm_workspace(isz, M, N, K))
     ws = hip.DeviceMatrix(1, need // 4, np.float32) if need else None
+    call = lambda: hip.gemm(dA, dB, dD, dC, 1.0, 1.0, workspace=ws)
     for _ in range(warmup):
-        hip.gemm(dA, dB, dD, workspace=ws)
+        call()
     hip.sync()
     # short kernels: keep launching until the clocks have settled (the first milliseconds after
     # idle run at ramping clocks and would be what a 20-launch measurement sees)
     t_settle = time.perf_counter()
     while time.perf_counter() - t_settle < settle_s:
         for _ in range(10):
-            hip.gemm(dA, dB, dD, workspace=ws)
+            call()
         hip.sync()
     timer = hip.Timer()
     t0 = time.perf_counter()
     timer.start()
     for _ in range(steps):
-        hip.gemm(dA, dB, dD, workspace=ws)
+        call()
     kernel_ms = timer.stop() / steps            # HIP events on the launch stream
     hip.sync()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     flops = 2.0 * M * N * K
-    abytes = float(isz) * (M * K + K * N + M * N)
+    abytes = float(isz) * (M * K + K * N + M * N + (M * N if C is not None else 0))
     tflops = flops / (kernel_ms * 1e-3) / 1e12
     gbs = abytes / (kernel_ms * 1e-3) / 1e9
     if bound == "mfma":
         peak = {"f32": PEAK_F32_TFLOPS, "f16": PEAK_F16_TFLOPS, "f64": PEAK_F64_TFLOPS}[dt]
         roof = {"bound": "mfma", "achieved": round(tflops, 3), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(tflops / peak, 4), "traffic": MEASURED_TRAFFIC.get(name)}
+                "frac": round(tflops / peak, 4)}
     else:
         roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC.get(name)}
+                "frac": round(gbs / PEAK_HBM_GBS, 4)}
+    roof.update(traffic_fields(name))
     p = hip.plan(isz, M, N, K)
     out = {"workload": desc, "dtype": dt, "value": round(tflops, 3), "unit": "TFLOP/s",
            "hbm_gbs_algorithmic": round(gbs, 1), "kernel_ms": round(kernel_ms, 5), "wall_ms_per_step": round(wall_ms, 5),
            "plan": {"path": int(p.path), "tile": [int(p.tile_m), int(p.tile_n)], "grid": int(p.grid), "edge": int(p.edge),
-                    "workspace_bytes": need},
+                    "k_splits": int(p.k_splits), "workspace_bytes": need},
            "roofline": roof}
-    result = (out, (A, B, dD.download()) if keep_inputs else None)    # the result goes to the CPU leg's comparison
-    for d in (dA, dB, dD, ws):
+    result = (out, (A, B, C, dD.download()) if keep_inputs else None)    # the result goes to the CPU leg's comparison
+    for d in (dA, dB, dC, dD, ws):
         if d is not None:
             d.free()
     return result
@@ -169,8 +211,8 @@ def run_conv(steps, warmup, settle_s=0.25, c=None):
         c["KW"], c["KH"], c["W"], c["H"], c["C"], c["OC"], ow * oh, c["OC"], K)
     if c is CONV:
         roof = {"bound": "mfma", "achieved": round(tf, 3), "peak": PEAK_F32_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(tf / PEAK_F32_TFLOPS, 4),
-                "traffic": 1.80e8}               # FETCH_SIZE 55 474 x 2.0 KiB + WRITE_SIZE 64 516 KiB
+                "frac": round(tf / PEAK_F32_TFLOPS, 4)}
+        roof.update(traffic_fields("conv2d"))
     else:                                        # 16 flop per byte: the memory system bounds it
         roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}
@@ -219,35 +261,88 @@ def run_complex(double, n, steps, warmup, settle_s=0.25):
     return out
 
 
-def cpu_baseline(name, A, B, D_gpu):
-    """Times the AVX2 restatement of the reference CPU GEMM once on this host, checks it bit-for-bit
-    against the scalar fma chain on sampled rows, and compares the GPU's whole result with it."""
+# how the CPU leg runs each fp32 workload: (thread counts, calls per thread count -- the best one is reported)
+CPU_LEGS = {
+    "fp32_8192": ((16,), 1),            # ~1.4 s per call
+    "fp32_1024": ((16,), 5),            # the one configuration the reference publishes a CPU time for (9.98 ms on its authors' host)
+    "fp32_ragged": ((16,), 5),
+    "fp32_ragged_abc": ((16,), 5),
+    "fp32_tall_skinny": ((16,), 2),
+    "fp32_gemv": ((1, 16), 3),          # the reference itself is only correct single-threaded on this shape
+}
+
+
+def cpu_baseline(name, A, B, C, D_gpu):
+    """Times the AVX2 restatement of the reference CPU GEMM on this host (best of a few calls for the short
+    workloads), checks it bit-for-bit against the scalar fma chain on sampled rows, and compares the GPU's
+    whole result with it.  Returns (cpu_baseline, gpu_parity)."""
     from oracle import binding as oracle
     import ctypes
     _, M, N, K, _, _, desc = WORKLOADS[name]
     L = oracle.lib()
-    threads = min(int(L.cpu_port_max_threads()), os.cpu_count() or 1)
     a, lda = oracle.aligned_f32(M, K); a[:, :K] = A
     b, ldb = oracle.aligned_f32(K, N); b[:, :N] = B
     d, ldd = oracle.aligned_f32(M, N)
+    c, ldc = (None, 0)
+    if C is not None:
+        c, ldc = oracle.aligned_f32(M, N); c[:, :N] = C
     scratch, _ = oracle.aligned_f32(1, int(L.cpu_port_scratch_floats(K, N)))
     fp = ctypes.POINTER(ctypes.c_float)
-    args = [x.ctypes.data_as(fp) for x in (a, b)] + [None, d.ctypes.data_as(fp), M, N, K, lda, ldb, 0, ldd,
-                                                     scratch.ctypes.data_as(fp), threads]
-    t0 = time.perf_counter()
-    rc = L.cpu_port_gemm_f32(*args)
-    secs = time.perf_counter() - t0
-    assert rc == 0
+    thread_counts, calls = CPU_LEGS[name]
+    runs = []
+    for want in thread_counts:
+        threads = max(1, min(want, int(L.cpu_port_max_threads()), os.cpu_count() or 1))
+        args = [a.ctypes.data_as(fp), b.ctypes.data_as(fp), c.ctypes.data_as(fp) if c is not None else None,
+                d.ctypes.data_as(fp), M, N, K, lda, ldb, ldc, ldd, scratch.ctypes.data_as(fp), threads]
+        best = 1e30
+        for _ in range(calls):
+            t0 = time.perf_counter()
+            rc = L.cpu_port_gemm_f32(*args)
+            best = min(best, time.perf_counter() - t0)
+            assert rc == 0
+        runs.append({"cores": threads, "ms": round(best * 1e3, 3), "value": round(2.0 * M * N * K / best / 1e12, 4)})
     rows = np.unique(np.random.default_rng(0).integers(0, M, 16)).astype(np.uint32)
-    chain = oracle.gemm_f32(A, B, rows=rows)
+    chain = oracle.gemm_f32(A, B, C, rows=rows)
     same = bool(np.array_equal(d[rows, :N].view(np.uint32), chain.view(np.uint32)))
     ref_max = float(np.max(np.abs(d[:, :N])))
     gpu_err = float(np.max(np.abs(D_gpu - d[:, :N]))) / (ref_max * math.sqrt(K))
-    return {"value": round(2.0 * M * N * K / secs / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": "one full call of the same workload (%s), %.2f s wall" % (desc.split(",")[0], secs),
-            "bit_equal_to_fma_chain": same,
-            "gpu_parity": {"rel_err": float("%.3g" % gpu_err), "bar": 1e-5, "elements": int(M) * int(N),
-                           "measure": "max|gpu - cpu| / (max|cpu| sqrt(K)) over the whole output"}}
+    top = max(runs, key=lambda r: r["value"])
+    base = {"value": top["value"], "unit": "TFLOP/s", "cores": top["cores"], "kind": "port", "ms": top["ms"],
+            "sample": "the whole workload (%s), best of %d call%s" % (desc.split(",")[0], calls, "" if calls == 1 else "s"),
+            "bit_equal_to_fma_chain": same}
+    if len(runs) > 1:
+        base["by_thread_count"] = runs
+    parity = {"rel_err": float("%.3g" % gpu_err), "bar": 1e-5, "elements": int(M) * int(N), "against": "cpu_baseline",
+              "measure": "max|gpu - cpu| / (max|cpu| sqrt(K)) over the whole output"}
+    return base, parity
+
+
+def chain_parity(name, A, B, C, D_gpu, rows=48):
+    """GPU result against the oracle's k-ascending fma chain on sampled rows, for the workloads the reference has no
+    CPU form of (fp16) or whose CPU form is not restated here (fp64)."""
+    from oracle import binding as oracle
+    dt, M, N, K = WORKLOADS[name][:4]
+    pick = np.unique(np.concatenate([[0, M - 1], np.random.default_rng(1).integers(0, M, rows)])).astype(np.uint32)
+    if dt == "f16":
+        ref = oracle.gemm_f16(A, B, rows=pick).astype(np.float64); bar = 2e-3
+    elif dt == "f64":
+        ref = oracle.gemm_f64(A, B, rows=pick); bar = 1e-14
+    else:
+        ref = oracle.gemm_f32(A, B, C, rows=pick).astype(np.float64); bar = 1e-5
+    err = float(np.max(np.abs(D_gpu[pick].astype(np.float64) - ref))) / (float(np.max(np.abs(ref))) * math.sqrt(K))
+    return {"rel_err": float("%.3g" % err), "bar": bar, "elements": int(len(pick)) * int(N), "against": "fma chain oracle",
+            "measure": "max|gpu - chain| / (max|chain| sqrt(K)) over %d sampled rows" % len(pick)}
+
+
+def cpu_and_parity(name, out, inputs):
+    """Adds "cpu_baseline" and "gpu_parity" to a workload's record."""
+    A, B, C, D_gpu = inputs
+    if name in CPU_LEGS:
+        out["cpu_baseline"], out["gpu_parity"] = cpu_baseline(name, A, B, C, D_gpu)
+    else:
+        out["cpu_baseline"] = None           # no CPU form in the reference (fp16) / none restated here (fp64, the long-K split)
+        out["gpu_parity"] = chain_parity(name, A, B, C, D_gpu)
+    return out
 
 
 def api_wall_time(name, repeats=10):
@@ -283,6 +378,7 @@ def main():
 
     # the de:: API's own wall time, before this process takes the GPU
     api = api_wall_time(args.workload) if (args.workload in WORKLOADS and not args.no_extra) else None
+    api16 = api_wall_time("fp16_4096") if (args.workload == "fp32_8192" and not args.no_extra) else None
 
     from decx_amd import hip
     hip.init(0)
@@ -332,17 +428,22 @@ def main():
         for name in WORKLOADS:
             if name != args.workload:
                 small = WORKLOADS[name][1] * WORKLOADS[name][2] * WORKLOADS[name][3] < 2 ** 38
-                others.append(run_workload(name, 200 if small else args.steps, args.warmup, settle_s=0.25)[0])
+                o, inp = run_workload(name, 200 if small else args.steps, args.warmup, keep_inputs=not args.no_cpu, settle_s=0.25)
+                if not args.no_cpu:
+                    cpu_and_parity(name, o, inp)
+                if name == "fp16_4096" and api16 is not None:
+                    o["api_wall"] = api16
+                others.append(o)
+                del inp
         others.append(run_conv(200, args.warmup))
         others.append(run_conv(200, args.warmup, c=CONV_RGB))
         others.append(run_complex(False, 4096, args.steps, args.warmup))
         others.append(run_complex(True, 2048, 50, args.warmup))
         line["other_workloads"] = others
     if not args.no_cpu:
-        if main_out["dtype"] == "f32":
-            line["cpu_baseline"] = cpu_baseline(args.workload, *inputs)
-        else:
-            line["cpu_baseline"] = None          # the reference has no fp16 CPU GEMM
+        cpu_and_parity(args.workload, line, inputs)
+        if line["cpu_baseline"] is not None:     # where the first round's readers look for it
+            line["cpu_baseline"]["gpu_parity"] = line["gpu_parity"]
     print(json.dumps(line))
 
 

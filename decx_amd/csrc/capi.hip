@@ -1,6 +1,7 @@
 // The C ABI declared in include/decx_hip.h: argument checking, the tile planner, and
 // thin wrappers over the HIP runtime.  No C++ type crosses this boundary.
 #include "../../include/decx_hip.h"
+#include "../../include/decx_hip_profiling.h"
 #include "gemm_common.hpp"
 
 #include <cstring>
@@ -35,7 +36,7 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 // small tiles win while the grid would otherwise leave CUs idle.  Ties go to the larger tile.
 int choose_tile_f64(uint32_t M, uint32_t N)
 {
-    int best = TILE_64x64;
+    int best = TILE_SMALL;
     double best_cost = 1e300;
     for (int s = TILE_COUNT - 1; s >= 0; --s) {
         const TileInfo ti = tile_info_f64(s);
@@ -48,7 +49,7 @@ int choose_tile_f64(uint32_t M, uint32_t N)
 
 int choose_tile(bool f16, uint32_t M, uint32_t N, bool aligned)
 {
-    int best = TILE_64x64;
+    int best = TILE_SMALL;
     double best_cost = 1e300;
     for (int s = TILE_COUNT - 1; s >= 0; --s) {
         const TileInfo ti = f16 ? tile_info_f16(s, aligned) : tile_info_f32(s, aligned, N);
@@ -91,7 +92,7 @@ SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
     if (elem_bytes == 4 && K >= 4096) {
         // 64 x 64 tiles, up to five workgroups per CU.  score = (workgroups on the busiest CU / the average) x what a
         // CU loses with m workgroups against a full one; the ranges p that make t * p an even three to five per CU win.
-        const TileInfo small = tile_info_f32(TILE_64x64, true, N);
+        const TileInfo small = tile_info_f32(TILE_SMALL, true, N);
         const uint64_t t = (uint64_t)((M + small.bm - 1) / small.bm) * ((N + small.bn - 1) / small.bn);
         const auto score = [&](uint32_t p) {
             const uint64_t wgs = t * p, m = (wgs + cus - 1) / cus;
@@ -105,7 +106,7 @@ SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
                 if (score(p2) < best_score) { best_score = score(p2); best = p2; }
             if (best > 1) {
                 const uint32_t len = ((K + best - 1) / best + 31) / 32 * 32;
-                return {TILE_64x64, (K + len - 1) / len, len};
+                return {TILE_SMALL, (K + len - 1) / len, len};
             }
         }
     }
@@ -118,7 +119,7 @@ SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
             while (p2 * 2 * t <= cus && p2 < 8 && K / (p2 * 2) >= 2048) p2 *= 2;
             if (p2 > 1 && t * p2 * 20 >= 11ull * cus) {
                 const uint32_t len = ((K + p2 - 1) / p2 + 31) / 32 * 32;
-                return {TILE_128x128, (K + len - 1) / len, len};
+                return {TILE_MEDIUM, (K + len - 1) / len, len};
             }
         }
     }
@@ -129,7 +130,7 @@ SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
         uint32_t best = 1;
         double best_cost = tile_cost(ti, tiles_of((uint32_t)ti.bm), cus) / 1.15;   // ti.bm == ti.bn for the smaller tiles
         if (ti.bm != ti.bn) best_cost = tile_cost(ti, (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn), cus) / 1.15;
-        for (int sh = TILE_128x128; sh <= TILE_64x64; ++sh) {
+        for (int sh = TILE_MEDIUM; sh <= TILE_SMALL; ++sh) {
             const TileInfo t2 = tile_info_f64(sh);
             const uint64_t t = tiles_of((uint32_t)t2.bm);
             for (uint32_t p2 = 2; p2 <= 8 && K / p2 >= 1024; ++p2) {
@@ -540,7 +541,9 @@ static int run_gemm_complex(const T* A, const T* B, const T* C, T* D, uint32_t M
     const uint32_t ldx = (uint32_t)(((size_t)2 * N + 15) / 16 * 16);
     if (rc == DECX_HIP_OK && K > 0) rc = launch_complex_expand_b<T>(B, (T*)workspace, K, N, ldb, ldx, ar, ai, S);
     if (rc != DECX_HIP_OK) return rc;
-    // real GEMM M x 2N x 2K accumulating onto D when C was given (K == 0 leaves D = beta * C, or zero)
+    // real GEMM M x 2N x 2K accumulating onto D when C was given (K == 0 leaves D = beta * C, or zero; no element of
+    // B' is read then and the caller may have passed no workspace: any non-null pointer stands in)
+    if (K == 0 && !workspace) workspace = D;
     if constexpr (sizeof(T) == 4)
         return run_gemm<false>(A, workspace, C ? D : nullptr, D, M, 2 * N, 2 * K, 2 * lda, ldx, 2 * ldd, 2 * ldd, 1.f, 1.f, stream,
                                DECX_HIP_TILE_AUTO, 0);

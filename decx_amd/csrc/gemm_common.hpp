@@ -27,7 +27,6 @@ struct GemmArgs {
     float alpha, beta;
     double alpha64, beta64;      // the same two scalars for the fp64 kernels
     uint32_t tiles_m, tiles_n;   // number of block tiles along M and N
-    uint32_t xcd_remap;          // 1: grid size is a multiple of 8, use the per-XCD ordering
     uint32_t vec_ok;             // 1: every base pointer is 16-byte aligned and every pitch a multiple of 16 bytes
     // Split K (direct-load kernels, grid.y = number of splits): split z multiplies k in [z * split_len,
     // min(K, (z + 1) * split_len)) and writes its M x N partial product (fp32 for fp32 and fp16 operands, fp64
@@ -57,13 +56,15 @@ constexpr int kGroupM = 4;      // tile-rows per L2 patch (4 x 8 tiles run toget
 
 // Maps the hardware block index to a tile.  Hardware deals consecutive block ids to
 // consecutive XCDs; each XCD has a private L2.  Step 1 gives every XCD a contiguous
-// range of logical ids, step 2 walks logical ids in groups of kGroupM tile-rows so the
+// range of logical ids (the first 8 * (nb / 8) blocks; the up to 7 that remain keep their
+// ids, at the end of the last range), step 2 walks logical ids in groups of kGroupM tile-rows so the
 // 32 tiles resident on one XCD form a compact patch that shares A rows and B columns.
 __device__ __forceinline__ void block_to_tile(const GemmArgs& g, uint32_t& tile_m, uint32_t& tile_n)
 {
     const uint32_t nb = g.tiles_m * g.tiles_n;
     uint32_t id = blockIdx.x;
-    if (g.xcd_remap) id = (id % kXcds) * (nb / kXcds) + id / kXcds;
+    const uint32_t per_xcd = nb / kXcds;
+    if (id < per_xcd * kXcds) id = (id % kXcds) * per_xcd + id / kXcds;
     const uint32_t group_m = g.group_m ? g.group_m : (uint32_t)kGroupM;
     const uint32_t per_group = group_m * g.tiles_n;
     const uint32_t group = id / per_group;
@@ -76,11 +77,14 @@ __device__ __forceinline__ void block_to_tile(const GemmArgs& g, uint32_t& tile_
 
 // ---- tile-shape table shared by the planner and the launchers -----------------
 
+// Size classes; the block tile each stands for depends on the element type and the kernel family (tile_info_*):
+// LARGE 256 x 256 (fp16, and the register-staged fp32 kernels) or 256 x 128 (fp32 and fp64 direct-to-LDS),
+// MEDIUM 128 x 128, SMALL 64 x 64 (128 x 32 for fp32 outputs of at most kNarrowN columns).
 enum TileShape : int {
-    TILE_256x256 = 0,
-    TILE_128x128 = 1,
-    TILE_64x64   = 2,
-    TILE_COUNT   = 3,
+    TILE_LARGE  = 0,
+    TILE_MEDIUM = 1,
+    TILE_SMALL  = 2,
+    TILE_COUNT  = 3,
 };
 
 // per_cu: workgroups of the shape that fit a CU together.  full: throughput of a CU filled with them, alone: of
@@ -120,8 +124,8 @@ __host__ inline double tile_cost(const TileInfo& ti, uint64_t tiles, uint32_t cu
 __host__ inline TileInfo tile_info_f32(int shape, bool aligned = true, uint32_t N = 0xffffffffu)
 {
     switch (shape) {
-    case TILE_256x256: return aligned ? TileInfo{256, 128, 256, 2, 1.00f, 0.95f} : TileInfo{256, 256, 512, 1, 1.00f, 1.00f};
-    case TILE_128x128: return {128, 128, 256, aligned ? 4 : 2, aligned ? 1.00f : 0.80f, aligned ? 0.88f : 0.72f};
+    case TILE_LARGE: return aligned ? TileInfo{256, 128, 256, 2, 1.00f, 0.95f} : TileInfo{256, 256, 512, 1, 1.00f, 1.00f};
+    case TILE_MEDIUM: return {128, 128, 256, aligned ? 4 : 2, aligned ? 1.00f : 0.80f, aligned ? 0.88f : 0.72f};
     default:
         if (aligned && N <= kNarrowN) return {128, 32, 256, 4, 0.96f, 0.667f};
         return { 64,  64, 256, aligned ? 5 : 2, aligned ? 0.96f : 0.70f, aligned ? 0.667f : 0.49f};
@@ -132,20 +136,20 @@ __host__ inline TileInfo tile_info_f32(int shape, bool aligned = true, uint32_t 
 __host__ inline TileInfo tile_info_f16(int shape, bool aligned = true)
 {
     switch (shape) {
-    case TILE_256x256: return {256, 256, aligned ? 512 : 256, 1, 1.00f, aligned ? 1.38f : 1.00f};
-    case TILE_128x128: return {128, 128, aligned ? 512 : 128, 2, aligned ? 0.84f : 0.60f, aligned ? 0.70f : 0.50f};
+    case TILE_LARGE: return {256, 256, aligned ? 512 : 256, 1, 1.00f, aligned ? 1.38f : 1.00f};
+    case TILE_MEDIUM: return {128, 128, aligned ? 512 : 128, 2, aligned ? 0.84f : 0.60f, aligned ? 0.70f : 0.50f};
     default:           return { 64,  64, aligned ? 256 :  64, aligned ? 4 : 2, aligned ? 0.55f : 0.25f, aligned ? 0.27f : 0.12f};
     }
 }
 
-// fp64 (TFLOP/s per CU): 256 x 128 (what TILE_256x256 stands for) 0.283 alone or full; 128 x 128 0.27 alone or two per
+// fp64 (TFLOP/s per CU): 256 x 128 (what TILE_LARGE stands for) 0.283 alone or full; 128 x 128 0.27 alone or two per
 // CU; 64 x 64 0.22 alone (1024^3), 0.27 two per CU (3072^3).  All three run 8 wavefronts per workgroup: with 4, the
 // two smaller tiles reach 0.24 (their accumulators leave no room for the four workgroups per CU that the fp32 tiles use).
 __host__ inline TileInfo tile_info_f64(int shape)
 {
     switch (shape) {
-    case TILE_256x256: return {256, 128, 512, 1, 1.00f, 1.00f};
-    case TILE_128x128: return {128, 128, 512, 2, 0.96f, 0.96f};
+    case TILE_LARGE: return {256, 128, 512, 1, 1.00f, 1.00f};
+    case TILE_MEDIUM: return {128, 128, 512, 2, 0.96f, 0.96f};
     default:           return { 64,  64, 512, 2, 0.95f, 0.77f};
     }
 }

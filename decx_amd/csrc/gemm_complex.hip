@@ -21,7 +21,9 @@ template <typename T>
 __global__ void __launch_bounds__(256) complex_expand_b_kernel(const T* __restrict__ B, T* __restrict__ Bx, uint32_t K, uint32_t N,
                                                                uint32_t ldb, uint32_t ldx, T ar, T ai)
 {
-    const uint32_t n = blockIdx.x * 64 + (threadIdx.x & 63), k = blockIdx.y * 4 + (threadIdx.x >> 6);
+    // 64 columns x 4 rows per workgroup on a 1-D grid (grid.y would cap the rows at 4 x 65 535)
+    const uint32_t cols = (N + 63) / 64;
+    const uint32_t n = (blockIdx.x % cols) * 64 + (threadIdx.x & 63), k = (blockIdx.x / cols) * 4 + (threadIdx.x >> 6);
     if (n >= N || k >= K) return;
     const T br = B[((size_t)k * ldb + n) * 2], bi = B[((size_t)k * ldb + n) * 2 + 1];
     const T re = ar * br - ai * bi, im = ar * bi + ai * br;
@@ -36,7 +38,8 @@ template <typename T>
 __global__ void __launch_bounds__(256) complex_scale_kernel(const T* __restrict__ C, T* __restrict__ D, uint32_t M, uint32_t N,
                                                             uint32_t ldc, uint32_t ldd, T br, T bi)
 {
-    const uint32_t n = blockIdx.x * 64 + (threadIdx.x & 63), m = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const uint32_t cols = (N + 63) / 64;
+    const uint32_t n = (blockIdx.x % cols) * 64 + (threadIdx.x & 63), m = (blockIdx.x / cols) * 4 + (threadIdx.x >> 6);
     if (n >= N || m >= M) return;
     const T cr = C[((size_t)m * ldc + n) * 2], ci = C[((size_t)m * ldc + n) * 2 + 1];
     D[((size_t)m * ldd + n) * 2] = br * cr - bi * ci;
@@ -48,13 +51,17 @@ __global__ void __launch_bounds__(256) complex_scale_kernel(const T* __restrict_
 template <typename T>
 int launch_complex_expand_b(const T* B, T* Bx, uint32_t K, uint32_t N, uint32_t ldb, uint32_t ldx, T ar, T ai, hipStream_t stream)
 {
-    hipLaunchKernelGGL((complex_expand_b_kernel<T>), dim3((N + 63) / 64, (K + 3) / 4), dim3(256), 0, stream, B, Bx, K, N, ldb, ldx, ar, ai);
+    const uint64_t blocks = (uint64_t)((N + 63) / 64) * ((K + 3) / 4);
+    if (blocks > 0x7fffffffull) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL((complex_expand_b_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, B, Bx, K, N, ldb, ldx, ar, ai);
     return (int)hipGetLastError();
 }
 template <typename T>
 int launch_complex_scale(const T* C, T* D, uint32_t M, uint32_t N, uint32_t ldc, uint32_t ldd, T br, T bi, hipStream_t stream)
 {
-    hipLaunchKernelGGL((complex_scale_kernel<T>), dim3((N + 63) / 64, (M + 3) / 4), dim3(256), 0, stream, C, D, M, N, ldc, ldd, br, bi);
+    const uint64_t blocks = (uint64_t)((N + 63) / 64) * ((M + 3) / 4);
+    if (blocks > 0x7fffffffull) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL((complex_scale_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, C, D, M, N, ldc, ldd, br, bi);
     return (int)hipGetLastError();
 }
 

@@ -222,7 +222,6 @@ static int launch_shape(const GemmArgs& args, hipStream_t stream)
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
-    g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
     hipLaunchKernelGGL((gemm_f16_kernel<BM, BN, BK, WAVES_M, WAVES_N>), dim3(nb), dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
     return (int)hipGetLastError();
 }
@@ -231,9 +230,9 @@ int launch_gemm_f16(int shape, bool edge, const GemmArgs& args, hipStream_t stre
 {
     if (!edge && args.vec_ok && args.K > 0 && dma_offsets_fit(args, 2)) return launch_gemm_f16_dma(shape, args, stream);
     switch (shape) {
-    case TILE_256x256: return launch_shape<256, 256, 64, 2, 2>(args, stream);
-    case TILE_128x128: return launch_shape<128, 128, 64, 2, 1>(args, stream);
-    case TILE_64x64:   return launch_shape< 64,  64, 64, 1, 1>(args, stream);
+    case TILE_LARGE: return launch_shape<256, 256, 64, 2, 2>(args, stream);
+    case TILE_MEDIUM: return launch_shape<128, 128, 64, 2, 1>(args, stream);
+    case TILE_SMALL:   return launch_shape< 64,  64, 64, 1, 1>(args, stream);
     default:           return (int)hipErrorInvalidValue;
     }
 }

@@ -395,7 +395,6 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
-    g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
     if (g.split_len) {
         const uint32_t splits = (g.K + g.split_len - 1) / g.split_len;
         hipLaunchKernelGGL((gemm_f16_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, true>), dim3(nb, splits),
@@ -423,13 +422,13 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
 int launch_gemm_f16_dma(int shape, const GemmArgs& args, hipStream_t stream)
 {
     switch (shape) {
-    case TILE_256x256: return launch_dma<256, 256, 2, 4, 64, 2>(args, stream);
-    case TILE_128x128: {
+    case TILE_LARGE: return launch_dma<256, 256, 2, 4, 64, 2>(args, stream);
+    case TILE_MEDIUM: {
         const uint64_t blocks = (uint64_t)((args.M + 127) / 128) * ((args.N + 127) / 128);
         return blocks <= 256 ? launch_dma<128, 128, 2, 4, 64, 4>(args, stream)
                              : launch_dma<128, 128, 2, 4, 64, 2>(args, stream);
     }
-    case TILE_64x64: {
+    case TILE_SMALL: {
         const uint64_t blocks = (uint64_t)((args.M + 63) / 64) * ((args.N + 63) / 64);
         return blocks <= 512 ? launch_dma<64, 64, 2, 2, 64, 4>(args, stream)
                              : launch_dma<64, 64, 2, 2, 64, 2>(args, stream);

@@ -249,7 +249,6 @@ static int launch_shape(const GemmArgs& args, hipStream_t stream)
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
-    g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
     hipLaunchKernelGGL((gemm_f32_kernel<BM, BN, BK, WAVES_M, WAVES_N>), dim3(nb), dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
     return (int)hipGetLastError();
 }
@@ -258,9 +257,9 @@ int launch_gemm_f32(int shape, bool edge, const GemmArgs& args, hipStream_t stre
 {
     if (!edge && args.vec_ok && args.K > 0 && dma_offsets_fit(args, 4)) return launch_gemm_f32_dma(shape, args, stream);
     switch (shape) {
-    case TILE_256x256: return launch_shape<256, 256, 16, 4, 2>(args, stream);
-    case TILE_128x128: return launch_shape<128, 128, 16, 2, 2>(args, stream);
-    case TILE_64x64:   return launch_shape< 64,  64, 16, 2, 2>(args, stream);
+    case TILE_LARGE: return launch_shape<256, 256, 16, 4, 2>(args, stream);
+    case TILE_MEDIUM: return launch_shape<128, 128, 16, 2, 2>(args, stream);
+    case TILE_SMALL:   return launch_shape< 64,  64, 16, 2, 2>(args, stream);
     default:           return (int)hipErrorInvalidValue;
     }
 }

@@ -494,7 +494,6 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
-    g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
     // 256 x 128 tiles, two independent workgroups per CU: patches two tile-rows high fetch least (8192^3: 5.5 GB through
     // L2 against 6.2 GB with four rows and 11.7 GB with eight, at the same speed)
     if constexpr (BM == 256 && BN == 128 && CONV == 0) g.group_m = 2;
@@ -514,7 +513,7 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
 }  // namespace
 
 // M, N, K >= 1; 16-byte aligned bases and pitches (the caller checks).  Measured on MI355X:
-//   256 x 128 (TILE_256x256, the largest tile): 4 wavefronts of 128 x 64, 16-deep slabs in a ring of 2, two workgroups
+//   256 x 128 (TILE_LARGE, the largest tile): 4 wavefronts of 128 x 64, 16-deep slabs in a ring of 2, two workgroups
 //     per CU, each with its own slab barrier: 149.3 TFLOP/s at 8192^3.  One 256 x 256 workgroup of 8 such wavefronts
 //     per CU (ring of 4) reaches 147.7-148.4 and leaves more of the chip idle on grids that are no multiple of the
 //     CU count (6144^3: 110 against 133); with 64 x 128 wave tiles, 16 wavefronts, 32-deep slabs or rings of 3 to
@@ -527,9 +526,9 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
 int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
 {
     switch (shape) {
-    case TILE_256x256: return launch_dma<256, 128, 2, 2, 16, 2, false>(args, stream);
-    case TILE_128x128: return launch_dma<128, 128, 2, 2, 16, 2, true>(args, stream);
-    case TILE_64x64:                                           // outputs of at most 32 columns: 128 x 32 tiles, no idle half
+    case TILE_LARGE: return launch_dma<256, 128, 2, 2, 16, 2, false>(args, stream);
+    case TILE_MEDIUM: return launch_dma<128, 128, 2, 2, 16, 2, true>(args, stream);
+    case TILE_SMALL:                                           // outputs of at most 32 columns: 128 x 32 tiles, no idle half
         return args.N <= kNarrowN ? launch_dma<128, 32, 4, 1, 32, 2, true>(args, stream)
                                   : launch_dma< 64, 64, 2, 2, 32, 2, true>(args, stream);
     default:           return (int)hipErrorInvalidValue;
@@ -556,14 +555,14 @@ int launch_conv2d_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
 {
     // runs that are a whole number of slabs (e.g. 3 x 112 channels: 21 slabs of 16 floats) let all copy lanes hop
     // together; image_bytes bounds the lanes' 32-bit offsets
-    const uint32_t slab_bytes = (shape == TILE_64x64 ? 32u : 16u) * 4u;
+    const uint32_t slab_bytes = (shape == TILE_SMALL ? 32u : 16u) * 4u;
     const bool uniform = args.conv_seg_bytes % slab_bytes == 0 && args.conv_image_bytes < (1ull << 31);
     switch (shape) {
-    case TILE_256x256: return uniform ? launch_dma<256, 256, 2, 4, 16, 4, false, 2>(args, stream)     // 137 TFLOP/s on the 3 x 3 x 112 workload; 256 x 128: 136
+    case TILE_LARGE: return uniform ? launch_dma<256, 256, 2, 4, 16, 4, false, 2>(args, stream)     // 137 TFLOP/s on the 3 x 3 x 112 workload; 256 x 128: 136
                                       : launch_dma<256, 256, 2, 4, 16, 4, false, 1>(args, stream);
-    case TILE_128x128: return uniform ? launch_dma<128, 128, 2, 2, 16, 2, true, 2>(args, stream)
+    case TILE_MEDIUM: return uniform ? launch_dma<128, 128, 2, 2, 16, 2, true, 2>(args, stream)
                                       : launch_dma<128, 128, 2, 2, 16, 2, true, 1>(args, stream);
-    case TILE_64x64:
+    case TILE_SMALL:
         if (args.N <= kNarrowN)                                // at most 32 kernels, all the reference's own path takes
             return uniform ? launch_dma<128, 32, 4, 1, 32, 2, true, 2>(args, stream)
                            : launch_dma<128, 32, 4, 1, 32, 2, true, 1>(args, stream);

@@ -311,7 +311,9 @@ gemm_f64_dma_kernel(const GemmArgs g_in)
 // One thread per output element, k ascending: any alignment, any K (also 0).
 __global__ void __launch_bounds__(256) gemm_f64_plain_kernel(const GemmArgs g)
 {
-    const uint32_t col = blockIdx.x * 16 + (threadIdx.x & 15), row = blockIdx.y * 16 + (threadIdx.x >> 4);
+    // tiles of 16 x 16 outputs on a 1-D grid (neither dimension is bound by the 65 535 blocks of grid.y)
+    const uint32_t tiles_n = (g.N + 15) / 16;
+    const uint32_t col = (blockIdx.x % tiles_n) * 16 + (threadIdx.x & 15), row = (blockIdx.x / tiles_n) * 16 + (threadIdx.x >> 4);
     if (row >= g.M || col >= g.N) return;
     const double* a = (const double*)g.A + (size_t)row * g.lda;
     const double* b = (const double*)g.B + col;
@@ -330,7 +332,6 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
-    g.xcd_remap = (nb % kXcds == 0) ? 1u : 0u;
     if (g.split_len) {
         const uint32_t splits = (g.K + g.split_len - 1) / g.split_len;
         hipLaunchKernelGGL((gemm_f64_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, true>), dim3(nb, splits),
@@ -344,20 +345,21 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
 
 }  // namespace
 
-// shape: TILE_256x256 stands for the largest fp64 tile, 256 x 128 (eight wavefronts of 64 x 64).  The smaller tiles
+// shape: TILE_LARGE stands for the largest fp64 tile, 256 x 128 (eight wavefronts of 64 x 64).  The smaller tiles
 // run eight wavefronts too (128 x 128: 64 x 32 each, 64 x 64: 16 x 32 each): measured 70 against 61 TFLOP/s at
 // 2048^3 and 56 against 50 at 1024^3 with four.
 int launch_gemm_f64(int shape, bool plain, const GemmArgs& args, hipStream_t stream)
 {
     if (plain || !args.vec_ok || args.K == 0 || !dma_offsets_fit(args, 8)) {
-        const dim3 grid((args.N + 15) / 16, (args.M + 15) / 16);
-        hipLaunchKernelGGL(gemm_f64_plain_kernel, grid, dim3(256), 0, stream, args);
+        const uint64_t tiles = (uint64_t)((args.N + 15) / 16) * ((args.M + 15) / 16);
+        if (tiles > 0x7fffffffull) return (int)hipErrorInvalidValue;
+        hipLaunchKernelGGL(gemm_f64_plain_kernel, dim3((unsigned)tiles), dim3(256), 0, stream, args);
         return (int)hipGetLastError();
     }
     switch (shape) {
-    case TILE_256x256: return launch_dma<256, 128, 4, 2, 16, 3>(args, stream);
-    case TILE_128x128: return launch_dma<128, 128, 2, 4, 16, 2>(args, stream);
-    case TILE_64x64:   return launch_dma< 64,  64, 4, 2, 16, 4>(args, stream);
+    case TILE_LARGE: return launch_dma<256, 128, 4, 2, 16, 3>(args, stream);
+    case TILE_MEDIUM: return launch_dma<128, 128, 2, 4, 16, 2>(args, stream);
+    case TILE_SMALL:   return launch_dma< 64,  64, 4, 2, 16, 4>(args, stream);
     default:           return (int)hipErrorInvalidValue;
     }
 }

@@ -9,7 +9,7 @@ import numpy as np
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "lib", "libdecx_hip.so")
 
-TILE_AUTO, TILE_256, TILE_128, TILE_64, PATH_GEMV, PATH_GEVM = -1, 0, 1, 2, 16, 17
+TILE_AUTO, TILE_LARGE, TILE_MEDIUM, TILE_SMALL, PATH_GEMV, PATH_GEVM = -1, 0, 1, 2, 16, 17
 
 _vp = ctypes.c_void_p
 _u32 = ctypes.c_uint32
@@ -274,7 +274,7 @@ def _align(v, a):
     return (v + a - 1) // a * a
 
 
-def conv2d(image, kernels, stride_x=1, stride_y=1, extend=False, stream=None, pad_value=np.nan):
+def conv2d(image, kernels, stride_x=1, stride_y=1, extend=False, stream=None, pad_value=np.nan, channel_pad_value=0.0):
     """dst[oy][ox][oc] = sum image[oy*sy+kh][ox*sx+kw][ic] * kernels[oc][kh][kw][ic] through decx_hip_conv2d_f32_depth.
     image [H][W][C], kernels [OC][KH][KW][C] (numpy fp32).  Device layouts follow the original's device tensors:
     channel pitch = C rounded up to 4, row pitch = W rounded up to 8 columns; unused columns hold `pad_value`,
@@ -296,7 +296,7 @@ def conv2d(image, kernels, stride_x=1, stride_y=1, extend=False, stream=None, pa
         PH, PW, host_img = H, W, image
     wp = _align(PW, 8)
     raw = np.full((PH, wp, dp), pad_value, np.float32)
-    raw[:, :PW, :] = 0
+    raw[:, :PW, :] = channel_pad_value
     raw[:, :PW, :C] = host_img
     d_img = DeviceMatrix(PH, wp * dp, np.float32, data=raw.reshape(PH, wp * dp))
     kdp, kwp = _align(C, 4), _align(KW, 8)

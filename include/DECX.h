@@ -19,8 +19,10 @@
  * it is part of the API's spelling; everything behind it is HIP on gfx950, reached
  * through the C ABI in decx_hip.h.
  *
- * Not provided here: de::blas::cpu::GEMM (the CPU path is not part of this module), and
- * the vector / tensor containers, which the matrix product does not use.
+ * Further down: the vector containers and the vector x matrix forms (de::Vector, de::GPU_Vector,
+ * srcs/includes/DECX/classes/Vector.h, GPU_Vector.h, BLAS.h:79-80) and the tensor containers with
+ * de::nn::cuda::Conv2D (Tensor.h, GPU_Tensor.h, TensorArray.h, BLAS.h:109-110), which call the same kernels.
+ * Not provided here: de::blas::cpu::GEMM (the CPU path is not part of this module).
  */
 #ifndef DECX_AMD_PUBLIC_H_
 #define DECX_AMD_PUBLIC_H_

@@ -48,17 +48,18 @@ typedef struct decx_hip_device_props {
     uint64_t global_mem_bytes;
 } decx_hip_device_props;
 
-/* Tile shapes the planner chooses between (block tile BM x BN).  DECX_HIP_TILE_256x256 is the largest tile of
- * the element type: 256 x 256 in fp16, 256 x 128 in fp32 on 16-byte aligned operands (256 x 256 otherwise) and
- * in fp64.  DECX_HIP_TILE_64x64 is the smallest: 64 x 64, or 128 x 32 for aligned fp32 outputs of at most 32
- * columns (all the kernel counts the reference's convolution takes).  decx_hip_gemm_plan reports the actual BM x BN. */
+/* Tile size classes the planner chooses between.  The block tile BM x BN a class stands for depends on the element
+ * type: DECX_HIP_TILE_LARGE is 256 x 256 in fp16, 256 x 128 in fp32 on 16-byte aligned operands (256 x 256 otherwise)
+ * and in fp64; DECX_HIP_TILE_MEDIUM is 128 x 128; DECX_HIP_TILE_SMALL is 64 x 64, or 128 x 32 for aligned fp32
+ * outputs of at most 32 columns (all the kernel counts the reference's convolution takes).  decx_hip_gemm_plan
+ * reports the actual BM x BN. */
 enum {
-    DECX_HIP_TILE_AUTO    = -1,
-    DECX_HIP_TILE_256x256 = 0,
-    DECX_HIP_TILE_128x128 = 1,
-    DECX_HIP_TILE_64x64   = 2,
-    DECX_HIP_PATH_GEMV    = 16,    /* N == 1: bandwidth-bound row-dot kernel */
-    DECX_HIP_PATH_GEVM    = 17     /* M == 1: bandwidth-bound column-sum kernel */
+    DECX_HIP_TILE_AUTO   = -1,
+    DECX_HIP_TILE_LARGE  = 0,
+    DECX_HIP_TILE_MEDIUM = 1,
+    DECX_HIP_TILE_SMALL  = 2,
+    DECX_HIP_PATH_GEMV   = 16,    /* N == 1: bandwidth-bound row-dot kernel */
+    DECX_HIP_PATH_GEVM   = 17     /* M == 1: bandwidth-bound column-sum kernel */
 };
 
 typedef struct decx_hip_plan {
@@ -281,7 +282,7 @@ DECX_HIP_API int decx_hip_gemm_f16_tile(const uint16_t* A, const uint16_t* B, co
                                         uint32_t M, uint32_t N, uint32_t K,
                                         uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
                                         float alpha, float beta, void* stream, int tile, int force_edge);
-/* fp64: DECX_HIP_TILE_256x256 selects the largest fp64 tile (256 x 128); force_plain != 0 forces the
+/* fp64: DECX_HIP_TILE_LARGE selects the largest fp64 tile (256 x 128); force_plain != 0 forces the
  * one-thread-per-element kernel. */
 DECX_HIP_API int decx_hip_gemm_f64_tile(const double* A, const double* B, const double* C, double* D,
                                         uint32_t M, uint32_t N, uint32_t K,
@@ -294,12 +295,6 @@ DECX_HIP_API int decx_hip_gemm_f64_tile(const double* A, const double* B, const 
  * Works without a GPU: before decx_hip_init() it assumes 256 compute units. */
 DECX_HIP_API int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int aligned,
                                     decx_hip_plan* out);
-
-/* A plain device-to-device copy kernel (128-bit loads and stores, `bytes` a multiple of 16,
- * both pointers 16-byte aligned).  It has no counterpart in the reference: it exists so that
- * hardware traffic counters can be scaled against a launch whose HBM traffic is known
- * (reads = writes = `bytes`). */
-DECX_HIP_API int decx_hip_calibration_copy(void* dst, const void* src, size_t bytes, void* stream);
 
 /* IEEE binary16 <-> binary32, round to nearest even; host-side helpers behind
  * de::Float2Half / de::Half2Float (srcs/common/FP16/float_half_convert.cu:35-46). */

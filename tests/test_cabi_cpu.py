@@ -59,7 +59,7 @@ def test_planner_choices():
     for eb, (M, N, K) in [(4, (8192, 8192, 8192)), (2, (4096, 4096, 4096)), (4, (65536, 256, 1024))]:
         p = hip.plan(eb, M, N, K)
         # the largest tile: 256 x 128 in fp32 (two workgroups per CU), 256 x 256 in fp16
-        assert (p.path, p.edge, p.tile_m, p.tile_n) == (hip.TILE_256, 0, 256, 128 if eb == 4 else 256)
+        assert (p.path, p.edge, p.tile_m, p.tile_n) == (hip.TILE_LARGE, 0, 256, 128 if eb == 4 else 256)
         assert p.grid == (M // p.tile_m) * (N // p.tile_n)
     assert hip.plan(4, 8192, 8192, 8192, aligned=False).tile_n == 256     # the register-staged family keeps 256 x 256
     # small and ragged problems take smaller tiles so the chip fills; they stay on the direct-to-LDS
@@ -149,3 +149,25 @@ def test_error_strings():
     assert L.decx_hip_error_string(0) == b"success"
     assert b"invalid argument" in L.decx_hip_error_string(-1)
     assert L.decx_hip_error_string(-99) == b"unknown error"
+
+
+def test_device_pass_applies_the_no_packed_fp32_switch(tmp_path):
+    """The build's feature switch keeps packed-fp32 VALU forms out of gfx950 code: the same float2 multiply-add
+    compiles to v_pk_fma_f32 without it and to scalar fmas with it (the host pass, which warns that it does not know
+    the feature, is not what is compiled here)."""
+    import subprocess
+    from decx_amd import build
+    src = tmp_path / "pk.hip"
+    src.write_text("#include <hip/hip_runtime.h>\n"
+                   "__global__ void k(float2* a, const float2* b, const float2* c) { const int i = threadIdx.x;\n"
+                   "  const float2 x = b[i], y = c[i], z = a[i]; a[i] = make_float2(x.x * y.x + z.x, x.y * y.y + z.y); }\n")
+    def asm(flags):
+        out = tmp_path / "pk.s"
+        subprocess.run([build.HIPCC, "--offload-arch=gfx950", "-O3", "--cuda-device-only", "-S", str(src), "-o", str(out)] + flags,
+                       check=True, capture_output=True)
+        return out.read_text()
+    switch = [f for f in build.HIP_FLAGS if f in ("-Xclang", "-target-feature", "-packed-fp32-ops")]
+    assert switch == ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+    assert "v_pk_fma_f32" in asm([])
+    with_switch = asm(switch)
+    assert "v_pk_" not in with_switch and "v_fma_f32" in with_switch

@@ -93,3 +93,17 @@ def test_conv2d_invalid_arguments(hip):
     # the same call with the number of channels that exist: 1 .. the channel pitch
     withdepth = lambda depth: L.decx_hip_conv2d_f32_depth(d.ptr, d.ptr, d.ptr, 2, 2, 4, 3, 3, depth, 4, 8, 1, 1, 4, 4, 8, None)
     assert withdepth(3) == 0 and withdepth(4) == 0 and withdepth(0) == -1 and withdepth(5) == -1
+
+
+@pytest.mark.parametrize("C", [1, 2, 3])
+@pytest.mark.parametrize("extend", [False, True])
+def test_padding_channel_of_grey_and_rgb_images_is_never_read_into_a_result(hip, oracle, C, extend):
+    """Channel pitch 4 with 1 to 3 real channels and few kernels: the lane-per-pixel kernel leaves the padding
+    channels out of its arithmetic, so NaN in them must not reach the output (the GEMM form would multiply them by
+    zero weights: NaN)."""
+    W, H, OC, KW, KH = 96, 40, 8, 3, 3
+    image, kernels = data(W, H, C, OC, KW, KH, 900 + C)
+    ref = oracle.conv2d_f32(image, kernels, 1, 1, extend)
+    got, _ = hip.conv2d(image, kernels, 1, 1, extend, channel_pad_value=np.nan)
+    assert np.isfinite(got).all(), "a padding channel reached the result"
+    assert rel_err(got, ref, KW * KH * C) <= TOL

@@ -103,3 +103,24 @@ def test_workspace_contract(hip):
     assert L.decx_hip_gemm_c32(*args, ws.ptr, 2 * 4 * 16 * 4 - 1, None) == -1         # workspace too small
     assert L.decx_hip_gemm_c32(*args, None, 1 << 20, None) == -1
     hip.sync()
+
+
+@pytest.mark.parametrize("dtype", [np.complex64, np.complex128])
+def test_k_zero_needs_no_workspace(hip, dtype):
+    """K == 0: D = beta * C (or zero); the workspace query returns 0 and a null workspace is accepted."""
+    L = hip.lib()
+    M, N = 37, 21
+    rng = np.random.default_rng(5)
+    C = (rng.standard_normal((M, N)) + 1j * rng.standard_normal((M, N))).astype(dtype)
+    rb = 4 if dtype == np.complex64 else 8
+    assert L.decx_hip_gemm_complex_workspace(rb, N, 0) == 0
+    dA = hip.DeviceMatrix(M, 1, dtype, 4); dB = hip.DeviceMatrix(1, N, dtype, 24)
+    dC = hip.DeviceMatrix(M, N, dtype, 24, C); dD = hip.DeviceMatrix(M, N, dtype, 24)
+    fn = L.decx_hip_gemm_c32 if rb == 4 else L.decx_hip_gemm_c64
+    hip.check(fn(dA.ptr, dB.ptr, dC.ptr, dD.ptr, M, N, 0, 4, 24, 24, 24, 1.0, 0.0, 0.5, -2.0, None, 0, None), "complex K = 0")
+    hip.sync()
+    want = (C.astype(np.complex128) * (0.5 - 2.0j))
+    assert np.max(np.abs(dD.download() - want)) <= 1e-5 * np.max(np.abs(want))
+    hip.check(fn(dA.ptr, dB.ptr, None, dD.ptr, M, N, 0, 4, 24, 0, 24, 1.0, 0.0, 1.0, 0.0, None, 0, None), "complex K = 0, no C")
+    hip.sync()
+    assert np.all(dD.download() == 0)

@@ -372,3 +372,17 @@ def test_reference_accumulate_form_agrees_on_the_rows_it_gets_right(oracle):
         pytest.skip("the reference's accumulate form crashed in this process (it does so intermittently)")
     want = oracle.gemm_f32(A, B, C)
     assert np.array_equal(bits(D[::8]), bits(want[::8]))
+
+
+def test_port_clock_tracks_the_compiled_reference(oracle):
+    """The AVX2 restatement is what the benchmark times as the CPU baseline on the GPU box: on this host, at 8
+    threads, its best call must be bit-equal to the compiled reference's and take about as long (within 15 % on a
+    quiet machine; the bound here leaves room for a shared one)."""
+    _need_reference(oracle)
+    from oracle import time_port_vs_reference as t
+    rows = t.measure(threads=8, repeats=5)
+    for r in rows:
+        if r["reference_ms"] is None:
+            pytest.skip("the compiled reference crashed in every child process")
+        assert r["bit_equal"], r
+        assert 0.6 <= r["port_over_reference"] <= 1.6, r
