@@ -5,6 +5,7 @@
 #include "gemm_common.hpp"
 
 #include <cstring>
+#include <mutex>
 
 using namespace decx_hip;
 
@@ -26,6 +27,27 @@ constexpr size_t kScratchBytes = (size_t)DECX_HIP_STATIC_WORKSPACE_BYTES;
 constexpr int kMaxDevices = 16;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 void* g_scratch[kMaxDevices] = {};
+
+// Tile counters of the fp32 split-K kernels (one per tile; the workgroups of a tile count themselves in, the last
+// one sums the tile and puts its counter back to zero, so the array is all zero between launches).  Every launch
+// takes the next window of the array, so that launches in flight on different streams do not share counters as
+// long as their windows together stay below kSplitCounters.
+constexpr uint32_t kSplitCounters = 1u << 16;
+static __device__ uint32_t split_counters[kSplitCounters];
+uint32_t* g_split_counters[kMaxDevices] = {};
+std::mutex g_counter_mutex;
+uint32_t g_counter_cursor = 0;
+
+uint32_t* take_split_counters(uint32_t tiles)
+{
+    uint32_t* const base = g_dev.device >= 0 && g_dev.device < kMaxDevices ? g_split_counters[g_dev.device] : nullptr;
+    if (!base || tiles > kSplitCounters) return nullptr;
+    std::lock_guard<std::mutex> lock(g_counter_mutex);
+    if (g_counter_cursor + tiles > kSplitCounters) g_counter_cursor = 0;
+    uint32_t* const window = base + g_counter_cursor;
+    g_counter_cursor += tiles;
+    return window;
+}
 
 inline int hip_rc(hipError_t e) { return (int)e; }
 inline hipStream_t as_stream(void* s) { return (hipStream_t)s; }
@@ -146,16 +168,36 @@ SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
     return {shape, 1, 0};
 }
 
+// Bytes of workspace a split of `splits` ranges needs.  fp32: one slot of BM x BN floats per workgroup (the tiles of
+// the shape the split runs on); fp16 / fp64: `splits` partial products of M rows at a pitch of N rounded up to 4.
+size_t split_workspace_bytes(int elem_bytes, int shape, uint32_t M, uint32_t N, uint32_t splits)
+{
+    if (elem_bytes == 4) {
+        const TileInfo ti = tile_info_f32(shape, true, N);
+        const uint64_t tiles = (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
+        return (size_t)(tiles * splits * (uint64_t)(ti.bm * ti.bn) * 4u);
+    }
+    return (size_t)splits * M * ((N + 3) / 4 * 4) * (size_t)(elem_bytes == 8 ? 8 : 4);
+}
+
 // Fills the split fields of g when the plan says so and the workspace is large enough; returns the number of splits
 // and, with more than one, the tile shape they run on.
 uint32_t arm_split(GemmArgs& g, int elem_bytes, void* workspace, size_t workspace_bytes, int& shape)
 {
     if (!workspace || !aligned16(workspace)) return 1;
     const SplitChoice sp = split_plan(elem_bytes, g.M, g.N, g.K);
-    const uint32_t ldw = (g.N + 3) / 4 * 4;
-    const size_t part = (size_t)(elem_bytes == 8 ? 8 : 4);
-    if (sp.splits <= 1 || workspace_bytes < (size_t)sp.splits * g.M * ldw * part) return 1;
-    g.split_len = sp.len; g.split_ldd = ldw; g.split_stride = (uint64_t)g.M * ldw; g.split_ws = workspace;
+    if (sp.splits <= 1 || workspace_bytes < split_workspace_bytes(elem_bytes, sp.shape, g.M, g.N, sp.splits)) return 1;
+    if (elem_bytes == 4) {                                      // one kernel: slots and tile counters
+        const TileInfo ti = tile_info_f32(sp.shape, true, g.N);
+        const uint64_t tiles = (uint64_t)((g.M + ti.bm - 1) / ti.bm) * ((g.N + ti.bn - 1) / ti.bn);
+        uint32_t* const counters = tiles <= kSplitCounters ? take_split_counters((uint32_t)tiles) : nullptr;
+        if (!counters) return 1;
+        g.split_counters = counters;
+    } else {
+        const uint32_t ldw = (g.N + 3) / 4 * 4;
+        g.split_ldd = ldw; g.split_stride = (uint64_t)g.M * ldw;
+    }
+    g.split_len = sp.len; g.split_ws = workspace;
     shape = sp.shape;
     return sp.splits;
 }
@@ -219,8 +261,9 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
     if (workspace && tile == DECX_HIP_TILE_AUTO && !edge && g.vec_ok && dma_offsets_fit(g, F16 ? 2 : 4)) {
         const uint32_t splits = arm_split(g, F16 ? 2 : 4, workspace, workspace_bytes, shape);
         if (splits > 1) {
-            const int rl = F16 ? launch_gemm_f16(shape, false, g, as_stream(stream)) : launch_gemm_f32(shape, false, g, as_stream(stream));
-            return rl != 0 ? rl : launch_split_reduce(F16 ? 2 : 4, g, splits, as_stream(stream));
+            if (!F16) return launch_gemm_f32(shape, false, g, as_stream(stream));       // the last workgroup of a tile sums it
+            const int rl = launch_gemm_f16(shape, false, g, as_stream(stream));
+            return rl != 0 ? rl : launch_split_reduce(2, g, splits, as_stream(stream));
         }
     }
     return F16 ? launch_gemm_f16(shape, edge, g, as_stream(stream))
@@ -279,6 +322,11 @@ int decx_hip_init(int device)
         void* p = nullptr;
         if ((e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) != hipSuccess) return hip_rc(e);
         g_scratch[device] = p;
+    }
+    if (device < kMaxDevices && !g_split_counters[device]) {
+        void* p = nullptr;
+        if ((e = hipGetSymbolAddress(&p, HIP_SYMBOL(split_counters))) != hipSuccess) return hip_rc(e);
+        g_split_counters[device] = (uint32_t*)p;
     }
     g_dev.device = device;
     g_dev.compute_units = g_dev.prop.multiProcessorCount > 0 ? g_dev.prop.multiProcessorCount : 256;
@@ -404,7 +452,7 @@ size_t decx_hip_gemm_workspace(int elem_bytes, uint32_t M, uint32_t N, uint32_t 
         return sp.splits > 1 ? (size_t)sp.splits * ((N + 3) / 4 * 4) * (elem_bytes == 8 ? 8 : 4) : 0;
     }
     const SplitChoice sp = split_plan(elem_bytes, M, N, K);
-    return sp.splits > 1 ? (size_t)sp.splits * M * ((N + 3) / 4 * 4) * (elem_bytes == 8 ? 8 : 4) : 0;
+    return sp.splits > 1 ? split_workspace_bytes(elem_bytes, sp.shape, M, N, sp.splits) : 0;
 }
 
 size_t decx_hip_gemm_f32_workspace(uint32_t M, uint32_t N, uint32_t K) { return decx_hip_gemm_workspace(4, M, N, K); }

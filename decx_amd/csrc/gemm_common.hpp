@@ -29,14 +29,17 @@ struct GemmArgs {
     uint32_t tiles_m, tiles_n;   // number of block tiles along M and N
     uint32_t vec_ok;             // 1: every base pointer is 16-byte aligned and every pitch a multiple of 16 bytes
     // Split K (direct-load kernels, grid.y = number of splits): split z multiplies k in [z * split_len,
-    // min(K, (z + 1) * split_len)) and writes its M x N partial product (fp32 for fp32 and fp16 operands, fp64
-    // for fp64), pitch split_ldd, to split_ws + z * split_stride elements; a second kernel adds the partial
-    // products in split order.
+    // min(K, (z + 1) * split_len)).  fp16 and fp64: it writes its M x N partial product (fp32 for fp16 operands),
+    // pitch split_ldd, to split_ws + z * split_stride elements, and a second kernel adds the partial products in
+    // split order.  fp32: every workgroup stores its accumulators to its slot of split_ws and counts itself in at
+    // split_counters[tile]; the one that arrives last adds all slots of the tile in split order (its own included,
+    // so the result does not depend on who is last), writes D and puts the counter back to zero.
     uint32_t group_m;            // tile-rows per L2 patch of the block -> tile map (0: the default, kGroupM)
     uint32_t split_len;          // 0: no split
     uint32_t split_ldd;
     uint64_t split_stride;
     void*    split_ws;
+    uint32_t* split_counters;    // one per tile, zero before and after every launch
     // Convolution as an implicit GEMM (used by the CONV instantiations only): row p of the A operand is the
     // patch under output pixel (p / conv_wout, p % conv_wout) of an image stored [row][column][channel]; its K
     // elements are KH runs of conv_seg_bytes contiguous bytes (KW columns x channel pitch), conv_seg_stride bytes

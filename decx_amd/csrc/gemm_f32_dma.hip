@@ -75,7 +75,9 @@ template <int TN> __device__ __forceinline__ float lane_of(const typename BFrag<
 // CONV: 0 plain GEMM; 1 convolution, every copy lane walks the image on its own; 2 convolution whose runs of
 // contiguous bytes are whole slabs, so that all lanes hop to the next image row in the same slab.
 // SPLIT: grid.y workgroups share each tile, each with its own range of K (a separate instantiation, so that the
-// plain kernel keeps reading its arguments straight from the kernel-argument segment).
+// plain kernel keeps reading its arguments straight from the kernel-argument segment).  They meet in the workspace:
+// every workgroup stores its accumulators to its slot and counts itself in at the tile's counter; the last one to
+// arrive adds the slots in range order and runs the epilogue.  No workgroup waits for another.
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, int CONV = 0, bool SPLIT = false>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_f32_dma_kernel(const GemmArgs g_in)
@@ -88,9 +90,6 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
         g_split.A = (const unsigned char*)g_in.A + (size_t)k0 * 4;
         g_split.B = (const unsigned char*)g_in.B + (size_t)k0 * g_in.ldb * 4;
         g_split.K = g_in.K - k0 < g_in.split_len ? g_in.K - k0 : g_in.split_len;
-        g_split.D = (float*)g_in.split_ws + (size_t)blockIdx.y * g_in.split_stride;
-        g_split.ldd = g_in.split_ldd;
-        g_split.C = nullptr;
     }
     const GemmArgs& g = [&]() -> const GemmArgs& { if constexpr (SPLIT) return g_split; else return g_in; }();
     constexpr int WAVES = WAVES_M * WAVES_N;
@@ -406,6 +405,62 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
             if (more) wait_loads_and_barrier<LOADS * (STAGES - 2)>(); else wait_loads_and_barrier<0>();
         }
         multiply_chunk(std::integral_constant<int, CHUNKS - 1>{});
+    }
+
+    if constexpr (SPLIT) {
+        // Every lane's accumulators go to the workgroup's slot, [register][thread]: whole lines per wave.  Slots are
+        // written and read with device-scope accesses (they pass the XCD's own L2, which is not coherent with the other
+        // seven), so that no cache-wide write-back or invalidation is needed around the count -- those would throw out
+        // the operand lines the workgroups still multiplying live on.
+        constexpr int NT = WAVES * 64;
+        const uint32_t splits = gridDim.y;
+        float* const slots = (float*)g.split_ws + (size_t)blockIdx.x * splits * (BM * BN);
+        float* const mine = slots + (size_t)blockIdx.y * (BM * BN);
+        // 16-byte pieces, [piece][thread]; `sc1`: device scope (written through / fetched past this XCD's L2)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const floatx4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                    float* const dst = mine + (size_t)(((i * TN + j) * 4 + q) * NT + t) * 4;
+                    asm volatile("global_store_dwordx4 %0, %1, off sc1" :: "v"(dst), "v"(v) : "memory");
+                }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this lane's stores have arrived
+        __syncthreads();                                   // everyone's have (the ring is free: every LDS read precedes the last slab barrier)
+        uint32_t* const flag = (uint32_t*)lds;
+        if (t == 0) {
+            const uint32_t before = __hip_atomic_fetch_add(g.split_counters + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *flag = (before + 1 == splits) ? 1u : 0u;
+        }
+        __syncthreads();
+        if (__builtin_amdgcn_readfirstlane(*flag) == 0) return;
+        for (uint32_t z = 0; z < splits; ++z) {            // range order, this workgroup's own slot included
+            const float* p = slots + (size_t)z * (BM * BN);
+            floatx4 v[TM][TN][4];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const float* const src = p + (size_t)(((i * TN + j) * 4 + q) * NT + t) * 4;
+                        asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[i][j][q]) : "v"(src) : "memory");
+                    }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        asm volatile("" : "+v"(v[i][j][q]));               // not before the wait above
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = (z == 0) ? v[i][j][q][e] : acc[i][j][4 * q + e] + v[i][j][q][e];
+                    }
+        }
+        if (t == 0) __hip_atomic_store(g.split_counters + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // Epilogue: register r of lane (l32, h) is row 8*(r/4) + 4*h + r%4 of a 32x32 tile; the

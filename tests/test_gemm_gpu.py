@@ -568,3 +568,35 @@ def test_stream_and_events(hip):
     hip.sync(s)
     assert ms > 0 and np.array_equal(dD.download(), A)
     assert L.decx_hip_stream_destroy(s) == 0
+
+
+@pytest.mark.parametrize("M,N,K", [(300, 300, 8192), (1280, 1024, 8192), (1000, 1500, 777)])
+def test_f32_split_k_slots_carry_nothing_from_launch_to_launch(hip, oracle, M, N, K):
+    """The workgroups of a tile meet in the workspace (slots written and read at device scope, a counter per tile
+    that ends every launch at zero).  Two input sets take turns on the same workspace: a slot, a cache line or a
+    counter left over from the launch before would show as a result that differs from the set's first one."""
+    need = hip.lib().decx_hip_gemm_f32_workspace(M, N, K)
+    if need == 0:
+        pytest.skip("the planner does not split this shape")
+    ws = hip.DeviceMatrix(1, need // 4, np.float32)
+    pa, pn = device_pitch(K, np.float32), device_pitch(N, np.float32)
+    sets = []
+    for s in range(2):
+        A = synth.uniform_f32(M, K, 700 + s); B = synth.uniform_f32(K, N, 710 + s)
+        sets.append((A, B, hip.DeviceMatrix(M, K, np.float32, pa, A), hip.DeviceMatrix(K, N, np.float32, pn, B)))
+    dD = hip.DeviceMatrix(M, N, np.float32, pn)
+    first = [None, None]
+    for it in range(60):
+        A, B, dA, dB = sets[it % 2]
+        hip.gemm(dA, dB, dD, workspace=ws)
+        if it % 2 == 1 or it < 2 or it % 7 == 0:             # most launches follow each other without a host round trip
+            hip.sync()
+            got = dD.download()
+            if first[it % 2] is None:
+                first[it % 2] = got
+                rows = np.arange(0, M, max(1, M // 24), dtype=np.uint32)
+                assert rel_err(got[rows], oracle.gemm_f32(A, B, rows=rows), K) <= TOL_F32
+            else:
+                assert np.array_equal(got.view(np.uint32), first[it % 2].view(np.uint32)), "launch %d" % it
+    for d in [ws, dD] + [x for t in sets for x in t[2:]]:
+        d.free()
