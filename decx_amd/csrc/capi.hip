@@ -111,9 +111,13 @@ SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
     // 57 -> 43 us with 128 x 128 tiles on 2 ranges, 768 x 768 x 16384 61 -> 37 (4 ranges); 2048 x 2048 x 8192 and
     // 1024 x 2048 x 4096 gain nothing and stay whole.
     const auto tiles_of = [&](uint32_t b) { return (uint64_t)((M + b - 1) / b) * ((N + b - 1) / b); };
-    if (elem_bytes == 4 && K >= 4096) {
+    if (elem_bytes == 4 && K >= 512) {
         // 64 x 64 tiles, up to five workgroups per CU.  score = (workgroups on the busiest CU / the average) x what a
         // CU loses with m workgroups against a full one; the ranges p that make t * p an even three to five per CU win.
+        // Long K (>= 4096): ranges of at least 1024.  Shorter K: the split costs every tile a trip through the
+        // workspace, which pays only when the tiles alone load the CUs unevenly -- more than one per CU, not a whole
+        // number of them (1000 x 1500 x 777: 384 tiles, 1.5 per CU, 29.0 -> 26.1 us on 2 ranges; 1536^3: 576 tiles,
+        // 72.3 -> 65.4 us; 1024^3 with one tile per CU and 2048^3 with four gain nothing and stay whole).
         const TileInfo small = tile_info_f32(TILE_SMALL, true, N);
         const uint64_t t = (uint64_t)((M + small.bm - 1) / small.bm) * ((N + small.bn - 1) / small.bn);
         const auto score = [&](uint32_t p) {
@@ -121,10 +125,12 @@ SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
             static const double loss[6] = {1.0, 1.35, 1.10, 1.03, 1.0, 1.0};
             return (double)(m * cus) / (double)wgs * (m <= 5 ? loss[m] : 1.0) + 0.01 * p;
         };
-        if (t <= 3ull * cus) {
+        const bool long_k = K >= 4096;
+        const uint32_t min_len = long_k ? 1024u : 256u, max_p = long_k ? 8u : 3u;
+        if (t <= 3ull * cus && (long_k || (t > cus && t % cus != 0))) {
             uint32_t best = 1;
-            double best_score = score(1) / 1.15;                    // the second kernel must be worth it
-            for (uint32_t p2 = 2; p2 <= 8 && K / p2 >= 1024 && t * p2 <= (uint64_t)small.per_cu * cus; ++p2)
+            double best_score = score(1) / 1.15;                    // the trip through the workspace must be worth it
+            for (uint32_t p2 = 2; p2 <= max_p && K / p2 >= min_len && t * p2 <= (uint64_t)small.per_cu * cus; ++p2)
                 if (score(p2) < best_score) { best_score = score(p2); best = p2; }
             if (best > 1) {
                 const uint32_t len = ((K + best - 1) / best + 31) / 32 * 32;

@@ -65,7 +65,9 @@ def test_planner_choices():
     # small and ragged problems take smaller tiles so the chip fills; they stay on the direct-to-LDS
     # kernels as long as the operands are 16-byte aligned
     p = hip.plan(4, 1000, 1500, 777)
-    assert p.edge == 0 and p.tile_m < 256 and p.grid == -(-1000 // p.tile_m) * -(-1500 // p.tile_n)
+    # 384 tiles of 64 x 64 are 1.5 per CU: with a workspace K is cut in two and every CU gets three workgroups
+    assert p.edge == 0 and p.tile_m < 256 and p.k_splits == 2 and p.grid == 2 * -(-1000 // p.tile_m) * -(-1500 // p.tile_n)
+    assert hip.plan(4, 1024, 1024, 1024).k_splits == 1 and hip.plan(4, 2048, 2048, 2048).k_splits == 1
     assert hip.plan(4, 1000, 1500, 777, aligned=False).edge == 1
     assert hip.plan(2, 1000, 1500, 777).edge == 0 and hip.plan(2, 1000, 1500, 777).tile_m == 64
     assert hip.plan(2, 2048, 2048, 2048).tile_m == 128 and hip.plan(2, 1000, 1500, 777, aligned=False).edge == 1
