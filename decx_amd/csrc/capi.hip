@@ -216,16 +216,12 @@ int gevm_maybe_split(bool f16, bool out_f32, const void* x, const void* B, const
 {
     const SplitPlan sp = plan_gevm_split(f16 ? 2 : 4, N, K, g_dev.compute_units);
     const uint32_t ldw = (N + 3) / 4 * 4;
-    const bool reducible = incy == 1 && (!c || (incc == 1 && !(f16 && out_f32)));
-    if (sp.splits > 1 && reducible && workspace && aligned16(workspace) && workspace_bytes >= (size_t)sp.splits * ldw * 4) {
-        const int rv = launch_gevm(f16, out_f32, x, B, nullptr, y, K, N, ldb, incx, 1, 1, 1.f, 1.f, stream, sp.len,
-                                   (float*)workspace, ldw);
-        if (rv != 0) return rv;
-        GemmArgs r;
-        std::memset(&r, 0, sizeof r);
-        r.C = c; r.D = y; r.M = 1; r.N = N; r.ldc = N; r.ldd = N; r.alpha = alpha; r.beta = beta;
-        r.split_ws = workspace; r.split_ldd = ldw; r.split_stride = ldw;
-        return launch_split_reduce(f16 && !out_f32 ? 2 : 4, r, sp.splits, stream);
+    if (sp.splits > 1 && workspace && aligned16(workspace) && workspace_bytes >= (size_t)sp.splits * ldw * 4) {
+        const uint32_t groups = (N + (f16 ? 64u : 32u) - 1) / (f16 ? 64u : 32u);
+        uint32_t* const counters = take_split_counters(groups);         // the last workgroup of a column group adds its ranges
+        if (counters)
+            return launch_gevm(f16, out_f32, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream, sp.len, (float*)workspace, ldw,
+                               counters);
     }
     return launch_gevm(f16, out_f32, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream);
 }
@@ -517,14 +513,10 @@ static int run_gemm_f64(const double* A, const double* B, const double* C, doubl
         const SplitPlan sp = plan_gevm_split(8, N, K, g_dev.compute_units);
         const uint32_t ldw = (N + 3) / 4 * 4;
         if (sp.splits > 1 && workspace && aligned16(workspace) && workspace_bytes >= (size_t)sp.splits * ldw * 8) {
-            const int rv = launch_gevm_f64(A, B, nullptr, D, K, N, ldb, 1, 1, 1, 1.0, 1.0, as_stream(stream), sp.len,
-                                           (double*)workspace, ldw);
-            if (rv != 0) return rv;
-            GemmArgs r;
-            std::memset(&r, 0, sizeof r);
-            r.C = C; r.D = D; r.M = 1; r.N = N; r.ldc = ldc; r.ldd = ldd; r.alpha64 = alpha; r.beta64 = beta;
-            r.split_ws = workspace; r.split_ldd = ldw; r.split_stride = ldw;
-            return launch_split_reduce(8, r, sp.splits, as_stream(stream));
+            uint32_t* const counters = take_split_counters((N + 15) / 16);
+            if (counters)
+                return launch_gevm_f64(A, B, C, D, K, N, ldb, 1, 1, 1, alpha, beta, as_stream(stream), sp.len, (double*)workspace, ldw,
+                                       counters);
         }
         return launch_gevm_f64(A, B, C, D, K, N, ldb, 1, 1, 1, alpha, beta, as_stream(stream));
     }

@@ -209,12 +209,12 @@ int launch_gemv(bool f16, bool out_f32, const void* A, const void* x, const void
                 uint32_t lda, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream);
 int launch_gevm(bool f16, bool out_f32, const void* x, const void* B, const void* c, void* y, uint32_t K, uint32_t N,
                 uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, hipStream_t stream,
-                uint32_t split_len = 0, float* partial = nullptr, uint32_t partial_stride = 0);
+                uint32_t split_len = 0, float* partial = nullptr, uint32_t partial_stride = 0, uint32_t* counters = nullptr);
 SplitPlan plan_gevm_split(int elem_bytes, uint32_t N, uint32_t K, uint32_t cus);
 int launch_gemv_f64(const double* A, const double* x, const double* c, double* y, uint32_t M, uint32_t K, uint32_t lda,
                     uint32_t incx, uint32_t incc, uint32_t incy, double alpha, double beta, hipStream_t stream);
 int launch_gevm_f64(const double* x, const double* B, const double* c, double* y, uint32_t K, uint32_t N, uint32_t ldb,
                     uint32_t incx, uint32_t incc, uint32_t incy, double alpha, double beta, hipStream_t stream,
-                    uint32_t split_len = 0, double* partial = nullptr, uint32_t partial_stride = 0);
+                    uint32_t split_len = 0, double* partial = nullptr, uint32_t partial_stride = 0, uint32_t* counters = nullptr);
 
 }  // namespace decx_hip

@@ -431,8 +431,8 @@ def test_column_operand_gathered_through_a_workspace(hip, oracle, dtype, M, K):
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 @pytest.mark.parametrize("K,N", [(8192, 2048), (20000, 70), (16500, 7), (33000, 513)])
 def test_row_operand_few_columns_split_through_a_workspace(hip, oracle, dtype, K, N):
-    """M = 1 with few columns and a long K: with a workspace, ranges of K go to workgroups of their own and their
-    partial sums are added in range order by a second kernel.  Parity, identical results from run to run,
+    """M = 1 with few columns and a long K: with a workspace, ranges of K go to workgroups of their own and the last
+    workgroup of a column group to finish adds their partial sums in range order.  Parity, identical results from run to run,
     C / alpha / beta, untouched padding; a workspace that is too small means the single-kernel path."""
     f16 = dtype == np.float16
     A = synth.normal_half(1, K, 181) if f16 else synth.uniform_f32(1, K, 181)
@@ -441,8 +441,8 @@ def test_row_operand_few_columns_split_through_a_workspace(hip, oracle, dtype, K
     need = hip.lib().decx_hip_gemm_workspace(dtype().itemsize, 1, N, K)
     assert need > 0 and need % 16 == 0
     assert hip.plan(dtype().itemsize, 1, N, K).k_splits > 1
-    assert hip.lib().decx_hip_gemm_workspace(dtype().itemsize, 1, 512, 8192) == 0       # too short to pay for a second kernel
-    assert hip.lib().decx_hip_gemm_workspace(dtype().itemsize, 1, 8192, 8192) == 0      # enough column groups
+    assert hip.lib().decx_hip_gemm_workspace(dtype().itemsize, 1, 512, 8192) == 0       # too little to share out
+    assert hip.lib().decx_hip_gemm_workspace(4, 1, 8192, 8192) == 0                     # fp32: a column group per CU already
     ws = hip.DeviceMatrix(1, need // 4, np.float32)
     ws.upload_raw(np.full((1, ws.pitch), np.nan, np.float32))
     pk, pn = device_pitch(K, dtype), device_pitch(N, dtype)
