@@ -104,7 +104,8 @@ def test_planner_choices():
     assert [hip.plan(4, M, 1, 4096).tile_m for M in (9000, 5000, 3000, 1500, 600, 100)] == [32, 16, 8, 4, 2, 1]
     p = hip.plan(4, 1, 512, 32768)
     assert (p.path, p.tile_n) == (hip.PATH_GEVM, 32) and p.k_splits > 1 and p.grid == 16 * p.k_splits
-    assert hip.plan(4, 1, 512, 8192).k_splits == 1 and hip.plan(2, 1, 8192, 8192).k_splits == 1
+    assert hip.plan(4, 1, 512, 8192).k_splits == 1 and hip.plan(4, 1, 8192, 8192).k_splits == 1
+    assert hip.plan(2, 1, 8192, 8192).k_splits == 2        # 128 groups of whole cache lines, two ranges: a workgroup per CU
     assert hip.plan(8, 8192, 1, 8192).path == hip.PATH_GEMV and hip.plan(8, 1, 8192, 8192).path == hip.PATH_GEVM
     assert hip.plan(8, 1, 8192, 8192).tile_n == 16
     bad = hip.Plan()
