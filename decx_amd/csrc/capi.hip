@@ -91,9 +91,55 @@ int check_gemm(const void* A, const void* B, const void* C, const void* D, uint3
     return DECX_HIP_OK;
 }
 
+struct SplitChoice { int shape; uint32_t splits, len; };
+
+// fp32 splits run on the smallest tile (64 x 64, or 128 x 32 for narrow outputs), whatever the whole product would
+// take, and add their ranges inside the kernel.  The number of ranges is the one a small model of the kernel's time
+// likes best, in microseconds:
+//   workgroups = tiles x ranges, each as long as its range; four fit a CU (32 KB of LDS each: a fifth does not get
+//   in), so whole rounds of 4 x CUs workgroups run at the full-CU rate and the remainder, m on the busiest CU, at
+//   the measured rate of m co-resident workgroups (alone 1 / 1.2 of a full CU, two 1 / 1.05, three 1 / 1.02);
+//   a remainder of more than half a workgroup per CU right after ONE full round lands unevenly (the CUs that finish
+//   first take several): it counts as two;
+//   every range costs a trip of the output through the workspace (0.15 us per MB) and every four ranges a round trip
+//   of the last workgroup's loads.
+// Fitted to 20 output shapes x K = 777 ... 16384 x 1 ... 8 ranges (estimate within 4 % of the measurement on most,
+// the pick within 1 % of the best on average).  The whole product is kept unless the split promises 4 %.
+SplitChoice split_plan_f32(uint32_t M, uint32_t N, uint32_t K, int whole_shape, const TileInfo& whole)
+{
+    const uint32_t cus = g_dev.compute_units;
+    const TileInfo small = tile_info_f32(TILE_SMALL, true, N);
+    const uint64_t t = (uint64_t)((M + small.bm - 1) / small.bm) * ((N + small.bn - 1) / small.bn);
+    if (K < 512 || t > 4ull * cus) return {whole_shape, 1, 0};
+    constexpr double kTileK = 0.01477;                          // us per tile and k, a CU with four workgroups
+    constexpr double kLaunch = 4.0, kCuFlopPerUs = 0.586e6;     // launch to launch; the largest tile on a full chip
+    static const double rate_loss[5] = {0.0, 1.2, 1.05, 1.02, 1.0};
+    const double out_mb = (double)M * N * 4.0 / 1e6;
+    const auto estimate = [&](uint32_t len, uint32_t ranges) {
+        const uint64_t wgs = t * ranges, slots = 4ull * cus;
+        const uint64_t full = wgs / slots, rem = wgs % slots;
+        uint64_t m = (rem + cus - 1) / cus;
+        if (full == 1 && rem > cus / 2 && rem <= cus) m = 2;
+        const double rounds = 4.0 * (double)full + (double)m * rate_loss[m];
+        return kTileK * len * rounds + kLaunch + 0.15 * ranges * out_mb + 1.0 + 0.4 * ((ranges + 3) / 4);
+    };
+    const uint64_t whole_tiles = (uint64_t)((M + whole.bm - 1) / whole.bm) * ((N + whole.bn - 1) / whole.bn);
+    const double whole_us = tile_cost(whole, whole_tiles, cus) * 2.0 * K / kCuFlopPerUs + kLaunch;
+    uint32_t best_len = 0, best_ranges = 1;
+    double best_us = whole_us / 1.04;
+    const uint32_t max_p = K / 256 < 64u ? K / 256 : 64u;
+    for (uint32_t p = 2; p <= max_p; ++p) {
+        const uint32_t len = ((K + p - 1) / p + 31) / 32 * 32, ranges = (K + len - 1) / len;
+        if (ranges < 2) continue;
+        const double us = estimate(len, ranges);
+        if (us < best_us) { best_us = us; best_len = len; best_ranges = ranges; }
+    }
+    if (best_ranges > 1) return {TILE_SMALL, best_ranges, best_len};
+    return {whole_shape, 1, 0};
+}
+
 // Split K is planned for products on 16-byte aligned operands whose tiles would leave CUs idle or unevenly loaded.
 // elem_bytes: 2, 4 or 8.  `shape` is the tile the split runs on (it may differ from the one the whole product takes).
-struct SplitChoice { int shape; uint32_t splits, len; };
 SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
 {
     if (M == 0 || N == 0) return {0, 1, 0};
@@ -102,42 +148,15 @@ SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
     const int shape = elem_bytes == 8 ? choose_tile_f64(M, N) : choose_tile(elem_bytes == 2, M, N, true);
     const TileInfo ti = elem_bytes == 8 ? tile_info_f64(shape)
                                         : elem_bytes == 2 ? tile_info_f16(shape, true) : tile_info_f32(shape, true, N);
+    if (elem_bytes == 4) return split_plan_f32(M, N, K, shape, ti);
     // outputs of at most half as many tiles as there are CUs: up to two workgroups per CU
     const SplitPlan sp = plan_split_k((uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn), K, cus);
     if (sp.splits > 1) return {shape, sp.splits, sp.len};
     // Outputs of a few hundred small tiles and a long K: one or two workgroups per CU run well below the rate of a
-    // full CU, and 1.5 per CU leave half the chip waiting for the other half.  Measured: fp32 1280 x 1024 x 8192
-    // 259 -> 186 us with 64 x 64 tiles on 3 ranges, 768 x 768 x 16384 292 -> 165 (7 ranges); fp16 1536 x 1024 x 8192
+    // full CU, and 1.5 per CU leave half the chip waiting for the other half.  Measured: fp16 1536 x 1024 x 8192
     // 57 -> 43 us with 128 x 128 tiles on 2 ranges, 768 x 768 x 16384 61 -> 37 (4 ranges); 2048 x 2048 x 8192 and
     // 1024 x 2048 x 4096 gain nothing and stay whole.
     const auto tiles_of = [&](uint32_t b) { return (uint64_t)((M + b - 1) / b) * ((N + b - 1) / b); };
-    if (elem_bytes == 4 && K >= 512) {
-        // 64 x 64 tiles, up to five workgroups per CU.  score = (workgroups on the busiest CU / the average) x what a
-        // CU loses with m workgroups against a full one; the ranges p that make t * p an even three to five per CU win.
-        // Long K (>= 4096): ranges of at least 1024.  Shorter K: the split costs every tile a trip through the
-        // workspace, which pays only when the tiles alone load the CUs unevenly -- more than one per CU, not a whole
-        // number of them (1000 x 1500 x 777: 384 tiles, 1.5 per CU, 29.0 -> 26.1 us on 2 ranges; 1536^3: 576 tiles,
-        // 72.3 -> 65.4 us; 1024^3 with one tile per CU and 2048^3 with four gain nothing and stay whole).
-        const TileInfo small = tile_info_f32(TILE_SMALL, true, N);
-        const uint64_t t = (uint64_t)((M + small.bm - 1) / small.bm) * ((N + small.bn - 1) / small.bn);
-        const auto score = [&](uint32_t p) {
-            const uint64_t wgs = t * p, m = (wgs + cus - 1) / cus;
-            static const double loss[6] = {1.0, 1.35, 1.10, 1.03, 1.0, 1.0};
-            return (double)(m * cus) / (double)wgs * (m <= 5 ? loss[m] : 1.0) + 0.01 * p;
-        };
-        const bool long_k = K >= 4096;
-        const uint32_t min_len = long_k ? 1024u : 256u, max_p = long_k ? 8u : 3u;
-        if (t <= 3ull * cus && (long_k || (t > cus && t % cus != 0))) {
-            uint32_t best = 1;
-            double best_score = score(1) / 1.15;                    // the trip through the workspace must be worth it
-            for (uint32_t p2 = 2; p2 <= max_p && K / p2 >= min_len && t * p2 <= (uint64_t)small.per_cu * cus; ++p2)
-                if (score(p2) < best_score) { best_score = score(p2); best = p2; }
-            if (best > 1) {
-                const uint32_t len = ((K + best - 1) / best + 31) / 32 * 32;
-                return {TILE_SMALL, (K + len - 1) / len, len};
-            }
-        }
-    }
     if (elem_bytes == 2 && K >= 6144) {
         // 128 x 128 tiles towards one workgroup per CU, a power of two of ranges at least 2048 long, and only when
         // that occupies more than half the chip (1024 x 1024 x 6144 on 2 ranges: 26.6 -> 28.9 us)
@@ -209,7 +228,7 @@ uint32_t arm_split(GemmArgs& g, int elem_bytes, void* workspace, size_t workspac
 }
 
 // y = alpha * x.B (+ beta * c).  Few columns and a long K: with a workspace, ranges of K go to workgroups of their
-// own and a second kernel adds their partial sums in range order; that kernel writes a dense y and reads c in y's type.
+// own, and the last of a column group to finish adds their partial sums in range order.
 int gevm_maybe_split(bool f16, bool out_f32, const void* x, const void* B, const void* c, void* y, uint32_t K, uint32_t N,
                      uint32_t ldb, uint32_t incx, uint32_t incc, uint32_t incy, float alpha, float beta, void* workspace,
                      size_t workspace_bytes, hipStream_t stream)

@@ -119,8 +119,9 @@ __host__ inline double tile_cost(const TileInfo& ti, uint64_t tiles, uint32_t cu
 
 // fp32, measured on MI355X (TFLOP/s per CU, direct-to-LDS kernels): 256 x 128 (the largest tile; 256 x 256 in the
 // register-staged family) 0.56 alone, 0.586 two per CU; 128 x 128
-// 0.52 alone (2048^3), 0.586 four per CU (4096^3, 6144^3); 64 x 64 0.39 alone (1024^3), 0.56 five per CU (3072^3,
-// 4096^3).  The predicated register-staged kernels (operands that are not 16-byte aligned) run at about
+// 0.52 alone (2048^3), 0.586 four per CU (4096^3, 6144^3); 64 x 64 0.47 alone (long K; 0.39 at 1024^3 with the launch
+// in it), 0.56 four per CU (3072^3, 4096^3; 160 KB of LDS would hold five of them, but time against the number of
+// tiles steps as for four).  The predicated register-staged kernels (operands that are not 16-byte aligned) run at about
 // 1 : 0.8 : 0.7 of the largest tile, two workgroups per CU.
 // N: columns of the output; at most kNarrowN of them turn the smallest aligned tile into 128 x 32 (the same area, no
 // idle half: 65536 x 32 x 1024 46.8 us against 81.9 us for 64 columns on 64 x 64 tiles).
@@ -131,7 +132,7 @@ __host__ inline TileInfo tile_info_f32(int shape, bool aligned = true, uint32_t 
     case TILE_MEDIUM: return {128, 128, 256, aligned ? 4 : 2, aligned ? 1.00f : 0.80f, aligned ? 0.88f : 0.72f};
     default:
         if (aligned && N <= kNarrowN) return {128, 32, 256, 4, 0.96f, 0.667f};
-        return { 64,  64, 256, aligned ? 5 : 2, aligned ? 0.96f : 0.70f, aligned ? 0.667f : 0.49f};
+        return { 64,  64, 256, aligned ? 4 : 2, aligned ? 0.96f : 0.70f, aligned ? 0.80f : 0.49f};
     }
 }
 // fp16 (TFLOP/s per CU): 256 x 256 4.64 on a full chip, 6.4 with at most half the CUs busy; 128 x 128 3.1 alone,

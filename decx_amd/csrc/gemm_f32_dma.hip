@@ -436,29 +436,44 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
         }
         __syncthreads();
         if (__builtin_amdgcn_readfirstlane(*flag) == 0) return;
-        for (uint32_t z = 0; z < splits; ++z) {            // range order, this workgroup's own slot included
-            const float* p = slots + (size_t)z * (BM * BN);
-            floatx4 v[TM][TN][4];
+        // Range order, this workgroup's own slot included.  A lane holds PIECES 16-byte pieces of a slot; they are
+        // summed GROUP pieces at a time (16 registers of loads in flight next to the accumulators keep two workgroups
+        // of the largest tile on a CU), and small tiles fetch the same pieces of BATCH slots together (one slot at a
+        // time costs a round trip to memory per range).
+        constexpr int PIECES = TM * TN * 4;
+        constexpr int GROUP = PIECES <= 16 ? PIECES : 16, BATCH = 16 / GROUP;
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+        for (int c0 = 0; c0 < PIECES; c0 += GROUP) {
+            for (uint32_t z0 = 0; z0 < splits; z0 += BATCH) {
+                floatx4 v[BATCH][GROUP];
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
+                for (int zb = 0; zb < BATCH; ++zb) {
+                    if (zb == 0 || z0 + zb < splits) {         // slots beyond the last range are neither loaded nor added
+                        const float* p = slots + (size_t)(z0 + zb) * (BM * BN);
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const float* const src = p + (size_t)(((i * TN + j) * 4 + q) * NT + t) * 4;
-                        asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[i][j][q]) : "v"(src) : "memory");
+                        for (int c = 0; c < GROUP; ++c) {
+                            const float* const src = p + (size_t)((c0 + c) * NT + t) * 4;
+                            asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[zb][c]) : "v"(src) : "memory");
+                        }
                     }
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+                for (int zb = 0; zb < BATCH; ++zb) {
+                    if (zb == 0 || z0 + zb < splits) {
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
+                        for (int c = 0; c < GROUP; ++c) {
+                            const int tile = (c0 + c) / 4, q = (c0 + c) % 4;
+                            asm volatile("" : "+v"(v[zb][c]));                 // not before the wait above
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        asm volatile("" : "+v"(v[i][j][q]));               // not before the wait above
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = (z == 0) ? v[i][j][q][e] : acc[i][j][4 * q + e] + v[i][j][q][e];
+                            for (int e = 0; e < 4; ++e) {
+                                const float a = acc[tile / TN][tile % TN][4 * q + e], w = v[zb][c][e];
+                                acc[tile / TN][tile % TN][4 * q + e] = (z0 + zb == 0) ? w : a + w;
+                            }
+                        }
                     }
+                }
+            }
         }
         if (t == 0) __hip_atomic_store(g.split_counters + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -574,7 +589,7 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
 //     CU count (6144^3: 110 against 133); with 64 x 128 wave tiles, 16 wavefronts, 32-deep slabs or rings of 3 to
 //     5 stages it lands between 138 and 144.
 //   128 x 128 and 64 x 64: 4 wavefronts, chunk-ahead fragments, and a ring of only 2 stages (32 KB): what hides the
-//     copy latency for these is not a deep ring but several workgroups per CU (4 and 5 fit), e.g. 128 x 128 at
+//     copy latency for these is not a deep ring but several workgroups per CU (4 fit), e.g. 128 x 128 at
 //     6144^3 147 TFLOP/s against 130 with 4 stages, 64 x 64 at 3072^3 139 against 127; with a single workgroup per CU
 //     (1024^3) both rings measure the same.  Deeper rings, 64-deep slabs, a second accumulator chain and splitting K
 //     over two wavefront groups changed nothing or lost.

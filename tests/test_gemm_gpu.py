@@ -332,7 +332,7 @@ def test_f16_split_k_through_a_workspace(hip, oracle, M, N, K):
 
 
 @pytest.mark.parametrize("dtype,M,N,K,tile,splits", [
-    (np.float32, 1280, 1024, 4096, 64, 4),          # 320 tiles of 64 x 64: 1.25 per CU, on 4 ranges five per CU
+    (np.float32, 1280, 1024, 4096, 64, 8),          # 320 tiles of 64 x 64: 1.25 per CU, on 8 ranges ten per CU, four at a time
     (np.float32, 900, 700, 4100, 64, 3),            # ragged output, K not a multiple of the range
     (np.float16, 1280, 1024, 6144, 128, 2),         # 80 tiles of 128 x 128 on 2 ranges
     (np.float16, 768, 768, 8200, 128, 4),
@@ -379,7 +379,8 @@ def test_split_k_for_a_few_hundred_tiles(hip, oracle, dtype, M, N, K, tile, spli
 def test_f32_split_k_is_planned_only_where_it_pays(hip):
     L = hip.lib()
     assert L.decx_hip_gemm_f32_workspace(8192, 8192, 8192) == 0           # enough tiles
-    assert L.decx_hip_gemm_f32_workspace(300, 300, 512) == 0              # K too short to cut
+    assert L.decx_hip_gemm_f32_workspace(300, 300, 400) == 0              # K too short to cut
+    assert L.decx_hip_gemm_f32_workspace(1024, 1024, 1024) == 0           # a tile per CU, K too short to pay for the exchange
     assert L.decx_hip_gemm_f32_workspace(1, 8192, 8192) == 0              # a row vector is dense already
     assert L.decx_hip_gemm_f32_workspace(0, 5, 5000) == 0
 
