@@ -193,35 +193,33 @@ SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
     return {shape, 1, 0};
 }
 
-// Bytes of workspace a split of `splits` ranges needs.  fp32: one slot of BM x BN floats per workgroup (the tiles of
-// the shape the split runs on); fp16 / fp64: `splits` partial products of M rows at a pitch of N rounded up to 4.
-size_t split_workspace_bytes(int elem_bytes, int shape, uint32_t M, uint32_t N, uint32_t splits)
+// Block tile of a size class in the direct-to-LDS family of an element type.
+TileInfo dma_tile_info(int elem_bytes, int shape, uint32_t N)
 {
-    if (elem_bytes == 4) {
-        const TileInfo ti = tile_info_f32(shape, true, N);
-        const uint64_t tiles = (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
-        return (size_t)(tiles * splits * (uint64_t)(ti.bm * ti.bn) * 4u);
-    }
-    return (size_t)splits * M * ((N + 3) / 4 * 4) * (size_t)(elem_bytes == 8 ? 8 : 4);
+    return elem_bytes == 8 ? tile_info_f64(shape) : elem_bytes == 2 ? tile_info_f16(shape, true) : tile_info_f32(shape, true, N);
 }
 
-// Fills the split fields of g when the plan says so and the workspace is large enough; returns the number of splits
-// and, with more than one, the tile shape they run on.
+// Bytes of workspace a split of `splits` ranges needs: one slot of BM x BN accumulators (fp32; fp64 for fp64 operands)
+// per workgroup, the tiles being those of the shape the split runs on.
+size_t split_workspace_bytes(int elem_bytes, int shape, uint32_t M, uint32_t N, uint32_t splits)
+{
+    const TileInfo ti = dma_tile_info(elem_bytes, shape, N);
+    const uint64_t tiles = (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
+    return (size_t)(tiles * splits * (uint64_t)(ti.bm * ti.bn) * (elem_bytes == 8 ? 8u : 4u));
+}
+
+// Fills the split fields of g when the plan says so, the workspace is large enough and the tiles have counters; returns
+// the number of splits and, with more than one, the tile shape they run on.
 uint32_t arm_split(GemmArgs& g, int elem_bytes, void* workspace, size_t workspace_bytes, int& shape)
 {
     if (!workspace || !aligned16(workspace)) return 1;
     const SplitChoice sp = split_plan(elem_bytes, g.M, g.N, g.K);
     if (sp.splits <= 1 || workspace_bytes < split_workspace_bytes(elem_bytes, sp.shape, g.M, g.N, sp.splits)) return 1;
-    if (elem_bytes == 4) {                                      // one kernel: slots and tile counters
-        const TileInfo ti = tile_info_f32(sp.shape, true, g.N);
-        const uint64_t tiles = (uint64_t)((g.M + ti.bm - 1) / ti.bm) * ((g.N + ti.bn - 1) / ti.bn);
-        uint32_t* const counters = tiles <= kSplitCounters ? take_split_counters((uint32_t)tiles) : nullptr;
-        if (!counters) return 1;
-        g.split_counters = counters;
-    } else {
-        const uint32_t ldw = (g.N + 3) / 4 * 4;
-        g.split_ldd = ldw; g.split_stride = (uint64_t)g.M * ldw;
-    }
+    const TileInfo ti = dma_tile_info(elem_bytes, sp.shape, g.N);
+    const uint64_t tiles = (uint64_t)((g.M + ti.bm - 1) / ti.bm) * ((g.N + ti.bn - 1) / ti.bn);
+    uint32_t* const counters = tiles <= kSplitCounters ? take_split_counters((uint32_t)tiles) : nullptr;
+    if (!counters) return 1;
+    g.split_counters = counters;
     g.split_len = sp.len; g.split_ws = workspace;
     shape = sp.shape;
     return sp.splits;
@@ -280,12 +278,7 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
     int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile(F16, M, N, g.vec_ok != 0) : tile;
     const bool edge = force_edge != 0 || K == 0;
     if (workspace && tile == DECX_HIP_TILE_AUTO && !edge && g.vec_ok && dma_offsets_fit(g, F16 ? 2 : 4)) {
-        const uint32_t splits = arm_split(g, F16 ? 2 : 4, workspace, workspace_bytes, shape);
-        if (splits > 1) {
-            if (!F16) return launch_gemm_f32(shape, false, g, as_stream(stream));       // the last workgroup of a tile sums it
-            const int rl = launch_gemm_f16(shape, false, g, as_stream(stream));
-            return rl != 0 ? rl : launch_split_reduce(2, g, splits, as_stream(stream));
-        }
+        arm_split(g, F16 ? 2 : 4, workspace, workspace_bytes, shape);    // with ranges, the last workgroup of a tile sums them
     }
     return F16 ? launch_gemm_f16(shape, edge, g, as_stream(stream))
                : launch_gemm_f32(shape, edge, g, as_stream(stream));
@@ -551,11 +544,7 @@ static int run_gemm_f64(const double* A, const double* B, const double* C, doubl
                 lda % 2 == 0 && ldb % 2 == 0 && ldd % 2 == 0 && (!C || ldc % 2 == 0)) ? 1u : 0u;
     int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile_f64(M, N) : tile;
     if (workspace && tile == DECX_HIP_TILE_AUTO && !force_plain && K > 0 && g.vec_ok && dma_offsets_fit(g, 8)) {
-        const uint32_t splits = arm_split(g, 8, workspace, workspace_bytes, shape);
-        if (splits > 1) {
-            const int rl = launch_gemm_f64(shape, false, g, as_stream(stream));
-            return rl != 0 ? rl : launch_split_reduce(8, g, splits, as_stream(stream));
-        }
+        arm_split(g, 8, workspace, workspace_bytes, shape);
     }
     return launch_gemm_f64(shape, force_plain != 0, g, as_stream(stream));
 }

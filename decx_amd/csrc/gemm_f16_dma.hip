@@ -56,14 +56,6 @@ __device__ __forceinline__ halfx8 join(shortx4 lo, shortx4 hi)
     return u.v;
 }
 
-template <int I, int N, class F> __device__ __forceinline__ void static_for(F&& f)
-{
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
-
 template <int N> __device__ __forceinline__ void wait_loads_and_barrier()
 {
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(N) : "memory");
@@ -85,7 +77,8 @@ template <int MFMAS, int READS> __device__ __forceinline__ void interleave()
 
 }  // namespace
 
-// SPLIT: grid.y workgroups share each tile, each with its own range of K, writing its partial product in fp32.
+// SPLIT: grid.y workgroups share each tile, each with its own range of K; the one that finishes last adds their fp32
+// partial products and rounds once (split_k_exchange).
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool SPLIT = false>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_f16_dma_kernel(const GemmArgs g_in)
@@ -178,13 +171,13 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
 #pragma unroll
             for (int i = 0; i < A_LOADS; ++i) {
                 const uint32_t dst = stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u;
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(a_voff[i]), "s"(a_base) : "memory", "m0");
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(a_voff[i]), "s"(a_base) : "memory", "m0");
             }
             a_base += RB;
 #pragma unroll
             for (int i = 0; i < B_LOADS; ++i) {
                 const uint32_t dst = stage_off + A_STAGE_BYTES + (uint32_t)(wave * B_LOADS + i) * 1024u;
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(b_voff[i]), "s"(b_base) : "memory", "m0");
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(b_voff[i]), "s"(b_base) : "memory", "m0");
             }
             b_base += b_step;
         } else {
@@ -307,19 +300,21 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
 
     // Epilogue.  Lane (kg, l16) holds, of the 16 x 16 tile (i, j), row l16 and the 4 adjacent columns 4 kg .. 4 kg + 3.
     if constexpr (SPLIT) {
-        float* __restrict__ P = (float*)g.split_ws + (size_t)blockIdx.y * g.split_stride;
+        // piece c of a lane: the four fp32 accumulators of its 16 x 16 tile (c % TM, c / TM).  The ring is free: every
+        // LDS read precedes the last slab barrier.
+        const bool last = split_k_exchange<WAVES * 64, TM * TN, floatx4>(g_in, (uint32_t*)lds,
+            [&](auto cc) { constexpr int c = decltype(cc)::value; return accT[c / TM][c % TM]; },
+            [&](auto cc, const floatx4& v, bool first) {
+                constexpr int c = decltype(cc)::value;
+                floatx4& a = accT[c / TM][c % TM];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const uint32_t row = m0 + wm0 + 16 * i + l16;
-            if (row < g.M) {
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    const uint32_t col = n0 + wn0 + 16 * j + 4 * kg;
-                    if (col < g.split_ldd) *(floatx4*)(P + (size_t)row * g.split_ldd + col) = accT[j][i];
+                for (int e = 0; e < 4; ++e) {
+                    const float old = a[e], w = v[e];
+                    a[e] = first ? w : old + w;
                 }
-            }
-        }
-        return;
+            });
+        if (!last) return;
+        __syncthreads();                                   // the flag word lies in the rows the epilogue stages through
     }
     const _Float16* __restrict__ C = (const _Float16*)g.C;
     _Float16* __restrict__ D = (_Float16*)g.D;

@@ -27,14 +27,6 @@
 
 namespace decx_hip {
 
-template <int I, int N, class F> __device__ __forceinline__ void static_for(F&& f)
-{
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
-
 template <int TN> struct BFrag;
 template <> struct BFrag<1> { typedef float type; };
 template <> struct BFrag<2> { typedef floatx2 type; };

@@ -18,7 +18,9 @@
 // ds_write), so late loads are absorbed by the ring and by the other workgroups of the CU.  The direct
 // loads are inline assembly and the slab barrier is a bare `s_barrier` behind an explicit vmcnt
 // wait, because the compiler would otherwise wait for every outstanding load in front of each
-// LDS read and at each __syncthreads().  Fragment reads are pinned behind MFMAs with
+// LDS read and at each __syncthreads().  (The compiler does not look into inline assembly for
+// hazards: the `s_nop 0` between the write of M0, which carries the LDS destination, and the
+// load that reads it is the wait state this part asks for.)  Fragment reads are pinned behind MFMAs with
 // `sched_group_barrier`; the MFMAs of the last k step of a slab are issued after the slab
 // barrier, behind the first fragment reads of the next slab.
 //   * tile shapes from 256 x 128 (four wavefronts of 128 x 64, two workgroups per CU; the
@@ -46,14 +48,6 @@ namespace decx_hip {
 namespace {
 
 typedef __attribute__((address_space(3))) void lds_void;
-
-template <int I, int N, class F> __device__ __forceinline__ void static_for(F&& f)
-{
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
 
 template <int N> __device__ __forceinline__ void wait_loads_and_barrier()
 {
@@ -197,7 +191,7 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
             constexpr int i = idx;
             const uint32_t dst = stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u;
             if constexpr (CONV != 1) {
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(a_voff[i]), "s"(a_base) : "memory", "m0");
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(a_voff[i]), "s"(a_base) : "memory", "m0");
                 if constexpr (i == A_LOADS - 1) {
                     a_base += BK * 4;
                     if constexpr (CONV == 2) {
@@ -206,7 +200,7 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
                     }
                 }
             } else {
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(a_src[i]) : "memory", "m0");
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(a_src[i]) : "memory", "m0");
                 a_src[i] += BK * 4;
                 a_seg[i] += BK * 4;
                 while (a_seg[i] >= g.conv_seg_bytes) {
@@ -217,7 +211,7 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
         } else {
             constexpr int i = idx - A_LOADS;
             const uint32_t dst = stage_off + A_STAGE_BYTES + (uint32_t)(wave * B_LOADS + i) * 1024u;
-            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(b_voff[i]), "s"(b_base) : "memory", "m0");
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(b_voff[i]), "s"(b_base) : "memory", "m0");
             if constexpr (i == B_LOADS - 1) b_base += b_step;
         }
     };
@@ -408,74 +402,24 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
     }
 
     if constexpr (SPLIT) {
-        // Every lane's accumulators go to the workgroup's slot, [register][thread]: whole lines per wave.  Slots are
-        // written and read with device-scope accesses (they pass the XCD's own L2, which is not coherent with the other
-        // seven), so that no cache-wide write-back or invalidation is needed around the count -- those would throw out
-        // the operand lines the workgroups still multiplying live on.
-        constexpr int NT = WAVES * 64;
-        const uint32_t splits = gridDim.y;
-        float* const slots = (float*)g.split_ws + (size_t)blockIdx.x * splits * (BM * BN);
-        float* const mine = slots + (size_t)blockIdx.y * (BM * BN);
-        // 16-byte pieces, [piece][thread]; `sc1`: device scope (written through / fetched past this XCD's L2)
+        // piece c of a lane: registers 4 (c % 4) .. + 3 of its 32 x 32 tile c / 4.  The ring is free: every LDS read
+        // precedes the last slab barrier.
+        const bool last = split_k_exchange<WAVES * 64, TM * TN * 4, floatx4>(g_in, (uint32_t*)lds,
+            [&](auto cc) {
+                constexpr int c = decltype(cc)::value, tile = c / 4, q = c % 4;
+                const floatx16& a = acc[tile / TN][tile % TN];
+                return floatx4{a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]};
+            },
+            [&](auto cc, const floatx4& v, bool first) {
+                constexpr int c = decltype(cc)::value, tile = c / 4, q = c % 4;
+                floatx16& a = acc[tile / TN][tile % TN];
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const floatx4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-                    float* const dst = mine + (size_t)(((i * TN + j) * 4 + q) * NT + t) * 4;
-                    asm volatile("global_store_dwordx4 %0, %1, off sc1" :: "v"(dst), "v"(v) : "memory");
+                for (int e = 0; e < 4; ++e) {
+                    const float old = a[4 * q + e], w = v[e];
+                    a[4 * q + e] = first ? w : old + w;
                 }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this lane's stores have arrived
-        __syncthreads();                                   // everyone's have (the ring is free: every LDS read precedes the last slab barrier)
-        uint32_t* const flag = (uint32_t*)lds;
-        if (t == 0) {
-            const uint32_t before = __hip_atomic_fetch_add(g.split_counters + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            *flag = (before + 1 == splits) ? 1u : 0u;
-        }
-        __syncthreads();
-        if (__builtin_amdgcn_readfirstlane(*flag) == 0) return;
-        // Range order, this workgroup's own slot included.  A lane holds PIECES 16-byte pieces of a slot; they are
-        // summed GROUP pieces at a time (16 registers of loads in flight next to the accumulators keep two workgroups
-        // of the largest tile on a CU), and small tiles fetch the same pieces of BATCH slots together (one slot at a
-        // time costs a round trip to memory per range).
-        constexpr int PIECES = TM * TN * 4;
-        constexpr int GROUP = PIECES <= 16 ? PIECES : 16, BATCH = 16 / GROUP;
-#pragma unroll
-        for (int c0 = 0; c0 < PIECES; c0 += GROUP) {
-            for (uint32_t z0 = 0; z0 < splits; z0 += BATCH) {
-                floatx4 v[BATCH][GROUP];
-#pragma unroll
-                for (int zb = 0; zb < BATCH; ++zb) {
-                    if (zb == 0 || z0 + zb < splits) {         // slots beyond the last range are neither loaded nor added
-                        const float* p = slots + (size_t)(z0 + zb) * (BM * BN);
-#pragma unroll
-                        for (int c = 0; c < GROUP; ++c) {
-                            const float* const src = p + (size_t)((c0 + c) * NT + t) * 4;
-                            asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[zb][c]) : "v"(src) : "memory");
-                        }
-                    }
-                }
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#pragma unroll
-                for (int zb = 0; zb < BATCH; ++zb) {
-                    if (zb == 0 || z0 + zb < splits) {
-#pragma unroll
-                        for (int c = 0; c < GROUP; ++c) {
-                            const int tile = (c0 + c) / 4, q = (c0 + c) % 4;
-                            asm volatile("" : "+v"(v[zb][c]));                 // not before the wait above
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                const float a = acc[tile / TN][tile % TN][4 * q + e], w = v[zb][c][e];
-                                acc[tile / TN][tile % TN][4 * q + e] = (z0 + zb == 0) ? w : a + w;
-                            }
-                        }
-                    }
-                }
-            }
-        }
-        if (t == 0) __hip_atomic_store(g.split_counters + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            });
+        if (!last) return;
     }
 
     // Epilogue: register r of lane (l32, h) is row 8*(r/4) + 4*h + r%4 of a 32x32 tile; the
@@ -524,39 +468,6 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
 
 namespace {
 
-__device__ __forceinline__ float  fma_as(float a, float b, float c)    { return __builtin_fmaf(a, b, c); }
-__device__ __forceinline__ double fma_as(double a, double b, double c) { return __builtin_fma(a, b, c); }
-
-// one thread per four columns: D = sum of the partial products in split order (+ the C term).  TA: type of the
-// partial products and of the arithmetic, TO: type of C and D.
-template <typename TA, typename TO>
-__global__ void __launch_bounds__(256) split_reduce_kernel(const GemmArgs g, uint32_t splits, TA alpha, TA beta)
-{
-    const uint32_t quads = g.split_ldd / 4;
-    const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (uint64_t)g.M * quads) return;
-    const uint32_t row = (uint32_t)(idx / quads), col = (uint32_t)(idx % quads) * 4;
-    const TA* p = (const TA*)g.split_ws + (size_t)row * g.split_ldd + col;
-    TA sum[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) sum[e] = p[e];
-    for (uint32_t z = 1; z < splits; ++z) {
-        const TA* q = p + (size_t)z * g.split_stride;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) sum[e] += q[e];
-    }
-    const TO* C = (const TO*)g.C;
-    TO* D = (TO*)g.D;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        if (col + e < g.N) {
-            TA o = sum[e];
-            if (C) o = fma_as((TA)C[(size_t)row * g.ldc + col + e], beta, alpha * o);   // one fma in TA, as the unsplit epilogue
-            D[(size_t)row * g.ldd + col + e] = (TO)o;
-        }
-    }
-}
-
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, int CONV = 0>
 int launch_dma(const GemmArgs& args, hipStream_t stream)
 {
@@ -567,12 +478,14 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     // 256 x 128 tiles, two independent workgroups per CU: patches two tile-rows high fetch least (8192^3: 5.5 GB through
     // L2 against 6.2 GB with four rows and 11.7 GB with eight, at the same speed)
     if constexpr (BM == 256 && BN == 128 && CONV == 0) g.group_m = 2;
-    if constexpr (CONV == 0) {
-        if (g.split_len) {
+    if (g.split_len) {                                     // the planner splits K on the smallest tiles only
+        if constexpr (CONV == 0 && BM * BN == 64 * 64) {
             const uint32_t splits = (g.K + g.split_len - 1) / g.split_len;
             hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD, 0, true>), dim3(nb, splits),
                                dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
             return (int)hipGetLastError();
+        } else {
+            return (int)hipErrorInvalidValue;
         }
     }
     hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD, CONV>), dim3(nb),
@@ -603,19 +516,6 @@ int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream)
                                   : launch_dma< 64, 64, 2, 2, 32, 2, true>(args, stream);
     default:           return (int)hipErrorInvalidValue;
     }
-}
-
-int launch_split_reduce(int elem_bytes, const GemmArgs& args, uint32_t splits, hipStream_t stream)
-{
-    const uint64_t threads = (uint64_t)args.M * (args.split_ldd / 4);
-    const dim3 grid((unsigned)((threads + 255) / 256)), block(256);
-    if (elem_bytes == 8)
-        hipLaunchKernelGGL((split_reduce_kernel<double, double>), grid, block, 0, stream, args, splits, args.alpha64, args.beta64);
-    else if (elem_bytes == 2)
-        hipLaunchKernelGGL((split_reduce_kernel<float, _Float16>), grid, block, 0, stream, args, splits, args.alpha, args.beta);
-    else
-        hipLaunchKernelGGL((split_reduce_kernel<float, float>), grid, block, 0, stream, args, splits, args.alpha, args.beta);
-    return (int)hipGetLastError();
 }
 
 // 2-D convolution as an implicit GEMM: M = output pixels, N = output channels, K = kernel rows x (kernel columns x

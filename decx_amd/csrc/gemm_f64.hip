@@ -30,14 +30,6 @@ typedef double doublex2 __attribute__((ext_vector_type(2)));
 typedef double doublex4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void lds_void;
 
-template <int I, int N, class F> __device__ __forceinline__ void static_for(F&& f)
-{
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
-
 template <int N> __device__ __forceinline__ void wait_loads_and_barrier()
 {
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(N) : "memory");
@@ -45,7 +37,8 @@ template <int N> __device__ __forceinline__ void wait_loads_and_barrier()
 
 }  // namespace
 
-// SPLIT: grid.y workgroups share each tile, each with its own range of K, writing a partial product.
+// SPLIT: grid.y workgroups share each tile, each with its own range of K; the one that finishes last adds their
+// partial products (split_k_exchange).
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool SPLIT = false>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_f64_dma_kernel(const GemmArgs g_in)
@@ -58,9 +51,6 @@ gemm_f64_dma_kernel(const GemmArgs g_in)
         g_split.A = (const unsigned char*)g_in.A + (size_t)k0 * 8;
         g_split.B = (const unsigned char*)g_in.B + (size_t)k0 * g_in.ldb * 8;
         g_split.K = g_in.K - k0 < g_in.split_len ? g_in.K - k0 : g_in.split_len;
-        g_split.D = (double*)g_in.split_ws + (size_t)blockIdx.y * g_in.split_stride;
-        g_split.ldd = g_in.split_ldd;
-        g_split.C = nullptr;
     }
     const GemmArgs& g = [&]() -> const GemmArgs& { if constexpr (SPLIT) return g_split; else return g_in; }();
     constexpr int WAVES = WAVES_M * WAVES_N;
@@ -136,12 +126,12 @@ gemm_f64_dma_kernel(const GemmArgs g_in)
         if constexpr (idx < A_LOADS) {
             constexpr int i = idx;
             const uint32_t dst = stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u;
-            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(a_voff[i]), "s"(a_base) : "memory", "m0");
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(a_voff[i]), "s"(a_base) : "memory", "m0");
             if constexpr (i == A_LOADS - 1) a_base += RBYTES;
         } else {
             constexpr int i = idx - A_LOADS;
             const uint32_t dst = stage_off + A_STAGE_BYTES + (uint32_t)(wave * B_LOADS + i) * 1024u;
-            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(b_voff[i]), "s"(b_base) : "memory", "m0");
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(b_voff[i]), "s"(b_base) : "memory", "m0");
             if constexpr (i == B_LOADS - 1) b_base += b_step;
         }
     };
@@ -271,6 +261,27 @@ gemm_f64_dma_kernel(const GemmArgs g_in)
         if (more) wait_loads_and_barrier<LOADS * (STAGES - 2)>(); else wait_loads_and_barrier<0>();
     }
     multiply(std::integral_constant<int, STEPS - 1>{});
+
+    if constexpr (SPLIT) {
+        // piece c of a lane: elements 2 (c % 2), + 1 of its 16 x 16 tile c / 2.  The ring is free: every LDS read
+        // precedes the last slab barrier.
+        const bool last = split_k_exchange<WAVES * 64, TM * TN * 2, doublex2>(g_in, (uint32_t*)lds,
+            [&](auto cc) {
+                constexpr int c = decltype(cc)::value, tile = c / 2, e0 = 2 * (c % 2);
+                const doublex4& a = acc[tile / TN][tile % TN];
+                return doublex2{a[e0], a[e0 + 1]};
+            },
+            [&](auto cc, const doublex2& v, bool first) {
+                constexpr int c = decltype(cc)::value, tile = c / 2, e0 = 2 * (c % 2);
+                doublex4& a = acc[tile / TN][tile % TN];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const double old = a[e0 + e], w = v[e];
+                    a[e0 + e] = first ? w : old + w;
+                }
+            });
+        if (!last) return;
+    }
 
     // Epilogue: element i of tile (ti, tj) is row 16 ti + 4 i + q; tiles 2 jj, 2 jj + 1 are the adjacent columns
     // 32 jj + 2 l16, + 1.
