@@ -91,106 +91,98 @@ int check_gemm(const void* A, const void* B, const void* C, const void* D, uint3
     return DECX_HIP_OK;
 }
 
+// Split K is planned for products on 16-byte aligned operands whose tiles would leave CUs idle or unevenly loaded.
+// The ranges are added inside the kernel (split_k_exchange), so a split costs no second launch, and it runs on one of
+// the smaller tiles whatever the whole product would take.  Tile and number of ranges are the pair that a small model
+// of the kernel's time likes best, in microseconds:
+//   workgroups = tiles x ranges, each as long as its range.  `fit` of them share a CU: whole rounds of fit x CUs
+//   workgroups run at the full-CU rate and the remainder, m on the busiest CU, at the measured rate of m co-resident
+//   workgroups (ns_per_k[m], per workgroup; slopes of time against K at exactly m tiles per CU);
+//   fp32: a remainder of more than half a workgroup per CU right after ONE full round lands unevenly (the CUs that
+//   finish first take several) and counts as two;
+//   fp16 on 128 x 128 tiles: a workgroup that has its CU to itself runs faster the fewer CUs are busy (the power cap);
+//   every range costs a trip of the output through the workspace (us_per_mb) and the last workgroup a round trip to
+//   memory per 16 pieces a lane loads (us_per_trip: where several workgroups share a CU the others hide most of it).
+// fp32 fitted to 20 output shapes x K = 777 ... 16384 x 1 ... 8 ranges, fp16 and fp64 to 12 and 9 shapes x 2 ... 32
+// ranges: the estimate is within 4 % of the measurement on most, the pick within 1 % (fp16: 2.5 %) of the best on
+// average.  The whole product is kept unless the split promises 4 %.
 struct SplitChoice { int shape; uint32_t splits, len; };
+struct SplitTile {
+    int shape, fit, pieces;          // size class, workgroups per CU, 16-byte pieces of accumulators per lane
+    double ns_per_k[5];              // per workgroup with m = 1 .. fit of them on the CU
+};
+struct SplitModel {
+    SplitTile tiles[2]; int n_tiles;
+    uint32_t len_align, acc_bytes;   // ranges are multiples of the deepest slab; bytes of an accumulator
+    double us_fixed, us_per_trip, us_per_mb, whole_flop_per_us;      // the last: the largest tile, per CU of a full chip
+    bool uneven_second_round;
+};
+// 64 x 64 tiles of 32 KB LDS: four fit a CU (160 KB would hold five, but time against the number of tiles steps as for four)
+static const SplitModel kSplitF32 = {{{TILE_SMALL, 4, 4, {0, 17.72, 15.51, 15.07, 14.77}}, {}}, 1, 32, 4, 1.0, 0.4, 0.15, 0.586e6, true};
+static const SplitModel kSplitF16 = {{{TILE_SMALL, 4, 4, {0, 4.33, 3.21, 3.18, 3.07}}, {TILE_MEDIUM, 2, 8, {0, 7.67, 6.95}}}, 2,
+                                     64, 4, 0.5, 2.0, 0.15, 5.2e6, false};
+static const SplitModel kSplitF64 = {{{TILE_SMALL, 2, 4, {0, 34.0, 30.3}}, {}}, 1, 32, 8, 0.5, 2.0, 0.30, 0.283e6, false};
 
-// fp32 splits run on the smallest tile (64 x 64, or 128 x 32 for narrow outputs), whatever the whole product would
-// take, and add their ranges inside the kernel.  The number of ranges is the one a small model of the kernel's time
-// likes best, in microseconds:
-//   workgroups = tiles x ranges, each as long as its range; four fit a CU (32 KB of LDS each: a fifth does not get
-//   in), so whole rounds of 4 x CUs workgroups run at the full-CU rate and the remainder, m on the busiest CU, at
-//   the measured rate of m co-resident workgroups (alone 1 / 1.2 of a full CU, two 1 / 1.05, three 1 / 1.02);
-//   a remainder of more than half a workgroup per CU right after ONE full round lands unevenly (the CUs that finish
-//   first take several): it counts as two;
-//   every range costs a trip of the output through the workspace (0.15 us per MB) and every four ranges a round trip
-//   of the last workgroup's loads.
-// Fitted to 20 output shapes x K = 777 ... 16384 x 1 ... 8 ranges (estimate within 4 % of the measurement on most,
-// the pick within 1 % of the best on average).  The whole product is kept unless the split promises 4 %.
-SplitChoice split_plan_f32(uint32_t M, uint32_t N, uint32_t K, int whole_shape, const TileInfo& whole)
+TileInfo dma_tile_info(int elem_bytes, int shape, uint32_t N);
+
+SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int whole_shape, const TileInfo& whole)
 {
+    const SplitModel& md = elem_bytes == 8 ? kSplitF64 : elem_bytes == 2 ? kSplitF16 : kSplitF32;
     const uint32_t cus = g_dev.compute_units;
-    const TileInfo small = tile_info_f32(TILE_SMALL, true, N);
-    const uint64_t t = (uint64_t)((M + small.bm - 1) / small.bm) * ((N + small.bn - 1) / small.bn);
-    if (K < 512 || t > 4ull * cus) return {whole_shape, 1, 0};
-    constexpr double kTileK = 0.01477;                          // us per tile and k, a CU with four workgroups
-    constexpr double kLaunch = 4.0, kCuFlopPerUs = 0.586e6;     // launch to launch; the largest tile on a full chip
-    static const double rate_loss[5] = {0.0, 1.2, 1.05, 1.02, 1.0};
-    const double out_mb = (double)M * N * 4.0 / 1e6;
-    const auto estimate = [&](uint32_t len, uint32_t ranges) {
-        const uint64_t wgs = t * ranges, slots = 4ull * cus;
+    constexpr double kLaunch = 4.0;                             // launch to launch
+    if (K < 512) return {whole_shape, 1, 0};
+    const double out_mb = (double)M * N * md.acc_bytes / 1e6;
+    const auto tiles_of = [&](int shape) {
+        const TileInfo ti = dma_tile_info(elem_bytes, shape, N);
+        return (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
+    };
+    const auto estimate = [&](const SplitTile& st, uint64_t t, uint32_t len, uint32_t ranges) {
+        const uint64_t wgs = t * ranges, slots = (uint64_t)st.fit * cus;
         const uint64_t full = wgs / slots, rem = wgs % slots;
         uint64_t m = (rem + cus - 1) / cus;
-        if (full == 1 && rem > cus / 2 && rem <= cus) m = 2;
-        const double rounds = 4.0 * (double)full + (double)m * rate_loss[m];
-        return kTileK * len * rounds + kLaunch + 0.15 * ranges * out_mb + 1.0 + 0.4 * ((ranges + 3) / 4);
+        if (md.uneven_second_round && full == 1 && rem > cus / 2 && rem <= cus) m = 2;
+        double lone = st.ns_per_k[1];
+        if (elem_bytes == 2 && st.shape == TILE_MEDIUM)        // 6.0 ns with half the CUs busy, 7.67 with all
+            lone = wgs <= cus / 2 ? 6.0 : 6.0 + 1.67 * (double)(wgs - cus / 2) / (double)(cus - cus / 2);
+        const double ns = (double)len * ((double)full * st.fit * st.ns_per_k[st.fit] + (m == 1 ? lone : (double)m * st.ns_per_k[m]));
+        double us = ns * 1e-3 + kLaunch;
+        if (ranges > 1) {
+            const uint32_t group = st.pieces < 16 ? st.pieces : 16, batch = 16 / group;
+            const uint32_t trips = (ranges + batch - 1) / batch * (st.pieces / group);
+            us += md.us_fixed + md.us_per_trip * trips + md.us_per_mb * ranges * out_mb;
+        }
+        return us;
     };
     const uint64_t whole_tiles = (uint64_t)((M + whole.bm - 1) / whole.bm) * ((N + whole.bn - 1) / whole.bn);
-    const double whole_us = tile_cost(whole, whole_tiles, cus) * 2.0 * K / kCuFlopPerUs + kLaunch;
-    uint32_t best_len = 0, best_ranges = 1;
+    double whole_us = tile_cost(whole, whole_tiles, cus) * 2.0 * K / md.whole_flop_per_us + kLaunch;
+    for (int i = 0; i < md.n_tiles; ++i)                        // the model's own figure where the whole product runs on one of its tiles
+        if (md.tiles[i].shape == whole_shape)
+            whole_us = estimate(md.tiles[i], tiles_of(whole_shape), (K + md.len_align - 1) / md.len_align * md.len_align, 1);
+    SplitChoice best = {whole_shape, 1, 0};
     double best_us = whole_us / 1.04;
     const uint32_t max_p = K / 256 < 64u ? K / 256 : 64u;
-    for (uint32_t p = 2; p <= max_p; ++p) {
-        const uint32_t len = ((K + p - 1) / p + 31) / 32 * 32, ranges = (K + len - 1) / len;
-        if (ranges < 2) continue;
-        const double us = estimate(len, ranges);
-        if (us < best_us) { best_us = us; best_len = len; best_ranges = ranges; }
+    for (int i = 0; i < md.n_tiles; ++i) {
+        const SplitTile& st = md.tiles[i];
+        const uint64_t t = tiles_of(st.shape);
+        if (t > 4ull * cus) continue;
+        for (uint32_t p = 2; p <= max_p && t * p <= 4096; ++p) {
+            const uint32_t len = ((K + p - 1) / p + md.len_align - 1) / md.len_align * md.len_align, ranges = (K + len - 1) / len;
+            if (ranges < 2) continue;
+            const double us = estimate(st, t, len, ranges);
+            if (us < best_us) { best_us = us; best = {st.shape, ranges, len}; }
+        }
     }
-    if (best_ranges > 1) return {TILE_SMALL, best_ranges, best_len};
-    return {whole_shape, 1, 0};
+    return best;
 }
 
-// Split K is planned for products on 16-byte aligned operands whose tiles would leave CUs idle or unevenly loaded.
-// elem_bytes: 2, 4 or 8.  `shape` is the tile the split runs on (it may differ from the one the whole product takes).
+// elem_bytes: 2, 4 or 8.  `shape` of the result is the tile the split runs on (it may differ from the one the whole
+// product takes).
 SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
 {
     if (M == 0 || N == 0) return {0, 1, 0};
     if (M == 1 || N == 1) return {0, 1, 0};                         // the vector corners have their own kernels
-    const uint32_t cus = g_dev.compute_units;
     const int shape = elem_bytes == 8 ? choose_tile_f64(M, N) : choose_tile(elem_bytes == 2, M, N, true);
-    const TileInfo ti = elem_bytes == 8 ? tile_info_f64(shape)
-                                        : elem_bytes == 2 ? tile_info_f16(shape, true) : tile_info_f32(shape, true, N);
-    if (elem_bytes == 4) return split_plan_f32(M, N, K, shape, ti);
-    // outputs of at most half as many tiles as there are CUs: up to two workgroups per CU
-    const SplitPlan sp = plan_split_k((uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn), K, cus);
-    if (sp.splits > 1) return {shape, sp.splits, sp.len};
-    // Outputs of a few hundred small tiles and a long K: one or two workgroups per CU run well below the rate of a
-    // full CU, and 1.5 per CU leave half the chip waiting for the other half.  Measured: fp16 1536 x 1024 x 8192
-    // 57 -> 43 us with 128 x 128 tiles on 2 ranges, 768 x 768 x 16384 61 -> 37 (4 ranges); 2048 x 2048 x 8192 and
-    // 1024 x 2048 x 4096 gain nothing and stay whole.
-    const auto tiles_of = [&](uint32_t b) { return (uint64_t)((M + b - 1) / b) * ((N + b - 1) / b); };
-    if (elem_bytes == 2 && K >= 6144) {
-        // 128 x 128 tiles towards one workgroup per CU, a power of two of ranges at least 2048 long, and only when
-        // that occupies more than half the chip (1024 x 1024 x 6144 on 2 ranges: 26.6 -> 28.9 us)
-        const uint64_t t = tiles_of(128);
-        if (t * 2 < cus) {
-            uint32_t p2 = 1;
-            while (p2 * 2 * t <= cus && p2 < 8 && K / (p2 * 2) >= 2048) p2 *= 2;
-            if (p2 > 1 && t * p2 * 20 >= 11ull * cus) {
-                const uint32_t len = ((K + p2 - 1) / p2 + 31) / 32 * 32;
-                return {TILE_MEDIUM, (K + len - 1) / len, len};
-            }
-        }
-    }
-    if (elem_bytes == 8 && K >= 4096) {
-        // the two smaller tiles, two workgroups per CU each: the ranges that fill whole rounds by the planner's own
-        // estimate (1280 x 1024 x 8192 runs 320 tiles of 64 x 64, 1.25 per CU, at 55 % of peak when whole)
-        int best_shape = shape;
-        uint32_t best = 1;
-        double best_cost = tile_cost(ti, tiles_of((uint32_t)ti.bm), cus) / 1.15;   // ti.bm == ti.bn for the smaller tiles
-        if (ti.bm != ti.bn) best_cost = tile_cost(ti, (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn), cus) / 1.15;
-        for (int sh = TILE_MEDIUM; sh <= TILE_SMALL; ++sh) {
-            const TileInfo t2 = tile_info_f64(sh);
-            const uint64_t t = tiles_of((uint32_t)t2.bm);
-            for (uint32_t p2 = 2; p2 <= 8 && K / p2 >= 1024; ++p2) {
-                const double c = tile_cost(t2, t * p2, cus) / p2 * (1.0 + 0.01 * p2);
-                if (c < best_cost) { best_cost = c; best = p2; best_shape = sh; }
-            }
-        }
-        if (best > 1) {
-            const uint32_t len = ((K + best - 1) / best + 31) / 32 * 32;
-            return {best_shape, (K + len - 1) / len, len};
-        }
-    }
-    return {shape, 1, 0};
+    return split_plan_model(elem_bytes, M, N, K, shape, dma_tile_info(elem_bytes, shape, N));
 }
 
 // Block tile of a size class in the direct-to-LDS family of an element type.
@@ -766,6 +758,11 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
         if (out->edge) { out->tile_m = out->tile_n = 16; out->grid = ((M + 15) / 16) * ((N + 15) / 16); }
         else {
             const SplitChoice sc = split_plan(8, M, N, K);
+            if (sc.splits > 1 && sc.shape != shape) {               // the split runs on another tile than the whole product
+                const TileInfo ts = tile_info_f64(sc.shape);
+                out->path = sc.shape; out->tile_m = ts.bm; out->tile_n = ts.bn;
+                out->grid = ((M + ts.bm - 1) / ts.bm) * ((N + ts.bn - 1) / ts.bn);
+            }
             out->k_splits = sc.splits; out->grid *= out->k_splits;
         }
         return DECX_HIP_OK;

@@ -256,19 +256,7 @@ int launch_gemm_f64(int shape, bool plain, const GemmArgs& args, hipStream_t str
 // direct-to-LDS fp32 kernel for any M, N, K >= 1 on 16-byte aligned bases and pitches, in the three tile shapes
 int launch_gemm_f32_dma(int shape, const GemmArgs& args, hipStream_t stream);
 
-// Split K pays when the tiles alone would leave most CUs without work and K is long enough to cut: aim at two
-// workgroups per CU, pieces of at least 256 and a multiple of 32 (the deepest slab).
-struct SplitPlan { uint32_t splits, len; };
-__host__ inline SplitPlan plan_split_k(uint64_t tiles, uint32_t K, uint32_t cus)
-{
-    if (tiles == 0 || tiles * 2 > cus || K < 1024) return {1, 0};
-    uint32_t splits = (uint32_t)((2ull * cus + tiles - 1) / tiles);
-    if (splits > K / 256) splits = K / 256;
-    if (splits > 64) splits = 64;
-    if (splits < 2) return {1, 0};
-    const uint32_t len = ((K + splits - 1) / splits + 31) / 32 * 32;
-    return {(K + len - 1) / len, len};
-}
+struct SplitPlan { uint32_t splits, len; };     // ranges of K and their length
 // the same kernels with the A operand gathered from an image (GemmArgs::conv_*): 2-D convolution without an im2col buffer
 int launch_conv2d_f32_dma(int shape, const GemmArgs& args, hipStream_t stream);
 // shallow patches and at most 32 kernels: a lane per output pixel on the vector pipe (conv_direct.hip)

@@ -416,15 +416,16 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
 //     than two workgroups per CU are there to hide the copies (1536^3: 447 against 388).
 int launch_gemm_f16_dma(int shape, const GemmArgs& args, hipStream_t stream)
 {
+    const uint32_t splits = args.split_len ? (args.K + args.split_len - 1) / args.split_len : 1u;     // workgroups per tile
     switch (shape) {
     case TILE_LARGE: return launch_dma<256, 256, 2, 4, 64, 2>(args, stream);
     case TILE_MEDIUM: {
-        const uint64_t blocks = (uint64_t)((args.M + 127) / 128) * ((args.N + 127) / 128);
+        const uint64_t blocks = (uint64_t)((args.M + 127) / 128) * ((args.N + 127) / 128) * splits;
         return blocks <= 256 ? launch_dma<128, 128, 2, 4, 64, 4>(args, stream)
                              : launch_dma<128, 128, 2, 4, 64, 2>(args, stream);
     }
     case TILE_SMALL: {
-        const uint64_t blocks = (uint64_t)((args.M + 63) / 64) * ((args.N + 63) / 64);
+        const uint64_t blocks = (uint64_t)((args.M + 63) / 64) * ((args.N + 63) / 64) * splits;
         return blocks <= 512 ? launch_dma<64, 64, 2, 2, 64, 4>(args, stream)
                              : launch_dma<64, 64, 2, 2, 64, 2>(args, stream);
     }

@@ -96,8 +96,13 @@ def test_planner_choices():
     assert hip.plan(4, 2048, 2048, 8192).k_splits == 1 and hip.plan(4, 1280, 1024, 2048).k_splits == 3    # 1.25 tiles per CU: 65.6 -> 47.1 us
     p = hip.plan(2, 1536, 1024, 8192)                      # fp16: 96 tiles of 128 x 128 on 2 ranges
     assert (p.tile_m, p.k_splits) == (128, 2)
-    assert hip.plan(2, 1024, 1024, 6144).k_splits == 1     # 64 tiles on 2 ranges would leave half the chip idle
-    assert hip.plan(2, 768, 768, 16384).k_splits == 4 and hip.plan(2, 2048, 2048, 8192).k_splits == 1
+    p = hip.plan(2, 1024, 1024, 6144)                      # 64 tiles of 128 x 128 on 4 ranges, one per CU: 29.6 -> 23.5 us
+    assert (p.tile_m, p.k_splits) == (128, 4)
+    assert hip.plan(2, 768, 768, 16384).k_splits == 6 and hip.plan(2, 2048, 2048, 8192).k_splits == 1
+    p = hip.plan(2, 300, 300, 8192)                        # few tiles: 8 ranges on 64 x 64 (12.9 us; the 20 that two
+    assert (p.tile_m, p.k_splits) == (64, 8)               # workgroups per CU would ask for: 17.8, the whole product 38.8)
+    p = hip.plan(8, 1280, 1024, 2048)                      # fp64: 320 tiles of 64 x 64 on 4 ranges, 128.5 -> 91.3 us
+    assert (p.tile_m, p.k_splits) == (64, 4)
     p = hip.plan(8, 1280, 1024, 8192)
     assert p.tile_m == 64 and p.k_splits > 1 and hip.plan(8, 4096, 4096, 4096).k_splits == 1
     # the vector corners: rows per workgroup of the row-dot kernel, ranges of K for few columns, fp64 on the same kernels
