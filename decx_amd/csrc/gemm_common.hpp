@@ -96,9 +96,10 @@ template <int I, int N, class F> __device__ __forceinline__ void static_for(F&& 
 // operand lines that workgroups still multiplying live on.  Nobody waits for anybody, so the grid drains in any order.
 // The sum runs GROUP pieces at a time (16 registers of loads in flight next to the accumulators), and tiles with few
 // pieces per lane fetch the same pieces of BATCH slots together (one slot at a time costs a round trip to memory per
-// split).  `flag`: a word of LDS that no wave still reads for anything else.
-template <int NT, int PIECES, typename V, class Get, class Put>
-__device__ __forceinline__ bool split_k_exchange(const GemmArgs& g, uint32_t* flag, Get&& get, Put&& put)
+// split).  `flag`: a word of LDS that no wave still reads for anything else.  on_last() runs in the last workgroup
+// before it loads the first slot.
+template <int NT, int PIECES, typename V, class Get, class Put, class OnLast>
+__device__ __forceinline__ bool split_k_exchange(const GemmArgs& g, uint32_t* flag, Get&& get, Put&& put, OnLast&& on_last)
 {
     static_assert(sizeof(V) == 16, "pieces are 16 bytes");
     constexpr int GROUP = PIECES <= 16 ? PIECES : 16, BATCH = 16 / GROUP;
@@ -130,6 +131,7 @@ __device__ __forceinline__ bool split_k_exchange(const GemmArgs& g, uint32_t* fl
     }
     __syncthreads();
     if (__builtin_amdgcn_readfirstlane(*flag) == 0) return false;
+    on_last();                                             // e.g. the loads of C: in flight together with the first slots
     static_for<0, PIECES / GROUP>([&](auto gc) {
         constexpr int c0 = decltype(gc)::value * GROUP;
         for (uint32_t z0 = 0; z0 < splits; z0 += BATCH) {

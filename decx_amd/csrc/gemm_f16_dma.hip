@@ -312,7 +312,8 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
                     const float old = a[e], w = v[e];
                     a[e] = first ? w : old + w;
                 }
-            });
+            },
+            [] {});
         if (!last) return;
         __syncthreads();                                   // the flag word lies in the rows the epilogue stages through
     }

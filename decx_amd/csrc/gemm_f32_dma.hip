@@ -72,7 +72,7 @@ template <int TN> __device__ __forceinline__ float lane_of(const typename BFrag<
 // plain kernel keeps reading its arguments straight from the kernel-argument segment).  They meet in the workspace:
 // every workgroup stores its accumulators to its slot and counts itself in at the tile's counter; the last one to
 // arrive adds the slots in range order and runs the epilogue.  No workgroup waits for another.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, int CONV = 0, bool SPLIT = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, int CONV = 0, bool SPLIT = false, bool SPLIT_WITH_C = false>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_f32_dma_kernel(const GemmArgs g_in)
 {
@@ -262,6 +262,25 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
 #pragma unroll
     for (int p = 0; p < STAGES - 1; ++p)
         if ((uint32_t)p < slabs) issue_loads(p);
+
+    // Split K on tiles of one 32 x 32 block per wave: the workgroup that finds itself the one to write the tile loads
+    // its 16 values of C per lane together with the first slots, instead of a round trip to memory later, in the
+    // epilogue (1000 x 1500 x 777 with C: 30.2 -> 28.0 us).  It is an instantiation of its own, launched when there is a
+    // C: the 16 registers cost the same kernel WITHOUT C a microsecond (26.1 -> 27.0 us), as fetching C in front of
+    // the K loop cost whole products (1024^3: 21.6 -> 23.0 us), which keep their late loads.
+    constexpr bool C_EARLY = SPLIT_WITH_C;
+    static_assert(!SPLIT_WITH_C || (SPLIT && TM * TN == 1 && CONV == 0), "early C: split K on 32 x 32 wave tiles");
+    float c_early[C_EARLY ? 16 : 1];
+    auto load_c_early = [&]() {
+        const float* __restrict__ Cp = (const float*)g.C;
+        if (!Cp) return;                                   // uniform: products without C pay a scalar branch
+        const uint32_t col = n0 + b_col;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const uint32_t row = m0 + wm0 + 8 * (r / 4) + 4 * h + (r % 4);
+            c_early[r] = (row < g.M && col < g.N) ? Cp[(size_t)row * g.ldc + col] : 0.f;
+        }
+    };
     if (slabs >= (uint32_t)(STAGES - 1)) wait_loads_and_barrier<LOADS * (STAGES - 2)>();
     else wait_loads_and_barrier<0>();
 
@@ -418,7 +437,8 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
                     const float old = a[4 * q + e], w = v[e];
                     a[4 * q + e] = first ? w : old + w;
                 }
-            });
+            },
+            [&] { if constexpr (C_EARLY) load_c_early(); });
         if (!last) return;
     }
 
@@ -439,11 +459,16 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
             float v[TN];
 #pragma unroll
             for (int j = 0; j < TN; ++j) v[j] = acc[i][j][r];
+            if constexpr (C_EARLY) {
+                if (C) v[0] = __builtin_fmaf(c_early[r], g.beta, g.alpha * v[0]);
+            }
             if (interior) {
-                if (C) {
-                    const bfrag cv = *(const bfrag*)(C + (size_t)row * g.ldc + col0);
+                if constexpr (!C_EARLY) {
+                    if (C) {
+                        const bfrag cv = *(const bfrag*)(C + (size_t)row * g.ldc + col0);
 #pragma unroll
-                    for (int j = 0; j < TN; ++j) v[j] = __builtin_fmaf(lane_of<TN>(cv, j), g.beta, g.alpha * v[j]);
+                        for (int j = 0; j < TN; ++j) v[j] = __builtin_fmaf(lane_of<TN>(cv, j), g.beta, g.alpha * v[j]);
+                    }
                 }
                 bfrag o;
                 if constexpr (TN == 1) o = v[0];
@@ -457,7 +482,9 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
                 for (int j = 0; j < TN; ++j) {
                     if (col0 + j < g.N) {
                         float o = v[j];
-                        if (C) o = __builtin_fmaf(C[(size_t)row * g.ldc + col0 + j], g.beta, g.alpha * o);
+                        if constexpr (!C_EARLY) {
+                            if (C) o = __builtin_fmaf(C[(size_t)row * g.ldc + col0 + j], g.beta, g.alpha * o);
+                        }
                         D[d_row + col0 + j] = o;
                     }
                 }
@@ -481,8 +508,12 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     if (g.split_len) {                                     // the planner splits K on the smallest tiles only
         if constexpr (CONV == 0 && BM * BN == 64 * 64) {
             const uint32_t splits = (g.K + g.split_len - 1) / g.split_len;
-            hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD, 0, true>), dim3(nb, splits),
-                               dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
+            if (g.C)
+                hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD, 0, true, true>),
+                                   dim3(nb, splits), dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
+            else
+                hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD, 0, true, false>),
+                                   dim3(nb, splits), dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
             return (int)hipGetLastError();
         } else {
             return (int)hipErrorInvalidValue;

@@ -279,7 +279,8 @@ gemm_f64_dma_kernel(const GemmArgs g_in)
                     const double old = a[e0 + e], w = v[e];
                     a[e0 + e] = first ? w : old + w;
                 }
-            });
+            },
+            [] {});
         if (!last) return;
     }
 
