@@ -571,21 +571,30 @@ def test_stream_and_events(hip):
     assert L.decx_hip_stream_destroy(s) == 0
 
 
-@pytest.mark.parametrize("M,N,K", [(300, 300, 8192), (1280, 1024, 8192), (1000, 1500, 777)])
-def test_f32_split_k_slots_carry_nothing_from_launch_to_launch(hip, oracle, M, N, K):
+@pytest.mark.parametrize("dtype,M,N,K", [
+    (np.float32, 300, 300, 8192), (np.float32, 1280, 1024, 8192), (np.float32, 1000, 1500, 777),
+    (np.float16, 300, 300, 8192), (np.float16, 1280, 1024, 6144), (np.float16, 640, 640, 8192),
+    (np.float64, 300, 300, 8192), (np.float64, 1280, 1024, 2048),
+])
+def test_split_k_slots_carry_nothing_from_launch_to_launch(hip, oracle, dtype, M, N, K):
     """The workgroups of a tile meet in the workspace (slots written and read at device scope, a counter per tile
     that ends every launch at zero).  Two input sets take turns on the same workspace: a slot, a cache line or a
     counter left over from the launch before would show as a result that differs from the set's first one."""
-    need = hip.lib().decx_hip_gemm_f32_workspace(M, N, K)
-    if need == 0:
+    esz = np.dtype(dtype).itemsize
+    need = hip.lib().decx_hip_gemm_workspace(esz, M, N, K)
+    if need == 0 or hip.plan(esz, M, N, K).k_splits < 2:
         pytest.skip("the planner does not split this shape")
     ws = hip.DeviceMatrix(1, need // 4, np.float32)
-    pa, pn = device_pitch(K, np.float32), device_pitch(N, np.float32)
+    pa, pn = device_pitch(K, dtype), device_pitch(N, dtype)
+    make = {2: synth.normal_half, 4: synth.uniform_f32, 8: synth.uniform_f64}[esz]
+    ref = {2: oracle.gemm_f16, 4: oracle.gemm_f32, 8: oracle.gemm_f64}[esz]
+    tol = {2: TOL_F16, 4: TOL_F32, 8: 1e-14}[esz]
+    bits = {2: np.uint16, 4: np.uint32, 8: np.uint64}[esz]
     sets = []
     for s in range(2):
-        A = synth.uniform_f32(M, K, 700 + s); B = synth.uniform_f32(K, N, 710 + s)
-        sets.append((A, B, hip.DeviceMatrix(M, K, np.float32, pa, A), hip.DeviceMatrix(K, N, np.float32, pn, B)))
-    dD = hip.DeviceMatrix(M, N, np.float32, pn)
+        A = make(M, K, 700 + s); B = make(K, N, 710 + s)
+        sets.append((A, B, hip.DeviceMatrix(M, K, dtype, pa, A), hip.DeviceMatrix(K, N, dtype, pn, B)))
+    dD = hip.DeviceMatrix(M, N, dtype, pn)
     first = [None, None]
     for it in range(60):
         A, B, dA, dB = sets[it % 2]
@@ -596,8 +605,8 @@ def test_f32_split_k_slots_carry_nothing_from_launch_to_launch(hip, oracle, M, N
             if first[it % 2] is None:
                 first[it % 2] = got
                 rows = np.arange(0, M, max(1, M // 24), dtype=np.uint32)
-                assert rel_err(got[rows], oracle.gemm_f32(A, B, rows=rows), K) <= TOL_F32
+                assert rel_err(got[rows], ref(A, B, rows=rows), K) <= tol
             else:
-                assert np.array_equal(got.view(np.uint32), first[it % 2].view(np.uint32)), "launch %d" % it
+                assert np.array_equal(got.view(bits), first[it % 2].view(bits)), "launch %d" % it
     for d in [ws, dD] + [x for t in sets for x in t[2:]]:
         d.free()
