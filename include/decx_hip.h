@@ -118,17 +118,17 @@ DECX_HIP_API int decx_hip_gemm_f32(const float* A, const float* B, const float* 
                                    uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
                                    float alpha, float beta, void* stream);
 
-/* The same product with a device workspace the library may use to split K: when the output has too few tiles to
- * occupy the chip and K is long (e.g. 300 x 300 x 8192), several workgroups share a tile, each multiplying a
- * range of K into a partial product in the workspace, and a second kernel adds the partial products in a fixed
- * order (results do not vary from run to run).  decx_hip_gemm_f32_workspace returns the bytes that make the
+/* The same product with a device workspace the library may use to split K: when the tiles of the output would leave
+ * CUs idle or unevenly loaded (e.g. 300 x 300 x 8192, 1280 x 1024 x 8192), several workgroups share a tile, each
+ * multiplying a range of K and leaving its partial product in the workspace, and the one of them that finishes last
+ * adds the partial products in a fixed order (results do not vary from run to run) and writes the tile: one launch.  decx_hip_gemm_f32_workspace returns the bytes that make the
  * split possible for a shape (0: the plain kernel is used anyway); a smaller or null workspace is never an
  * error.  The workspace must be 16-byte aligned and is free again when the call's work on `stream` is done.
  * For N == 1 (fp32, fp16) the workspace serves another purpose: B is then the single column of a pitched K x 1
  * matrix, every element in a cache line of its own, and with K * elem_bytes of workspace it is copied once into
  * a dense vector in front of the matrix-vector kernel (8192 x 8192: 46.9 -> 43.9 us); the query returns that
  * size where the copy pays.  For M == 1 with few columns and a long K (1 x 512 x 32768) ranges of K go to workgroups
- * of their own, their partial sums to the workspace, and a second kernel adds them in range order (69 -> 23 us).
+ * of their own, their partial sums to the workspace, and the last of a column group adds them in range order (69 -> 23 us).
  * Plays the part of the scratch the reference's planner keeps for itself (cuda_GEMM_LS_planner: the transposed
  * A, srcs/modules/BLAS/GEMM/CUDA/large_squares/common/cuda_GEMM_LS_planner.cu:95-160). */
 DECX_HIP_API size_t decx_hip_gemm_f32_workspace(uint32_t M, uint32_t N, uint32_t K);
@@ -223,11 +223,11 @@ DECX_HIP_API int decx_hip_gevm_f16(const uint16_t* x, const uint16_t* B, const u
                                    uint32_t incx, uint32_t incc, uint32_t incy,
                                    float alpha, float beta, int y_is_f32, void* stream);
 /* Vector x matrix with a device workspace (decx_hip_gemm_workspace(elem_bytes, 1, N, K) bytes, 16-byte aligned): when
- * the matrix has few columns and a long K, ranges of K go to workgroups of their own and a second kernel adds their
- * partial sums in a fixed order -- the part of the reference's second pass reduce_sum2D_v_fp32_Async behind
- * cu_vec_m_mat_fp32 (srcs/modules/BLAS/GEMM/CUDA/extreme_shapes/VMM_callers.cuh:67-202), taken only where one
- * kernel would leave most CUs idle.  Needs incy == 1 (and incc == 1, c of y's type); otherwise, or with a smaller or
- * null workspace, the single-kernel path runs. */
+ * the matrix has few columns and a long K, ranges of K go to workgroups of their own and the last of a column group to
+ * finish adds their partial sums in a fixed order -- the part of the reference's second pass reduce_sum2D_v_fp32_Async
+ * behind cu_vec_m_mat_fp32 (srcs/modules/BLAS/GEMM/CUDA/extreme_shapes/VMM_callers.cuh:67-202), inside the one
+ * kernel and taken only where whole columns per workgroup would leave most CUs idle.  With a smaller or null workspace
+ * every workgroup sums its columns over all of K. */
 DECX_HIP_API int decx_hip_gevm_f32_ws(const float* x, const float* B, const float* c, float* y,
                                       uint32_t K, uint32_t N, uint32_t ldb,
                                       uint32_t incx, uint32_t incc, uint32_t incy,

@@ -120,7 +120,7 @@ def test_gevm_against_oracle(hip, oracle, tin, tout, tol, K, N, strided):
 @pytest.mark.parametrize("K,N", [(8192, 2048), (33000, 100)])
 def test_gevm_split_over_k_through_a_workspace(hip, oracle, tin, tout, tol, K, N):
     """Few columns and a long K through decx_hip_gevm_*_ws: ranges of K on workgroups of their own, partial sums added
-    in range order.  Strided x is fine; a strided y, or a c the second kernel cannot read, take the single kernel."""
+    in range order by the last workgroup of each column group.  Dense and strided x, y and c."""
     esz = np.dtype(tin).itemsize
     B = inputs(tin, K, N, 221); x = inputs(tin, 1, K, 222).reshape(-1); c = inputs(tin, 1, N, 223).reshape(-1)
     need = hip.lib().decx_hip_gemm_workspace(esz, 1, N, K)
