@@ -83,11 +83,12 @@ MEASURED_TRAFFIC = {
 
 
 def sources_sha256(source):
-    """SHA-256 over a kernel's source file and the header all kernels share (block -> tile map, split-K exchange)."""
+    """SHA-256 over a kernel's source file and the headers the kernels share: the argument block and block -> tile map,
+    and where the ranges of a split K meet."""
     import hashlib
     h = hashlib.sha256()
     try:
-        for f in (source, "decx_amd/csrc/gemm_common.hpp"):
+        for f in (source, "decx_amd/csrc/gemm_common.hpp", "decx_amd/csrc/split_k_exchange.hpp"):
             h.update(open(os.path.join(ROOT, f), "rb").read())
     except OSError:
         return None

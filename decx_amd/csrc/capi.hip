@@ -3,6 +3,7 @@
 #include "../../include/decx_hip.h"
 #include "../../include/decx_hip_profiling.h"
 #include "gemm_common.hpp"
+#include "split_k_exchange.hpp"
 
 #include <cstring>
 #include <mutex>
@@ -28,10 +29,11 @@ constexpr int kMaxDevices = 16;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 void* g_scratch[kMaxDevices] = {};
 
-// Tile counters of the fp32 split-K kernels (one per tile; the workgroups of a tile count themselves in, the last
-// one sums the tile and puts its counter back to zero, so the array is all zero between launches).  Every launch
-// takes the next window of the array, so that launches in flight on different streams do not share counters as
-// long as their windows together stay below kSplitCounters.
+// Counters of the split-K kernels (per tile, or per column group of a vector x matrix product: one, plus one per group
+// of ranges when there are many; the workgroups of a tile count themselves in, the last one sums the tile and puts
+// the counter back to zero, so the array is all zero between launches).  Every launch takes the next window of the
+// array, so that launches in flight on different streams do not share counters as long as their windows together
+// stay below kSplitCounters.
 constexpr uint32_t kSplitCounters = 1u << 16;
 static __device__ uint32_t split_counters[kSplitCounters];
 uint32_t* g_split_counters[kMaxDevices] = {};
@@ -147,8 +149,10 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
         const double ns = (double)len * ((double)full * st.fit * st.ns_per_k[st.fit] + (m == 1 ? lone : (double)m * st.ns_per_k[m]));
         double us = ns * 1e-3 + kLaunch;
         if (ranges > 1) {
-            const uint32_t group = st.pieces < 16 ? st.pieces : 16, batch = 16 / group;
-            const uint32_t trips = (ranges + batch - 1) / batch * (st.pieces / group);
+            const uint32_t group = st.pieces < 16 ? st.pieces : 16, batch = 16 / group, per_slot = st.pieces / group;
+            uint32_t trips = (ranges + batch - 1) / batch * per_slot;
+            if (ranges > kSplitFlat)                           // two levels: a group of kSplitGroup, the group sums, and a second store and count
+                trips = ((kSplitGroup + batch - 1) / batch + ((ranges + kSplitGroup - 1) / kSplitGroup + batch - 1) / batch) * per_slot + 1;
             us += md.us_fixed + md.us_per_trip * trips + md.us_per_mb * ranges * out_mb;
         }
         return us;
@@ -165,7 +169,8 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
         const SplitTile& st = md.tiles[i];
         const uint64_t t = tiles_of(st.shape);
         if (t > 4ull * cus) continue;
-        for (uint32_t p = 2; p <= max_p && t * p <= 4096; ++p) {
+        const uint32_t tile_max_p = st.shape == TILE_SMALL ? max_p : (max_p < kSplitFlat ? max_p : kSplitFlat);     // only the smallest tiles sum on two levels
+        for (uint32_t p = 2; p <= tile_max_p && t * p <= 4096; ++p) {
             const uint32_t len = ((K + p - 1) / p + md.len_align - 1) / md.len_align * md.len_align, ranges = (K + len - 1) / len;
             if (ranges < 2) continue;
             const double us = estimate(st, t, len, ranges);
@@ -209,7 +214,8 @@ uint32_t arm_split(GemmArgs& g, int elem_bytes, void* workspace, size_t workspac
     if (sp.splits <= 1 || workspace_bytes < split_workspace_bytes(elem_bytes, sp.shape, g.M, g.N, sp.splits)) return 1;
     const TileInfo ti = dma_tile_info(elem_bytes, sp.shape, g.N);
     const uint64_t tiles = (uint64_t)((g.M + ti.bm - 1) / ti.bm) * ((g.N + ti.bn - 1) / ti.bn);
-    uint32_t* const counters = tiles <= kSplitCounters ? take_split_counters((uint32_t)tiles) : nullptr;
+    const uint64_t n_counters = tiles * split_counters_per_tile(sp.splits);
+    uint32_t* const counters = n_counters <= kSplitCounters ? take_split_counters((uint32_t)n_counters) : nullptr;
     if (!counters) return 1;
     g.split_counters = counters;
     g.split_len = sp.len; g.split_ws = workspace;

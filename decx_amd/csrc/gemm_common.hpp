@@ -33,7 +33,7 @@ struct GemmArgs {
     // min(K, (z + 1) * split_len)).  Every workgroup stores its accumulators (fp32, or fp64 for fp64 operands) to its
     // slot of split_ws and counts itself in at split_counters[tile]; the one that arrives last adds all slots of the
     // tile in split order (its own included, so the result does not depend on who is last), writes D and puts the
-    // counter back to zero (split_k_exchange below).
+    // counter back to zero (split_k_exchange.hpp).
     uint32_t group_m;            // tile-rows per L2 patch of the block -> tile map (0: the default, kGroupM)
     uint32_t split_len;          // 0: no split
     void*    split_ws;
@@ -74,95 +74,6 @@ __device__ __forceinline__ void block_to_tile(const GemmArgs& g, uint32_t& tile_
     const uint32_t in_group = id % per_group;
     tile_m = first_m + in_group % rows;
     tile_n = in_group / rows;
-}
-
-// Compile-time loop: f(std::integral_constant<int, I>{}) for I in [I, N).
-template <int I, int N, class F> __device__ __forceinline__ void static_for(F&& f)
-{
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
-
-// Where the workgroups that share a split-K tile meet (grid = (tiles, splits), NT threads each).  A lane's accumulators
-// are PIECES 16-byte pieces, piece c read by get(c) and given back by put(c, value, first): put stores `value` when
-// `first`, else adds it.  Every workgroup writes its pieces to its slot of the workspace, [piece][thread] so that a wave
-// writes whole lines, and counts itself in; the function returns false in all but the workgroup that arrives last,
-// and in that one after it has summed every slot in split order (its own included: the sum does not depend on who is
-// last) into the accumulators and put the counter back to zero.
-// Slots are written and read with device-scope accesses (`sc1`: they pass the XCD's own L2, which is not coherent with
-// the other seven), so no cache-wide write-back or invalidation is needed around the count -- those would throw out the
-// operand lines that workgroups still multiplying live on.  Nobody waits for anybody, so the grid drains in any order.
-// The sum runs GROUP pieces at a time (16 registers of loads in flight next to the accumulators), and tiles with few
-// pieces per lane fetch the same pieces of BATCH slots together (one slot at a time costs a round trip to memory per
-// split).  `flag`: a word of LDS that no wave still reads for anything else.  on_last() runs in the last workgroup
-// before it loads the first slot.
-template <int NT, int PIECES, typename V, class Get, class Put, class OnLast>
-__device__ __forceinline__ bool split_k_exchange(const GemmArgs& g, uint32_t* flag, Get&& get, Put&& put, OnLast&& on_last)
-{
-    static_assert(sizeof(V) == 16, "pieces are 16 bytes");
-    constexpr int GROUP = PIECES <= 16 ? PIECES : 16, BATCH = 16 / GROUP;
-    static_assert(PIECES % GROUP == 0 && GROUP * BATCH == 16, "pieces per lane: 1, 2, 4, 8, or a multiple of 16");
-    const int t = threadIdx.x;
-    const uint32_t splits = gridDim.y;
-    constexpr size_t SLOT = (size_t)NT * PIECES;           // pieces per slot
-    V* const slots = (V*)g.split_ws + (size_t)blockIdx.x * splits * SLOT;
-    V* const mine = slots + (size_t)blockIdx.y * SLOT;
-    // The stores below are inline asm, and the compiler does not count the wait states an MFMA needs before its result
-    // registers may be read for an instruction it cannot see into (accumulators that live in VGPRs go to the stores
-    // without a copy in between): every MFMA stays in front of the fence and has drained behind it.
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-    static_for<0, PIECES>([&](auto cc) {
-        constexpr int c = decltype(cc)::value;
-        const V v = get(cc);
-        V* const dst = mine + (size_t)c * NT + t;
-        // s_nop: a store of more than 64 bits reads its data registers up to two cycles after it issues, and the
-        // compiler, which inserts that gap for its own stores, does not know that this is one
-        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" :: "v"(dst), "v"(v) : "memory");
-    });
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // this lane's stores have arrived
-    __syncthreads();                                       // everyone's have
-    if (t == 0) {
-        const uint32_t before = __hip_atomic_fetch_add(g.split_counters + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        *flag = (before + 1 == splits) ? 1u : 0u;
-    }
-    __syncthreads();
-    if (__builtin_amdgcn_readfirstlane(*flag) == 0) return false;
-    on_last();                                             // e.g. the loads of C: in flight together with the first slots
-    static_for<0, PIECES / GROUP>([&](auto gc) {
-        constexpr int c0 = decltype(gc)::value * GROUP;
-        for (uint32_t z0 = 0; z0 < splits; z0 += BATCH) {
-            V v[BATCH][GROUP];
-#pragma unroll
-            for (int zb = 0; zb < BATCH; ++zb) {
-                if (zb == 0 || z0 + zb < splits) {         // slots beyond the last split are neither loaded nor added
-                    const V* const p = slots + (size_t)(z0 + zb) * SLOT;
-#pragma unroll
-                    for (int c = 0; c < GROUP; ++c) {
-                        const V* const src = p + (size_t)(c0 + c) * NT + t;
-                        asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[zb][c]) : "v"(src) : "memory");
-                    }
-                }
-            }
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#pragma unroll
-            for (int zb = 0; zb < BATCH; ++zb) {
-                if (zb == 0 || z0 + zb < splits) {
-#pragma unroll
-                    for (int c = 0; c < GROUP; ++c) asm volatile("" : "+v"(v[zb][c]));     // not before the wait above
-                    static_for<0, GROUP>([&](auto cc) {
-                        constexpr int c = decltype(cc)::value;
-                        put(std::integral_constant<int, c0 + c>{}, v[zb][c], z0 + zb == 0);
-                    });
-                }
-            }
-        }
-    });
-    if (t == 0) __hip_atomic_store(g.split_counters + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return true;
 }
 
 // ---- tile-shape table shared by the planner and the launchers -----------------

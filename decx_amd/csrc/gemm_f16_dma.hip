@@ -39,6 +39,7 @@
 // of the transposing read takes 4 k rows x 32 bytes from each of two k groups 8 rows apart, and the 16
 // pieces land in 16 different bank groups.  Both permutations are applied on the global side of the copy.
 #include "gemm_common.hpp"
+#include "split_k_exchange.hpp"
 #include <type_traits>
 
 namespace decx_hip {
@@ -302,7 +303,7 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     if constexpr (SPLIT) {
         // piece c of a lane: the four fp32 accumulators of its 16 x 16 tile (c % TM, c / TM).  The ring is free: every
         // LDS read precedes the last slab barrier.
-        const bool last = split_k_exchange<WAVES * 64, TM * TN, floatx4>(g_in, (uint32_t*)lds,
+        const bool last = split_k_exchange<WAVES * 64, TM * TN, floatx4, (BM <= 64)>(g_in, (uint32_t*)lds,
             [&](auto cc) { constexpr int c = decltype(cc)::value; return accT[c / TM][c % TM]; },
             [&](auto cc, const floatx4& v, bool first) {
                 constexpr int c = decltype(cc)::value;
@@ -315,7 +316,6 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
             },
             [] {});
         if (!last) return;
-        __syncthreads();                                   // the flag word lies in the rows the epilogue stages through
     }
     const _Float16* __restrict__ C = (const _Float16*)g.C;
     _Float16* __restrict__ D = (_Float16*)g.D;
@@ -391,11 +391,15 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
-    if (g.split_len) {
-        const uint32_t splits = (g.K + g.split_len - 1) / g.split_len;
-        hipLaunchKernelGGL((gemm_f16_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, true>), dim3(nb, splits),
-                           dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
-        return (int)hipGetLastError();
+    if (g.split_len) {                                     // the planner splits K on the two smaller tiles only
+        if constexpr (BM <= 128) {
+            const uint32_t splits = (g.K + g.split_len - 1) / g.split_len;
+            hipLaunchKernelGGL((gemm_f16_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, true>), dim3(nb, splits),
+                               dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
+            return (int)hipGetLastError();
+        } else {
+            return (int)hipErrorInvalidValue;
+        }
     }
     hipLaunchKernelGGL((gemm_f16_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES>), dim3(nb), dim3(WAVES_M * WAVES_N * 64),
                        0, stream, g);

@@ -22,6 +22,7 @@
 // within a lane half; epilogue D = fma(C, beta, alpha * acc) as the reference's F kernels
 // do (GEMM_fp32_B128_kernels.cu:725-744).
 #include "gemm_common.hpp"
+#include "split_k_exchange.hpp"
 
 #include <type_traits>
 

@@ -41,6 +41,7 @@
 // are shifted by 128 bytes so the two half-waves read different banks.  Both permutations
 // are applied on the global side of the copy: a direct load always writes 1 KB contiguous.
 #include "gemm_common.hpp"
+#include "split_k_exchange.hpp"
 #include <type_traits>
 
 namespace decx_hip {

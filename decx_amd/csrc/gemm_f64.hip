@@ -20,6 +20,7 @@
 //
 // A plain one-thread-per-element kernel serves operands that are not 16-byte aligned, and K == 0.
 #include "gemm_common.hpp"
+#include "split_k_exchange.hpp"
 #include <type_traits>
 
 namespace decx_hip {
@@ -344,11 +345,15 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
-    if (g.split_len) {
-        const uint32_t splits = (g.K + g.split_len - 1) / g.split_len;
-        hipLaunchKernelGGL((gemm_f64_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, true>), dim3(nb, splits),
-                           dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
-        return (int)hipGetLastError();
+    if (g.split_len) {                                     // the planner splits K on the smallest tile only
+        if constexpr (BM == 64) {
+            const uint32_t splits = (g.K + g.split_len - 1) / g.split_len;
+            hipLaunchKernelGGL((gemm_f64_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, true>), dim3(nb, splits),
+                               dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
+            return (int)hipGetLastError();
+        } else {
+            return (int)hipErrorInvalidValue;
+        }
     }
     hipLaunchKernelGGL((gemm_f64_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES>), dim3(nb), dim3(WAVES_M * WAVES_N * 64),
                        0, stream, g);

@@ -575,6 +575,8 @@ def test_stream_and_events(hip):
     (np.float32, 300, 300, 8192), (np.float32, 1280, 1024, 8192), (np.float32, 1000, 1500, 777),
     (np.float16, 300, 300, 8192), (np.float16, 1280, 1024, 6144), (np.float16, 640, 640, 8192),
     (np.float64, 300, 300, 8192), (np.float64, 1280, 1024, 2048),
+    # more than 8 ranges: groups of four are added first, then the group sums
+    (np.float32, 100, 120, 20000), (np.float16, 128, 128, 16384), (np.float16, 70, 130, 40000), (np.float64, 100, 120, 4096),
 ])
 def test_split_k_slots_carry_nothing_from_launch_to_launch(hip, oracle, dtype, M, N, K):
     """The workgroups of a tile meet in the workspace (slots written and read at device scope, a counter per tile
@@ -584,6 +586,8 @@ def test_split_k_slots_carry_nothing_from_launch_to_launch(hip, oracle, dtype, M
     need = hip.lib().decx_hip_gemm_workspace(esz, M, N, K)
     if need == 0 or hip.plan(esz, M, N, K).k_splits < 2:
         pytest.skip("the planner does not split this shape")
+    if K >= 16384 or (M, N) == (100, 120):
+        assert hip.plan(esz, M, N, K).k_splits > 8
     ws = hip.DeviceMatrix(1, need // 4, np.float32)
     pa, pn = device_pitch(K, dtype), device_pitch(N, dtype)
     make = {2: synth.normal_half, 4: synth.uniform_f32, 8: synth.uniform_f64}[esz]
