@@ -5,6 +5,7 @@
 #include "gemm_common.hpp"
 #include "split_k_exchange.hpp"
 
+#include <chrono>
 #include <cstring>
 #include <mutex>
 
@@ -418,7 +419,17 @@ int decx_hip_stream_create(void** stream)
     return hip_rc(e);
 }
 int decx_hip_stream_destroy(void* stream) { return stream ? hip_rc(hipStreamDestroy(as_stream(stream))) : DECX_HIP_OK; }
-int decx_hip_stream_sync(void* stream) { return hip_rc(hipStreamSynchronize(as_stream(stream))); }
+// Polls for a quarter of a millisecond before it blocks: a blocking wait is woken by an interrupt, some 10 us after the
+// work is done, which is a tenth of an fp16 4096^3 product.
+int decx_hip_stream_sync(void* stream)
+{
+    const auto t0 = std::chrono::steady_clock::now();
+    do {
+        const hipError_t e = hipStreamQuery(as_stream(stream));
+        if (e != hipErrorNotReady) return hip_rc(e);
+    } while (std::chrono::steady_clock::now() - t0 < std::chrono::microseconds(250));
+    return hip_rc(hipStreamSynchronize(as_stream(stream)));
+}
 
 int decx_hip_event_create(void** event)
 {
