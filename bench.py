@@ -204,7 +204,7 @@ CONV = {"W": 256, "H": 256, "C": 112, "OC": 256, "KW": 3, "KH": 3}     # 64 516 
 CONV_RGB = {"W": 1920, "H": 1080, "C": 3, "OC": 8, "KW": 3, "KH": 3}    # a filter bank over an RGB frame: 36 taps, bound by HBM
 
 
-def run_conv(steps, warmup, settle_s=0.25, c=None):
+def run_conv(steps, warmup, settle_s=0.25, c=None, parity=False):
     """fp32 3 x 3 convolution of a 256 x 256 x 112 image with 256 kernels through decx_hip_conv2d_f32_depth (implicit GEMM,
     operands resident): the workload the tall-skinny GEMM shape 65536 x 256 x 1024 stands for.  c: another
     configuration (CONV_RGB: a shallow patch and few kernels, which the library runs a lane per output pixel)."""
@@ -252,12 +252,28 @@ def run_conv(steps, warmup, settle_s=0.25, c=None):
         roof.update(traffic_fields("conv2d_rgb"))
     out = {"workload": desc, "dtype": "f32", "value": round(tf, 3), "unit": "TFLOP/s", "hbm_gbs_algorithmic": round(gbs, 1),
            "kernel_ms": round(ms, 5), "roofline": roof}
+    if parity:
+        # bands of output rows against the oracle's fmaf chain over (kernel row, kernel column, channel) on the image
+        # rows under them
+        from oracle import binding as oracle
+        got = d_out.download().reshape(oh, owp, c["OC"])[:, :ow, :]
+        kernels = kmat.reshape(c["KH"], c["KW"], dp, c["OC"])[:, :, :c["C"], :].transpose(3, 0, 1, 2)
+        worst, scale, count = 0.0, 1e-30, 0
+        for r0 in (0, oh // 2 - 1, oh - 2):
+            ref = oracle.conv2d_f32(img[r0:r0 + 2 + c["KH"] - 1, :c["W"], :c["C"]], kernels).astype(np.float64)
+            worst = max(worst, float(np.max(np.abs(got[r0:r0 + 2].astype(np.float64) - ref))))
+            scale = max(scale, float(np.max(np.abs(ref)))); count += ref.size
+        taps = c["KH"] * c["KW"] * c["C"]
+        out["cpu_baseline"] = None               # the reference has no CPU convolution
+        out["gpu_parity"] = {"rel_err": float("%.3g" % (worst / (scale * math.sqrt(taps)))), "bar": 1e-5, "elements": count,
+                             "against": "fmaf chain oracle (oracle/conv_oracle.c)",
+                             "measure": "max|gpu - chain| / (max|chain| sqrt(taps)) over 6 output rows"}
     for d in (d_img, d_kmat, d_out):
         d.free()
     return out
 
 
-def run_complex(double, n, steps, warmup, settle_s=0.25):
+def run_complex(double, n, steps, warmup, settle_s=0.25, parity=False):
     """Complex GEMM D = A.B (interleaved re / im, n x n x n) through decx_hip_gemm_c32 / _c64 with a caller-held
     workspace: one pass expanding B, then one real GEMM on the fp32 / fp64 matrix pipe.  8 real flops per complex
     multiply-add; the expansion pass is inside the timed region."""
@@ -290,6 +306,19 @@ def run_complex(double, n, steps, warmup, settle_s=0.25):
            "hbm_gbs_algorithmic": round(3.0 * n * n * 2 * rb / (ms * 1e-3) / 1e9, 1), "kernel_ms": round(ms, 5),
            "roofline": {"bound": "mfma", "achieved": round(tf, 3), "peak": peak, "unit": "TFLOP/s", "frac": round(tf / peak, 4),
                         "traffic": None}}
+    if parity:
+        # sampled rows against the real chain oracle on the same expansion of B
+        from oracle import binding as oracle
+        rt = np.float64 if double else np.float32
+        pick = np.unique(np.concatenate([[0, n - 1], np.random.default_rng(1).integers(0, n, 14)])).astype(np.uint32)
+        fn = oracle.gemm_f64 if double else oracle.gemm_f32
+        ref = fn(np.ascontiguousarray(a).view(rt), oracle.complex_embed(b), rows=pick).astype(np.float64)
+        got = np.ascontiguousarray(dD.download()[pick]).view(rt).astype(np.float64)
+        err = float(np.max(np.abs(got - ref))) / (float(np.max(np.abs(ref))) * math.sqrt(2 * n))
+        out["cpu_baseline"] = None               # the reference's complex CPU GEMM is not restated as a timed port
+        out["gpu_parity"] = {"rel_err": float("%.3g" % err), "bar": 1e-14 if double else 1e-5, "elements": int(len(pick)) * 2 * n,
+                             "against": "fma chain oracle on the real expansion",
+                             "measure": "max|gpu - chain| / (max|chain| sqrt(2K)) over %d sampled rows" % len(pick)}
     for d in (dA, dB, dD, ws):
         d.free()
     return out
@@ -434,10 +463,10 @@ def main():
         return
 
     if args.workload in ("conv2d", "conv2d_rgb"):
-        print(json.dumps(run_conv(args.steps, args.warmup, c=CONV if args.workload == "conv2d" else CONV_RGB)))
+        print(json.dumps(run_conv(args.steps, args.warmup, c=CONV if args.workload == "conv2d" else CONV_RGB, parity=not args.no_cpu)))
         return
     if args.workload in ("c64_4096", "c128_2048"):
-        print(json.dumps(run_complex(args.workload == "c128_2048", 4096 if args.workload == "c64_4096" else 2048, args.steps, args.warmup)))
+        print(json.dumps(run_complex(args.workload == "c128_2048", 4096 if args.workload == "c64_4096" else 2048, args.steps, args.warmup, parity=not args.no_cpu)))
         return
 
     main_out, inputs = run_workload(args.workload, args.steps, args.warmup, keep_inputs=not args.no_cpu,
@@ -469,10 +498,10 @@ def main():
                     o["api_wall"] = api16
                 others.append(o)
                 del inp
-        others.append(run_conv(200, args.warmup))
-        others.append(run_conv(200, args.warmup, c=CONV_RGB))
-        others.append(run_complex(False, 4096, args.steps, args.warmup))
-        others.append(run_complex(True, 2048, 50, args.warmup))
+        others.append(run_conv(200, args.warmup, parity=not args.no_cpu))
+        others.append(run_conv(200, args.warmup, c=CONV_RGB, parity=not args.no_cpu))
+        others.append(run_complex(False, 4096, args.steps, args.warmup, parity=not args.no_cpu))
+        others.append(run_complex(True, 2048, 50, args.warmup, parity=not args.no_cpu))
         line["other_workloads"] = others
     if not args.no_cpu:
         cpu_and_parity(args.workload, line, inputs)
