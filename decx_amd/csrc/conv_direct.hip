@@ -8,6 +8,13 @@
 // a patch element are the same for all lanes, so they come through scalar loads and cost no vector
 // instruction; the vector pipe does one fma per (pixel, patch element, kernel), which is the arithmetic itself.
 //
+// What bounds it is the memory system's rate for traffic that is mostly writes (1920 x 1080 x 3, 8 kernels: 25 MB in,
+// 66 MB out in 24 us; a plain copy kernel moves 4.6 TB/s of reads plus writes on this part, i.e. 20 us for these 91 MB):
+// the same arithmetic on the matrix cores (v_mfma_f32_4x4x1_16b_f32 with the weights of four kernels as one operand and
+// the lane's own patch element as the other leaves every lane with its pixel's four outputs, bit for bit the same chain,
+// in a sixteenth of the instructions) measured 23.2 us there and lost on smaller and larger images (640 x 480: 8.5
+// against 6.9 us, 3840 x 2160: 143 against 126), so it is not in here.
+//
 // Same operands and layouts as the GEMM form (image [row][column][channel pitch], kernels packed
 // [patch element][kernel] with zero rows for padded channels, destination [row][column][channel pitch]), same
 // k-ascending fma chain per output as the CPU oracle.  Replaces, for these sizes, the same reference path:
@@ -19,6 +26,16 @@ namespace decx_hip {
 
 namespace {
 
+// Hardware deals consecutive workgroups to the 8 XCDs in turn, and each XCD has an L2 of its own.  An output row
+// needs KH rows of the image, most of which the rows above and below need as well: workgroup b takes the b / 8-th tile
+// of XCD b % 8's contiguous share of the pixels, so that an XCD works its way down a band of rows and finds the rows it
+// fetched for the last output row in its L2 (1920 x 1080 x 3, 3 x 3: 67.9 MB fetched per launch before, the image is 24.9).
+__device__ __forceinline__ uint32_t xcd_contiguous(uint32_t block, uint32_t blocks)
+{
+    const uint32_t per_xcd = blocks / kXcds;
+    return block < per_xcd * kXcds ? (block % kXcds) * per_xcd + block / kXcds : block;
+}
+
 // NACC: accumulators per pixel = kernels rounded up to a multiple of 4 (never beyond the pitch of the packed kernels).
 // REAL: channels of a 16-byte group that exist; below 4 only for a channel pitch of 4 with 1 to 3 channels (grey, RGB),
 // whose padding channel meets zero weights and is left out of the arithmetic.
@@ -29,7 +46,7 @@ conv2d_direct_kernel(const float* __restrict__ image, const float* __restrict__ 
                      uint64_t row_floats, uint32_t px_floats, uint64_t py_floats, uint32_t kmat_pitch,
                      uint32_t dst_dpitch, uint32_t dst_wpitch)
 {
-    const uint32_t p = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t p = xcd_contiguous(blockIdx.x, gridDim.x) * 256 + threadIdx.x;
     const bool live = p < pixels;
     const uint32_t q = live ? p : pixels - 1;              // idle lanes of the last workgroup repeat the last pixel
     const uint32_t oy = q / out_w, ox = q % out_w;
