@@ -76,9 +76,9 @@ MEASURED_TRAFFIC = {
     "conv2d": {"bytes": 1.08e8, "counters": "FETCH_SIZE 20 383 x 2.0 KiB + WRITE_SIZE 64 516 KiB",
                "kernel": "gemm_f32_dma_kernel<256, 256, 2, 4, 16, 4, false, 2, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
                "source_sha256": "6b285174a7da1174be80ab3543edb7e39772b75aecc853511ba3b6c106c8665e", "profile": "profiles/conv2d_implicit_gemm_256x256x112_3x3x256.md"},
-    "conv2d_rgb": {"bytes": 1.34e8, "counters": "FETCH_SIZE 33 138 x 2.0 KiB + WRITE_SIZE 64 613 KiB",
+    "conv2d_rgb": {"bytes": 1.00e8, "counters": "FETCH_SIZE 16 455 x 2.0 KiB + WRITE_SIZE 64 613 KiB",
                    "kernel": "conv2d_direct_kernel<8, 3>", "source": "decx_amd/csrc/conv_direct.hip",
-                   "source_sha256": "fd7361603433186e146b774c91a6854620390bcbf5b5767b9f1d0f8a981c4930", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
+                   "source_sha256": "1a7a0a29a0ddfd248c3fdb51c6df7bd2e4515bdeb8ff951c0af73a5327f6658e", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
 }
 
 
