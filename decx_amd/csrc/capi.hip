@@ -109,7 +109,7 @@ int check_gemm(const void* A, const void* B, const void* C, const void* D, uint3
 // fp32 fitted to 20 output shapes x K = 777 ... 16384 x 1 ... 8 ranges, fp16 and fp64 to 12 and 9 shapes x 2 ... 32
 // ranges: the estimate is within 4 % of the measurement on most, the pick within 1 % (fp16: 2.5 %) of the best on
 // average.  The whole product is kept unless the split promises 4 %.
-struct SplitChoice { int shape; uint32_t splits, len; };
+struct SplitChoice { int shape; uint32_t splits, len, first; };     // first: tiles in front that stay whole
 struct SplitTile {
     int shape, fit, pieces;          // size class, workgroups per CU, 16-byte pieces of accumulators per lane
     double ns_per_k[5];              // per workgroup with m = 1 .. fit of them on the CU
@@ -133,28 +133,32 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
     const SplitModel& md = elem_bytes == 8 ? kSplitF64 : elem_bytes == 2 ? kSplitF16 : kSplitF32;
     const uint32_t cus = g_dev.compute_units;
     constexpr double kLaunch = 4.0;                             // launch to launch
-    if (K < 512) return {whole_shape, 1, 0};
+    if (K < 512) return {whole_shape, 1, 0, 0};
     const double out_mb = (double)M * N * md.acc_bytes / 1e6;
     const auto tiles_of = [&](int shape) {
         const TileInfo ti = dma_tile_info(elem_bytes, shape, N);
         return (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
     };
-    const auto estimate = [&](const SplitTile& st, uint64_t t, uint32_t len, uint32_t ranges) {
-        const uint64_t wgs = t * ranges, slots = (uint64_t)st.fit * cus;
+    // `whole` tiles in front run unsplit (full rounds of workgroups: whole is a multiple of fit x CUs), the other
+    // t - whole on `ranges` ranges of `len`
+    const auto estimate = [&](const SplitTile& st, uint64_t t, uint32_t len, uint32_t ranges, uint64_t whole = 0) {
+        const uint64_t wgs = (t - whole) * ranges, slots = (uint64_t)st.fit * cus;
         const uint64_t full = wgs / slots, rem = wgs % slots;
         uint64_t m = (rem + cus - 1) / cus;
         if (md.uneven_second_round && full == 1 && rem > cus / 2 && rem <= cus) m = 2;
         double lone = st.ns_per_k[1];
         if (elem_bytes == 2 && st.shape == TILE_MEDIUM)        // 6.0 ns with half the CUs busy, 7.67 with all
             lone = wgs <= cus / 2 ? 6.0 : 6.0 + 1.67 * (double)(wgs - cus / 2) / (double)(cus - cus / 2);
-        const double ns = (double)len * ((double)full * st.fit * st.ns_per_k[st.fit] + (m == 1 ? lone : (double)m * st.ns_per_k[m]));
+        const uint32_t k_whole = (K + md.len_align - 1) / md.len_align * md.len_align;
+        const double ns = (double)len * ((double)full * st.fit * st.ns_per_k[st.fit] + (m == 1 ? lone : (double)m * st.ns_per_k[m])) +
+                          (double)k_whole * (double)(whole / slots) * st.fit * st.ns_per_k[st.fit];
         double us = ns * 1e-3 + kLaunch;
         if (ranges > 1) {
             const uint32_t group = st.pieces < 16 ? st.pieces : 16, batch = 16 / group, per_slot = st.pieces / group;
             uint32_t trips = (ranges + batch - 1) / batch * per_slot;
             if (ranges > kSplitFlat)                           // two levels: a group of kSplitGroup, the group sums, and a second store and count
                 trips = ((kSplitGroup + batch - 1) / batch + ((ranges + kSplitGroup - 1) / kSplitGroup + batch - 1) / batch) * per_slot + 1;
-            us += md.us_fixed + md.us_per_trip * trips + md.us_per_mb * ranges * out_mb;
+            us += md.us_fixed + md.us_per_trip * trips + md.us_per_mb * ranges * out_mb * (double)(t - whole) / (double)t;
         }
         return us;
     };
@@ -163,19 +167,23 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
     for (int i = 0; i < md.n_tiles; ++i)                        // the model's own figure where the whole product runs on one of its tiles
         if (md.tiles[i].shape == whole_shape)
             whole_us = estimate(md.tiles[i], tiles_of(whole_shape), (K + md.len_align - 1) / md.len_align * md.len_align, 1);
-    SplitChoice best = {whole_shape, 1, 0};
+    SplitChoice best = {whole_shape, 1, 0, 0};
     double best_us = whole_us / 1.04;
     const uint32_t max_p = K / 256 < 64u ? K / 256 : 64u;
     for (int i = 0; i < md.n_tiles; ++i) {
         const SplitTile& st = md.tiles[i];
-        const uint64_t t = tiles_of(st.shape);
-        if (t > 4ull * cus) continue;
+        const uint64_t t = tiles_of(st.shape), slots = (uint64_t)st.fit * cus;
+        if (t > 16ull * cus) continue;
         const uint32_t tile_max_p = st.shape == TILE_SMALL ? max_p : (max_p < kSplitFlat ? max_p : kSplitFlat);     // only the smallest tiles sum on two levels
-        for (uint32_t p = 2; p <= tile_max_p && t * p <= 4096; ++p) {
-            const uint32_t len = ((K + p - 1) / p + md.len_align - 1) / md.len_align * md.len_align, ranges = (K + len - 1) / len;
-            if (ranges < 2) continue;
-            const double us = estimate(st, t, len, ranges);
-            if (us < best_us) { best_us = us; best = {st.shape, ranges, len}; }
+        // all tiles split, or only those of the ragged last round (the full rounds in front stay whole)
+        for (uint64_t whole = 0; whole <= t / slots * slots; whole += (t / slots * slots ? t / slots * slots : 1)) {
+            if (whole == t || (whole == 0 && t > 4ull * cus)) continue;
+            for (uint32_t p = 2; p <= tile_max_p && (t - whole) * p <= 4096; ++p) {
+                const uint32_t len = ((K + p - 1) / p + md.len_align - 1) / md.len_align * md.len_align, ranges = (K + len - 1) / len;
+                if (ranges < 2) continue;
+                const double us = estimate(st, t, len, ranges, whole);
+                if (us < best_us) { best_us = us; best = {st.shape, ranges, len, (uint32_t)whole}; }
+            }
         }
     }
     return best;
@@ -185,8 +193,8 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
 // product takes).
 SplitChoice split_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K)
 {
-    if (M == 0 || N == 0) return {0, 1, 0};
-    if (M == 1 || N == 1) return {0, 1, 0};                         // the vector corners have their own kernels
+    if (M == 0 || N == 0) return {0, 1, 0, 0};
+    if (M == 1 || N == 1) return {0, 1, 0, 0};                      // the vector corners have their own kernels
     const int shape = elem_bytes == 8 ? choose_tile_f64(M, N) : choose_tile(elem_bytes == 2, M, N, true);
     return split_plan_model(elem_bytes, M, N, K, shape, dma_tile_info(elem_bytes, shape, N));
 }
@@ -199,11 +207,11 @@ TileInfo dma_tile_info(int elem_bytes, int shape, uint32_t N)
 
 // Bytes of workspace a split of `splits` ranges needs: one slot of BM x BN accumulators (fp32; fp64 for fp64 operands)
 // per workgroup, the tiles being those of the shape the split runs on.
-size_t split_workspace_bytes(int elem_bytes, int shape, uint32_t M, uint32_t N, uint32_t splits)
+size_t split_workspace_bytes(int elem_bytes, const SplitChoice& sp, uint32_t M, uint32_t N)
 {
-    const TileInfo ti = dma_tile_info(elem_bytes, shape, N);
+    const TileInfo ti = dma_tile_info(elem_bytes, sp.shape, N);
     const uint64_t tiles = (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
-    return (size_t)(tiles * splits * (uint64_t)(ti.bm * ti.bn) * (elem_bytes == 8 ? 8u : 4u));
+    return (size_t)((tiles - sp.first) * sp.splits * (uint64_t)(ti.bm * ti.bn) * (elem_bytes == 8 ? 8u : 4u));
 }
 
 // Fills the split fields of g when the plan says so, the workspace is large enough and the tiles have counters; returns
@@ -212,14 +220,14 @@ uint32_t arm_split(GemmArgs& g, int elem_bytes, void* workspace, size_t workspac
 {
     if (!workspace || !aligned16(workspace)) return 1;
     const SplitChoice sp = split_plan(elem_bytes, g.M, g.N, g.K);
-    if (sp.splits <= 1 || workspace_bytes < split_workspace_bytes(elem_bytes, sp.shape, g.M, g.N, sp.splits)) return 1;
+    if (sp.splits <= 1 || workspace_bytes < split_workspace_bytes(elem_bytes, sp, g.M, g.N)) return 1;
     const TileInfo ti = dma_tile_info(elem_bytes, sp.shape, g.N);
     const uint64_t tiles = (uint64_t)((g.M + ti.bm - 1) / ti.bm) * ((g.N + ti.bn - 1) / ti.bn);
-    const uint64_t n_counters = tiles * split_counters_per_tile(sp.splits);
+    const uint64_t n_counters = (tiles - sp.first) * split_counters_per_tile(sp.splits);
     uint32_t* const counters = n_counters <= kSplitCounters ? take_split_counters((uint32_t)n_counters) : nullptr;
     if (!counters) return 1;
     g.split_counters = counters;
-    g.split_len = sp.len; g.split_ws = workspace;
+    g.split_len = sp.len; g.split_count = sp.splits; g.split_first = sp.first; g.split_ws = workspace;
     shape = sp.shape;
     return sp.splits;
 }
@@ -475,7 +483,7 @@ size_t decx_hip_gemm_workspace(int elem_bytes, uint32_t M, uint32_t N, uint32_t 
         return sp.splits > 1 ? (size_t)sp.splits * ((N + 3) / 4 * 4) * (elem_bytes == 8 ? 8 : 4) : 0;
     }
     const SplitChoice sp = split_plan(elem_bytes, M, N, K);
-    return sp.splits > 1 ? split_workspace_bytes(elem_bytes, sp.shape, M, N, sp.splits) : 0;
+    return sp.splits > 1 ? split_workspace_bytes(elem_bytes, sp, M, N) : 0;
 }
 
 size_t decx_hip_gemm_f32_workspace(uint32_t M, uint32_t N, uint32_t K) { return decx_hip_gemm_workspace(4, M, N, K); }
@@ -780,7 +788,8 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
                 out->path = sc.shape; out->tile_m = ts.bm; out->tile_n = ts.bn;
                 out->grid = ((M + ts.bm - 1) / ts.bm) * ((N + ts.bn - 1) / ts.bn);
             }
-            out->k_splits = sc.splits; out->grid *= out->k_splits;
+            out->k_splits = sc.splits; out->whole_tiles = sc.first;
+            out->grid = sc.first + (out->grid - sc.first) * sc.splits;
         }
         return DECX_HIP_OK;
     }
@@ -819,7 +828,8 @@ int decx_hip_gemm_plan(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int a
             out->path = sc.shape; out->tile_m = ts.bm; out->tile_n = ts.bn;
             out->grid = ((M + ts.bm - 1) / ts.bm) * ((N + ts.bn - 1) / ts.bn);
         }
-        out->k_splits = sc.splits; out->grid *= out->k_splits;
+        out->k_splits = sc.splits; out->whole_tiles = sc.first;
+        out->grid = sc.first + (out->grid - sc.first) * sc.splits;
     }
     return DECX_HIP_OK;
 }

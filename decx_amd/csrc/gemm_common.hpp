@@ -29,13 +29,16 @@ struct GemmArgs {
     double alpha64, beta64;      // the same two scalars for the fp64 kernels
     uint32_t tiles_m, tiles_n;   // number of block tiles along M and N
     uint32_t vec_ok;             // 1: every base pointer is 16-byte aligned and every pitch a multiple of 16 bytes
-    // Split K (direct-load kernels, grid.y = number of splits): split z multiplies k in [z * split_len,
-    // min(K, (z + 1) * split_len)).  Every workgroup stores its accumulators (fp32, or fp64 for fp64 operands) to its
+    // Split K (direct-load kernels; a 1-D grid of split_first whole tiles, then split 0 of every split tile, split 1 of
+    // every split tile, ...): split z multiplies k in [z * split_len, min(K, (z + 1) * split_len)).  Every workgroup stores its accumulators (fp32, or fp64 for fp64 operands) to its
     // slot of split_ws and counts itself in at split_counters[tile]; the one that arrives last adds all slots of the
     // tile in split order (its own included, so the result does not depend on who is last), writes D and puts the
     // counter back to zero (split_k_exchange.hpp).
     uint32_t group_m;            // tile-rows per L2 patch of the block -> tile map (0: the default, kGroupM)
     uint32_t split_len;          // 0: no split
+    uint32_t split_count;        // splits per split tile
+    uint32_t split_first;        // tiles below this index are multiplied whole, by one workgroup each (the full rounds of
+                                 // workgroups); only the tiles of the ragged last round are split
     void*    split_ws;
     uint32_t* split_counters;    // one per tile, zero before and after every launch
     // Convolution as an implicit GEMM (used by the CONV instantiations only): row p of the A operand is the
@@ -60,12 +63,13 @@ constexpr int kGroupM = 4;      // tile-rows per L2 patch (4 x 8 tiles run toget
 // range of logical ids (the first 8 * (nb / 8) blocks; the up to 7 that remain keep their
 // ids, at the end of the last range), step 2 walks logical ids in groups of kGroupM tile-rows so the
 // 32 tiles resident on one XCD form a compact patch that shares A rows and B columns.
-__device__ __forceinline__ void block_to_tile(const GemmArgs& g, uint32_t& tile_m, uint32_t& tile_n)
+// `id`: the block's index among the `nb` blocks dealt to the XCDs in turn that it belongs to (all tiles of a whole
+// product; the whole tiles, or one split of the split tiles, of a split one), `first`: the tile the first of them takes.
+__device__ __forceinline__ void block_to_tile(const GemmArgs& g, uint32_t id, uint32_t nb, uint32_t first, uint32_t& tile_m, uint32_t& tile_n)
 {
-    const uint32_t nb = g.tiles_m * g.tiles_n;
-    uint32_t id = blockIdx.x;
     const uint32_t per_xcd = nb / kXcds;
     if (id < per_xcd * kXcds) id = (id % kXcds) * per_xcd + id / kXcds;
+    id += first;
     const uint32_t group_m = g.group_m ? g.group_m : (uint32_t)kGroupM;
     const uint32_t per_group = group_m * g.tiles_n;
     const uint32_t group = id / per_group;
@@ -74,6 +78,25 @@ __device__ __forceinline__ void block_to_tile(const GemmArgs& g, uint32_t& tile_
     const uint32_t in_group = id % per_group;
     tile_m = first_m + in_group % rows;
     tile_n = in_group / rows;
+}
+__device__ __forceinline__ void block_to_tile(const GemmArgs& g, uint32_t& tile_m, uint32_t& tile_n)
+{
+    block_to_tile(g, blockIdx.x, g.tiles_m * g.tiles_n, 0, tile_m, tile_n);
+}
+
+// Where a block of a split-K launch works: its tile's index, its split and the number of splits of its tile (1 for the
+// whole tiles in front).
+struct SplitBlock { uint32_t tile, z, splits; };
+__device__ __forceinline__ SplitBlock split_block(const GemmArgs& g, uint32_t& tile_m, uint32_t& tile_n)
+{
+    const uint32_t tiles = g.tiles_m * g.tiles_n;
+    if (blockIdx.x < g.split_first) {
+        block_to_tile(g, blockIdx.x, g.split_first, 0, tile_m, tile_n);
+        return {0u, 0u, 1u};                               // (whole tiles have no slot)
+    }
+    const uint32_t r = blockIdx.x - g.split_first, rest = tiles - g.split_first;
+    block_to_tile(g, r % rest, rest, g.split_first, tile_m, tile_n);
+    return {r % rest, r / rest, g.split_count};
 }
 
 // ---- tile-shape table shared by the planner and the launchers -----------------

@@ -86,12 +86,19 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
 {
     struct Nothing {};
     std::conditional_t<SPLIT, GemmArgs, Nothing> g_split;
-    if constexpr (SPLIT) {
+    uint32_t tile_m, tile_n;
+    SplitBlock sb = {0u, 0u, 1u};
+    if constexpr (SPLIT) {                                 // this workgroup's tile, its share of K and its partial product
+        sb = split_block(g_in, tile_m, tile_n);
         g_split = g_in;
-        const uint32_t k0 = blockIdx.y * g_in.split_len;
-        g_split.A = (const unsigned char*)g_in.A + (size_t)k0 * 2;
-        g_split.B = (const unsigned char*)g_in.B + (size_t)k0 * g_in.ldb * 2;
-        g_split.K = g_in.K - k0 < g_in.split_len ? g_in.K - k0 : g_in.split_len;
+        if (sb.splits > 1) {
+            const uint32_t k0 = sb.z * g_in.split_len;
+            g_split.A = (const unsigned char*)g_in.A + (size_t)k0 * 2;
+            g_split.B = (const unsigned char*)g_in.B + (size_t)k0 * g_in.ldb * 2;
+            g_split.K = g_in.K - k0 < g_in.split_len ? g_in.K - k0 : g_in.split_len;
+        }
+    } else {
+        block_to_tile(g_in, tile_m, tile_n);
     }
     const GemmArgs& g = [&]() -> const GemmArgs& { if constexpr (SPLIT) return g_split; else return g_in; }();
     constexpr int WAVES = WAVES_M * WAVES_N;
@@ -113,8 +120,6 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     __shared__ __attribute__((aligned(1024))) unsigned char lds[LDS_BYTES];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)lds;
 
-    uint32_t tile_m, tile_n;
-    block_to_tile(g, tile_m, tile_n);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
 
     const int t = threadIdx.x, lane = t & 63;
@@ -303,7 +308,7 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     if constexpr (SPLIT) {
         // piece c of a lane: the four fp32 accumulators of its 16 x 16 tile (c % TM, c / TM).  The ring is free: every
         // LDS read precedes the last slab barrier.
-        const bool last = split_k_exchange<WAVES * 64, TM * TN, floatx4, (BM <= 64)>(g_in, (uint32_t*)lds,
+        const bool last = sb.splits == 1 || split_k_exchange<WAVES * 64, TM * TN, floatx4, (BM <= 64)>(g_in, sb, (uint32_t*)lds,
             [&](auto cc) { constexpr int c = decltype(cc)::value; return accT[c / TM][c % TM]; },
             [&](auto cc, const floatx4& v, bool first) {
                 constexpr int c = decltype(cc)::value;
@@ -393,8 +398,8 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     const uint32_t nb = g.tiles_m * g.tiles_n;
     if (g.split_len) {                                     // the planner splits K on the two smaller tiles only
         if constexpr (BM <= 128) {
-            const uint32_t splits = (g.K + g.split_len - 1) / g.split_len;
-            hipLaunchKernelGGL((gemm_f16_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, true>), dim3(nb, splits),
+            const uint32_t splits = g.split_count;
+            hipLaunchKernelGGL((gemm_f16_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, true>), dim3(g.split_first + (nb - g.split_first) * splits),
                                dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
             return (int)hipGetLastError();
         } else {
@@ -421,16 +426,20 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
 //     than two workgroups per CU are there to hide the copies (1536^3: 447 against 388).
 int launch_gemm_f16_dma(int shape, const GemmArgs& args, hipStream_t stream)
 {
-    const uint32_t splits = args.split_len ? (args.K + args.split_len - 1) / args.split_len : 1u;     // workgroups per tile
+    // workgroups of a launch on b x b tiles: whole tiles, and splits of the others
+    const auto workgroups = [&](uint32_t b) {
+        const uint64_t tiles = (uint64_t)((args.M + b - 1) / b) * ((args.N + b - 1) / b);
+        return args.split_len ? args.split_first + (tiles - args.split_first) * args.split_count : tiles;
+    };
     switch (shape) {
     case TILE_LARGE: return launch_dma<256, 256, 2, 4, 64, 2>(args, stream);
     case TILE_MEDIUM: {
-        const uint64_t blocks = (uint64_t)((args.M + 127) / 128) * ((args.N + 127) / 128) * splits;
+        const uint64_t blocks = workgroups(128);
         return blocks <= 256 ? launch_dma<128, 128, 2, 4, 64, 4>(args, stream)
                              : launch_dma<128, 128, 2, 4, 64, 2>(args, stream);
     }
     case TILE_SMALL: {
-        const uint64_t blocks = (uint64_t)((args.M + 63) / 64) * ((args.N + 63) / 64) * splits;
+        const uint64_t blocks = workgroups(64);
         return blocks <= 512 ? launch_dma<64, 64, 2, 2, 64, 4>(args, stream)
                              : launch_dma<64, 64, 2, 2, 64, 2>(args, stream);
     }

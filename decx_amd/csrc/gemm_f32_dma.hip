@@ -79,12 +79,19 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
 {
     struct Nothing {};
     std::conditional_t<SPLIT, GemmArgs, Nothing> g_split;
-    if constexpr (SPLIT) {                                 // this workgroup's share of K and its partial product
+    uint32_t tile_m, tile_n;
+    SplitBlock sb = {0u, 0u, 1u};
+    if constexpr (SPLIT) {                                 // this workgroup's tile, its share of K and its partial product
+        sb = split_block(g_in, tile_m, tile_n);
         g_split = g_in;
-        const uint32_t k0 = blockIdx.y * g_in.split_len;
-        g_split.A = (const unsigned char*)g_in.A + (size_t)k0 * 4;
-        g_split.B = (const unsigned char*)g_in.B + (size_t)k0 * g_in.ldb * 4;
-        g_split.K = g_in.K - k0 < g_in.split_len ? g_in.K - k0 : g_in.split_len;
+        if (sb.splits > 1) {
+            const uint32_t k0 = sb.z * g_in.split_len;
+            g_split.A = (const unsigned char*)g_in.A + (size_t)k0 * 4;
+            g_split.B = (const unsigned char*)g_in.B + (size_t)k0 * g_in.ldb * 4;
+            g_split.K = g_in.K - k0 < g_in.split_len ? g_in.K - k0 : g_in.split_len;
+        }
+    } else {
+        block_to_tile(g_in, tile_m, tile_n);
     }
     const GemmArgs& g = [&]() -> const GemmArgs& { if constexpr (SPLIT) return g_split; else return g_in; }();
     constexpr int WAVES = WAVES_M * WAVES_N;
@@ -113,8 +120,6 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
     __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE_BYTES];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)lds;
 
-    uint32_t tile_m, tile_n;
-    block_to_tile(g, tile_m, tile_n);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
 
     const int t = threadIdx.x, lane = t & 63;
@@ -424,7 +429,7 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
     if constexpr (SPLIT) {
         // piece c of a lane: registers 4 (c % 4) .. + 3 of its 32 x 32 tile c / 4.  The ring is free: every LDS read
         // precedes the last slab barrier.
-        const bool last = split_k_exchange<WAVES * 64, TM * TN * 4, floatx4>(g_in, (uint32_t*)lds,
+        const bool last = sb.splits == 1 || split_k_exchange<WAVES * 64, TM * TN * 4, floatx4>(g_in, sb, (uint32_t*)lds,
             [&](auto cc) {
                 constexpr int c = decltype(cc)::value, tile = c / 4, q = c % 4;
                 const floatx16& a = acc[tile / TN][tile % TN];
@@ -441,6 +446,7 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
             },
             [&] { if constexpr (C_EARLY) load_c_early(); });
         if (!last) return;
+        if constexpr (C_EARLY) { if (sb.splits == 1) load_c_early(); }      // a whole tile
     }
 
     // Epilogue: register r of lane (l32, h) is row 8*(r/4) + 4*h + r%4 of a 32x32 tile; the
@@ -508,13 +514,13 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     if constexpr (BM == 256 && BN == 128 && CONV == 0) g.group_m = 2;
     if (g.split_len) {                                     // the planner splits K on the smallest tiles only
         if constexpr (CONV == 0 && BM * BN == 64 * 64) {
-            const uint32_t splits = (g.K + g.split_len - 1) / g.split_len;
+            const uint32_t splits = g.split_count;
             if (g.C)
                 hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD, 0, true, true>),
-                                   dim3(nb, splits), dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
+                                   dim3(g.split_first + (nb - g.split_first) * splits), dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
             else
                 hipLaunchKernelGGL((gemm_f32_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, CHUNK_AHEAD, 0, true, false>),
-                                   dim3(nb, splits), dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
+                                   dim3(g.split_first + (nb - g.split_first) * splits), dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
             return (int)hipGetLastError();
         } else {
             return (int)hipErrorInvalidValue;

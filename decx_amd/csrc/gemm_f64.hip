@@ -46,12 +46,19 @@ gemm_f64_dma_kernel(const GemmArgs g_in)
 {
     struct Nothing {};
     std::conditional_t<SPLIT, GemmArgs, Nothing> g_split;
-    if constexpr (SPLIT) {
+    uint32_t tile_m, tile_n;
+    SplitBlock sb = {0u, 0u, 1u};
+    if constexpr (SPLIT) {                                 // this workgroup's tile, its share of K and its partial product
+        sb = split_block(g_in, tile_m, tile_n);
         g_split = g_in;
-        const uint32_t k0 = blockIdx.y * g_in.split_len;
-        g_split.A = (const unsigned char*)g_in.A + (size_t)k0 * 8;
-        g_split.B = (const unsigned char*)g_in.B + (size_t)k0 * g_in.ldb * 8;
-        g_split.K = g_in.K - k0 < g_in.split_len ? g_in.K - k0 : g_in.split_len;
+        if (sb.splits > 1) {
+            const uint32_t k0 = sb.z * g_in.split_len;
+            g_split.A = (const unsigned char*)g_in.A + (size_t)k0 * 8;
+            g_split.B = (const unsigned char*)g_in.B + (size_t)k0 * g_in.ldb * 8;
+            g_split.K = g_in.K - k0 < g_in.split_len ? g_in.K - k0 : g_in.split_len;
+        }
+    } else {
+        block_to_tile(g_in, tile_m, tile_n);
     }
     const GemmArgs& g = [&]() -> const GemmArgs& { if constexpr (SPLIT) return g_split; else return g_in; }();
     constexpr int WAVES = WAVES_M * WAVES_N;
@@ -72,8 +79,6 @@ gemm_f64_dma_kernel(const GemmArgs g_in)
     __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE_BYTES];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void*)lds;
 
-    uint32_t tile_m, tile_n;
-    block_to_tile(g, tile_m, tile_n);
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
 
     const int t = threadIdx.x, lane = t & 63;
@@ -266,7 +271,7 @@ gemm_f64_dma_kernel(const GemmArgs g_in)
     if constexpr (SPLIT) {
         // piece c of a lane: elements 2 (c % 2), + 1 of its 16 x 16 tile c / 2.  The ring is free: every LDS read
         // precedes the last slab barrier.
-        const bool last = split_k_exchange<WAVES * 64, TM * TN * 2, doublex2>(g_in, (uint32_t*)lds,
+        const bool last = sb.splits == 1 || split_k_exchange<WAVES * 64, TM * TN * 2, doublex2>(g_in, sb, (uint32_t*)lds,
             [&](auto cc) {
                 constexpr int c = decltype(cc)::value, tile = c / 2, e0 = 2 * (c % 2);
                 const doublex4& a = acc[tile / TN][tile % TN];
@@ -347,8 +352,8 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     const uint32_t nb = g.tiles_m * g.tiles_n;
     if (g.split_len) {                                     // the planner splits K on the smallest tile only
         if constexpr (BM == 64) {
-            const uint32_t splits = (g.K + g.split_len - 1) / g.split_len;
-            hipLaunchKernelGGL((gemm_f64_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, true>), dim3(nb, splits),
+            const uint32_t splits = g.split_count;
+            hipLaunchKernelGGL((gemm_f64_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, true>), dim3(g.split_first + (nb - g.split_first) * splits),
                                dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
             return (int)hipGetLastError();
         } else {

@@ -24,7 +24,8 @@ __host__ __device__ inline uint32_t split_counters_per_tile(uint32_t splits)
     return splits <= kSplitFlat ? 1u : 1u + (splits + kSplitGroup - 1) / kSplitGroup;
 }
 
-// grid = (tiles, splits), NT threads per workgroup.  A lane's accumulators are PIECES 16-byte pieces, piece c read by
+// sb: the block's split tile (counted from the first split tile), split and number of splits; NT threads per workgroup.
+// A lane's accumulators are PIECES 16-byte pieces, piece c read by
 // get(c) and given back by put(c, value, first): put stores `value` when `first`, else adds it.  Every workgroup
 // writes its pieces to its slot of the workspace, [piece][thread] so that a wave writes whole lines, and counts itself
 // in on the tile's counter; the function returns false in all but the workgroup that arrives last, and in that one
@@ -44,16 +45,16 @@ __host__ __device__ inline uint32_t split_counters_per_tile(uint32_t splits)
 // TWO_LEVEL false: one level whatever the number of splits (a kernel whose registers the second copy of the sum would
 // cost a workgroup per CU, and which the planner gives few splits anyway).
 template <int NT, int PIECES, typename V, bool TWO_LEVEL = true, class Get, class Put, class OnLast>
-__device__ __forceinline__ bool split_k_exchange(const GemmArgs& g, uint32_t* flag, Get&& get, Put&& put, OnLast&& on_last)
+__device__ __forceinline__ bool split_k_exchange(const GemmArgs& g, const SplitBlock& sb, uint32_t* flag, Get&& get, Put&& put, OnLast&& on_last)
 {
     static_assert(sizeof(V) == 16, "pieces are 16 bytes");
     constexpr int GROUP = PIECES <= 16 ? PIECES : 16, BATCH = 16 / GROUP;
     static_assert(PIECES % GROUP == 0 && GROUP * BATCH == 16, "pieces per lane: 1, 2, 4, 8, or a multiple of 16");
     const int t = threadIdx.x;
-    const uint32_t splits = gridDim.y, z = blockIdx.y;
+    const uint32_t splits = sb.splits, z = sb.z;
     constexpr size_t SLOT = (size_t)NT * PIECES;           // pieces per slot
-    V* const slots = (V*)g.split_ws + (size_t)blockIdx.x * splits * SLOT;
-    uint32_t* const counters = g.split_counters + (size_t)blockIdx.x * split_counters_per_tile(splits);
+    V* const slots = (V*)g.split_ws + (size_t)sb.tile * splits * SLOT;
+    uint32_t* const counters = g.split_counters + (size_t)sb.tile * split_counters_per_tile(splits);
 
     // this lane's pieces -> slot `s`
     const auto store_slot = [&](uint32_t s) {

@@ -27,7 +27,7 @@ class DeviceProps(ctypes.Structure):
 
 class Plan(ctypes.Structure):
     _fields_ = [("path", ctypes.c_int32), ("edge", ctypes.c_int32), ("tile_m", _u32), ("tile_n", _u32),
-                ("grid", _u32), ("k_splits", _u32)]
+                ("grid", _u32), ("k_splits", _u32), ("whole_tiles", _u32)]
 
 
 # name -> (restype, argtypes): every symbol include/decx_hip.h declares

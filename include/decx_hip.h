@@ -67,10 +67,12 @@ typedef struct decx_hip_plan {
     int32_t  edge;                 /* 1: the predicated register-staged kernel runs (operands not 16-byte
                                       aligned, or K == 0); 0: a direct-to-LDS kernel */
     uint32_t tile_m, tile_n;       /* block tile */
-    uint32_t grid;                 /* workgroups launched (tiles x k_splits) */
+    uint32_t grid;                 /* workgroups launched: whole_tiles + (tiles - whole_tiles) x k_splits */
     uint32_t k_splits;             /* ranges K is cut into when the *_ws entry point gets its workspace; 1: no split.
                                       With more than one, path / tile are those of the split (it may run on a smaller
                                       tile than the whole product takes without a workspace) */
+    uint32_t whole_tiles;          /* with k_splits > 1: tiles that are multiplied whole all the same -- the full rounds
+                                      of workgroups; only the tiles of the ragged last round are split.  0: all are */
 } decx_hip_plan;
 
 /* ---- device, memory, streams, events --------------------------------------------------

@@ -101,6 +101,12 @@ def test_planner_choices():
     assert hip.plan(2, 768, 768, 16384).k_splits == 6 and hip.plan(2, 2048, 2048, 8192).k_splits == 1
     p = hip.plan(2, 300, 300, 8192)                        # few tiles: 8 ranges on 64 x 64 (12.9 us; the 20 that two
     assert (p.tile_m, p.k_splits) == (64, 8)               # workgroups per CU would ask for: 17.8, the whole product 38.8)
+    # more tiles than the chip holds at once: the full rounds stay whole, only the ragged last round is split
+    p = hip.plan(4, 2112, 2112, 2112)                      # 1089 tiles: 1024 whole, 65 on 7 ranges each (161.5 -> 143.7 us)
+    assert (p.tile_m, p.k_splits, p.whole_tiles, p.grid) == (64, 7, 1024, 1024 + 65 * 7)
+    p = hip.plan(8, 1536, 1536, 1536)                      # fp64, two workgroups per CU: 512 whole + 64 x 4 (146 -> 112 us)
+    assert (p.tile_m, p.k_splits, p.whole_tiles, p.grid) == (64, 4, 512, 512 + 64 * 4)
+    assert hip.plan(4, 2048, 2048, 2048).whole_tiles == 0 and hip.plan(4, 1000, 1500, 777).whole_tiles == 0
     p = hip.plan(8, 1280, 1024, 2048)                      # fp64: 320 tiles of 64 x 64 on 4 ranges, 128.5 -> 91.3 us
     assert (p.tile_m, p.k_splits) == (64, 4)
     p = hip.plan(8, 1280, 1024, 8192)

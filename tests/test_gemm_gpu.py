@@ -577,6 +577,8 @@ def test_stream_and_events(hip):
     (np.float64, 300, 300, 8192), (np.float64, 1280, 1024, 2048),
     # more than 8 ranges: groups of four are added first, then the group sums
     (np.float32, 100, 120, 20000), (np.float16, 128, 128, 16384), (np.float16, 70, 130, 40000), (np.float64, 100, 120, 4096),
+    # more tiles than fit the chip at once: the full rounds stay whole, the tiles of the ragged last round are split
+    (np.float32, 2112, 2112, 1024), (np.float64, 1536, 1400, 1536),
 ])
 def test_split_k_slots_carry_nothing_from_launch_to_launch(hip, oracle, dtype, M, N, K):
     """The workgroups of a tile meet in the workspace (slots written and read at device scope, a counter per tile
@@ -588,6 +590,9 @@ def test_split_k_slots_carry_nothing_from_launch_to_launch(hip, oracle, dtype, M
         pytest.skip("the planner does not split this shape")
     if K >= 16384 or (M, N) == (100, 120):
         assert hip.plan(esz, M, N, K).k_splits > 8
+    if M >= 1536:
+        plan = hip.plan(esz, M, N, K)
+        assert plan.whole_tiles > 0 and plan.grid == plan.whole_tiles + (-(-M // 64) * -(-N // 64) - plan.whole_tiles) * plan.k_splits
     ws = hip.DeviceMatrix(1, need // 4, np.float32)
     pa, pn = device_pitch(K, dtype), device_pitch(N, dtype)
     make = {2: synth.normal_half, 4: synth.uniform_f32, 8: synth.uniform_f64}[esz]
