@@ -178,6 +178,10 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
         // all tiles split, or only those of the ragged last round (the full rounds in front stay whole)
         for (uint64_t whole = 0; whole <= t / slots * slots; whole += (t / slots * slots ? t / slots * slots : 1)) {
             if (whole == t || (whole == 0 && t > 4ull * cus)) continue;
+            // fp16: the rates above are those of launches of some tens of microseconds; full rounds of 128 x 128 tiles
+            // run for longer than that, into the power cap, and then 15 % slower (3072^3: estimate 55 us, measured
+            // 66.7, whole on 256 x 256 tiles 60.4): full rounds in front only where the whole product takes the same tile
+            if (elem_bytes == 2 && whole > 0 && st.shape != whole_shape) continue;
             for (uint32_t p = 2; p <= tile_max_p && (t - whole) * p <= 4096; ++p) {
                 const uint32_t len = ((K + p - 1) / p + md.len_align - 1) / md.len_align * md.len_align, ranges = (K + len - 1) / len;
                 if (ranges < 2) continue;

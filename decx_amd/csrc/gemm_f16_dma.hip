@@ -330,9 +330,11 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
         return w.u;
     };
     const bool interior = (m0 + BM <= g.M) && (n0 + BN <= g.N);
-    // Interior tiles go through LDS once more (the ring is free: every wave has passed the last slab barrier): a lane
+    // The tile goes through LDS once more (the ring is free: every wave has passed the last slab barrier): a lane
     // holds 8 bytes of a row, 4 lanes 32 contiguous bytes.  Each wave turns 16 rows x WN columns around in a private
-    // buffer (two of them, taking turns) and stores whole rows: WN * 2 contiguous bytes per row.
+    // buffer (two of them, taking turns) and stores whole rows: WN * 2 contiguous bytes per row.  Tiles on a ragged
+    // edge take the same way and leave out rows beyond M and 16-byte pieces beyond N; only a piece that straddles N is
+    // stored element by element (stored that way as a whole, a 256 x 256 edge tile took a third longer than an interior one).
     constexpr int ROW_BYTES = WN * 2, PPR = WN / 8, RPG = 256 / ROW_BYTES, ROWS_PER_STORE = 64 / PPR, STORES = 16 / ROWS_PER_STORE;
     static_assert(PPR == 4 || PPR == 8 || PPR == 16, "staging rows of 64, 128 or 256 bytes");
     static_assert(WAVES * 2 * 16 * ROW_BYTES <= LDS_BYTES, "staging rows must fit in the ring");
@@ -345,45 +347,47 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     for (int i = 0; i < TM; ++i) {
         const uint32_t row = m0 + wm0 + 16 * i + l16;
         unsigned char* stage_rows = lds + (wave * 2 + (i & 1)) * (16 * ROW_BYTES);
-        if (interior) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                float v[4];
+        for (int j = 0; j < TN; ++j) {
+            float v[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = accT[j][i][e];
-                if (C) {
-                    const uint32_t col = n0 + wn0 + 16 * j + 4 * kg;
+            for (int e = 0; e < 4; ++e) v[e] = accT[j][i][e];
+            if (C) {
+                const uint32_t col = n0 + wn0 + 16 * j + 4 * kg;
+                if (interior || (row < g.M && col + 4 <= g.N)) {
                     const halfx4 cv = *(const halfx4*)(C + (size_t)row * g.ldc + col);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf((float)cv[e], g.beta, g.alpha * v[e]);
+                } else if (row < g.M) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < g.N) v[e] = __builtin_fmaf((float)C[(size_t)row * g.ldc + col + e], g.beta, g.alpha * v[e]);
                 }
-                const uintx2 out = {pack2(v[0], v[1]), pack2(v[2], v[3])};
-                // piece p (16 bytes) of row l16, half kg & 1 of it; pieces XOR-permuted so that the 32 lanes of a write
-                // and the 16 lanes of a read-back each cover all banks once
-                const int p = 2 * j + (kg >> 1);
-                *(uintx2*)(stage_rows + l16 * ROW_BYTES + ((p ^ ((l16 / RPG) % PPR)) * 16) + (kg & 1) * 8) = out;
             }
-            wave_sync();
-#pragma unroll
-            for (int t2 = 0; t2 < STORES; ++t2) {
-                const int r = ROWS_PER_STORE * t2 + lane / PPR, pc = lane % PPR;
-                const uintx4 v = *(const uintx4*)(stage_rows + r * ROW_BYTES + ((pc ^ ((r / RPG) % PPR)) * 16));
-                *(uintx4*)(D + (size_t)(m0 + wm0 + 16 * i + r) * g.ldd + n0 + wn0 + 8 * pc) = v;
-            }
-            wave_sync();
-        } else if (row < g.M) {
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const uint32_t col = n0 + wn0 + 16 * j + 4 * kg + e;
-                    if (col < g.N) {
-                        float v = accT[j][i][e];
-                        if (C) v = __builtin_fmaf((float)C[(size_t)row * g.ldc + col], g.beta, g.alpha * v);
-                        D[(size_t)row * g.ldd + col] = (_Float16)v;
-                    }
-                }
+            const uintx2 out = {pack2(v[0], v[1]), pack2(v[2], v[3])};
+            // piece p (16 bytes) of row l16, half kg & 1 of it; pieces XOR-permuted so that the 32 lanes of a write
+            // and the 16 lanes of a read-back each cover all banks once
+            const int p = 2 * j + (kg >> 1);
+            *(uintx2*)(stage_rows + l16 * ROW_BYTES + ((p ^ ((l16 / RPG) % PPR)) * 16) + (kg & 1) * 8) = out;
         }
+        wave_sync();
+#pragma unroll
+        for (int t2 = 0; t2 < STORES; ++t2) {
+            const int r = ROWS_PER_STORE * t2 + lane / PPR, pc = lane % PPR;
+            const uintx4 v = *(const uintx4*)(stage_rows + r * ROW_BYTES + ((pc ^ ((r / RPG) % PPR)) * 16));
+            const uint32_t grow = m0 + wm0 + 16 * i + r, gcol = n0 + wn0 + 8 * pc;
+            _Float16* out = D + (size_t)grow * g.ldd + gcol;
+            if (interior || (grow < g.M && gcol + 8 <= g.N)) {
+                *(uintx4*)out = v;
+            } else if (grow < g.M && gcol < g.N) {
+                union { uintx4 u; _Float16 h[8]; } w;
+                w.u = v;
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (gcol + e < g.N) out[e] = w.h[e];
+            }
+        }
+        wave_sync();
     }
 }
 

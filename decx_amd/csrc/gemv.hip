@@ -19,8 +19,10 @@
 //   workgroup (2048 x 8192: 24.3 -> 16.1 us with a dense x, 512 x 32768: 60.9 -> 23.8); x is staged in LDS once per
 //   workgroup, as fp32, in chunks of 4096 -- x may be strided (the single column of a
 //   pitched K x 1 matrix puts every element in its own cache line), so staging it once per
-//   32 rows keeps that gather small; A is read with 128-bit loads; per lane an fp32 fma
-//   chain, then a butterfly over the 64 lanes.
+//   32 rows keeps that gather small -- and a chunk of x is loaded into registers while the chunk
+//   before is being multiplied, so that its latency hides behind the rows (8192 x 8192: fp32 43.1 -> 42.0 us,
+//   fp16 26.1 -> 23.9; gevm the same way: 39.2 -> 37.8 and 24.3 -> 23.3); A is read with 128-bit loads; per
+//   lane an fp32 fma chain, then a butterfly over the 64 lanes.
 // gevm: a workgroup owns 128 bytes of columns (32 fp32 / 64 fp16); 8 lanes cover those with
 //   one 128-bit load each, the other lane bits and the 16 wavefronts stride over k
 //   (128 rows per sweep); partial sums meet in a shuffle over the row lanes and in LDS over
@@ -37,6 +39,7 @@ constexpr int GEMV_THREADS = 1024;
 constexpr int GEMV_WAVES = GEMV_THREADS / 64;
 constexpr int GEMV_ROWS_PER_BLOCK = 2 * GEMV_WAVES;
 constexpr int GEMV_KC = 4096;            // elements of x staged per chunk (16 KB of LDS, 32 KB for fp64)
+constexpr int GEMV_XPT = GEMV_KC / GEMV_THREADS;   // of which a thread carries this many
 
 typedef double doublex2 __attribute__((ext_vector_type(2)));
 
@@ -103,20 +106,47 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
     // workgroup starts at another chunk and each wavefront at another step inside it (sums commute).
     const uint32_t chunks = (K + GEMV_KC - 1) / GEMV_KC;
     const uint32_t chunk0 = chunks ? (blockIdx.x * 3u) % chunks : 0u;
+    // x travels one chunk ahead in registers, its loads dealt out among the steps of the chunk before: a strided x
+    // (the column of a pitched K x 1 matrix) touches a cache line per element, and with one workgroup per CU the loads
+    // of the rows queue behind whatever is issued in a burst.
+    constexpr uint32_t STEP = 64 * N16;
+    constexpr int PER = GEMV_KC / (int)STEP / GEMV_XPT;    // steps per load of x: fp32 4, fp16 2, fp64 8
+    constexpr int XG = PER >= 4 ? 1 : 4 / PER;             // loads of x per group of at least 4 steps
+    constexpr int GROUPS = GEMV_XPT / XG;
+    T xr[GEMV_XPT];
+    const auto fetch_x = [&](uint32_t kc, int j) {
+        const uint32_t i = t + j * GEMV_THREADS;
+        xr[j] = kc + i < K ? x[(size_t)(kc + i) * incx] : T(0);
+    };
+    if (chunks) {
+#pragma unroll
+        for (int j = 0; j < GEMV_XPT; ++j) fetch_x(chunk0 * GEMV_KC, j);
+    }
     for (uint32_t ci = 0; ci < chunks; ++ci) {
         const uint32_t chunk = chunk0 + ci < chunks ? chunk0 + ci : chunk0 + ci - chunks;
         const uint32_t kc = chunk * GEMV_KC;
         const uint32_t len = (K - kc) < (uint32_t)GEMV_KC ? (K - kc) : (uint32_t)GEMV_KC;
         __syncthreads();                                   // previous chunk fully consumed
-        for (uint32_t i = t; i < len; i += GEMV_THREADS) xs[i] = to_acc(x[(size_t)(kc + i) * incx]);
+#pragma unroll
+        for (int j = 0; j < GEMV_XPT; ++j) xs[t + j * GEMV_THREADS] = to_acc(xr[j]);
         __syncthreads();
+        const bool more = ci + 1 < chunks;
+        const uint32_t kc_next = (chunk + 1 < chunks ? chunk + 1 : 0u) * GEMV_KC;
         const uint32_t lenv = vec_ok ? (len / N16) * N16 : 0u;   // part done with 128-bit loads
-        if (has0) {
-            constexpr uint32_t STEP = 64 * N16;
-            const uint32_t steps = (lenv + STEP - 1) / STEP;
-            const uint32_t step0 = steps ? ((blockIdx.x * GEMV_WAVES + wave - sub) * 5u) % steps : 0u;   // one start per row
+        const uint32_t steps = (lenv + STEP - 1) / STEP;
+        const uint32_t mine = has0 && steps > (uint32_t)sub ? (steps - sub + WPR - 1) / WPR : 0u;   // steps of this wavefront
+        const uint32_t step0 = steps ? ((blockIdx.x * GEMV_WAVES + wave - sub) * 5u) % steps : 0u;   // one start per row
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+            if (more) {
+#pragma unroll
+                for (int j = 0; j < XG; ++j) fetch_x(kc_next, g * XG + j);
+            }
+            // the last chunk has no loads of x to make room for: its steps stay in one loop
+            const uint32_t lo = more ? mine * g / GROUPS : (g == 0 ? 0u : mine), hi = more ? mine * (g + 1) / GROUPS : mine;
 #pragma unroll 4
-            for (uint32_t i = sub; i < steps; i += WPR) {
+            for (uint32_t ii = lo; ii < hi; ++ii) {
+                const uint32_t i = sub + ii * WPR;
                 const uint32_t step = step0 + i < steps ? step0 + i : step0 + i - steps;
                 const uint32_t k = step * STEP + lane * N16;
                 if (k < lenv) {
@@ -131,6 +161,8 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
                     }
                 }
             }
+        }
+        if (has0) {
             for (uint32_t k = lenv + lane + 64u * sub; k < len; k += 64u * WPR) {   // the tail, or a whole unaligned row
                 s0 = fma_acc(to_acc(a0[kc + k]), xs[k], s0);
                 if (has1) s1 = fma_acc(to_acc(a1[kc + k]), xs[k], s1);
@@ -192,11 +224,22 @@ gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restric
 #pragma unroll
     for (int e = 0; e < N16; ++e) acc[e] = 0;
 
+    T xr[GEMV_XPT];                                        // x one chunk ahead, as in gemv_kernel
+    const auto fetch_x = [&](uint32_t kc) {
+#pragma unroll
+        for (int j = 0; j < GEMV_XPT; ++j) {
+            const uint32_t i = t + j * GEMV_THREADS;
+            xr[j] = kc + i < K ? x[(size_t)(kc + i) * incx] : T(0);
+        }
+    };
+    if (K) fetch_x(0);
     for (uint32_t kc = 0; kc < K; kc += GEMV_KC) {
         const uint32_t len = (K - kc) < (uint32_t)GEMV_KC ? (K - kc) : (uint32_t)GEMV_KC;
         __syncthreads();
-        for (uint32_t i = t; i < len; i += GEMV_THREADS) xs[i] = to_acc(x[(size_t)(kc + i) * incx]);
+#pragma unroll
+        for (int j = 0; j < GEMV_XPT; ++j) xs[t + j * GEMV_THREADS] = to_acc(xr[j]);
         __syncthreads();
+        if (kc + GEMV_KC < K) fetch_x(kc + GEMV_KC);
         if (n0 < N) {
 #pragma unroll 2
             for (uint32_t k = wave * RL + row_lane; k < len; k += GEMV_WAVES * RL) {
@@ -317,7 +360,8 @@ uint32_t gemv_rows_per_block(uint32_t M)
 // A strided x (the single column of a pitched K x 1 matrix) costs every workgroup of gemv one cache
 // line request per element; gathered once into a dense buffer it costs one per 32 (fp32) or 64.
 // The copy is a launch of its own (about 4.5 us with its loads, all L2 misses): it pays from the sizes
-// below (8192 x 8192: 46.7 -> 43.9 us, 512 x 32768: 44.7 -> 23.8, 256 x 8192: 10.8 -> 7.2, 4096 x 2048: 7.7 -> 7.9).
+// below (8192 x 8192: 45.4 -> 41.8 us, with a dense x 38.5; 512 x 32768: 44.7 -> 23.8, 256 x 8192: 10.8 -> 7.2,
+// 4096 x 2048: 7.7 -> 7.9).
 bool gemv_gather_pays(uint32_t M, uint32_t K, uint32_t incx)
 {
     if (incx <= 1) return false;
