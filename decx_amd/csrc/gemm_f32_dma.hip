@@ -469,7 +469,7 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
             if constexpr (C_EARLY) {
                 if (C) v[0] = __builtin_fmaf(c_early[r], g.beta, g.alpha * v[0]);
             }
-            if (interior) {
+            if (interior || (row < g.M && col0 + TN <= g.N)) {      // the lane's TN columns exist: one store
                 if constexpr (!C_EARLY) {
                     if (C) {
                         const bfrag cv = *(const bfrag*)(C + (size_t)row * g.ldc + col0);
@@ -512,7 +512,10 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     // 256 x 128 tiles, two independent workgroups per CU: patches two tile-rows high fetch least (8192^3: 5.5 GB through
     // L2 against 6.2 GB with four rows and 11.7 GB with eight, at the same speed)
     if constexpr (BM == 256 && BN == 128 && CONV == 0) g.group_m = 2;
-    if (g.split_len) {                                     // the planner splits K on the smallest tiles only
+    // The planner splits K on the smallest tiles only.  (On 128 x 128 tiles the exchange costs the kernel a workgroup per
+    // CU -- 149 VGPRs beside the 64 accumulators, two workgroups where three fit -- and whole rounds in front of a split
+    // last round then gain 1 % at 5120^3 and lose at 2560^3, 3072^3 and 3584^3.)
+    if (g.split_len) {
         if constexpr (CONV == 0 && BM * BN == 64 * 64) {
             const uint32_t splits = g.split_count;
             if (g.C)

@@ -304,7 +304,7 @@ gemm_f64_dma_kernel(const GemmArgs g_in)
             for (int jj = 0; jj < TP; ++jj) {
                 const uint32_t col = n0 + b_col + 32 * jj;
                 double v0 = acc[ti][2 * jj][i], v1 = acc[ti][2 * jj + 1][i];
-                if (interior) {
+                if (interior || (row < g.M && col + 2 <= g.N)) {
                     if (C) {
                         const doublex2 cv = *(const doublex2*)(C + (size_t)row * g.ldc + col);
                         v0 = __builtin_fma(cv[0], g.beta64, g.alpha64 * v0);

@@ -72,6 +72,16 @@ template <typename T> __device__ __forceinline__ void load16(const T* p, typenam
     }
 }
 
+// the same in two halves: the 16 bytes as they are (a load that nothing waits for yet), and their widening
+template <typename T> struct Raw16 { typedef floatx4 type; };
+template <> struct Raw16<_Float16> { typedef halfx8 type; };
+template <> struct Raw16<double> { typedef doublex2 type; };
+template <typename T> __device__ __forceinline__ void widen16(const typename Raw16<T>::type& v, typename Acc<T>::type (&out)[Per16<T>::n])
+{
+#pragma unroll
+    for (int e = 0; e < Per16<T>::n; ++e) out[e] = (typename Acc<T>::type)v[e];
+}
+
 template <typename A> __device__ __forceinline__ A wave_sum(A v)
 {
 #pragma unroll
@@ -108,7 +118,9 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
     const uint32_t chunk0 = chunks ? (blockIdx.x * 3u) % chunks : 0u;
     // x travels one chunk ahead in registers, its loads dealt out among the steps of the chunk before: a strided x
     // (the column of a pitched K x 1 matrix) touches a cache line per element, and with one workgroup per CU the loads
-    // of the rows queue behind whatever is issued in a burst.
+    // of the rows queue behind whatever is issued in a burst.  (Asking for the first rows of A ahead of x as well, as
+    // gevm_kernel does for B, takes this kernel beyond 64 VGPRs and with that from two workgroups per CU to one:
+    // 16384 x 1024 13.2 -> 15.3 us, fp16 6.5 -> 9.9.)
     constexpr uint32_t STEP = 64 * N16;
     constexpr int PER = GEMV_KC / (int)STEP / GEMV_XPT;    // steps per load of x: fp32 4, fp16 2, fp64 8
     constexpr int XG = PER >= 4 ? 1 : 4 / PER;             // loads of x per group of at least 4 steps
@@ -233,6 +245,19 @@ gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restric
         }
     };
     if (K) fetch_x(0);
+    // The first rows of B are asked for before x is in LDS: the memory system has work from the first cycle on, not
+    // only after the round trip of x and two barriers.
+    constexpr int PRE = 4;
+    typename Raw16<T>::type pre[PRE];
+    const uint32_t len0 = K < (uint32_t)GEMV_KC ? K : (uint32_t)GEMV_KC;
+    const bool pre_ok = whole && n0 < N;
+    if (pre_ok) {
+#pragma unroll
+        for (int u = 0; u < PRE; ++u) {
+            const uint32_t k = wave * RL + row_lane + u * (GEMV_WAVES * RL);
+            if (k < len0) pre[u] = *(const typename Raw16<T>::type*)(B + (size_t)k * ldb + n0);
+        }
+    }
     for (uint32_t kc = 0; kc < K; kc += GEMV_KC) {
         const uint32_t len = (K - kc) < (uint32_t)GEMV_KC ? (K - kc) : (uint32_t)GEMV_KC;
         __syncthreads();
@@ -240,9 +265,24 @@ gevm_kernel(const T* __restrict__ x, const T* __restrict__ B, const T* __restric
         for (int j = 0; j < GEMV_XPT; ++j) xs[t + j * GEMV_THREADS] = to_acc(xr[j]);
         __syncthreads();
         if (kc + GEMV_KC < K) fetch_x(kc + GEMV_KC);
+        uint32_t k_first = wave * RL + row_lane;
+        if (kc == 0 && pre_ok) {
+#pragma unroll
+            for (int u = 0; u < PRE; ++u) {
+                const uint32_t k = wave * RL + row_lane + u * (GEMV_WAVES * RL);
+                if (k < len) {
+                    A_t bv[N16];
+                    widen16<T>(pre[u], bv);
+                    const A_t xv = xs[k];
+#pragma unroll
+                    for (int e = 0; e < N16; ++e) acc[e] = fma_acc(xv, bv[e], acc[e]);
+                }
+            }
+            k_first += PRE * (GEMV_WAVES * RL);
+        }
         if (n0 < N) {
-#pragma unroll 2
-            for (uint32_t k = wave * RL + row_lane; k < len; k += GEMV_WAVES * RL) {
+#pragma unroll 4
+            for (uint32_t k = k_first; k < len; k += GEMV_WAVES * RL) {
                 const T* p = B + (size_t)(kc + k) * ldb + n0;
                 const A_t xv = xs[k];
                 if (whole) {
