@@ -469,7 +469,7 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
             if constexpr (C_EARLY) {
                 if (C) v[0] = __builtin_fmaf(c_early[r], g.beta, g.alpha * v[0]);
             }
-            if (interior || (row < g.M && col0 + TN <= g.N)) {      // the lane's TN columns exist: one store
+            if (interior) {       // (one store also on edge tiles wherever the lane's TN columns all exist: 141 VGPRs in place of 64)
                 if constexpr (!C_EARLY) {
                     if (C) {
                         const bfrag cv = *(const bfrag*)(C + (size_t)row * g.ldc + col0);
