@@ -619,3 +619,43 @@ def test_split_k_slots_carry_nothing_from_launch_to_launch(hip, oracle, dtype, M
                 assert np.array_equal(got.view(bits), first[it % 2].view(bits)), "launch %d" % it
     for d in [ws, dD] + [x for t in sets for x in t[2:]]:
         d.free()
+
+
+@pytest.mark.parametrize("dtype,M,N,K", [(np.float32, 1000, 1500, 777), (np.float16, 640, 640, 8192), (np.float64, 1536, 1400, 1536)])
+def test_split_k_on_two_streams_at_once(hip, oracle, dtype, M, N, K):
+    """Every launch takes its own window of tile counters, so products that split K may run side by side on two streams
+    (each with a workspace of its own): the results are those of the same products run alone, bit for bit."""
+    import ctypes
+    esz = np.dtype(dtype).itemsize
+    need = hip.lib().decx_hip_gemm_workspace(esz, M, N, K)
+    if need == 0 or hip.plan(esz, M, N, K).k_splits < 2:
+        pytest.skip("the planner does not split this shape")
+    L = hip.lib()
+    pa, pn = device_pitch(K, dtype), device_pitch(N, dtype)
+    make = {2: synth.normal_half, 4: synth.uniform_f32, 8: synth.uniform_f64}[esz]
+    bits = {2: np.uint16, 4: np.uint32, 8: np.uint64}[esz]
+    lanes = []
+    for s in range(2):
+        st = ctypes.c_void_p()
+        assert L.decx_hip_stream_create(ctypes.byref(st)) == 0
+        A = make(M, K, 900 + s); B = make(K, N, 910 + s)
+        lanes.append(dict(stream=st, A=hip.DeviceMatrix(M, K, dtype, pa, A), B=hip.DeviceMatrix(K, N, dtype, pn, B),
+                          D=hip.DeviceMatrix(M, N, dtype, pn), ws=hip.DeviceMatrix(1, need // 4, np.float32)))
+    alone = []
+    for ln in lanes:                                          # one after the other, on the default stream
+        hip.gemm(ln["A"], ln["B"], ln["D"], workspace=ln["ws"])
+        hip.sync()
+        alone.append(ln["D"].download())
+    for rep in range(5):
+        for ln in lanes:
+            ln["D"].upload_raw(np.full((M, pn), 3, dtype))
+        for it in range(12):                                  # launches of the two streams interleave on the chip
+            for ln in lanes:
+                hip.gemm(ln["A"], ln["B"], ln["D"], workspace=ln["ws"], stream=ln["stream"])
+        for ln, want in zip(lanes, alone):
+            hip.sync(ln["stream"])
+            assert np.array_equal(ln["D"].download().view(bits), want.view(bits)), "repetition %d" % rep
+    for ln in lanes:
+        assert L.decx_hip_stream_destroy(ln["stream"]) == 0
+        for k in ("A", "B", "D", "ws"):
+            ln[k].free()
