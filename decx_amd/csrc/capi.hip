@@ -113,6 +113,7 @@ struct SplitChoice { int shape; uint32_t splits, len, first; };     // first: ti
 struct SplitTile {
     int shape, fit, pieces;          // size class, workgroups per CU, 16-byte pieces of accumulators per lane
     double ns_per_k[5];              // per workgroup with m = 1 .. fit of them on the CU
+    double ns_per_k_one_round[5];    // the same in a launch of at most fit x CUs workgroups, where the kernel has a tighter loop (0: none)
 };
 struct SplitModel {
     SplitTile tiles[2]; int n_tiles;
@@ -121,7 +122,7 @@ struct SplitModel {
     bool uneven_second_round;
 };
 // 64 x 64 tiles of 32 KB LDS: four fit a CU (160 KB would hold five, but time against the number of tiles steps as for four)
-static const SplitModel kSplitF32 = {{{TILE_SMALL, 4, 4, {0, 17.72, 15.51, 15.07, 14.77}}, {}}, 1, 32, 4, 1.0, 0.4, 0.15, 0.586e6, true};
+static const SplitModel kSplitF32 = {{{TILE_SMALL, 4, 4, {0, 17.72, 15.51, 15.07, 14.77}, {0, 15.8, 14.4, 14.3, 14.16}}, {}}, 1, 32, 4, 1.0, 0.4, 0.15, 0.586e6, true};
 static const SplitModel kSplitF16 = {{{TILE_SMALL, 4, 4, {0, 4.33, 3.21, 3.18, 3.07}}, {TILE_MEDIUM, 2, 8, {0, 7.67, 6.95}}}, 2,
                                      64, 4, 0.5, 2.0, 0.15, 5.2e6, false};
 static const SplitModel kSplitF64 = {{{TILE_SMALL, 2, 4, {0, 34.0, 30.3}}, {}}, 1, 32, 8, 0.5, 2.0, 0.30, 0.283e6, false};
@@ -146,12 +147,13 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
         const uint64_t full = wgs / slots, rem = wgs % slots;
         uint64_t m = (rem + cus - 1) / cus;
         if (md.uneven_second_round && full == 1 && rem > cus / 2 && rem <= cus) m = 2;
-        double lone = st.ns_per_k[1];
+        const double* rate = (whole + wgs <= slots && st.ns_per_k_one_round[1] > 0) ? st.ns_per_k_one_round : st.ns_per_k;
+        double lone = rate[1];
         if (elem_bytes == 2 && st.shape == TILE_MEDIUM)        // 6.0 ns with half the CUs busy, 7.67 with all
             lone = wgs <= cus / 2 ? 6.0 : 6.0 + 1.67 * (double)(wgs - cus / 2) / (double)(cus - cus / 2);
         const uint32_t k_whole = (K + md.len_align - 1) / md.len_align * md.len_align;
-        const double ns = (double)len * ((double)full * st.fit * st.ns_per_k[st.fit] + (m == 1 ? lone : (double)m * st.ns_per_k[m])) +
-                          (double)k_whole * (double)(whole / slots) * st.fit * st.ns_per_k[st.fit];
+        const double ns = (double)len * ((double)full * st.fit * rate[st.fit] + (m == 1 ? lone : (double)m * rate[m])) +
+                          (double)k_whole * (double)(whole / slots) * st.fit * rate[st.fit];
         double us = ns * 1e-3 + kLaunch;
         if (ranges > 1) {
             const uint32_t group = st.pieces < 16 ? st.pieces : 16, batch = 16 / group, per_slot = st.pieces / group;
@@ -280,6 +282,7 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
     constexpr uint32_t per16 = F16 ? 8u : 4u;          // elements per 16 bytes
     GemmArgs g;
     std::memset(&g, 0, sizeof g);
+    g.cus = (uint32_t)g_dev.compute_units;
     g.A = A; g.B = B; g.C = C; g.D = D;
     g.M = M; g.N = N; g.K = K;
     g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldd = ldd;
@@ -556,6 +559,7 @@ static int run_gemm_f64(const double* A, const double* B, const double* C, doubl
 
     GemmArgs g;
     std::memset(&g, 0, sizeof g);
+    g.cus = (uint32_t)g_dev.compute_units;
     g.A = A; g.B = B; g.C = C; g.D = D;
     g.M = M; g.N = N; g.K = K;
     g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldd = ldd;
@@ -755,6 +759,7 @@ int decx_hip_conv2d_f32_depth(const float* image, const float* kmat, float* dst,
         return DECX_HIP_E_INVALID_ARG;
     GemmArgs g;
     std::memset(&g, 0, sizeof g);
+    g.cus = (uint32_t)g_dev.compute_units;
     g.A = image; g.B = kmat; g.C = nullptr; g.D = dst;
     g.M = out_w * out_h; g.N = out_c; g.K = k_h * k_w * img_dpitch;
     g.lda = g.K; g.ldb = kmat_pitch; g.ldc = 0; g.ldd = dst_dpitch;

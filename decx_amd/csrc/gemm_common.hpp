@@ -29,6 +29,7 @@ struct GemmArgs {
     double alpha64, beta64;      // the same two scalars for the fp64 kernels
     uint32_t tiles_m, tiles_n;   // number of block tiles along M and N
     uint32_t vec_ok;             // 1: every base pointer is 16-byte aligned and every pitch a multiple of 16 bytes
+    uint32_t cus;                // compute units of the device (0: not given, the kernels take 256)
     // Split K (direct-load kernels; a 1-D grid of split_first whole tiles, then split 0 of every split tile, split 1 of
     // every split tile, ...): split z multiplies k in [z * split_len, min(K, (z + 1) * split_len)).  Every workgroup stores its accumulators (fp32, or fp64 for fp64 operands) to its
     // slot of split_ws and counts itself in at split_counters[tile]; the one that arrives last adds all slots of the

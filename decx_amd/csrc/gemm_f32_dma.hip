@@ -400,16 +400,30 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
         };
         constexpr int READS = TM + 4, MFMAS = 4 * TM * TN;
 
-        for (uint32_t s = 0; s < slabs; ++s) {
-            const unsigned char* st = lds + (s % STAGES) * STAGE_BYTES;
-            const bool more = s + STAGES - 1 < slabs;
+        // One slab.  STAGE >= 0: the stage it sits in is known at compile time, and the slab that is asked for while this
+        // one multiplies is a whole one (direct loads, no questions asked); STAGE < 0: the general form.  A loop over
+        // STAGES such slabs is one block of code without a branch inside and without a vector ALU instruction between its
+        // MFMAs: every LDS address is a register that never changes plus an immediate.  A wavefront that has its SIMD
+        // to itself (one workgroup per CU) needs that: a VALU instruction issued behind an MFMA holds up the next MFMA
+        // of the same accumulator chain by about 20 cycles (measured on a bare chain of v_mfma_f32_32x32x2_f32: 64
+        // cycles each, 74 with two integer adds per four of them), and a taken branch leaves the matrix pipe empty
+        // (1024^3, one 64 x 64 tile per CU: 84 -> 70 cycles per MFMA, 21.5 -> 18.5 us).
+        auto slab_body = [&](uint32_t s, auto stage_c) {
+            constexpr int STAGE = decltype(stage_c)::value;
+            constexpr bool STEADY = STAGE >= 0;
+            const unsigned char* st;
+            if constexpr (STEADY) st = lds + STAGE * STAGE_BYTES; else st = lds + (s % STAGES) * STAGE_BYTES;
+            const bool more = STEADY || s + STAGES - 1 < slabs;
 
             read_chunk(st, std::integral_constant<int, 0>{});
             multiply_chunk(std::integral_constant<int, CHUNKS - 1>{});
             __builtin_amdgcn_sched_group_barrier(0x100, READS, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
             __builtin_amdgcn_sched_barrier(0);
-            if (more) issue_loads(s + STAGES - 1);
+            if constexpr (STEADY) {
+                static_for<0, LOADS>([&](auto ic) { issue_one((uint32_t)((STAGE + STAGES - 1) % STAGES), ic); });
+                __builtin_amdgcn_sched_barrier(0);             // the loads stay in front of the next chunk's reads
+            } else if (more) issue_loads(s + STAGES - 1);
 
             static_for<0, CHUNKS - 1>([&](auto cc) {
                 constexpr int c = decltype(cc)::value;
@@ -422,7 +436,21 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
             });
 
             if (more) wait_loads_and_barrier<LOADS * (STAGES - 2)>(); else wait_loads_and_barrier<0>();
-        }
+        };
+        // Slabs [0, steady): the slab STAGES - 1 ahead is a whole one; they are walked STAGES at a time in the tight form,
+        // in launches of at most one round of workgroups (four 64 x 64 tiles to a CU).  With more rounds the tight form loses: the
+        // wavefront that is oldest on its SIMD then wins every MFMA slot it is ready for, the workgroups of a round end
+        // far apart (2048^3, four per CU: between 69 and 139 us, against 108 to 142) and the rounds no longer tile
+        // (3072 x 2048 x 2048, six per CU: 207 us against 188; a VALU instruction per chunk put back on purpose mends
+        // 8 per CU, 245 against 249 us, but neither 6 nor 9 per CU), so those launches keep the general form, whose
+        // address arithmetic and branches happen to share the matrix pipe evenly.
+        const uint32_t steady = __builtin_amdgcn_readfirstlane(full_slabs > (uint32_t)(STAGES - 1) ? (full_slabs - (uint32_t)(STAGES - 1)) / STAGES * STAGES : 0u);
+        constexpr uint32_t FIT = BM * BN >= 128 * 128 ? 3u : 4u;                    // workgroups of this tile that share a CU
+        const bool one_round = gridDim.x <= FIT * (g_in.cus ? g_in.cus : 256u);
+        uint32_t s = 0;
+        if (one_round)
+            for (; s < steady; s += STAGES) static_for<0, STAGES>([&](auto jc) { slab_body(s + decltype(jc)::value, jc); });
+        for (; s < slabs; ++s) slab_body(s, std::integral_constant<int, -1>{});
         multiply_chunk(std::integral_constant<int, CHUNKS - 1>{});
     }
 

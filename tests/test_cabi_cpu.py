@@ -89,8 +89,8 @@ def test_planner_choices():
     assert p.k_splits > 1 and p.grid == 25 * p.k_splits and hip.plan(4, 8192, 8192, 8192).k_splits == 1
     assert hip.plan(4, 300, 300, 400).k_splits == 1 and hip.plan(2, 256, 256, 65536).k_splits > 1
     # a few hundred tiles that do not divide among 256 CUs and a long K: even rounds of workgroups on the small tile
-    p = hip.plan(4, 1280, 1024, 8192)                      # 320 tiles of 64 x 64 on 8 ranges: ten per CU, four at a time
-    assert (p.tile_m, p.k_splits, p.grid) == (64, 8, 320 * 8)     # 161 us; 4 ranges (five per CU, a lone fifth) 185, whole 251
+    p = hip.plan(4, 1280, 1024, 8192)                      # 320 tiles of 64 x 64 on 3 ranges: 960 workgroups, one round of
+    assert (p.tile_m, p.k_splits, p.grid) == (64, 3, 320 * 3)     # at most four per CU (163.7 us; 8 ranges, 2.5 rounds: 166.8, whole 251)
     p = hip.plan(4, 1536, 1024, 8192)                      # 384 tiles on 2 ranges: three per CU
     assert (p.tile_m, p.k_splits) == (64, 2)
     assert hip.plan(4, 2048, 2048, 8192).k_splits == 1 and hip.plan(4, 1280, 1024, 2048).k_splits == 3    # 1.25 tiles per CU: 65.6 -> 47.1 us
