@@ -325,9 +325,14 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
             bf[step & BFM] = *(const bfrag*)(st + b_off + (8 * (step / 4) + step % 4) * BN * 4);
         };
 
-        for (uint32_t s = 0; s < slabs; ++s) {
-            const unsigned char* st = lds + (s % STAGES) * STAGE_BYTES;
-            const bool more = s + STAGES - 1 < slabs;
+        // One slab; STAGE >= 0: its stage is known at compile time and the slab asked for meanwhile is a whole one (see
+        // the small-tile loop below for what that buys), STAGE < 0: the general form.
+        auto slab_body = [&](uint32_t s, auto stage_c) {
+            constexpr int STAGE = decltype(stage_c)::value;
+            constexpr bool STEADY = STAGE >= 0;
+            const unsigned char* st;
+            if constexpr (STEADY) st = lds + STAGE * STAGE_BYTES; else st = lds + (s % STAGES) * STAGE_BYTES;
+            const bool more = STEADY || s + STAGES - 1 < slabs;
 
 #pragma unroll
             for (int i = 0; i < TM; ++i) af[0][i] = *(const floatx4*)(st + a_off[0] + i * 32 * BK * 4);
@@ -337,9 +342,9 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
             __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
             __builtin_amdgcn_sched_barrier(0);
             // The stage that held slab s-1 is free: every wave passed the barrier after reading it.
-            const uint32_t nstage = (s + STAGES - 1) % STAGES;
-            const bool direct = s + STAGES - 1 < full_slabs;
-            if (more && !direct) issue_tail(nstage);
+            const uint32_t nstage = STEADY ? (uint32_t)((STAGE + STAGES - 1) % STAGES) : (s + STAGES - 1) % STAGES;
+            const bool direct = STEADY || s + STAGES - 1 < full_slabs;
+            if constexpr (!STEADY) { if (more && !direct) issue_tail(nstage); }
 
             static_for<0, STEPS - 1>([&](auto stc) {
                 constexpr int step = decltype(stc)::value;
@@ -367,7 +372,11 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
             // slab s+1 must have landed (ours: vmcnt; everyone's: barrier); the loads of the
             // STAGES-2 slabs behind it may stay in flight.
             if (more) wait_loads_and_barrier<LOADS * (STAGES - 2)>(); else wait_loads_and_barrier<0>();
-        }
+        };
+        const uint32_t steady = __builtin_amdgcn_readfirstlane(full_slabs > (uint32_t)(STAGES - 1) ? (full_slabs - (uint32_t)(STAGES - 1)) / STAGES * STAGES : 0u);
+        uint32_t s = 0;
+        for (; s < steady; s += STAGES) static_for<0, STAGES>([&](auto jc) { slab_body(s + decltype(jc)::value, jc); });
+        for (; s < slabs; ++s) slab_body(s, std::integral_constant<int, -1>{});
         multiply(std::integral_constant<int, STEPS - 1>{});
     } else {
         // Small wave tiles: a k step is one or two MFMAs, shorter than an LDS read, so fragments are
