@@ -137,23 +137,25 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
 
     const unsigned char* a_src[A_LOADS];
     const unsigned char* b_src[B_LOADS];
-    int a_chunk[A_LOADS], b_krow[B_LOADS];
+    // chunk of its row that copy lane i of A fetches / k row of copy lane i of B (functions, not arrays: the partial last
+    // slab is the only other place that wants them, and registers that live across the K loop are scarce)
+    auto a_chunk_of = [&](int i) { const int row = (64 / CPR) * (wave * A_LOADS + i) + lane / CPR; return (lane % CPR) ^ ((row / RPB) % CPR); };
+    auto b_krow_of = [&](int i) { return BROWS * (wave * B_LOADS + i) + lane / CBR; };
     const uint32_t last_row = g.M - 1, last_col_chunk = (g.N - 1) / 8;
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
         const int I = wave * A_LOADS + i;
         const int row = (64 / CPR) * I + lane / CPR;
-        a_chunk[i] = (lane % CPR) ^ ((row / RPB) % CPR);
         const uint32_t grow = (m0 + row) < last_row ? (m0 + row) : last_row;
-        a_src[i] = A + (size_t)grow * lda_b + a_chunk[i] * 16;
+        a_src[i] = A + (size_t)grow * lda_b + a_chunk_of(i) * 16;
     }
 #pragma unroll
     for (int i = 0; i < B_LOADS; ++i) {
         const int I = wave * B_LOADS + i;
-        b_krow[i] = BROWS * I + lane / CBR;
-        const int chunk = (lane % CBR) ^ b_key(b_krow[i]);
+        const int krow = b_krow_of(i);
+        const int chunk = (lane % CBR) ^ b_key(krow);
         const uint32_t gchunk = (n0 / 8 + chunk) < last_col_chunk ? (n0 / 8 + chunk) : last_col_chunk;
-        b_src[i] = B + (size_t)b_krow[i] * ldb_b + (size_t)gchunk * 16;
+        b_src[i] = B + (size_t)krow * ldb_b + (size_t)gchunk * 16;
     }
 
     const uint32_t full_slabs = g.K / BK, k_tail = g.K % BK;
@@ -170,29 +172,32 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     // Slabs are issued in ascending order.  A direct load takes its address as a scalar base (the tile's
     // first row of A / B's row k, running along K) plus a 32-bit lane offset that never changes, so that
     // advancing to the next slab is scalar arithmetic.
+    auto issue_direct = [&](uint32_t stage) {               // a whole slab, straight into LDS
+        const uint32_t stage_off = lds_base + stage * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) {
+            const uint32_t dst = stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(a_voff[i]), "s"(a_base) : "memory", "m0");
+        }
+        a_base += RB;
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) {
+            const uint32_t dst = stage_off + A_STAGE_BYTES + (uint32_t)(wave * B_LOADS + i) * 1024u;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(b_voff[i]), "s"(b_base) : "memory", "m0");
+        }
+        b_base += b_step;
+    };
     auto issue_loads = [&](uint32_t slab) {
         const uint32_t stage = slab % STAGES;
         if (slab < full_slabs) {
-            const uint32_t stage_off = lds_base + stage * STAGE_BYTES;
-#pragma unroll
-            for (int i = 0; i < A_LOADS; ++i) {
-                const uint32_t dst = stage_off + (uint32_t)(wave * A_LOADS + i) * 1024u;
-                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(a_voff[i]), "s"(a_base) : "memory", "m0");
-            }
-            a_base += RB;
-#pragma unroll
-            for (int i = 0; i < B_LOADS; ++i) {
-                const uint32_t dst = stage_off + A_STAGE_BYTES + (uint32_t)(wave * B_LOADS + i) * 1024u;
-                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(b_voff[i]), "s"(b_base) : "memory", "m0");
-            }
-            b_base += b_step;
+            issue_direct(stage);
         } else {
             // the partial last slab: through registers, zero beyond K
             unsigned char* st = lds + stage * STAGE_BYTES;
             const uint32_t k0 = full_slabs * BK;
 #pragma unroll
             for (int i = 0; i < A_LOADS; ++i) {
-                const uint32_t k = k0 + a_chunk[i] * 8;
+                const uint32_t k = k0 + a_chunk_of(i) * 8;
                 halfx8 v = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
                 if (k < g.K) {
                     v = *(const halfx8*)(a_base + a_voff[i]);             // inside the pitch: lda is a multiple of 8
@@ -204,7 +209,7 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
 #pragma unroll
             for (int i = 0; i < B_LOADS; ++i) {
                 halfx8 v = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
-                if (k0 + b_krow[i] < g.K) v = *(const halfx8*)(b_base + b_voff[i]);
+                if (k0 + b_krow_of(i) < g.K) v = *(const halfx8*)(b_base + b_voff[i]);
                 *(halfx8*)(st + A_STAGE_BYTES + (wave * B_LOADS + i) * 1024 + lane * 16) = v;
             }
         }
@@ -214,7 +219,7 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     // A fragment (tile i, k step ks): lane (kg, l16) takes row wm0 + 16 i + l16, k = 32 ks + 8 kg .. + 7: chunk 4 ks + kg.
     const int a_row = wm0 + l16;
     const int a_sw = (a_row / RPB) % CPR;                  // wm0 + 16 i leaves it unchanged (multiples of 16 rows)
-    const int a_off = a_row * RB;
+    int a_off = a_row * RB;
     // B fragment (tile j, k step ks, half r): the 16 lanes of group kg hand in the 4 k rows 32 ks + 8 kg + 4 r + (0..3),
     // lane s = l16 the row s / 4 and the 8-byte segment s % 4 of the 16 columns from wn0 + 16 j; lane l16 receives
     // column l16, 4 consecutive k.
@@ -281,16 +286,25 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
 #pragma unroll
     for (int j = 0; j < TN; ++j) fb[(KS - 1) & 1].b[j] = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
 
-    for (uint32_t s = 0; s < slabs; ++s) {
-        const unsigned char* st = lds + (s % STAGES) * STAGE_BYTES;
-        const bool more = s + STAGES - 1 < slabs;
+    // One slab.  STAGE >= 0: its stage is known at compile time and the slab that is asked for meanwhile is a whole one;
+    // a loop over STAGES such slabs is one block of code with neither a branch nor address arithmetic between its MFMAs
+    // (every LDS address a register that never changes plus an immediate).  STAGE < 0: the general form, for the last slabs.
+    auto slab_body = [&](uint32_t s, auto stage_c) {
+        constexpr int STAGE = decltype(stage_c)::value;
+        constexpr bool STEADY = STAGE >= 0;
+        const unsigned char* st;
+        if constexpr (STEADY) st = lds + STAGE * STAGE_BYTES; else st = lds + (s % STAGES) * STAGE_BYTES;
+        const bool more = STEADY || s + STAGES - 1 < slabs;
 
         read_unit(st, std::integral_constant<int, 0>{});
         multiply_unit(std::integral_constant<int, UNITS - 1>{});
         interleave<MFMAS, READS_FIRST>();
         __builtin_amdgcn_sched_barrier(0);
         // the stage that held slab s-1 is free: every wave passed the barrier after reading it
-        if (more) issue_loads(s + STAGES - 1);
+        if constexpr (STEADY) {
+            issue_direct((uint32_t)((STAGE + STAGES - 1) % STAGES));
+            __builtin_amdgcn_sched_barrier(0);
+        } else if (more) issue_loads(s + STAGES - 1);
 
         static_for<0, UNITS - 1>([&](auto uc) {
             constexpr int u = decltype(uc)::value;
@@ -301,7 +315,20 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
         });
 
         if (more) wait_loads_and_barrier<LOADS * (STAGES - 2)>(); else wait_loads_and_barrier<0>();
-    }
+    };
+    const uint32_t steady = __builtin_amdgcn_readfirstlane(full_slabs > (uint32_t)(STAGES - 1) ? (full_slabs - (uint32_t)(STAGES - 1)) / STAGES * STAGES : 0u);
+    uint32_t s = 0;
+    for (; s < steady; s += STAGES) static_for<0, STAGES>([&](auto jc) { slab_body(s + decltype(jc)::value, jc); });
+    // (the general form derives its LDS addresses from these afresh: computed in front of the loop above they would
+    // have to live across it, and it has no register to spare)
+    asm volatile("" : "+v"(a_off));
+#pragma unroll
+    for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(b_off[j]));
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) asm volatile("" : "+v"(a_voff[i]));
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) asm volatile("" : "+v"(b_voff[i]));
+    for (; s < slabs; ++s) slab_body(s, std::integral_constant<int, -1>{});
     multiply_unit(std::integral_constant<int, UNITS - 1>{});
 
     // Epilogue.  Lane (kg, l16) holds, of the 16 x 16 tile (i, j), row l16 and the 4 adjacent columns 4 kg .. 4 kg + 3.
