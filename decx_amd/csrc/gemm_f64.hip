@@ -224,9 +224,15 @@ gemm_f64_dma_kernel(const GemmArgs g_in)
     // the direct loads of a slab go out PER_STEP per k step, each group behind the first MFMA of its step
     constexpr int PER_STEP = (LOADS + STEPS - 2) / (STEPS - 1);
 
-    for (uint32_t s = 0; s < slabs; ++s) {
-        const unsigned char* st = lds + (s % STAGES) * STAGE_BYTES;
-        const bool more = s + STAGES - 1 < slabs;
+    // One slab.  STAGE >= 0: its stage is known at compile time and the slab that is asked for meanwhile is a whole one;
+    // a loop over STAGES such slabs is one block of code with neither a branch nor address arithmetic between its MFMAs.
+    // STAGE < 0: the general form, for the last slabs.
+    auto slab_body = [&](uint32_t s, auto stage_c) {
+        constexpr int STAGE = decltype(stage_c)::value;
+        constexpr bool STEADY = STAGE >= 0;
+        const unsigned char* st;
+        if constexpr (STEADY) st = lds + STAGE * STAGE_BYTES; else st = lds + (s % STAGES) * STAGE_BYTES;
+        const bool more = STEADY || s + STAGES - 1 < slabs;
 
         read_a(st, std::integral_constant<int, 0>{});
         static_for<0, BF_AHEAD>([&](auto stc) { read_b(st, stc); });
@@ -235,9 +241,9 @@ gemm_f64_dma_kernel(const GemmArgs g_in)
         __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
         __builtin_amdgcn_sched_barrier(0);
         // the stage that held slab s-1 is free: every wave passed the barrier after reading it
-        const uint32_t nstage = (s + STAGES - 1) % STAGES;
-        const bool direct = s + STAGES - 1 < full_slabs;
-        if (more && !direct) issue_tail(nstage);
+        const uint32_t nstage = STEADY ? (uint32_t)((STAGE + STAGES - 1) % STAGES) : (s + STAGES - 1) % STAGES;
+        const bool direct = STEADY || s + STAGES - 1 < full_slabs;
+        if constexpr (!STEADY) { if (more && !direct) issue_tail(nstage); }
 
         static_for<0, STEPS - 1>([&](auto stc) {
             constexpr int step = decltype(stc)::value;
@@ -265,7 +271,11 @@ gemm_f64_dma_kernel(const GemmArgs g_in)
         });
 
         if (more) wait_loads_and_barrier<LOADS * (STAGES - 2)>(); else wait_loads_and_barrier<0>();
-    }
+    };
+    const uint32_t steady = __builtin_amdgcn_readfirstlane(full_slabs > (uint32_t)(STAGES - 1) ? (full_slabs - (uint32_t)(STAGES - 1)) / STAGES * STAGES : 0u);
+    uint32_t s = 0;
+    for (; s < steady; s += STAGES) static_for<0, STAGES>([&](auto jc) { slab_body(s + decltype(jc)::value, jc); });
+    for (; s < slabs; ++s) slab_body(s, std::integral_constant<int, -1>{});
     multiply(std::integral_constant<int, STEPS - 1>{});
 
     if constexpr (SPLIT) {
