@@ -122,10 +122,10 @@ struct SplitModel {
     bool uneven_second_round;
 };
 // 64 x 64 tiles of 32 KB LDS: four fit a CU (160 KB would hold five, but time against the number of tiles steps as for four)
-static const SplitModel kSplitF32 = {{{TILE_SMALL, 4, 4, {0, 17.72, 15.51, 15.07, 14.77}, {0, 15.8, 14.4, 14.3, 14.16}}, {}}, 1, 32, 4, 1.0, 0.4, 0.15, 0.586e6, true};
-static const SplitModel kSplitF16 = {{{TILE_SMALL, 4, 4, {0, 4.33, 3.21, 3.18, 3.07}}, {TILE_MEDIUM, 2, 8, {0, 7.67, 6.95}}}, 2,
-                                     64, 4, 0.5, 2.0, 0.15, 5.2e6, false};
-static const SplitModel kSplitF64 = {{{TILE_SMALL, 2, 4, {0, 34.0, 30.3}}, {}}, 1, 32, 8, 0.5, 2.0, 0.30, 0.283e6, false};
+static const SplitModel kSplitF32 = {{{TILE_SMALL, 4, 4, {0, 17.72, 15.51, 15.07, 14.77}, {0, 15.8, 15.1, 15.0, 14.96}}, {}}, 1, 32, 4, 1.0, 0.4, 0.15, 0.600e6, true};
+static const SplitModel kSplitF16 = {{{TILE_SMALL, 4, 4, {0, 3.4, 3.3, 3.15, 3.1}}, {TILE_MEDIUM, 2, 8, {0, 7.4, 7.0}}}, 2,
+                                     64, 4, 0.5, 2.0, 0.15, 5.4e6, false};
+static const SplitModel kSplitF64 = {{{TILE_SMALL, 2, 4, {0, 28.2, 28.8}}, {}}, 1, 32, 8, 0.5, 2.0, 0.30, 0.300e6, false};
 
 TileInfo dma_tile_info(int elem_bytes, int shape, uint32_t N);
 
@@ -149,8 +149,8 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
         if (md.uneven_second_round && full == 1 && rem > cus / 2 && rem <= cus) m = 2;
         const double* rate = (whole + wgs <= slots && st.ns_per_k_one_round[1] > 0) ? st.ns_per_k_one_round : st.ns_per_k;
         double lone = rate[1];
-        if (elem_bytes == 2 && st.shape == TILE_MEDIUM)        // 6.0 ns with half the CUs busy, 7.67 with all
-            lone = wgs <= cus / 2 ? 6.0 : 6.0 + 1.67 * (double)(wgs - cus / 2) / (double)(cus - cus / 2);
+        if (elem_bytes == 2 && st.shape == TILE_MEDIUM)        // 5.4 ns with half the CUs busy, 7.4 with all
+            lone = wgs <= cus / 2 ? 5.4 : 5.4 + 2.0 * (double)(wgs - cus / 2) / (double)(cus - cus / 2);
         const uint32_t k_whole = (K + md.len_align - 1) / md.len_align * md.len_align;
         const double ns = (double)len * ((double)full * st.fit * rate[st.fit] + (m == 1 ? lone : (double)m * rate[m])) +
                           (double)k_whole * (double)(whole / slots) * st.fit * rate[st.fit];

@@ -139,22 +139,22 @@ __host__ inline double tile_cost(const TileInfo& ti, uint64_t tiles, uint32_t cu
     return t;
 }
 
-// fp32, measured on MI355X (TFLOP/s per CU, direct-to-LDS kernels): 256 x 128 (the largest tile; 256 x 256 in the
-// register-staged family) 0.56 alone, 0.586 two per CU; 128 x 128
-// 0.52 alone (2048^3), 0.586 four per CU (4096^3, 6144^3); 64 x 64 0.47 alone (long K; 0.39 at 1024^3 with the launch
-// in it), 0.56 four per CU (3072^3, 4096^3; 160 KB of LDS would hold five of them, but time against the number of
-// tiles steps as for four).  The predicated register-staged kernels (operands that are not 16-byte aligned) run at about
+// fp32, measured on MI355X (direct-to-LDS kernels; nanoseconds per k and workgroup with m workgroups on the CU, slopes
+// of time against K): 256 x 128 (the largest tile; 256 x 256 in the register-staged family) 108.9 alone, 109.6 two per
+// CU (the matrix pipe alone would take 106.7); 128 x 128 55.8 / 55.1 / 56.3 for one to three per CU (53.3), 58.4 in a
+// second round; 64 x 64 15.8 / 15.1 / 15.0 / 15.0 for one to four per CU (13.3), 15.5 per workgroup in launches of
+// several rounds.  The predicated register-staged kernels (operands that are not 16-byte aligned) run at about
 // 1 : 0.8 : 0.7 of the largest tile, two workgroups per CU.
 // N: columns of the output; at most kNarrowN of them turn the smallest aligned tile into 128 x 32 (the same area, no
 // idle half: 65536 x 32 x 1024 46.8 us against 81.9 us for 64 columns on 64 x 64 tiles).
 __host__ inline TileInfo tile_info_f32(int shape, bool aligned = true, uint32_t N = 0xffffffffu)
 {
     switch (shape) {
-    case TILE_LARGE: return aligned ? TileInfo{256, 128, 256, 2, 1.00f, 0.95f} : TileInfo{256, 256, 512, 1, 1.00f, 1.00f};
-    case TILE_MEDIUM: return {128, 128, 256, aligned ? 4 : 2, aligned ? 1.00f : 0.80f, aligned ? 0.88f : 0.72f};
+    case TILE_LARGE: return aligned ? TileInfo{256, 128, 256, 2, 1.00f, 1.00f} : TileInfo{256, 256, 512, 1, 1.00f, 1.00f};
+    case TILE_MEDIUM: return {128, 128, 256, aligned ? 3 : 2, aligned ? 0.97f : 0.80f, aligned ? 0.98f : 0.72f};
     default:
-        if (aligned && N <= kNarrowN) return {128, 32, 256, 4, 0.96f, 0.667f};
-        return { 64,  64, 256, aligned ? 4 : 2, aligned ? 0.96f : 0.70f, aligned ? 0.80f : 0.49f};
+        if (aligned && N <= kNarrowN) return {128, 32, 256, 4, 0.90f, 0.70f};
+        return { 64,  64, 256, aligned ? 4 : 2, aligned ? 0.90f : 0.70f, aligned ? 0.865f : 0.49f};
     }
 }
 // fp16 (TFLOP/s per CU): 256 x 256 4.64 on a full chip, 6.4 with at most half the CUs busy; 128 x 128 3.1 alone,
@@ -168,15 +168,16 @@ __host__ inline TileInfo tile_info_f16(int shape, bool aligned = true)
     }
 }
 
-// fp64 (TFLOP/s per CU): 256 x 128 (what TILE_LARGE stands for) 0.283 alone or full; 128 x 128 0.27 alone or two per
-// CU; 64 x 64 0.22 alone (1024^3), 0.27 two per CU (3072^3).  All three run 8 wavefronts per workgroup: with 4, the
-// two smaller tiles reach 0.24 (their accumulators leave no room for the four workgroups per CU that the fp32 tiles use).
+// fp64 (nanoseconds per k and workgroup): 256 x 128 (what TILE_LARGE stands for) 218.6 alone (the matrix pipe alone:
+// 213.4); 128 x 128 109.4 alone or two per CU; 64 x 64 28.2 alone, 28.8 two per CU.  All three run 8 wavefronts per
+// workgroup: with 4, the two smaller tiles are a tenth slower (their accumulators leave no room for the four workgroups
+// per CU that the fp32 tiles use).
 __host__ inline TileInfo tile_info_f64(int shape)
 {
     switch (shape) {
     case TILE_LARGE: return {256, 128, 512, 1, 1.00f, 1.00f};
-    case TILE_MEDIUM: return {128, 128, 512, 2, 0.96f, 0.96f};
-    default:           return { 64,  64, 512, 2, 0.95f, 0.77f};
+    case TILE_MEDIUM: return {128, 128, 512, 2, 1.00f, 1.00f};
+    default:           return { 64,  64, 512, 2, 0.95f, 0.97f};
     }
 }
 

@@ -72,7 +72,7 @@ def test_planner_choices():
     assert hip.plan(2, 1000, 1500, 777).edge == 0 and hip.plan(2, 1000, 1500, 777).tile_m == 64
     assert hip.plan(2, 2048, 2048, 2048).tile_m == 128 and hip.plan(2, 1000, 1500, 777, aligned=False).edge == 1
     assert hip.plan(4, 1024, 1024, 1024).tile_m == 64
-    assert hip.plan(4, 2048, 2048, 2048).tile_m == 64      # 1024 small tiles, four to a CU, beat 256 lone 128 x 128 ones
+    assert hip.plan(4, 2048, 2048, 2048).tile_m == 128     # 256 tiles of 128 x 128, one per CU: 121.5 us (1024 small ones, four per CU: 122.9)
     assert hip.plan(4, 6144, 6144, 6144).tile_m == 128
     assert hip.plan(4, 3000, 3000, 3000).tile_m == 64
     assert hip.plan(4, 1024, 1024, 1024, aligned=False).edge == 1
@@ -89,8 +89,8 @@ def test_planner_choices():
     assert p.k_splits > 1 and p.grid == 25 * p.k_splits and hip.plan(4, 8192, 8192, 8192).k_splits == 1
     assert hip.plan(4, 300, 300, 400).k_splits == 1 and hip.plan(2, 256, 256, 65536).k_splits > 1
     # a few hundred tiles that do not divide among 256 CUs and a long K: even rounds of workgroups on the small tile
-    p = hip.plan(4, 1280, 1024, 8192)                      # 320 tiles of 64 x 64 on 3 ranges: 960 workgroups, one round of
-    assert (p.tile_m, p.k_splits, p.grid) == (64, 3, 320 * 3)     # at most four per CU (163.7 us; 8 ranges, 2.5 rounds: 166.8, whole 251)
+    p = hip.plan(4, 1280, 1024, 8192)                      # 320 tiles of 64 x 64 on 8 ranges: ten per CU, four at a time
+    assert (p.tile_m, p.k_splits, p.grid) == (64, 8, 320 * 8)     # 164 us; 3 ranges (one round of 960 workgroups) the same, whole 239
     p = hip.plan(4, 1536, 1024, 8192)                      # 384 tiles on 2 ranges: three per CU
     assert (p.tile_m, p.k_splits) == (64, 2)
     assert hip.plan(4, 2048, 2048, 8192).k_splits == 1 and hip.plan(4, 1280, 1024, 2048).k_splits == 3    # 1.25 tiles per CU: 65.6 -> 47.1 us

@@ -332,10 +332,10 @@ def test_f16_split_k_through_a_workspace(hip, oracle, M, N, K):
 
 
 @pytest.mark.parametrize("dtype,M,N,K,tile,splits", [
-    (np.float32, 1280, 1024, 4096, 64, 3),          # 320 tiles of 64 x 64: 1.25 per CU; on 3 ranges 960 workgroups, one round of four per CU
+    (np.float32, 1280, 1024, 4096, 64, 8),          # 320 tiles of 64 x 64: 1.25 per CU, on 8 ranges ten per CU, four at a time
     (np.float32, 900, 700, 4100, 64, 3),            # ragged output, K not a multiple of the range
     (np.float16, 1280, 1024, 6144, 128, 3),         # 80 tiles of 128 x 128 on 3 ranges
-    (np.float16, 768, 768, 8200, 128, 6),
+    (np.float16, 768, 768, 8200, 128, 4),
 ])
 def test_split_k_for_a_few_hundred_tiles(hip, oracle, dtype, M, N, K, tile, splits):
     """Outputs of a few hundred small tiles and a long K: with a workspace the product runs on the tile shape that

@@ -62,9 +62,9 @@ def both(hip, M, N, K, seed, with_c, alpha=1.0, beta=1.0):
 
 
 def test_static_workspace_matches_the_allocated_one_call_after_call(hip, oracle):
-    # (M, N, K, C term): split K over 4, 20, 16 ranges, then the dense copy of a pitched x, then a product that needs
+    # (M, N, K, C term): split K over 5, 10, 16 ranges, then the dense copy of a pitched x, then a product that needs
     # no workspace at all.  Each smaller than the one before, so stale partial sums of the bigger call lie beyond.
-    cases = [(1024, 1024, 8192, True), (300, 300, 8192, False), (100, 120, 4096, True), (8192, 1, 8192, False),
+    cases = [(640, 640, 8192, True), (300, 300, 8192, False), (100, 120, 4096, True), (8192, 1, 8192, False),
              (200, 136, 120, True)]
     used_split = 0
     for i, (M, N, K, with_c) in enumerate(cases):
