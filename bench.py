@@ -37,48 +37,48 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
 # file of the kernel it was measured on with that file's SHA-256 at the time: when the kernel source has changed
 # since, the figure is withheld ("traffic": null, "traffic_stale": true) until the workload is profiled again.
 MEASURED_TRAFFIC = {
-    "fp32_8192": {"bytes": 6.12e9, "counters": "FETCH_SIZE 2.8588e6 x 2.0 KiB + WRITE_SIZE 2.621e5 KiB (FETCH_SIZE 2.66e6 ... 3.40e6 from run to run)",
+    "fp32_8192": {"bytes": 5.67e9, "counters": "FETCH_SIZE 2.6380e6 x 2.0 KiB + WRITE_SIZE 2.621e5 KiB (FETCH_SIZE 2.66e6 ... 3.40e6 from run to run)",
                   "kernel": "gemm_f32_dma_kernel<256, 128, 2, 2, 16, 2, false, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                  "source_sha256": "83b27cf25e8546a4509c45204c5c0b77da0d9f5d256a9dd23f0804976d93637d", "profile": "profiles/gemm_f32_dma_fp32_8192cubed.md"},
-    "fp16_4096": {"bytes": 2.35e8, "counters": "FETCH_SIZE 98 507 x 2.0 KiB + WRITE_SIZE 32 768 KiB",
+                  "source_sha256": "42b4675ace5ce46287a6879c4bcdc2d1fc1e5ffab56f8f94bb23aa2ccf21cb91", "profile": "profiles/gemm_f32_dma_fp32_8192cubed.md"},
+    "fp16_4096": {"bytes": 2.35e8, "counters": "FETCH_SIZE 98 520 x 2.0 KiB + WRITE_SIZE 32 768 KiB",
                   "kernel": "gemm_f16_dma_kernel<256, 256, 2, 4, 64, 2, false>", "source": "decx_amd/csrc/gemm_f16_dma.hip",
-                  "source_sha256": "33cd90d01dc3e3ec833842c257071145fec9f786e12b677fe6f1991bd7a922d4", "profile": "profiles/gemm_f16_dma_fp16_4096cubed.md"},
-    "fp64_4096": {"bytes": 1.21e9, "counters": "FETCH_SIZE 524 413 x 2.0 KiB + WRITE_SIZE 131 072 KiB",
+                  "source_sha256": "7672608b2dfaee6ab187426e6cf743154d6b9401f8b85203142c62e174a902fd", "profile": "profiles/gemm_f16_dma_fp16_4096cubed.md"},
+    "fp64_4096": {"bytes": 1.21e9, "counters": "FETCH_SIZE 524 441 x 2.0 KiB + WRITE_SIZE 131 072 KiB",
                   "kernel": "gemm_f64_dma_kernel<256, 128, 4, 2, 16, 3, false>", "source": "decx_amd/csrc/gemm_f64.hip",
-                  "source_sha256": "086a9772e456035cd79db946ccd67aa4490498f145e02d633b0e075b3cefb6c0", "profile": "profiles/gemm_f64_dma_fp64_4096cubed.md"},
-    "fp32_1024": {"bytes": 2.95e7, "counters": "FETCH_SIZE 12 345 x 2.0 KiB + WRITE_SIZE 4 096 KiB",
+                  "source_sha256": "8bfbb2f095545fa429bdc684d2eb76fc7ed7944b7f044310b2cc232485cf66a4", "profile": "profiles/gemm_f64_dma_fp64_4096cubed.md"},
+    "fp32_1024": {"bytes": 2.95e7, "counters": "FETCH_SIZE 12 352 x 2.0 KiB + WRITE_SIZE 4 096 KiB",
                   "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                  "source_sha256": "83b27cf25e8546a4509c45204c5c0b77da0d9f5d256a9dd23f0804976d93637d", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
-    "fp32_ragged": {"bytes": 5.65e7, "counters": "FETCH_SIZE 18 486 x 2.0 KiB + WRITE_SIZE 18 199 KiB (operands, and the slots of the 2 ranges of K)",
+                  "source_sha256": "42b4675ace5ce46287a6879c4bcdc2d1fc1e5ffab56f8f94bb23aa2ccf21cb91", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+    "fp32_ragged": {"bytes": 5.65e7, "counters": "FETCH_SIZE 18 503 x 2.0 KiB + WRITE_SIZE 18 199 KiB (operands, and the slots of the 2 ranges of K)",
                     "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                    "source_sha256": "83b27cf25e8546a4509c45204c5c0b77da0d9f5d256a9dd23f0804976d93637d", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
-    "fp32_ragged_abc": {"bytes": 6.25e7, "counters": "FETCH_SIZE 21 419 x 2.0 KiB + WRITE_SIZE 18 199 KiB",
+                    "source_sha256": "42b4675ace5ce46287a6879c4bcdc2d1fc1e5ffab56f8f94bb23aa2ccf21cb91", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+    "fp32_ragged_abc": {"bytes": 6.25e7, "counters": "FETCH_SIZE 21 423 x 2.0 KiB + WRITE_SIZE 18 199 KiB",
                         "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, true>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                        "source_sha256": "83b27cf25e8546a4509c45204c5c0b77da0d9f5d256a9dd23f0804976d93637d", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
-    "fp32_tall_skinny": {"bytes": 3.51e8, "counters": "FETCH_SIZE 138 688 x 2.0 KiB + WRITE_SIZE 65 536 KiB",
+                        "source_sha256": "42b4675ace5ce46287a6879c4bcdc2d1fc1e5ffab56f8f94bb23aa2ccf21cb91", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+    "fp32_tall_skinny": {"bytes": 3.58e8, "counters": "FETCH_SIZE 142 167 x 2.0 KiB + WRITE_SIZE 65 536 KiB",
                          "kernel": "gemm_f32_dma_kernel<256, 128, 2, 2, 16, 2, false, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                         "source_sha256": "83b27cf25e8546a4509c45204c5c0b77da0d9f5d256a9dd23f0804976d93637d", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
-    "fp32_mid_long_k": {"bytes": 3.76e8, "counters": "FETCH_SIZE 160 819 x 2.0 KiB + WRITE_SIZE 46 170 KiB (operands, and the slots of the 8 ranges of K)",
+                         "source_sha256": "42b4675ace5ce46287a6879c4bcdc2d1fc1e5ffab56f8f94bb23aa2ccf21cb91", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+    "fp32_mid_long_k": {"bytes": 3.76e8, "counters": "FETCH_SIZE 160 893 x 2.0 KiB + WRITE_SIZE 46 170 KiB (operands, and the slots of the 8 ranges of K)",
                         "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                        "source_sha256": "83b27cf25e8546a4509c45204c5c0b77da0d9f5d256a9dd23f0804976d93637d", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
+                        "source_sha256": "42b4675ace5ce46287a6879c4bcdc2d1fc1e5ffab56f8f94bb23aa2ccf21cb91", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
     "fp32_gemv": {"bytes": 2.70e8, "counters": "FETCH_SIZE (131 258 + 522) x 2.0 KiB + WRITE_SIZE (256 + 32) KiB: matrix-vector kernel + the copy of x",
                   "kernel": "gemv_kernel<float, float, 2, 1>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "ab015914fc6f336627eb2a698f9c11314809ae166f47d2169c418a465860f12a", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "4b643fb2db289936e88028f8ddcf8b14ab9fce401e801b59cb3779d7d23aed21", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp32_gevm": {"bytes": 2.69e8, "counters": "FETCH_SIZE 131 233 x 2.0 KiB + WRITE_SIZE 32 KiB",
                   "kernel": "gevm_kernel<float, float, 8>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "ab015914fc6f336627eb2a698f9c11314809ae166f47d2169c418a465860f12a", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "4b643fb2db289936e88028f8ddcf8b14ab9fce401e801b59cb3779d7d23aed21", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp16_gemv": {"bytes": 1.36e8, "counters": "FETCH_SIZE (65 647 + 522) x 2.0 KiB + WRITE_SIZE (256 + 16) KiB: matrix-vector kernel + the copy of x",
                   "kernel": "gemv_kernel<_Float16, _Float16, 2, 1>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "ab015914fc6f336627eb2a698f9c11314809ae166f47d2169c418a465860f12a", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "4b643fb2db289936e88028f8ddcf8b14ab9fce401e801b59cb3779d7d23aed21", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp16_gevm": {"bytes": 1.35e8, "counters": "FETCH_SIZE 65 685 x 2.0 KiB + WRITE_SIZE 92 KiB",
                   "kernel": "gevm_kernel<_Float16, _Float16, 8>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "ab015914fc6f336627eb2a698f9c11314809ae166f47d2169c418a465860f12a", "profile": "profiles/gemv_gevm_8192x8192.md"},
-    "conv2d": {"bytes": 1.08e8, "counters": "FETCH_SIZE 20 532 x 2.0 KiB + WRITE_SIZE 64 516 KiB",
+                  "source_sha256": "4b643fb2db289936e88028f8ddcf8b14ab9fce401e801b59cb3779d7d23aed21", "profile": "profiles/gemv_gevm_8192x8192.md"},
+    "conv2d": {"bytes": 1.08e8, "counters": "FETCH_SIZE 20 545 x 2.0 KiB + WRITE_SIZE 64 516 KiB",
                "kernel": "gemm_f32_dma_kernel<256, 256, 2, 4, 16, 4, false, 2, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-               "source_sha256": "83b27cf25e8546a4509c45204c5c0b77da0d9f5d256a9dd23f0804976d93637d", "profile": "profiles/conv2d_implicit_gemm_256x256x112_3x3x256.md"},
+               "source_sha256": "42b4675ace5ce46287a6879c4bcdc2d1fc1e5ffab56f8f94bb23aa2ccf21cb91", "profile": "profiles/conv2d_implicit_gemm_256x256x112_3x3x256.md"},
     "conv2d_rgb": {"bytes": 1.00e8, "counters": "FETCH_SIZE 16 455 x 2.0 KiB + WRITE_SIZE 64 613 KiB",
                    "kernel": "conv2d_direct_kernel<8, 3>", "source": "decx_amd/csrc/conv_direct.hip",
-                   "source_sha256": "89c37a455455a6410aa63de5c09e83c9e3f55f3e1a3cf3b9c9be3aa7e3842a7c", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
+                   "source_sha256": "91b8dd40c7d5ace863daedc2876c5cd9e2a7843c09a30451c9ac3dadcd1c8250", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
 }
 
 
