@@ -109,7 +109,7 @@ int check_gemm(const void* A, const void* B, const void* C, const void* D, uint3
 // fp32 fitted to 20 output shapes x K = 777 ... 16384 x 1 ... 8 ranges, fp16 and fp64 to 12 and 9 shapes x 2 ... 32
 // ranges: the estimate is within 4 % of the measurement on most, the pick within 1 % (fp16: 2.5 %) of the best on
 // average.  The whole product is kept unless the split promises 4 %.
-struct SplitChoice { int shape; uint32_t splits, len, first; };     // first: tiles in front that stay whole
+struct SplitChoice { int shape; uint32_t splits, len, first, urgent; };     // first: tiles in front that stay whole; urgent: GemmArgs::split_urgent
 struct SplitTile {
     int shape, fit, pieces;          // size class, workgroups per CU, 16-byte pieces of accumulators per lane
     double ns_per_k[5];              // per workgroup with m = 1 .. fit of them on the CU
@@ -120,12 +120,18 @@ struct SplitModel {
     uint32_t len_align, acc_bytes;   // ranges are multiples of the deepest slab; bytes of an accumulator
     double us_fixed, us_per_trip, us_per_mb, whole_flop_per_us;      // the last: the largest tile, per CU of a full chip
     bool uneven_second_round;
+    // Whole tiles that share their CUs with split ones (tiles[0] only; 0: not planned): microseconds of a launch beside
+    // its k steps, nanoseconds per k step of a CU, and the longest K at which the split workgroups run at a raised priority
+    double shared_us_fixed, shared_ns_per_k;
+    uint32_t urgent_max_k;
 };
 // 64 x 64 tiles of 32 KB LDS: four fit a CU (160 KB would hold five, but time against the number of tiles steps as for four)
-static const SplitModel kSplitF32 = {{{TILE_SMALL, 4, 4, {0, 17.72, 15.51, 15.07, 14.77}, {0, 15.8, 15.1, 15.0, 14.96}}, {}}, 1, 32, 4, 1.0, 0.4, 0.15, 0.600e6, true};
+static const SplitModel kSplitF32 = {{{TILE_SMALL, 4, 4, {0, 17.72, 15.51, 15.07, 14.77}, {0, 15.8, 15.1, 15.0, 14.96}}, {}}, 1, 32, 4, 1.0, 0.4, 0.15, 0.600e6, true,
+                                     6.2, 14.0, 2048};
 static const SplitModel kSplitF16 = {{{TILE_SMALL, 4, 4, {0, 3.4, 3.3, 3.15, 3.1}}, {TILE_MEDIUM, 2, 8, {0, 7.4, 7.0}}}, 2,
-                                     64, 4, 0.5, 2.0, 0.15, 5.4e6, false};
-static const SplitModel kSplitF64 = {{{TILE_SMALL, 2, 4, {0, 28.2, 28.8}}, {}}, 1, 32, 8, 0.5, 2.0, 0.30, 0.300e6, false};
+                                     64, 4, 0.5, 2.0, 0.15, 5.4e6, false, 0, 0, 0};
+static const SplitModel kSplitF64 = {{{TILE_SMALL, 2, 4, {0, 28.2, 28.8}}, {}}, 1, 32, 8, 0.5, 2.0, 0.30, 0.300e6, false,
+                                     5.7, 27.8, 1u << 30};
 
 TileInfo dma_tile_info(int elem_bytes, int shape, uint32_t N);
 
@@ -191,6 +197,30 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
                 if (us < best_us) { best_us = us; best = {st.shape, ranges, len, (uint32_t)whole}; }
             }
         }
+        // Or the CUs hold j whole tiles each (the first j x CUs workgroups of the grid: the hardware deals them out evenly)
+        // and the other tiles on so many ranges that every workgroup of the launch is resident from the start, m split ones
+        // on the busiest CU.  A CU then multiplies j K + m len steps, and does so at a better rate than in any launch of
+        // equal workgroups: the whole ones, which are older, take the matrix pipe whenever they are ready and the split
+        // ones the slots they leave (fp32, 1 + 1: 1280 x 1024 x 8192 163 -> 150 us, 1536^3 62.0 -> 55.1 with 2 + 1,
+        // 1000 x 1500 x 777 25.5 -> 23.4; fp64 1000 x 1500 x 777 48.2 -> 39.4, 1280 x 1024 x 2048 87.1 -> 77.3).  Where K is
+        // short the split ones run at a raised wave priority instead, finish first, and meet in the workspace behind the
+        // whole ones' last steps; where K is long that costs more than it hides, because the whole ones are then alone
+        // on their CU for most of the launch (fp32 K = 777: 24.2 -> 23.4 us, K = 1536 the same, K = 3072 71.1 -> 73.5).
+        if (i == 0 && md.shared_ns_per_k > 0) {
+            const uint32_t k_whole = (K + md.len_align - 1) / md.len_align * md.len_align;
+            for (uint64_t j = 1; j < (uint64_t)st.fit && j * cus < t; ++j) {
+                const uint64_t rest = t - j * cus, room = ((uint64_t)st.fit - j) * cus;
+                for (uint32_t p = 2; p <= max_p && rest * p <= room; ++p) {
+                    const uint32_t len = ((K + p - 1) / p + md.len_align - 1) / md.len_align * md.len_align, ranges = (K + len - 1) / len;
+                    if (ranges < 2 || ranges > kSplitFlat || rest * ranges > room) continue;
+                    const uint64_t m = (rest * ranges + cus - 1) / cus;
+                    const uint32_t group = st.pieces < 16 ? st.pieces : 16, batch = 16 / group, per_slot = st.pieces / group;
+                    const double us = md.shared_us_fixed + md.us_per_trip * ((ranges + batch - 1) / batch * per_slot) +
+                                      md.shared_ns_per_k * 1e-3 * ((double)j * k_whole + (double)m * len);
+                    if (us < best_us) { best_us = us; best = {st.shape, ranges, len, (uint32_t)(j * cus), K <= md.urgent_max_k ? 1u : 0u}; }
+                }
+            }
+        }
     }
     return best;
 }
@@ -234,6 +264,7 @@ uint32_t arm_split(GemmArgs& g, int elem_bytes, void* workspace, size_t workspac
     if (!counters) return 1;
     g.split_counters = counters;
     g.split_len = sp.len; g.split_count = sp.splits; g.split_first = sp.first; g.split_ws = workspace;
+    g.split_urgent = sp.urgent;
     shape = sp.shape;
     return sp.splits;
 }

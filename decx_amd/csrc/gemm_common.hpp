@@ -38,8 +38,11 @@ struct GemmArgs {
     uint32_t group_m;            // tile-rows per L2 patch of the block -> tile map (0: the default, kGroupM)
     uint32_t split_len;          // 0: no split
     uint32_t split_count;        // splits per split tile
-    uint32_t split_first;        // tiles below this index are multiplied whole, by one workgroup each (the full rounds of
-                                 // workgroups); only the tiles of the ragged last round are split
+    uint32_t split_first;        // tiles below this index are multiplied whole, by one workgroup each (full rounds of
+                                 // workgroups, or one to three per CU that share their CU with the split ones)
+    uint32_t split_urgent;       // 1: the workgroups of split tiles raise their wave priority (set where whole tiles
+                                 // share the CUs with them and K is short: the split ones then finish first and meet
+                                 // in the workspace while the whole ones still multiply)
     void*    split_ws;
     uint32_t* split_counters;    // one per tile, zero before and after every launch
     // Convolution as an implicit GEMM (used by the CONV instantiations only): row p of the A operand is the

@@ -56,6 +56,7 @@ gemm_f64_dma_kernel(const GemmArgs g_in)
             g_split.A = (const unsigned char*)g_in.A + (size_t)k0 * 8;
             g_split.B = (const unsigned char*)g_in.B + (size_t)k0 * g_in.ldb * 8;
             g_split.K = g_in.K - k0 < g_in.split_len ? g_in.K - k0 : g_in.split_len;
+            if (g_in.split_urgent) __builtin_amdgcn_s_setprio(3);
         }
     } else {
         block_to_tile(g_in, tile_m, tile_n);

@@ -65,8 +65,9 @@ def test_planner_choices():
     # small and ragged problems take smaller tiles so the chip fills; they stay on the direct-to-LDS
     # kernels as long as the operands are 16-byte aligned
     p = hip.plan(4, 1000, 1500, 777)
-    # 384 tiles of 64 x 64 are 1.5 per CU: with a workspace K is cut in two and every CU gets three workgroups
-    assert p.edge == 0 and p.tile_m < 256 and p.k_splits == 2 and p.grid == 2 * -(-1000 // p.tile_m) * -(-1500 // p.tile_n)
+    # 384 tiles of 64 x 64 are 1.5 per CU: with a workspace every CU gets one tile whole and one half of another
+    # (256 whole + 128 on two ranges of K: 23.5 us; all 384 on two ranges 25.6, the whole product 28.2)
+    assert p.edge == 0 and p.tile_m == 64 and (p.k_splits, p.whole_tiles, p.grid) == (2, 256, 256 + 2 * 128)
     assert hip.plan(4, 1024, 1024, 1024).k_splits == 1 and hip.plan(4, 2048, 2048, 2048).k_splits == 1
     assert hip.plan(4, 1000, 1500, 777, aligned=False).edge == 1
     assert hip.plan(2, 1000, 1500, 777).edge == 0 and hip.plan(2, 1000, 1500, 777).tile_m == 64
@@ -89,11 +90,16 @@ def test_planner_choices():
     assert p.k_splits > 1 and p.grid == 25 * p.k_splits and hip.plan(4, 8192, 8192, 8192).k_splits == 1
     assert hip.plan(4, 300, 300, 400).k_splits == 1 and hip.plan(2, 256, 256, 65536).k_splits > 1
     # a few hundred tiles that do not divide among 256 CUs and a long K: even rounds of workgroups on the small tile
-    p = hip.plan(4, 1280, 1024, 8192)                      # 320 tiles of 64 x 64 on 8 ranges: ten per CU, four at a time
-    assert (p.tile_m, p.k_splits, p.grid) == (64, 8, 320 * 8)     # 164 us; 3 ranges (one round of 960 workgroups) the same, whole 239
+    p = hip.plan(4, 1280, 1024, 8192)                      # 320 tiles of 64 x 64: a whole one per CU and 64 on 4 ranges, one of those per CU
+    assert (p.tile_m, p.k_splits, p.whole_tiles, p.grid) == (64, 4, 256, 256 + 64 * 4)     # 150 us; all on 8 ranges 163, whole 239
     p = hip.plan(4, 1536, 1024, 8192)                      # 384 tiles on 2 ranges: three per CU
     assert (p.tile_m, p.k_splits) == (64, 2)
-    assert hip.plan(4, 2048, 2048, 8192).k_splits == 1 and hip.plan(4, 1280, 1024, 2048).k_splits == 3    # 1.25 tiles per CU: 65.6 -> 47.1 us
+    assert hip.plan(4, 2048, 2048, 8192).k_splits == 1
+    p = hip.plan(4, 1280, 1024, 2048)                      # 1.25 tiles per CU: whole 65.6 us, all on 3 ranges 47.1, 256 whole + 64 on 4 ranges 44.4
+    assert (p.k_splits, p.whole_tiles) == (4, 256)
+    p = hip.plan(4, 1536, 1536, 1536)                      # 2.25 per CU: two whole and a quarter (62.0 -> 55.1 us)
+    assert (p.k_splits, p.whole_tiles, p.grid) == (4, 512, 512 + 64 * 4)
+    assert hip.plan(4, 1536, 1280, 1024).k_splits == 1     # 480 tiles: the 224 beyond one per CU do not fit beside them on two ranges
     p = hip.plan(2, 1536, 1024, 8192)                      # fp16: 96 tiles of 128 x 128 on 2 ranges
     assert (p.tile_m, p.k_splits) == (128, 2)
     p = hip.plan(2, 1024, 1024, 6144)                      # 64 tiles of 128 x 128 on 4 ranges, one per CU: 29.6 -> 23.5 us
@@ -106,9 +112,11 @@ def test_planner_choices():
     assert (p.tile_m, p.k_splits, p.whole_tiles, p.grid) == (64, 7, 1024, 1024 + 65 * 7)
     p = hip.plan(8, 1536, 1536, 1536)                      # fp64, two workgroups per CU: 512 whole + 64 x 4 (146 -> 112 us)
     assert (p.tile_m, p.k_splits, p.whole_tiles, p.grid) == (64, 4, 512, 512 + 64 * 4)
-    assert hip.plan(4, 2048, 2048, 2048).whole_tiles == 0 and hip.plan(4, 1000, 1500, 777).whole_tiles == 0
-    p = hip.plan(8, 1280, 1024, 2048)                      # fp64: 320 tiles of 64 x 64 on 4 ranges, 128.5 -> 91.3 us
-    assert (p.tile_m, p.k_splits) == (64, 4)
+    assert hip.plan(4, 2048, 2048, 2048).whole_tiles == 0 and hip.plan(4, 640, 640, 8192).whole_tiles == 0
+    p = hip.plan(8, 1280, 1024, 2048)                      # fp64: 320 tiles of 64 x 64, 256 whole + 64 on 4 ranges (whole 128.5 us, all on 4 ranges 87.1, this 77.3)
+    assert (p.tile_m, p.k_splits, p.whole_tiles) == (64, 4, 256)
+    p = hip.plan(8, 1000, 1500, 777)                       # 48.2 -> 39.4 us
+    assert (p.tile_m, p.k_splits, p.whole_tiles) == (64, 2, 256)
     p = hip.plan(8, 1280, 1024, 8192)
     assert p.tile_m == 64 and p.k_splits > 1 and hip.plan(8, 4096, 4096, 4096).k_splits == 1
     # the vector corners: rows per workgroup of the row-dot kernel, ranges of K for few columns, fp64 on the same kernels

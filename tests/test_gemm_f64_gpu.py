@@ -110,14 +110,14 @@ def test_split_k_through_a_workspace(hip, oracle, M, N, K):
 
 
 def test_split_k_for_a_few_hundred_tiles(hip, oracle):
-    """320 tiles of 64 x 64 (1.25 per CU) and a long K: with a workspace the planner cuts K so that whole rounds of
-    workgroups result.  Parity on sampled rows, the same result from run to run, untouched padding."""
+    """320 tiles of 64 x 64 (1.25 per CU) and a long K: with a workspace a tile per CU stays whole and the other 64 are
+    cut along K, one range per CU.  Parity on sampled rows, the same result from run to run, untouched padding."""
     M, N, K = 1280, 1024, 4100
     A = synth.uniform_f64(M, K, 961); B = synth.uniform_f64(K, N, 962)
     plan = hip.plan(8, M, N, K)
     assert plan.k_splits > 1 and plan.tile_m == 64
     need = hip.lib().decx_hip_gemm_workspace(8, M, N, K)
-    assert need >= plan.k_splits * M * N * 8
+    assert need == (20 * 16 - plan.whole_tiles) * plan.k_splits * 64 * 64 * 8        # a slot per workgroup of a split tile
     ws = hip.DeviceMatrix(1, need // 8, np.float64)
     ws.upload_raw(np.full((1, ws.pitch), np.nan, np.float64))
     r16 = lambda v: (v + 15) // 16 * 16

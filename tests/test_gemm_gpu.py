@@ -331,13 +331,16 @@ def test_f16_split_k_through_a_workspace(hip, oracle, M, N, K):
     ws.free()
 
 
-@pytest.mark.parametrize("dtype,M,N,K,tile,splits", [
-    (np.float32, 1280, 1024, 4096, 64, 8),          # 320 tiles of 64 x 64: 1.25 per CU, on 8 ranges ten per CU, four at a time
-    (np.float32, 900, 700, 4100, 64, 3),            # ragged output, K not a multiple of the range
-    (np.float16, 1280, 1024, 6144, 128, 3),         # 80 tiles of 128 x 128 on 3 ranges
-    (np.float16, 768, 768, 8200, 128, 4),
+@pytest.mark.parametrize("dtype,M,N,K,tile,splits,whole", [
+    (np.float32, 1280, 1024, 4096, 64, 4, 256),     # 320 tiles of 64 x 64, 1.25 per CU: a whole one per CU, the other 64 on 4 ranges
+    (np.float32, 1536, 1536, 1536, 64, 4, 512),     # 2.25 per CU: two whole per CU and a quarter of another
+    (np.float32, 1664, 2048, 2048, 64, 4, 768),     # 3.25 per CU
+    (np.float32, 1100, 1100, 1100, 64, 3, 256),     # ragged output, K not a multiple of the range, 68 split tiles on 204 workgroups
+    (np.float32, 900, 700, 4100, 64, 3, 0),         # fewer tiles than CUs: all of them on 3 ranges
+    (np.float16, 1280, 1024, 6144, 128, 3, 0),      # 80 tiles of 128 x 128 on 3 ranges
+    (np.float16, 768, 768, 8200, 128, 4, 0),
 ])
-def test_split_k_for_a_few_hundred_tiles(hip, oracle, dtype, M, N, K, tile, splits):
+def test_split_k_for_a_few_hundred_tiles(hip, oracle, dtype, M, N, K, tile, splits, whole):
     """Outputs of a few hundred small tiles and a long K: with a workspace the product runs on the tile shape that
     splits best, on the planned number of ranges.  Parity on sampled rows, a column checksum over the whole output
     against the product without a workspace, identical results from run to run, untouched padding."""
@@ -346,9 +349,9 @@ def test_split_k_for_a_few_hundred_tiles(hip, oracle, dtype, M, N, K, tile, spli
     B = synth.normal_half(K, N, 192) if f16 else synth.uniform_f32(K, N, 192)
     esz = dtype().itemsize
     plan = hip.plan(esz, M, N, K)
-    assert (plan.tile_m, plan.tile_n, plan.k_splits) == (tile, tile, splits)
+    assert (plan.tile_m, plan.tile_n, plan.k_splits, plan.whole_tiles) == (tile, tile, splits, whole)
     need = hip.lib().decx_hip_gemm_workspace(esz, M, N, K)
-    assert need >= splits * M * N * 4
+    assert need == (-(-M // tile) * -(-N // tile) - whole) * splits * tile * tile * 4      # a slot per workgroup of a split tile
     ws = hip.DeviceMatrix(1, need // 4, np.float32)
     ws.upload_raw(np.full((1, ws.pitch), np.nan, np.float32))
     pa, pn = device_pitch(K, dtype), device_pitch(N, dtype)
@@ -373,6 +376,56 @@ def test_split_k_for_a_few_hundred_tiles(hip, oracle, dtype, M, N, K, tile, spli
     col_a = split.astype(np.float64).sum(axis=0); col_b = whole.astype(np.float64).sum(axis=0)
     assert np.max(np.abs(col_a - col_b)) <= (2e-2 if f16 else 1e-4) * np.max(np.abs(col_b))
     for d in (dA, dB, ws):
+        d.free()
+
+
+@pytest.mark.parametrize("dtype,M,N,K,whole", [(np.float32, 1000, 1500, 777, 256), (np.float32, 1536, 1400, 1000, 512), (np.float64, 1000, 1500, 777, 256),
+                                              (np.float64, 1100, 1030, 2100, 256)])
+def test_whole_tiles_that_share_their_cus_with_split_ones(hip, oracle, dtype, M, N, K, whole):
+    """A few more tiles than a whole number per CU: the first ones of the grid stay whole and the others are cut along K
+    so that all workgroups are resident together (the split ones at a raised wave priority where K is short).  Every
+    form of the epilogue on both kinds of tile: A.B, alpha A.B + beta C and C aliased to D; all rows against the
+    oracle, identical from run to run, padding untouched."""
+    f64 = dtype == np.float64
+    esz = 8 if f64 else 4
+    plan = hip.plan(esz, M, N, K)
+    assert plan.whole_tiles == whole and plan.k_splits > 1 and plan.grid == whole + (plan.grid - whole) // plan.k_splits * plan.k_splits
+    rng = np.random.default_rng(77)
+    A = rng.uniform(-1, 1, (M, K)).astype(dtype); B = rng.uniform(-1, 1, (K, N)).astype(dtype); C = rng.uniform(-1, 1, (M, N)).astype(dtype)
+    need = hip.lib().decx_hip_gemm_workspace(esz, M, N, K)
+    ws = hip.DeviceMatrix(1, need // 4, np.float32)
+    ws.upload_raw(np.full((1, ws.pitch), np.nan, np.float32))
+    pa, pn = device_pitch(K, dtype), device_pitch(N, dtype)
+    dA = hip.DeviceMatrix(M, K, dtype, pa, A, pad_value=np.nan); dB = hip.DeviceMatrix(K, N, dtype, pn, B, pad_value=np.nan)
+    dC = hip.DeviceMatrix(M, N, dtype, pn, C, pad_value=np.nan)
+    rows = sample_rows(M, 96, 5)
+    ref_ab = (oracle.gemm_f64 if f64 else oracle.gemm_f32)(A, B, rows=rows).astype(np.float64)
+    tol = 1e-14 if f64 else TOL_F32
+
+    def product(c, alpha, beta, alias=False):
+        dD = hip.DeviceMatrix(M, N, dtype, pn)
+        raw0 = np.full((M, pn), -12345.0, dtype)
+        if alias:
+            raw0[:, :N] = C
+        dD.upload_raw(raw0)
+        hip.gemm(dA, dB, dD, C=dD if alias else c, alpha=alpha, beta=beta, workspace=ws)
+        hip.sync()
+        raw = dD.download_raw()
+        dD.free()
+        assert np.all(raw[:, N:] == dtype(-12345.0))
+        return raw[:, :N].copy()
+
+    ab = product(None, 1.0, 1.0)
+    assert rel_err(ab[rows], ref_ab, K) <= tol
+    assert np.array_equal(ab.view(np.uint8), product(None, 1.0, 1.0).view(np.uint8))
+    want = 0.5 * ref_ab - 2.0 * C[rows].astype(np.float64)
+    for alias in (False, True):
+        got = product(dC, 0.5, -2.0, alias)
+        assert np.max(np.abs(got[rows].astype(np.float64) - want)) <= tol * np.sqrt(K) * np.max(np.abs(want)), alias
+        # beyond the sampled rows: every element is alpha x (the product above) + beta x C, rounded once more at most
+        full = 0.5 * ab.astype(np.float64) - 2.0 * C.astype(np.float64)
+        assert np.max(np.abs(got.astype(np.float64) - full)) <= (1e-14 if f64 else 4e-6) * np.max(np.abs(full))
+    for d in (dA, dB, dC, ws):
         d.free()
 
 

@@ -83,7 +83,7 @@ def test_static_workspace_matches_the_allocated_one_call_after_call(hip, oracle)
 
 def test_static_workspace_rejects_what_does_not_fit(hip):
     L = hip.lib()
-    M, N, K = 1536, 1536, 1536                                  # 576 tiles on 3 ranges: 27 MiB of partial products
+    M, N, K = 480, 864, 4096                                    # 112 tiles on 16 ranges: 28 MiB of partial products
     need = L.decx_hip_gemm_f32_workspace(M, N, K)
     assert need > STATIC_BYTES, "pick another shape: this one fits the static workspace now"
     dA = hip.DeviceMatrix(M, K, np.float32, K, synth.uniform_f32(M, K, 1))
