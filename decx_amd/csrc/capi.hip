@@ -120,18 +120,21 @@ struct SplitModel {
     uint32_t len_align, acc_bytes;   // ranges are multiples of the deepest slab; bytes of an accumulator
     double us_fixed, us_per_trip, us_per_mb, whole_flop_per_us;      // the last: the largest tile, per CU of a full chip
     bool uneven_second_round;
-    // Whole tiles that share their CUs with split ones (tiles[0] only; 0: not planned): microseconds of a launch beside
-    // its k steps, nanoseconds per k step of a CU, and the longest K at which the split workgroups run at a raised priority
-    double shared_us_fixed, shared_ns_per_k;
+    // Whole tiles that share their CUs with split ones (on tiles[shared_tile]; rate 0: not planned): microseconds of a
+    // launch beside its k steps, nanoseconds per k step of a CU (plus shared_ns_busy x the share of the CUs that hold
+    // a split workgroup: fp16 runs into the power cap), and the longest K at which the split workgroups run at a
+    // raised priority
+    int shared_tile;
+    double shared_us_fixed, shared_ns_per_k, shared_ns_busy;
     uint32_t urgent_max_k;
 };
 // 64 x 64 tiles of 32 KB LDS: four fit a CU (160 KB would hold five, but time against the number of tiles steps as for four)
 static const SplitModel kSplitF32 = {{{TILE_SMALL, 4, 4, {0, 17.72, 15.51, 15.07, 14.77}, {0, 15.8, 15.1, 15.0, 14.96}}, {}}, 1, 32, 4, 1.0, 0.4, 0.15, 0.600e6, true,
-                                     6.2, 14.0, 2048};
+                                     0, 6.2, 14.0, 0, 2048};
 static const SplitModel kSplitF16 = {{{TILE_SMALL, 4, 4, {0, 3.4, 3.3, 3.15, 3.1}}, {TILE_MEDIUM, 2, 8, {0, 7.4, 7.0}}}, 2,
-                                     64, 4, 0.5, 2.0, 0.15, 5.4e6, false, 0, 0, 0};
+                                     64, 4, 0.5, 2.0, 0.15, 5.4e6, false, 1, 4.3, 6.5, 1.6, 0};
 static const SplitModel kSplitF64 = {{{TILE_SMALL, 2, 4, {0, 28.2, 28.8}}, {}}, 1, 32, 8, 0.5, 2.0, 0.30, 0.300e6, false,
-                                     5.7, 27.8, 1u << 30};
+                                     0, 5.7, 27.8, 0, 1u << 30};
 
 TileInfo dma_tile_info(int elem_bytes, int shape, uint32_t N);
 
@@ -158,7 +161,10 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
         if (elem_bytes == 2 && st.shape == TILE_MEDIUM)        // 5.4 ns with half the CUs busy, 7.4 with all
             lone = wgs <= cus / 2 ? 5.4 : 5.4 + 2.0 * (double)(wgs - cus / 2) / (double)(cus - cus / 2);
         const uint32_t k_whole = (K + md.len_align - 1) / md.len_align * md.len_align;
-        const double ns = (double)len * ((double)full * st.fit * rate[st.fit] + (m == 1 ? lone : (double)m * rate[m])) +
+        double last = m == 1 ? lone : (double)m * rate[m];          // the remainder's round, per k step
+        if (elem_bytes == 2 && st.shape == TILE_MEDIUM && full == 0 && m == 2)      // two on some CUs, one on the others: 5.8 ns with a
+            last = 2.0 * (5.6 + 1.4 * (double)(rem - cus) / (double)cus);           // quarter of the CUs doubly loaded, 6.0 with half, 7.0 with all
+        const double ns = (double)len * ((double)full * st.fit * rate[st.fit] + last) +
                           (double)k_whole * (double)(whole / slots) * st.fit * rate[st.fit];
         double us = ns * 1e-3 + kLaunch;
         if (ranges > 1) {
@@ -206,17 +212,20 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
         // short the split ones run at a raised wave priority instead, finish first, and meet in the workspace behind the
         // whole ones' last steps; where K is long that costs more than it hides, because the whole ones are then alone
         // on their CU for most of the launch (fp32 K = 777: 24.2 -> 23.4 us, K = 1536 the same, K = 3072 71.1 -> 73.5).
-        if (i == 0 && md.shared_ns_per_k > 0) {
+        // fp16 on 128 x 128 tiles, one whole and at most one split workgroup per CU: 2304 x 2304 x 4096 59.4 -> 50.3 us,
+        // 2560 x 2048 x 4096 58.4 -> 50.6, 3072 x 2048 x 8192 116.3 -> 104.2; the more CUs hold two, the slower each step.
+        if (i == md.shared_tile && md.shared_ns_per_k > 0) {
             const uint32_t k_whole = (K + md.len_align - 1) / md.len_align * md.len_align;
             for (uint64_t j = 1; j < (uint64_t)st.fit && j * cus < t; ++j) {
                 const uint64_t rest = t - j * cus, room = ((uint64_t)st.fit - j) * cus;
-                for (uint32_t p = 2; p <= max_p && rest * p <= room; ++p) {
+                for (uint32_t p = 2; p <= max_p && rest * p <= room && (elem_bytes != 2 || (K >= 4096 && K < 8192)); ++p) {     // (fp16: no gain measured below 4096, nor from 8192 on, where all tiles on 3 ranges do as well)
                     const uint32_t len = ((K + p - 1) / p + md.len_align - 1) / md.len_align * md.len_align, ranges = (K + len - 1) / len;
                     if (ranges < 2 || ranges > kSplitFlat || rest * ranges > room) continue;
                     const uint64_t m = (rest * ranges + cus - 1) / cus;
                     const uint32_t group = st.pieces < 16 ? st.pieces : 16, batch = 16 / group, per_slot = st.pieces / group;
                     const double us = md.shared_us_fixed + md.us_per_trip * ((ranges + batch - 1) / batch * per_slot) +
-                                      md.shared_ns_per_k * 1e-3 * ((double)j * k_whole + (double)m * len);
+                                      (md.shared_ns_per_k + md.shared_ns_busy * (double)(rest * ranges) / (double)room) * 1e-3 *
+                                          ((double)j * k_whole + (double)m * len);
                     if (us < best_us) { best_us = us; best = {st.shape, ranges, len, (uint32_t)(j * cus), K <= md.urgent_max_k ? 1u : 0u}; }
                 }
             }

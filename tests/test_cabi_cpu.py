@@ -105,6 +105,10 @@ def test_planner_choices():
     p = hip.plan(2, 1024, 1024, 6144)                      # 64 tiles of 128 x 128 on 4 ranges, one per CU: 29.6 -> 23.5 us
     assert (p.tile_m, p.k_splits) == (128, 4)
     assert hip.plan(2, 768, 768, 16384).k_splits == 6 and hip.plan(2, 2048, 2048, 8192).k_splits == 1
+    p = hip.plan(2, 2560, 2048, 4096)                      # 320 tiles of 128 x 128: 256 whole + 64 on 4 ranges (52.5 us; all on 3 ranges 57.4)
+    assert (p.tile_m, p.k_splits, p.whole_tiles) == (128, 4, 256)
+    assert hip.plan(2, 3072, 2048, 8192).k_splits == 1     # 1.5 per CU, power-bound either way: whole 100.9 us, 4 ranges 115.3
+    assert hip.plan(2, 2560, 2048, 2048).k_splits == 1 and hip.plan(2, 2560, 2048, 8192).whole_tiles == 0
     p = hip.plan(2, 300, 300, 8192)                        # few tiles: 8 ranges on 64 x 64 (12.9 us; the 20 that two
     assert (p.tile_m, p.k_splits) == (64, 8)               # workgroups per CU would ask for: 17.8, the whole product 38.8)
     # more tiles than the chip holds at once: the full rounds stay whole, only the ragged last round is split

@@ -339,6 +339,7 @@ def test_f16_split_k_through_a_workspace(hip, oracle, M, N, K):
     (np.float32, 900, 700, 4100, 64, 3, 0),         # fewer tiles than CUs: all of them on 3 ranges
     (np.float16, 1280, 1024, 6144, 128, 3, 0),      # 80 tiles of 128 x 128 on 3 ranges
     (np.float16, 768, 768, 8200, 128, 4, 0),
+    (np.float16, 2560, 2048, 4100, 128, 4, 256),    # 320 tiles of 128 x 128: a whole one per CU, 64 on 4 ranges
 ])
 def test_split_k_for_a_few_hundred_tiles(hip, oracle, dtype, M, N, K, tile, splits, whole):
     """Outputs of a few hundred small tiles and a long K: with a workspace the product runs on the tile shape that
