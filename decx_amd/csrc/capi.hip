@@ -138,6 +138,21 @@ static const SplitModel kSplitF64 = {{{TILE_SMALL, 2, 4, {0, 28.2, 28.8}}, {}}, 
 
 TileInfo dma_tile_info(int elem_bytes, int shape, uint32_t N);
 
+// K on about p ranges whose starts are multiples of `align` (the deepest slab): `len` for all but the last, which takes
+// what is left.  Rounding K / p up makes the last range the shortest, rounding it down the longest; the one whose
+// longest range is shorter wins (K = 777 on two: 416 + 361 or 384 + 393).
+struct RangeLen { uint32_t len, ranges, longest; };
+RangeLen range_len(uint32_t K, uint32_t p, uint32_t align)
+{
+    const uint32_t up = ((K + p - 1) / p + align - 1) / align * align, n_up = (K + up - 1) / up;
+    const uint32_t down = K / p / align * align;
+    if (down && (uint64_t)down * p < K && n_up == p) {
+        const uint32_t last = K - (p - 1) * down;
+        if (last < up) return {down, p, last};
+    }
+    return {up, n_up, up};
+}
+
 SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K, int whole_shape, const TileInfo& whole)
 {
     const SplitModel& md = elem_bytes == 8 ? kSplitF64 : elem_bytes == 2 ? kSplitF16 : kSplitF32;
@@ -197,10 +212,10 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
             // 66.7, whole on 256 x 256 tiles 60.4): full rounds in front only where the whole product takes the same tile
             if (elem_bytes == 2 && whole > 0 && st.shape != whole_shape) continue;
             for (uint32_t p = 2; p <= tile_max_p && (t - whole) * p <= 4096; ++p) {
-                const uint32_t len = ((K + p - 1) / p + md.len_align - 1) / md.len_align * md.len_align, ranges = (K + len - 1) / len;
-                if (ranges < 2) continue;
-                const double us = estimate(st, t, len, ranges, whole);
-                if (us < best_us) { best_us = us; best = {st.shape, ranges, len, (uint32_t)whole}; }
+                const RangeLen rl = range_len(K, p, md.len_align);
+                if (rl.ranges < 2) continue;
+                const double us = estimate(st, t, rl.longest, rl.ranges, whole);
+                if (us < best_us) { best_us = us; best = {st.shape, rl.ranges, rl.len, (uint32_t)whole}; }
             }
         }
         // Or the CUs hold j whole tiles each (the first j x CUs workgroups of the grid: the hardware deals them out evenly)
@@ -219,14 +234,15 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
             for (uint64_t j = 1; j < (uint64_t)st.fit && j * cus < t; ++j) {
                 const uint64_t rest = t - j * cus, room = ((uint64_t)st.fit - j) * cus;
                 for (uint32_t p = 2; p <= max_p && rest * p <= room && (elem_bytes != 2 || (K >= 4096 && K < 8192)); ++p) {     // (fp16: no gain measured below 4096, nor from 8192 on, where all tiles on 3 ranges do as well)
-                    const uint32_t len = ((K + p - 1) / p + md.len_align - 1) / md.len_align * md.len_align, ranges = (K + len - 1) / len;
+                    const RangeLen rl = range_len(K, p, md.len_align);
+                    const uint32_t len = rl.longest, ranges = rl.ranges;
                     if (ranges < 2 || ranges > kSplitFlat || rest * ranges > room) continue;
                     const uint64_t m = (rest * ranges + cus - 1) / cus;
                     const uint32_t group = st.pieces < 16 ? st.pieces : 16, batch = 16 / group, per_slot = st.pieces / group;
                     const double us = md.shared_us_fixed + md.us_per_trip * ((ranges + batch - 1) / batch * per_slot) +
                                       (md.shared_ns_per_k + md.shared_ns_busy * (double)(rest * ranges) / (double)room) * 1e-3 *
                                           ((double)j * k_whole + (double)m * len);
-                    if (us < best_us) { best_us = us; best = {st.shape, ranges, len, (uint32_t)(j * cus), K <= md.urgent_max_k ? 1u : 0u}; }
+                    if (us < best_us) { best_us = us; best = {st.shape, ranges, rl.len, (uint32_t)(j * cus), K <= md.urgent_max_k ? 1u : 0u}; }
                 }
             }
         }

@@ -31,7 +31,7 @@ struct GemmArgs {
     uint32_t vec_ok;             // 1: every base pointer is 16-byte aligned and every pitch a multiple of 16 bytes
     uint32_t cus;                // compute units of the device (0: not given, the kernels take 256)
     // Split K (direct-load kernels; a 1-D grid of split_first whole tiles, then split 0 of every split tile, split 1 of
-    // every split tile, ...): split z multiplies k in [z * split_len, min(K, (z + 1) * split_len)).  Every workgroup stores its accumulators (fp32, or fp64 for fp64 operands) to its
+    // every split tile, ...): split z multiplies k in [z * split_len, (z + 1) * split_len), the last one up to K (its range may be longer or shorter than the others').  Every workgroup stores its accumulators (fp32, or fp64 for fp64 operands) to its
     // slot of split_ws and counts itself in at split_counters[tile]; the one that arrives last adds all slots of the
     // tile in split order (its own included, so the result does not depend on who is last), writes D and puts the
     // counter back to zero (split_k_exchange.hpp).

@@ -95,7 +95,7 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
             const uint32_t k0 = sb.z * g_in.split_len;
             g_split.A = (const unsigned char*)g_in.A + (size_t)k0 * 2;
             g_split.B = (const unsigned char*)g_in.B + (size_t)k0 * g_in.ldb * 2;
-            g_split.K = g_in.K - k0 < g_in.split_len ? g_in.K - k0 : g_in.split_len;
+            g_split.K = sb.z + 1 == sb.splits ? g_in.K - k0 : g_in.split_len;     // the last range: what is left (more or less than split_len)
             if (g_in.split_urgent) __builtin_amdgcn_s_setprio(3);
         }
     } else {
