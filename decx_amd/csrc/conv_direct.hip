@@ -9,11 +9,12 @@
 // instruction; the vector pipe does one fma per (pixel, patch element, kernel), which is the arithmetic itself.
 //
 // What bounds it is the memory system's rate for traffic that is mostly writes (1920 x 1080 x 3, 8 kernels: 25 MB in,
-// 66 MB out in 24 us; a plain copy kernel moves 4.6 TB/s of reads plus writes on this part, i.e. 20 us for these 91 MB):
+// 66 MB out in 23 us; a plain copy kernel moves 4.6 TB/s of reads plus writes on this part, i.e. 20 us for these 91 MB):
 // the same arithmetic on the matrix cores (v_mfma_f32_4x4x1_16b_f32 with the weights of four kernels as one operand and
 // the lane's own patch element as the other leaves every lane with its pixel's four outputs, bit for bit the same chain,
 // in a sixteenth of the instructions) measured 23.2 us there and lost on smaller and larger images (640 x 480: 8.5
-// against 6.9 us, 3840 x 2160: 143 against 126), so it is not in here.
+// against 6.9 us, 3840 x 2160: 143 against 126), so it is not in here; with the stores below and the weights in LDS it
+// lost again (8 kernels 23.5 against 22.8 us, 16 kernels 46.8 against 34.5, 32 kernels at 1000 x 700: 40.7 against 24.3).
 //
 // Same operands and layouts as the GEMM form (image [row][column][channel pitch], kernels packed
 // [patch element][kernel] with zero rows for padded channels, destination [row][column][channel pitch]), same
@@ -55,7 +56,7 @@ conv2d_direct_kernel(const float* __restrict__ image, const float* __restrict__ 
 #pragma unroll
     for (int o = 0; o < NACC; ++o) acc[o] = 0.f;
 
-    const float* w = kmat;                                 // row k of the packed kernels: the same for every lane
+    const float* w = kmat;                             // row k of the packed kernels: the same for every lane
     for (uint32_t kh = 0; kh < k_h; ++kh) {
         const float* run = patch + (size_t)kh * row_floats;
         for (uint32_t e = 0; e < seg_floats; e += 4) {
@@ -69,12 +70,40 @@ conv2d_direct_kernel(const float* __restrict__ image, const float* __restrict__ 
             w += (size_t)4 * kmat_pitch;
         }
     }
+    // The output is written once and is larger than L2: nontemporal stores, and whole cache lines per store instruction.
+    // A lane's CHUNKS 16-byte pieces lie CHUNKS x 16 bytes from its neighbour's, so with two or more of them the wavefront
+    // first lays its 64 pixels out in LDS as they lie in memory (no barrier: the region is the wavefront's own, and a
+    // wavefront's LDS operations complete in order) and lane l then stores piece 64 i + l of the wavefront in its i-th
+    // store, at the offset that piece's pixel left in LDS.  1920 x 1080 x 3, 8 kernels of 3 x 3: 24.3 -> 22.9 us,
+    // 3840 x 2160: 124.5 -> 84.2, 640 x 480: 7.0 -> 5.7; 16 kernels: 47.6 -> 37.3; 1000 x 700, 32 kernels: 39.1 -> 24.7.
+    // (Nontemporal stores of the lanes' own pieces, half a line per instruction: 28.8 us for 8 kernels, 160 for 16.)
+    const uint64_t my_off = ((uint64_t)oy * dst_wpitch + ox) * dst_dpitch;
+    constexpr int CHUNKS = NACC / 4;
+    if constexpr (CHUNKS >= 2) {
+        if (out_c == (uint32_t)NACC) {
+            __shared__ uint64_t offs[256];
+            __shared__ __attribute__((aligned(16))) float tr[256 * NACC];
+            const uint32_t lane = threadIdx.x & 63u, wave0 = threadIdx.x & ~63u;
+            float* mine = tr + (size_t)threadIdx.x * NACC;
+#pragma unroll
+            for (int c = 0; c < CHUNKS; ++c) *(floatx4*)(mine + 4 * c) = floatx4{acc[4 * c], acc[4 * c + 1], acc[4 * c + 2], acc[4 * c + 3]};
+            offs[threadIdx.x] = live ? my_off : ~0ull;
+#pragma unroll
+            for (int i = 0; i < CHUNKS; ++i) {
+                const uint32_t j = (uint32_t)i * 64u + lane, px = j / (uint32_t)CHUNKS, c = j % (uint32_t)CHUNKS;
+                const floatx4 v = *(const floatx4*)(tr + (size_t)wave0 * NACC + (size_t)j * 4);
+                const uint64_t off = offs[wave0 + px];
+                if (off != ~0ull) __builtin_nontemporal_store(v, (floatx4*)(dst + off + 4 * c));
+            }
+            return;
+        }
+    }
     if (!live) return;
-    float* out = dst + ((size_t)oy * dst_wpitch + ox) * dst_dpitch;
+    float* out = dst + my_off;
 #pragma unroll
     for (int o = 0; o < NACC; o += 4) {
         if ((uint32_t)o + 4 <= out_c) {
-            *(floatx4*)(out + o) = floatx4{acc[o], acc[o + 1], acc[o + 2], acc[o + 3]};
+            __builtin_nontemporal_store(floatx4{acc[o], acc[o + 1], acc[o + 2], acc[o + 3]}, (floatx4*)(out + o));
         } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e)

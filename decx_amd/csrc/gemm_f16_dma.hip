@@ -406,7 +406,9 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
             const uint32_t grow = m0 + wm0 + 16 * i + r, gcol = n0 + wn0 + 8 * pc;
             _Float16* out = D + (size_t)grow * g.ldd + gcol;
             if (interior || (grow < g.M && gcol + 8 <= g.N)) {
-                *(uintx4*)out = v;
+                // the streaming hint: 2048^3 904 -> 943 TFLOP/s, 16384 x 2048 x 512 876 -> 958, 4096^3 1399 -> 1415
+                // (8192 x 8192 x 1024: 1196 -> 1166)
+                __builtin_nontemporal_store(v, (uintx4*)out);
             } else if (grow < g.M && gcol < g.N) {
                 union { uintx4 u; _Float16 h[8]; } w;
                 w.u = v;
