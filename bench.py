@@ -37,48 +37,48 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
 # file of the kernel it was measured on with that file's SHA-256 at the time: when the kernel source has changed
 # since, the figure is withheld ("traffic": null, "traffic_stale": true) until the workload is profiled again.
 MEASURED_TRAFFIC = {
-    "fp32_8192": {"bytes": 5.67e9, "counters": "FETCH_SIZE 2.6380e6 x 2.0 KiB + WRITE_SIZE 2.621e5 KiB (FETCH_SIZE 2.66e6 ... 3.40e6 from run to run)",
+    "fp32_8192": {"bytes": 5.67e9, "counters": "FETCH_SIZE 2.6370e6 x 2.0 KiB + WRITE_SIZE 2.621e5 KiB (FETCH_SIZE 2.64e6 ... 3.40e6 from run to run)",
                   "kernel": "gemm_f32_dma_kernel<256, 128, 2, 2, 16, 2, false, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                  "source_sha256": "42b4675ace5ce46287a6879c4bcdc2d1fc1e5ffab56f8f94bb23aa2ccf21cb91", "profile": "profiles/gemm_f32_dma_fp32_8192cubed.md"},
-    "fp16_4096": {"bytes": 2.35e8, "counters": "FETCH_SIZE 98 520 x 2.0 KiB + WRITE_SIZE 32 768 KiB",
+                  "source_sha256": "d5e666b1c8f89af4112699ae13c7634dee7620818705fa8a7f3e0b219405bb0b", "profile": "profiles/gemm_f32_dma_fp32_8192cubed.md"},
+    "fp16_4096": {"bytes": 2.35e8, "counters": "FETCH_SIZE 98 520 x 2.0 KiB + WRITE_SIZE 32 774 KiB",
                   "kernel": "gemm_f16_dma_kernel<256, 256, 2, 4, 64, 2, false>", "source": "decx_amd/csrc/gemm_f16_dma.hip",
-                  "source_sha256": "7672608b2dfaee6ab187426e6cf743154d6b9401f8b85203142c62e174a902fd", "profile": "profiles/gemm_f16_dma_fp16_4096cubed.md"},
-    "fp64_4096": {"bytes": 1.21e9, "counters": "FETCH_SIZE 524 441 x 2.0 KiB + WRITE_SIZE 131 072 KiB",
+                  "source_sha256": "cd9908bada071afe4720c1e7cad55a10d63243a30656e19f2f17bd9a8b71e764", "profile": "profiles/gemm_f16_dma_fp16_4096cubed.md"},
+    "fp64_4096": {"bytes": 1.21e9, "counters": "FETCH_SIZE 524 441 x 2.0 KiB + WRITE_SIZE 131 098 KiB",
                   "kernel": "gemm_f64_dma_kernel<256, 128, 4, 2, 16, 3, false>", "source": "decx_amd/csrc/gemm_f64.hip",
-                  "source_sha256": "8bfbb2f095545fa429bdc684d2eb76fc7ed7944b7f044310b2cc232485cf66a4", "profile": "profiles/gemm_f64_dma_fp64_4096cubed.md"},
+                  "source_sha256": "16b1410dda50b7db160f38aa84050bc47f2d2f20348dd2acf59a2f4dac12cade", "profile": "profiles/gemm_f64_dma_fp64_4096cubed.md"},
     "fp32_1024": {"bytes": 2.95e7, "counters": "FETCH_SIZE 12 352 x 2.0 KiB + WRITE_SIZE 4 096 KiB",
                   "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                  "source_sha256": "42b4675ace5ce46287a6879c4bcdc2d1fc1e5ffab56f8f94bb23aa2ccf21cb91", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
-    "fp32_ragged": {"bytes": 5.65e7, "counters": "FETCH_SIZE 18 503 x 2.0 KiB + WRITE_SIZE 18 199 KiB (operands, and the slots of the 2 ranges of K)",
+                  "source_sha256": "d5e666b1c8f89af4112699ae13c7634dee7620818705fa8a7f3e0b219405bb0b", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+    "fp32_ragged": {"bytes": 4.44e7, "counters": "FETCH_SIZE 16 666 x 2.0 KiB + WRITE_SIZE 9 983 KiB (operands, and the slots of the 128 tiles that are split in two; 256 tiles are whole)",
                     "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                    "source_sha256": "42b4675ace5ce46287a6879c4bcdc2d1fc1e5ffab56f8f94bb23aa2ccf21cb91", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
-    "fp32_ragged_abc": {"bytes": 6.25e7, "counters": "FETCH_SIZE 21 423 x 2.0 KiB + WRITE_SIZE 18 199 KiB",
+                    "source_sha256": "d5e666b1c8f89af4112699ae13c7634dee7620818705fa8a7f3e0b219405bb0b", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+    "fp32_ragged_abc": {"bytes": 5.04e7, "counters": "FETCH_SIZE 19 606 x 2.0 KiB + WRITE_SIZE 9 983 KiB",
                         "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, true>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                        "source_sha256": "42b4675ace5ce46287a6879c4bcdc2d1fc1e5ffab56f8f94bb23aa2ccf21cb91", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
-    "fp32_tall_skinny": {"bytes": 3.58e8, "counters": "FETCH_SIZE 142 167 x 2.0 KiB + WRITE_SIZE 65 536 KiB",
+                        "source_sha256": "d5e666b1c8f89af4112699ae13c7634dee7620818705fa8a7f3e0b219405bb0b", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+    "fp32_tall_skinny": {"bytes": 3.58e8, "counters": "FETCH_SIZE 141 956 x 2.0 KiB + WRITE_SIZE 65 536 KiB",
                          "kernel": "gemm_f32_dma_kernel<256, 128, 2, 2, 16, 2, false, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                         "source_sha256": "42b4675ace5ce46287a6879c4bcdc2d1fc1e5ffab56f8f94bb23aa2ccf21cb91", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
-    "fp32_mid_long_k": {"bytes": 3.76e8, "counters": "FETCH_SIZE 160 893 x 2.0 KiB + WRITE_SIZE 46 170 KiB (operands, and the slots of the 8 ranges of K)",
+                         "source_sha256": "d5e666b1c8f89af4112699ae13c7634dee7620818705fa8a7f3e0b219405bb0b", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+    "fp32_mid_long_k": {"bytes": 3.12e8, "counters": "FETCH_SIZE 147 873 x 2.0 KiB + WRITE_SIZE 9 226 KiB (operands, and the slots of the 64 tiles that are split in four; 256 tiles are whole)",
                         "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                        "source_sha256": "42b4675ace5ce46287a6879c4bcdc2d1fc1e5ffab56f8f94bb23aa2ccf21cb91", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
+                        "source_sha256": "d5e666b1c8f89af4112699ae13c7634dee7620818705fa8a7f3e0b219405bb0b", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
     "fp32_gemv": {"bytes": 2.70e8, "counters": "FETCH_SIZE (131 258 + 522) x 2.0 KiB + WRITE_SIZE (256 + 32) KiB: matrix-vector kernel + the copy of x",
                   "kernel": "gemv_kernel<float, float, 2, 1>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "4b643fb2db289936e88028f8ddcf8b14ab9fce401e801b59cb3779d7d23aed21", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "5cccc9d00320d0a2a62939fdf04484d79a04bf8a1533b3757ed0ef48c1a66532", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp32_gevm": {"bytes": 2.69e8, "counters": "FETCH_SIZE 131 233 x 2.0 KiB + WRITE_SIZE 32 KiB",
                   "kernel": "gevm_kernel<float, float, 8>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "4b643fb2db289936e88028f8ddcf8b14ab9fce401e801b59cb3779d7d23aed21", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "5cccc9d00320d0a2a62939fdf04484d79a04bf8a1533b3757ed0ef48c1a66532", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp16_gemv": {"bytes": 1.36e8, "counters": "FETCH_SIZE (65 647 + 522) x 2.0 KiB + WRITE_SIZE (256 + 16) KiB: matrix-vector kernel + the copy of x",
                   "kernel": "gemv_kernel<_Float16, _Float16, 2, 1>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "4b643fb2db289936e88028f8ddcf8b14ab9fce401e801b59cb3779d7d23aed21", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "5cccc9d00320d0a2a62939fdf04484d79a04bf8a1533b3757ed0ef48c1a66532", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp16_gevm": {"bytes": 1.35e8, "counters": "FETCH_SIZE 65 685 x 2.0 KiB + WRITE_SIZE 92 KiB",
                   "kernel": "gevm_kernel<_Float16, _Float16, 8>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "4b643fb2db289936e88028f8ddcf8b14ab9fce401e801b59cb3779d7d23aed21", "profile": "profiles/gemv_gevm_8192x8192.md"},
-    "conv2d": {"bytes": 1.08e8, "counters": "FETCH_SIZE 20 545 x 2.0 KiB + WRITE_SIZE 64 516 KiB",
+                  "source_sha256": "5cccc9d00320d0a2a62939fdf04484d79a04bf8a1533b3757ed0ef48c1a66532", "profile": "profiles/gemv_gevm_8192x8192.md"},
+    "conv2d": {"bytes": 1.08e8, "counters": "FETCH_SIZE 20 548 x 2.0 KiB + WRITE_SIZE 64 528 KiB",
                "kernel": "gemm_f32_dma_kernel<256, 256, 2, 4, 16, 4, false, 2, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-               "source_sha256": "42b4675ace5ce46287a6879c4bcdc2d1fc1e5ffab56f8f94bb23aa2ccf21cb91", "profile": "profiles/conv2d_implicit_gemm_256x256x112_3x3x256.md"},
-    "conv2d_rgb": {"bytes": 1.00e8, "counters": "FETCH_SIZE 16 455 x 2.0 KiB + WRITE_SIZE 64 613 KiB",
+               "source_sha256": "d5e666b1c8f89af4112699ae13c7634dee7620818705fa8a7f3e0b219405bb0b", "profile": "profiles/conv2d_implicit_gemm_256x256x112_3x3x256.md"},
+    "conv2d_rgb": {"bytes": 1.01e8, "counters": "FETCH_SIZE 16 457 x 2.0 KiB + WRITE_SIZE 66 133 KiB",
                    "kernel": "conv2d_direct_kernel<8, 3>", "source": "decx_amd/csrc/conv_direct.hip",
-                   "source_sha256": "91b8dd40c7d5ace863daedc2876c5cd9e2a7843c09a30451c9ac3dadcd1c8250", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
+                   "source_sha256": "743f8085e23b35e155b1707c1bdef9b228656d9b2d166446d7aec6af9d3c37e7", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
 }
 
 
@@ -121,7 +121,7 @@ WORKLOADS = {
     "fp32_ragged": ("f32", 1000, 1500, 777, "mfma", 2, "fp32 GEMM M=1000 N=1500 K=777, uniform[-1,1]"),
     "fp32_ragged_abc": ("f32", 1000, 1500, 777, "mfma", 2, "fp32 GEMM D=A.B+C M=1000 N=1500 K=777 (four-matrix entry, alpha=beta=1), uniform[-1,1]"),
     "fp32_tall_skinny": ("f32", 65536, 256, 1024, "mfma", 5, "fp32 GEMM M=65536 N=256 K=1024, uniform[-1,1]"),
-    "fp32_mid_long_k": ("f32", 1280, 1024, 8192, "mfma", 8, "fp32 GEMM M=1280 N=1024 K=8192 (320 small tiles, split along K through the workspace), uniform[-1,1]"),
+    "fp32_mid_long_k": ("f32", 1280, 1024, 8192, "mfma", 8, "fp32 GEMM M=1280 N=1024 K=8192 (320 small tiles: 256 whole, 64 split along K through the workspace), uniform[-1,1]"),
     "fp32_gemv": ("f32", 8192, 1, 8192, "hbm", 6, "fp32 GEMM M=8192 N=1 K=8192 (GEMV-like), uniform[-1,1]"),
     "fp32_gevm": ("f32", 1, 8192, 8192, "hbm", 6, "fp32 GEMM M=1 N=8192 K=8192 (vector x matrix), uniform[-1,1]"),
     "fp16_gemv": ("f16", 8192, 1, 8192, "hbm", 6, "fp16 GEMM M=8192 N=1 K=8192 (fp32 accumulate), normal(0,0.5)"),
