@@ -72,7 +72,8 @@ typedef struct decx_hip_plan {
                                       With more than one, path / tile are those of the split (it may run on a smaller
                                       tile than the whole product takes without a workspace) */
     uint32_t whole_tiles;          /* with k_splits > 1: tiles that are multiplied whole all the same -- the full rounds
-                                      of workgroups; only the tiles of the ragged last round are split.  0: all are */
+                                      of workgroups in front of a ragged last round, or one to three tiles per CU that
+                                      share their CU with the workgroups of the split ones.  0: all are split */
 } decx_hip_plan;
 
 /* ---- device, memory, streams, events --------------------------------------------------
