@@ -95,6 +95,24 @@ def test_conv2d_invalid_arguments(hip):
     assert withdepth(3) == 0 and withdepth(4) == 0 and withdepth(0) == -1 and withdepth(5) == -1
 
 
+@pytest.mark.parametrize("OC", [4, 8, 12, 16, 20, 24, 28, 32, 3, 6, 10, 30])
+@pytest.mark.parametrize("W,H", [(70, 50), (259, 21), (64, 9)])
+def test_every_store_path_of_the_lane_per_pixel_kernel(hip, oracle, OC, W, H):
+    """3 x 3 over RGB.  A multiple of four kernels from 8 up: a wavefront lays its 64 pixels out in LDS and stores whole
+    cache lines (here with image rows that end inside a wavefront: 68, 257 and 62 output pixels per row, the destination's
+    rows are longer, and the last wavefront has idle lanes); 4 kernels: one piece per lane; any other number: the last
+    piece element by element, the channels beyond the kernels untouched.  Bit-exact: the kernel runs the oracle's chain."""
+    image, kernels = data(W, H, 3, OC, 3, 3, 7000 + OC + W)
+    ref = oracle.conv2d_f32(image, kernels, 1, 1, False)
+    got, raw = hip.conv2d(image, kernels, 1, 1, False)
+    assert got.shape == ref.shape == (H - 2, W - 2, OC)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+    oh, ow = ref.shape[:2]
+    assert np.all(raw[:oh, ow:, :] == np.float32(-555.0)), "padding columns of dst were written"
+    assert np.all(raw[:oh, :ow, OC:] == np.float32(-555.0)), "padding channels of dst were written"
+    assert np.all(raw[oh:] == np.float32(-555.0)), "rows beyond the output were written"
+
+
 @pytest.mark.parametrize("C", [1, 2, 3])
 @pytest.mark.parametrize("extend", [False, True])
 def test_padding_channel_of_grey_and_rgb_images_is_never_read_into_a_result(hip, oracle, C, extend):
