@@ -495,21 +495,139 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
     float* __restrict__ D = (float*)g.D;
     const uint32_t col0 = n0 + b_col;
     const bool interior = (m0 + BM <= g.M) && (n0 + BN <= g.N);
+    const auto row_of = [&](int i, int r) { return m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * h + (r % 4); };
+    const auto d_row_of = [&](uint32_t row) {              // offset of the row's first element in D
+        if constexpr (CONV != 0) return (size_t)(row / g.conv_wout) * g.conv_dst_row + (size_t)(row % g.conv_wout) * g.ldd;
+        else return (size_t)row * g.ldd;
+    };
+    constexpr bool STRAIGHT = TM * TN < 8;     // (the 256 x 128 tile keeps the row-by-row form below: 142 VGPRs otherwise, one workgroup per CU)
+    // (the 128 x 128 tile takes it with a C only: without one it gains nothing there, and edge shapes lose 2 %)
+    if (STRAIGHT && interior && (TM * TN == 1 || (!C_EARLY && C != nullptr))) {
+        // Straight-line code: with a C, the loads of a batch of rows are all asked for before the first is used (a load,
+        // its wait, the fma and the store row by row made the C term cost 6 % at 2048^3 and 14 % at 65536 x 256 x 1024).
+        // D is written once, read by whoever comes next, often larger than L2: the streaming hint (65536 x 256 x 1024
+        // 244 -> 240 us, 2048^3 122.2 -> 120.6, 1024^3 18.65 -> 18.3, 8192^3 the same).  An address is a scalar base (the
+        // row: tile, wavefront, register) plus one 32-bit lane offset for all rows, so no row costs a register pair.
+        const bool with_c = !C_EARLY && C != nullptr;
+        const uint32_t lane_d = (uint32_t)(4 * h) * g.ldd * 4u + (uint32_t)b_col * 4u;
+        const uint32_t lane_c = (uint32_t)(4 * h) * g.ldc * 4u + (uint32_t)b_col * 4u;
+        // The row offsets run from row to row (1, 1, 1, 5 rows on: registers 4 q .. 4 q + 3 are rows 8 q .. 8 q + 3) behind
+        // an empty asm each, or the compiler computes the 16 TM offsets of a wavefront up front and they fill the register
+        // file; with and without C are two copies of the code, or both are computed and one selected.
+        size_t d_off = ((size_t)(m0 + (uint32_t)wm0) * g.ldd + n0) * 4, c_off = ((size_t)(m0 + (uint32_t)wm0) * g.ldc + n0) * 4;
+        const size_t d_step = (size_t)g.ldd * 4, c_step = (size_t)g.ldc * 4;
+        const auto d_ptr = [&](int i, int r) {
+            if constexpr (CONV != 0) return (bfrag*)(D + d_row_of(row_of(i, r)) + col0);
+            else {
+                bfrag* const p = (bfrag*)((unsigned char*)D + d_off + lane_d);
+                d_off += (r % 4 == 3 ? 5 : 1) * d_step;
+                asm volatile("" : "+s"(d_off));
+                return p;
+            }
+        };
+        const auto c_ptr = [&](int r) {
+            const bfrag* const p = (const bfrag*)((const unsigned char*)C + c_off + lane_c);
+            c_off += (r % 4 == 3 ? 5 : 1) * c_step;
+            asm volatile("" : "+s"(c_off));
+            return p;
+        };
+        // rows per batch: few where the accumulators fill the register file
+        constexpr int G = TM * TN >= 8 ? 4 : TM * TN >= 4 ? 8 : 16;
+        const auto store_all = [&](auto with_c_t) {
+            constexpr bool WITH_C = decltype(with_c_t)::value;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int r0 = 0; r0 < 16; r0 += G) {
+                    bfrag cv[G];
+                    if constexpr (WITH_C) {
+#pragma unroll
+                        for (int r = 0; r < G; ++r) cv[r] = *c_ptr(r0 + r);
+                    }
+#pragma unroll
+                    for (int q = 0; q < G; ++q) {
+                        const int r = r0 + q;
+                        float v[TN];
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) v[j] = acc[i][j][r];
+                        if constexpr (C_EARLY) {
+                            if (C) v[0] = __builtin_fmaf(c_early[r], g.beta, g.alpha * v[0]);
+                        }
+                        if constexpr (WITH_C) {
+#pragma unroll
+                            for (int j = 0; j < TN; ++j) v[j] = __builtin_fmaf(lane_of<TN>(cv[q], j), g.beta, g.alpha * v[j]);
+                        }
+                        bfrag o;
+                        if constexpr (TN == 1) o = v[0];
+                        else {
+#pragma unroll
+                            for (int j = 0; j < TN; ++j) o[j] = v[j];
+                        }
+                        __builtin_nontemporal_store(o, d_ptr(i, r));
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        };
+        if (with_c) store_all(std::true_type{}); else store_all(std::false_type{});
+        return;
+    }
+    if constexpr (STRAIGHT) {
+        // edge tiles, element by element; the C values of a batch of rows are asked for together here too (1000 x 1500 x 777
+        // on 64 x 64 tiles, 39 edge tiles of 384: the C term cost 14.8 %)
+        constexpr int G = TM * TN >= 4 ? 8 : 16;
+        const auto store_edge = [&](auto with_c_t) {
+            constexpr bool WITH_C = decltype(with_c_t)::value;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int r0 = 0; r0 < 16; r0 += G) {
+                    float cv[G][TN];
+                    if constexpr (WITH_C) {
+#pragma unroll
+                        for (int q = 0; q < G; ++q) {
+                            const uint32_t row = row_of(i, r0 + q);
+#pragma unroll
+                            for (int j = 0; j < TN; ++j)
+                                cv[q][j] = (row < g.M && col0 + j < g.N) ? C[(size_t)row * g.ldc + col0 + j] : 0.f;
+                        }
+                    }
+#pragma unroll
+                    for (int q = 0; q < G; ++q) {
+                        const int r = r0 + q;
+                        const uint32_t row = row_of(i, r);
+                        if (row >= g.M) continue;
+                        const size_t d_row = d_row_of(row);
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) {
+                            if (col0 + j < g.N) {
+                                float o = acc[i][j][r];
+                                if constexpr (C_EARLY) {
+                                    if (C && j == 0) o = __builtin_fmaf(c_early[r], g.beta, g.alpha * o);
+                                }
+                                if constexpr (WITH_C) o = __builtin_fmaf(cv[q][j], g.beta, g.alpha * o);
+                                D[d_row + col0 + j] = o;
+                            }
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        };
+        if (!C_EARLY && C != nullptr) { store_edge(std::true_type{}); return; }
+    }
+    // the largest tile: interior tiles row by row; edge tiles without a C to fetch, element by element (one store wherever
+    // the lane's TN columns all exist: 141 VGPRs in place of 64)
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const uint32_t row = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * h + (r % 4);
-            size_t d_row;                              // offset of the row's first element in D
-            if constexpr (CONV != 0) d_row = (size_t)(row / g.conv_wout) * g.conv_dst_row + (size_t)(row % g.conv_wout) * g.ldd;
-            else d_row = (size_t)row * g.ldd;
-            float v[TN];
+            const uint32_t row = row_of(i, r);
+            const size_t d_row = d_row_of(row);
+            if ((!STRAIGHT || TM * TN > 1) && interior) {
+                float v[TN];
 #pragma unroll
-            for (int j = 0; j < TN; ++j) v[j] = acc[i][j][r];
-            if constexpr (C_EARLY) {
-                if (C) v[0] = __builtin_fmaf(c_early[r], g.beta, g.alpha * v[0]);
-            }
-            if (interior) {       // (one store also on edge tiles wherever the lane's TN columns all exist: 141 VGPRs in place of 64)
+                for (int j = 0; j < TN; ++j) v[j] = acc[i][j][r];
                 if constexpr (!C_EARLY) {
                     if (C) {
                         const bfrag cv = *(const bfrag*)(C + (size_t)row * g.ldc + col0);
@@ -523,15 +641,15 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
 #pragma unroll
                     for (int j = 0; j < TN; ++j) o[j] = v[j];
                 }
-                // written once, read by whoever comes next, often larger than L2: the streaming hint (65536 x 256 x 1024
-                // 244 -> 240 us, 2048^3 122.2 -> 120.6, 1024^3 18.65 -> 18.3, 8192^3 the same)
                 __builtin_nontemporal_store(o, (bfrag*)(D + d_row + col0));
             } else if (row < g.M) {
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
                     if (col0 + j < g.N) {
-                        float o = v[j];
-                        if constexpr (!C_EARLY) {
+                        float o = acc[i][j][r];
+                        if constexpr (C_EARLY) {
+                            if (C && j == 0) o = __builtin_fmaf(c_early[r], g.beta, g.alpha * o);
+                        } else {
                             if (C) o = __builtin_fmaf(C[(size_t)row * g.ldc + col0 + j], g.beta, g.alpha * o);
                         }
                         D[d_row + col0 + j] = o;
