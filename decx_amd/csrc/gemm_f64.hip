@@ -311,12 +311,22 @@ gemm_f64_dma_kernel(const GemmArgs g_in)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t row = m0 + wm0 + 16 * ti + 4 * i + q;
+            // interior tiles ask for a row's C values before the first is used
+            doublex2 c_row[TP];
+            const bool c_ahead = C != nullptr && interior;
+            if (c_ahead) {
+#pragma unroll
+                for (int jj = 0; jj < TP; ++jj) c_row[jj] = *(const doublex2*)(C + (size_t)row * g.ldc + (n0 + b_col + 32 * jj));
+            }
 #pragma unroll
             for (int jj = 0; jj < TP; ++jj) {
                 const uint32_t col = n0 + b_col + 32 * jj;
                 double v0 = acc[ti][2 * jj][i], v1 = acc[ti][2 * jj + 1][i];
                 if (interior || (row < g.M && col + 2 <= g.N)) {
-                    if (C) {
+                    if (c_ahead) {
+                        v0 = __builtin_fma(c_row[jj][0], g.beta64, g.alpha64 * v0);
+                        v1 = __builtin_fma(c_row[jj][1], g.beta64, g.alpha64 * v1);
+                    } else if (C) {
                         const doublex2 cv = *(const doublex2*)(C + (size_t)row * g.ldc + col);
                         v0 = __builtin_fma(cv[0], g.beta64, g.alpha64 * v0);
                         v1 = __builtin_fma(cv[1], g.beta64, g.alpha64 * v1);
