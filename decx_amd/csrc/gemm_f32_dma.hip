@@ -551,7 +551,7 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
 #pragma unroll
                         for (int j = 0; j < TN; ++j) v[j] = acc[i][j][r];
                         if constexpr (C_EARLY) {
-                            if (C) v[0] = __builtin_fmaf(c_early[r], g.beta, g.alpha * v[0]);
+                            v[0] = __builtin_fmaf(c_early[r], g.beta, g.alpha * v[0]);     // (this instantiation runs with a C only)
                         }
                         if constexpr (WITH_C) {
 #pragma unroll
@@ -603,7 +603,7 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
                             if (col0 + j < g.N) {
                                 float o = acc[i][j][r];
                                 if constexpr (C_EARLY) {
-                                    if (C && j == 0) o = __builtin_fmaf(c_early[r], g.beta, g.alpha * o);
+                                    if (j == 0) o = __builtin_fmaf(c_early[r], g.beta, g.alpha * o);
                                 }
                                 if constexpr (WITH_C) o = __builtin_fmaf(cv[q][j], g.beta, g.alpha * o);
                                 D[d_row + col0 + j] = o;
@@ -648,7 +648,7 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
                     if (col0 + j < g.N) {
                         float o = acc[i][j][r];
                         if constexpr (C_EARLY) {
-                            if (C && j == 0) o = __builtin_fmaf(c_early[r], g.beta, g.alpha * o);
+                            if (j == 0) o = __builtin_fmaf(c_early[r], g.beta, g.alpha * o);
                         } else {
                             if (C) o = __builtin_fmaf(C[(size_t)row * g.ldc + col0 + j], g.beta, g.alpha * o);
                         }
