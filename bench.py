@@ -39,46 +39,46 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
 MEASURED_TRAFFIC = {
     "fp32_8192": {"bytes": 5.67e9, "counters": "FETCH_SIZE 2.6383e6 x 2.0 KiB + WRITE_SIZE 2.621e5 KiB (FETCH_SIZE 2.64e6 ... 3.40e6 from run to run)",
                   "kernel": "gemm_f32_dma_kernel<256, 128, 2, 2, 16, 2, false, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                  "source_sha256": "fc144dd4f6024eaeaa247125634d9a430904e2914977ee98e6de1e2abf0ba6bf", "profile": "profiles/gemm_f32_dma_fp32_8192cubed.md"},
+                  "source_sha256": "3d5258c6b04f9947025a532a207321072f8a0a86abba6952293d4b7b17921c75", "profile": "profiles/gemm_f32_dma_fp32_8192cubed.md"},
     "fp16_4096": {"bytes": 2.35e8, "counters": "FETCH_SIZE 98 543 x 2.0 KiB + WRITE_SIZE 32 778 KiB",
                   "kernel": "gemm_f16_dma_kernel<256, 256, 2, 4, 64, 2, false>", "source": "decx_amd/csrc/gemm_f16_dma.hip",
-                  "source_sha256": "12e1a9c6a9a2669e8416aea3470a96a2ffe28146e5a404c4007ddc6f1ab51461", "profile": "profiles/gemm_f16_dma_fp16_4096cubed.md"},
+                  "source_sha256": "8fe2bf39af426d7dd5e58cb40eacf4f3cbcc1192a266f8b5a923330679cec043", "profile": "profiles/gemm_f16_dma_fp16_4096cubed.md"},
     "fp64_4096": {"bytes": 1.21e9, "counters": "FETCH_SIZE 524 460 x 2.0 KiB + WRITE_SIZE 131 106 KiB",
                   "kernel": "gemm_f64_dma_kernel<256, 128, 4, 2, 16, 3, false>", "source": "decx_amd/csrc/gemm_f64.hip",
-                  "source_sha256": "dbc487b31ead39829cd20fc03729d367462fb35dd22d3480ad4f480b4773341f", "profile": "profiles/gemm_f64_dma_fp64_4096cubed.md"},
+                  "source_sha256": "b21c941385a6d73c7134f9f30ee5cf1ac1453522fda2b4a09e36683088de5226", "profile": "profiles/gemm_f64_dma_fp64_4096cubed.md"},
     "fp32_1024": {"bytes": 2.95e7, "counters": "FETCH_SIZE 12 342 x 2.0 KiB + WRITE_SIZE 4 096 KiB",
                   "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                  "source_sha256": "fc144dd4f6024eaeaa247125634d9a430904e2914977ee98e6de1e2abf0ba6bf", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+                  "source_sha256": "3d5258c6b04f9947025a532a207321072f8a0a86abba6952293d4b7b17921c75", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
     "fp32_ragged": {"bytes": 4.44e7, "counters": "FETCH_SIZE 16 663 x 2.0 KiB + WRITE_SIZE 9 983 KiB (operands, and the slots of the 128 tiles that are split in two; 256 tiles are whole)",
                     "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                    "source_sha256": "fc144dd4f6024eaeaa247125634d9a430904e2914977ee98e6de1e2abf0ba6bf", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+                    "source_sha256": "3d5258c6b04f9947025a532a207321072f8a0a86abba6952293d4b7b17921c75", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
     "fp32_ragged_abc": {"bytes": 5.04e7, "counters": "FETCH_SIZE 19 604 x 2.0 KiB + WRITE_SIZE 9 983 KiB",
                         "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, true>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                        "source_sha256": "fc144dd4f6024eaeaa247125634d9a430904e2914977ee98e6de1e2abf0ba6bf", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+                        "source_sha256": "3d5258c6b04f9947025a532a207321072f8a0a86abba6952293d4b7b17921c75", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
     "fp32_tall_skinny": {"bytes": 3.58e8, "counters": "FETCH_SIZE 142 267 x 2.0 KiB + WRITE_SIZE 65 536 KiB",
                          "kernel": "gemm_f32_dma_kernel<256, 128, 2, 2, 16, 2, false, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                         "source_sha256": "fc144dd4f6024eaeaa247125634d9a430904e2914977ee98e6de1e2abf0ba6bf", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+                         "source_sha256": "3d5258c6b04f9947025a532a207321072f8a0a86abba6952293d4b7b17921c75", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
     "fp32_mid_long_k": {"bytes": 3.12e8, "counters": "FETCH_SIZE 147 817 x 2.0 KiB + WRITE_SIZE 9 226 KiB (operands, and the slots of the 64 tiles that are split in four; 256 tiles are whole)",
                         "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                        "source_sha256": "fc144dd4f6024eaeaa247125634d9a430904e2914977ee98e6de1e2abf0ba6bf", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
+                        "source_sha256": "3d5258c6b04f9947025a532a207321072f8a0a86abba6952293d4b7b17921c75", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
     "fp32_gemv": {"bytes": 2.70e8, "counters": "FETCH_SIZE (131 258 + 522) x 2.0 KiB + WRITE_SIZE (256 + 32) KiB: matrix-vector kernel + the copy of x",
                   "kernel": "gemv_kernel<float, float, 2, 1>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "5cccc9d00320d0a2a62939fdf04484d79a04bf8a1533b3757ed0ef48c1a66532", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "f9881524ceb3a6641140288364cd04af404cc4af5f2621b325a961744ac47258", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp32_gevm": {"bytes": 2.69e8, "counters": "FETCH_SIZE 131 233 x 2.0 KiB + WRITE_SIZE 32 KiB",
                   "kernel": "gevm_kernel<float, float, 8>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "5cccc9d00320d0a2a62939fdf04484d79a04bf8a1533b3757ed0ef48c1a66532", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "f9881524ceb3a6641140288364cd04af404cc4af5f2621b325a961744ac47258", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp16_gemv": {"bytes": 1.36e8, "counters": "FETCH_SIZE (65 647 + 522) x 2.0 KiB + WRITE_SIZE (256 + 16) KiB: matrix-vector kernel + the copy of x",
                   "kernel": "gemv_kernel<_Float16, _Float16, 2, 1>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "5cccc9d00320d0a2a62939fdf04484d79a04bf8a1533b3757ed0ef48c1a66532", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "f9881524ceb3a6641140288364cd04af404cc4af5f2621b325a961744ac47258", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp16_gevm": {"bytes": 1.35e8, "counters": "FETCH_SIZE 65 685 x 2.0 KiB + WRITE_SIZE 92 KiB",
                   "kernel": "gevm_kernel<_Float16, _Float16, 8>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "5cccc9d00320d0a2a62939fdf04484d79a04bf8a1533b3757ed0ef48c1a66532", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "f9881524ceb3a6641140288364cd04af404cc4af5f2621b325a961744ac47258", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "conv2d": {"bytes": 1.08e8, "counters": "FETCH_SIZE 20 595 x 2.0 KiB + WRITE_SIZE 64 528 KiB",
                "kernel": "gemm_f32_dma_kernel<256, 256, 2, 4, 16, 4, false, 2, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-               "source_sha256": "fc144dd4f6024eaeaa247125634d9a430904e2914977ee98e6de1e2abf0ba6bf", "profile": "profiles/conv2d_implicit_gemm_256x256x112_3x3x256.md"},
+               "source_sha256": "3d5258c6b04f9947025a532a207321072f8a0a86abba6952293d4b7b17921c75", "profile": "profiles/conv2d_implicit_gemm_256x256x112_3x3x256.md"},
     "conv2d_rgb": {"bytes": 1.01e8, "counters": "FETCH_SIZE 16 457 x 2.0 KiB + WRITE_SIZE 66 130 KiB",
                    "kernel": "conv2d_direct_kernel<8, 3>", "source": "decx_amd/csrc/conv_direct.hip",
-                   "source_sha256": "743f8085e23b35e155b1707c1bdef9b228656d9b2d166446d7aec6af9d3c37e7", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
+                   "source_sha256": "84ef56bdb16515a688bf81f1e7616863ba4917ab9f569a9353d866eeee6872e4", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
 }
 
 

@@ -187,10 +187,12 @@ __host__ inline TileInfo tile_info_f64(int shape)
 int launch_gemm_f32(int shape, bool edge, const GemmArgs& args, hipStream_t stream);
 // fp64: direct-to-LDS kernels on 16-byte aligned operands, else (or with `plain`) a one-thread-per-element kernel
 // The direct-load kernels address a slab as scalar base + 32-bit lane offset: 256 rows of A and 64 rows
-// of B must span less than 2 GiB (any realistic pitch does; otherwise the register-staged kernels run).
+// of B must span less than 2 GiB (any realistic pitch does; otherwise the register-staged kernels run).  The fp32
+// epilogue addresses D and C the same way, with a lane offset of up to 4 rows and a row of the tile.
 inline bool dma_offsets_fit(const GemmArgs& g, uint32_t elem_bytes)
 {
-    return 256ull * g.lda * elem_bytes < (1ull << 31) && 64ull * g.ldb * elem_bytes + 16ull < (1ull << 31);
+    return 256ull * g.lda * elem_bytes < (1ull << 31) && 64ull * g.ldb * elem_bytes + 16ull < (1ull << 31) &&
+           8ull * g.ldd * elem_bytes < (1ull << 31) && (!g.C || 8ull * g.ldc * elem_bytes < (1ull << 31));
 }
 
 int launch_gemm_f64(int shape, bool plain, const GemmArgs& args, hipStream_t stream);
