@@ -37,30 +37,30 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
 # file of the kernel it was measured on with that file's SHA-256 at the time: when the kernel source has changed
 # since, the figure is withheld ("traffic": null, "traffic_stale": true) until the workload is profiled again.
 MEASURED_TRAFFIC = {
-    "fp32_8192": {"bytes": 5.67e9, "counters": "FETCH_SIZE 2.6383e6 x 2.0 KiB + WRITE_SIZE 2.621e5 KiB (FETCH_SIZE 2.64e6 ... 3.40e6 from run to run)",
+    "fp32_8192": {"bytes": 5.67e9, "counters": "FETCH_SIZE 2.6361e6 x 2.0 KiB + WRITE_SIZE 2.621e5 KiB (FETCH_SIZE 2.64e6 ... 3.40e6 from run to run)",
                   "kernel": "gemm_f32_dma_kernel<256, 128, 2, 2, 16, 2, false, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                  "source_sha256": "3d5258c6b04f9947025a532a207321072f8a0a86abba6952293d4b7b17921c75", "profile": "profiles/gemm_f32_dma_fp32_8192cubed.md"},
-    "fp16_4096": {"bytes": 2.35e8, "counters": "FETCH_SIZE 98 543 x 2.0 KiB + WRITE_SIZE 32 778 KiB",
+                  "source_sha256": "76fb449e905c676f571eeadb730abe3ca3c578d0851a8ba3d400b84d9dac7646", "profile": "profiles/gemm_f32_dma_fp32_8192cubed.md"},
+    "fp16_4096": {"bytes": 2.35e8, "counters": "FETCH_SIZE 98 543 x 2.0 KiB + WRITE_SIZE 32 772 KiB",
                   "kernel": "gemm_f16_dma_kernel<256, 256, 2, 4, 64, 2, false>", "source": "decx_amd/csrc/gemm_f16_dma.hip",
-                  "source_sha256": "8fe2bf39af426d7dd5e58cb40eacf4f3cbcc1192a266f8b5a923330679cec043", "profile": "profiles/gemm_f16_dma_fp16_4096cubed.md"},
-    "fp64_4096": {"bytes": 1.21e9, "counters": "FETCH_SIZE 524 460 x 2.0 KiB + WRITE_SIZE 131 106 KiB",
+                  "source_sha256": "01ecb755392386c03aae0f5c0f2b46e2726495319ab46b6fdf98e9d4d8ca4dbe", "profile": "profiles/gemm_f16_dma_fp16_4096cubed.md"},
+    "fp64_4096": {"bytes": 1.21e9, "counters": "FETCH_SIZE 524 460 x 2.0 KiB + WRITE_SIZE 131 099 KiB",
                   "kernel": "gemm_f64_dma_kernel<256, 128, 4, 2, 16, 3, false>", "source": "decx_amd/csrc/gemm_f64.hip",
-                  "source_sha256": "b21c941385a6d73c7134f9f30ee5cf1ac1453522fda2b4a09e36683088de5226", "profile": "profiles/gemm_f64_dma_fp64_4096cubed.md"},
-    "fp32_1024": {"bytes": 2.95e7, "counters": "FETCH_SIZE 12 342 x 2.0 KiB + WRITE_SIZE 4 096 KiB",
+                  "source_sha256": "a35256187572bedc339c2dec0b155b1a87bc39fb226006a00774161acea7cdf0", "profile": "profiles/gemm_f64_dma_fp64_4096cubed.md"},
+    "fp32_1024": {"bytes": 2.95e7, "counters": "FETCH_SIZE 12 335 x 2.0 KiB + WRITE_SIZE 4 096 KiB",
                   "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                  "source_sha256": "3d5258c6b04f9947025a532a207321072f8a0a86abba6952293d4b7b17921c75", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
-    "fp32_ragged": {"bytes": 4.44e7, "counters": "FETCH_SIZE 16 663 x 2.0 KiB + WRITE_SIZE 9 983 KiB (operands, and the slots of the 128 tiles that are split in two; 256 tiles are whole)",
+                  "source_sha256": "76fb449e905c676f571eeadb730abe3ca3c578d0851a8ba3d400b84d9dac7646", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+    "fp32_ragged": {"bytes": 4.44e7, "counters": "FETCH_SIZE 16 659 x 2.0 KiB + WRITE_SIZE 9 983 KiB (operands, and the slots of the 128 tiles that are split in two; 256 tiles are whole)",
                     "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                    "source_sha256": "3d5258c6b04f9947025a532a207321072f8a0a86abba6952293d4b7b17921c75", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
-    "fp32_ragged_abc": {"bytes": 5.04e7, "counters": "FETCH_SIZE 19 604 x 2.0 KiB + WRITE_SIZE 9 983 KiB",
+                    "source_sha256": "76fb449e905c676f571eeadb730abe3ca3c578d0851a8ba3d400b84d9dac7646", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+    "fp32_ragged_abc": {"bytes": 5.04e7, "counters": "FETCH_SIZE 19 601 x 2.0 KiB + WRITE_SIZE 9 983 KiB",
                         "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, true>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                        "source_sha256": "3d5258c6b04f9947025a532a207321072f8a0a86abba6952293d4b7b17921c75", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
-    "fp32_tall_skinny": {"bytes": 3.58e8, "counters": "FETCH_SIZE 142 267 x 2.0 KiB + WRITE_SIZE 65 536 KiB",
+                        "source_sha256": "76fb449e905c676f571eeadb730abe3ca3c578d0851a8ba3d400b84d9dac7646", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+    "fp32_tall_skinny": {"bytes": 3.58e8, "counters": "FETCH_SIZE 141 987 x 2.0 KiB + WRITE_SIZE 65 536 KiB",
                          "kernel": "gemm_f32_dma_kernel<256, 128, 2, 2, 16, 2, false, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                         "source_sha256": "3d5258c6b04f9947025a532a207321072f8a0a86abba6952293d4b7b17921c75", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
-    "fp32_mid_long_k": {"bytes": 3.12e8, "counters": "FETCH_SIZE 147 817 x 2.0 KiB + WRITE_SIZE 9 226 KiB (operands, and the slots of the 64 tiles that are split in four; 256 tiles are whole)",
+                         "source_sha256": "76fb449e905c676f571eeadb730abe3ca3c578d0851a8ba3d400b84d9dac7646", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+    "fp32_mid_long_k": {"bytes": 3.12e8, "counters": "FETCH_SIZE 147 752 x 2.0 KiB + WRITE_SIZE 9 226 KiB (operands, and the slots of the 64 tiles that are split in four; 256 tiles are whole)",
                         "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                        "source_sha256": "3d5258c6b04f9947025a532a207321072f8a0a86abba6952293d4b7b17921c75", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
+                        "source_sha256": "76fb449e905c676f571eeadb730abe3ca3c578d0851a8ba3d400b84d9dac7646", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
     "fp32_gemv": {"bytes": 2.70e8, "counters": "FETCH_SIZE (131 258 + 522) x 2.0 KiB + WRITE_SIZE (256 + 32) KiB: matrix-vector kernel + the copy of x",
                   "kernel": "gemv_kernel<float, float, 2, 1>", "source": "decx_amd/csrc/gemv.hip",
                   "source_sha256": "f9881524ceb3a6641140288364cd04af404cc4af5f2621b325a961744ac47258", "profile": "profiles/gemv_gevm_8192x8192.md"},
@@ -73,9 +73,9 @@ MEASURED_TRAFFIC = {
     "fp16_gevm": {"bytes": 1.35e8, "counters": "FETCH_SIZE 65 685 x 2.0 KiB + WRITE_SIZE 92 KiB",
                   "kernel": "gevm_kernel<_Float16, _Float16, 8>", "source": "decx_amd/csrc/gemv.hip",
                   "source_sha256": "f9881524ceb3a6641140288364cd04af404cc4af5f2621b325a961744ac47258", "profile": "profiles/gemv_gevm_8192x8192.md"},
-    "conv2d": {"bytes": 1.08e8, "counters": "FETCH_SIZE 20 595 x 2.0 KiB + WRITE_SIZE 64 528 KiB",
+    "conv2d": {"bytes": 1.08e8, "counters": "FETCH_SIZE 20 512 x 2.0 KiB + WRITE_SIZE 64 559 KiB",
                "kernel": "gemm_f32_dma_kernel<256, 256, 2, 4, 16, 4, false, 2, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-               "source_sha256": "3d5258c6b04f9947025a532a207321072f8a0a86abba6952293d4b7b17921c75", "profile": "profiles/conv2d_implicit_gemm_256x256x112_3x3x256.md"},
+               "source_sha256": "76fb449e905c676f571eeadb730abe3ca3c578d0851a8ba3d400b84d9dac7646", "profile": "profiles/conv2d_implicit_gemm_256x256x112_3x3x256.md"},
     "conv2d_rgb": {"bytes": 1.01e8, "counters": "FETCH_SIZE 16 457 x 2.0 KiB + WRITE_SIZE 66 130 KiB",
                    "kernel": "conv2d_direct_kernel<8, 3>", "source": "decx_amd/csrc/conv_direct.hip",
                    "source_sha256": "84ef56bdb16515a688bf81f1e7616863ba4917ab9f569a9353d866eeee6872e4", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},

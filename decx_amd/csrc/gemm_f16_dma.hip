@@ -82,6 +82,7 @@ template <int MFMAS, int READS> __device__ __forceinline__ void interleave()
 // partial products and rounds once (split_k_exchange).
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool SPLIT = false>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
+__attribute__((amdgpu_waves_per_eu((BM * BN >= 256 * 256 || STAGES > 2) ? 2 : 4)))     // as scheduled: one 256 x 256 workgroup per CU, two of 128 x 128, four of 64 x 64 (rings of 2 stages)
 gemm_f16_dma_kernel(const GemmArgs g_in)
 {
     struct Nothing {};

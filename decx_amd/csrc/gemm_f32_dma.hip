@@ -74,7 +74,12 @@ template <int TN> __device__ __forceinline__ float lane_of(const typename BFrag<
 // every workgroup stores its accumulators to its slot and counts itself in at the tile's counter; the last one to
 // arrive adds the slots in range order and runs the epilogue.  No workgroup waits for another.
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool CHUNK_AHEAD, int CONV = 0, bool SPLIT = false, bool SPLIT_WITH_C = false>
+// The wavefronts per SIMD every tile is scheduled for (two workgroups of the largest tile per CU, three of 128 x 128, four of
+// the smaller ones) are told to the compiler: it then keeps the accumulators in the unified register file's VGPR half and
+// fits the epilogue below into the budget, where its own choice was 142 VGPRs beside 128 accumulation registers (one
+// workgroup of the 256 x 128 tile per CU) for any epilogue that keeps loads in flight across rows.
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
+__attribute__((amdgpu_waves_per_eu(BM * BN >= 256 * 128 ? 2 : BM * BN >= 128 * 128 ? 3 : 4)))
 gemm_f32_dma_kernel(const GemmArgs g_in)
 {
     struct Nothing {};
@@ -500,8 +505,8 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
         if constexpr (CONV != 0) return (size_t)(row / g.conv_wout) * g.conv_dst_row + (size_t)(row % g.conv_wout) * g.ldd;
         else return (size_t)row * g.ldd;
     };
-    constexpr bool STRAIGHT = TM * TN < 8;     // (the 256 x 128 tile keeps the row-by-row form below: 142 VGPRs otherwise, one workgroup per CU)
-    // (the 128 x 128 tile takes it with a C only: without one it gains nothing there, and edge shapes lose 2 %)
+    constexpr bool STRAIGHT = true;
+    // (the 128 x 128 and 256 x 128 tiles take it with a C only: without one it gains nothing there, and edge shapes lose 2 %)
     if (STRAIGHT && interior && (TM * TN == 1 || (!C_EARLY && C != nullptr))) {
         // Straight-line code: with a C, the loads of a batch of rows are all asked for before the first is used (a load,
         // its wait, the fma and the store row by row made the C term cost 6 % at 2048^3 and 14 % at 65536 x 256 x 1024).
@@ -616,8 +621,7 @@ gemm_f32_dma_kernel(const GemmArgs g_in)
         };
         if (!C_EARLY && C != nullptr) { store_edge(std::true_type{}); return; }
     }
-    // the largest tile: interior tiles row by row; edge tiles without a C to fetch, element by element (one store wherever
-    // the lane's TN columns all exist: 141 VGPRs in place of 64)
+    // without a C to fetch: the interior tiles of the two larger tiles row by row, edge tiles element by element
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll

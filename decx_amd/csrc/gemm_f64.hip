@@ -42,6 +42,7 @@ template <int N> __device__ __forceinline__ void wait_loads_and_barrier()
 // partial products (split_k_exchange).
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool SPLIT = false>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
+__attribute__((amdgpu_waves_per_eu(BM * BN >= 128 * 128 ? 2 : 4)))     // as scheduled: one workgroup of 8 wavefronts per CU on the two larger tiles, two of 64 x 64
 gemm_f64_dma_kernel(const GemmArgs g_in)
 {
     struct Nothing {};
