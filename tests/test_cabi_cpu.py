@@ -105,6 +105,7 @@ def test_planner_choices():
     p = hip.plan(2, 1024, 1024, 6144)                      # 64 tiles of 128 x 128 on 4 ranges, one per CU: 29.6 -> 23.5 us
     assert (p.tile_m, p.k_splits) == (128, 4)
     assert hip.plan(2, 768, 768, 16384).k_splits == 6 and hip.plan(2, 2048, 2048, 8192).k_splits == 1
+    assert hip.plan(2, 4096, 512, 2048).k_splits == 1 and hip.plan(2, 896, 896, 4096).k_splits == 1    # on ranges: 20.7 and 18.3 us, whole 14.1 and 14.7
     p = hip.plan(2, 2560, 2048, 4096)                      # 320 tiles of 128 x 128: 256 whole + 64 on 4 ranges (52.5 us; all on 3 ranges 57.4)
     assert (p.tile_m, p.k_splits, p.whole_tiles) == (128, 4, 256)
     assert hip.plan(2, 3072, 2048, 8192).k_splits == 1     # 1.5 per CU, power-bound either way: whole 100.9 us, 4 ranges 115.3
