@@ -585,6 +585,37 @@ def test_c_may_alias_d(hip, oracle):
     assert rel_err(dD.download(), oracle.gemm_f32(A, B, C, 1.0, 1.0), K) <= TOL_F32
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.float64])
+@pytest.mark.parametrize("tile", [0, 1, 2])
+def test_c_term_on_interior_and_edge_tiles_of_every_tile(hip, oracle, dtype, tile):
+    """alpha A.B + beta C on an output that holds interior tiles, tiles on the right and lower edges and the corner tile of
+    every tile class, with C apart from D and with C = D (the epilogues ask for the C values of several rows ahead of
+    their use; every element is read before it is overwritten)."""
+    M, N, K = 650, 420, 130
+    f64 = dtype == np.float64
+    rng = np.random.default_rng(4242 + tile)
+    A = rng.uniform(-1, 1, (M, K)).astype(dtype); B = rng.uniform(-1, 1, (K, N)).astype(dtype); C = rng.uniform(-1, 1, (M, N)).astype(dtype)
+    ref = {np.float32: oracle.gemm_f32, np.float16: oracle.gemm_f16, np.float64: oracle.gemm_f64}[dtype](A, B, C, 0.75, -1.25)
+    tol = {np.float32: TOL_F32, np.float16: TOL_F16, np.float64: 1e-14}[dtype]
+    pk, pn = device_pitch(K, dtype), device_pitch(N, dtype)
+    dA = hip.DeviceMatrix(M, K, dtype, pk, A, pad_value=np.nan); dB = hip.DeviceMatrix(K, N, dtype, pn, B, pad_value=np.nan)
+    dC = hip.DeviceMatrix(M, N, dtype, pn, C, pad_value=np.nan)
+    for alias in (False, True):
+        dD = hip.DeviceMatrix(M, N, dtype, pn)
+        raw0 = np.full((M, pn), -12345.0, dtype)
+        if alias:
+            raw0[:, :N] = C
+        dD.upload_raw(raw0)
+        hip.gemm(dA, dB, dD, dD if alias else dC, 0.75, -1.25, tile=tile)
+        hip.sync()
+        raw = dD.download_raw()
+        dD.free()
+        assert np.all(raw[:, N:] == dtype(-12345.0)), "padding columns of D were written"
+        assert rel_err(raw[:, :N], ref, K) <= tol, alias
+    for d in (dA, dB, dC):
+        d.free()
+
+
 def test_empty_and_invalid_arguments(hip):
     L = hip.lib()
     d = hip.DeviceMatrix(4, 4, np.float32, data=np.ones((4, 4), np.float32))
