@@ -4,10 +4,14 @@
 #include "../../include/decx_hip_profiling.h"
 #include "gemm_common.hpp"
 #include "split_k_exchange.hpp"
+#include "split_counter_ring.hpp"
 
 #include <chrono>
 #include <cstring>
+#include <functional>
 #include <mutex>
+#include <thread>
+#include <vector>
 
 using namespace decx_hip;
 
@@ -33,23 +37,71 @@ void* g_scratch[kMaxDevices] = {};
 // Counters of the split-K kernels (per tile, or per column group of a vector x matrix product: one, plus one per group
 // of ranges when there are many; the workgroups of a tile count themselves in, the last one sums the tile and puts
 // the counter back to zero, so the array is all zero between launches).  Every launch takes the next window of the
-// array, so that launches in flight on different streams do not share counters as long as their windows together
-// stay below kSplitCounters.
+// array; a window only goes to a new launch once the launches that had it before are known to be over
+// (split_counter_ring.hpp: same stream, a completed event, or an idle stream), and a launch that cannot have one
+// runs unsplit.
 constexpr uint32_t kSplitCounters = 1u << 16;
 static __device__ uint32_t split_counters[kSplitCounters];
 uint32_t* g_split_counters[kMaxDevices] = {};
 std::mutex g_counter_mutex;
-uint32_t g_counter_cursor = 0;
 
-uint32_t* take_split_counters(uint32_t tiles)
+struct HipRingRuntime final : CounterRingRuntime {
+    std::vector<hipEvent_t> pool;
+    void* record_event(void* stream) override
+    {
+        hipEvent_t ev = nullptr;
+        if (!pool.empty()) { ev = pool.back(); pool.pop_back(); }
+        else if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+        if (hipEventRecord(ev, (hipStream_t)stream) != hipSuccess) { (void)hipGetLastError(); pool.push_back(ev); return nullptr; }
+        return ev;
+    }
+    bool event_done(void* event) override
+    {
+        const hipError_t e = hipEventQuery((hipEvent_t)event);
+        if (e != hipSuccess) (void)hipGetLastError();              // "not ready" is no error of the caller's
+        return e == hipSuccess;
+    }
+    void release_event(void* event) override { pool.push_back((hipEvent_t)event); }
+    bool stream_idle_or_gone(void* stream) override
+    {
+        const auto gone = [](hipError_t e) {
+            return e == hipErrorContextIsDestroyed || e == hipErrorInvalidHandle || e == hipErrorInvalidResourceHandle;
+        };
+        // (a stream that is recording a graph must not be queried: the query would end the recording with an error)
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        hipError_t e = hipStreamIsCapturing((hipStream_t)stream, &st);
+        if (e != hipSuccess) { (void)hipGetLastError(); return gone(e); }
+        if (st != hipStreamCaptureStatusNone) return false;
+        e = hipStreamQuery((hipStream_t)stream);
+        if (e != hipSuccess) (void)hipGetLastError();
+        return e == hipSuccess || gone(e);
+    }
+};
+HipRingRuntime g_ring_runtime;
+CounterRing* g_rings[kMaxDevices] = {};
+
+// A window of `n` counters for a launch on `stream`, or nullptr (run unsplit).  `ticket` goes to commit_split_counters()
+// right behind the launch.
+uint32_t* take_split_counters(uint32_t n, hipStream_t stream, uint64_t& ticket)
 {
-    uint32_t* const base = g_dev.device >= 0 && g_dev.device < kMaxDevices ? g_split_counters[g_dev.device] : nullptr;
-    if (!base || tiles > kSplitCounters) return nullptr;
+    ticket = 0;
+    const int d = g_dev.device;
+    if (d < 0 || d >= kMaxDevices || !g_split_counters[d] || !g_rings[d]) return nullptr;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &st) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    uint64_t key = (uint64_t)(uintptr_t)stream;
+    if (stream == hipStreamPerThread) key ^= (uint64_t)std::hash<std::thread::id>{}(std::this_thread::get_id()) << 8;
     std::lock_guard<std::mutex> lock(g_counter_mutex);
-    if (g_counter_cursor + tiles > kSplitCounters) g_counter_cursor = 0;
-    uint32_t* const window = base + g_counter_cursor;
-    g_counter_cursor += tiles;
-    return window;
+    const uint32_t at = g_rings[d]->take(g_ring_runtime, (void*)stream, key, n, st != hipStreamCaptureStatusNone, &ticket);
+    return at == CounterRing::kNone ? nullptr : g_split_counters[d] + at;
+}
+
+void commit_split_counters(uint64_t ticket)
+{
+    if (!ticket) return;
+    const int d = g_dev.device;
+    std::lock_guard<std::mutex> lock(g_counter_mutex);
+    if (d >= 0 && d < kMaxDevices && g_rings[d]) g_rings[d]->commit(g_ring_runtime, ticket);
 }
 
 inline int hip_rc(hipError_t e) { return (int)e; }
@@ -277,15 +329,17 @@ size_t split_workspace_bytes(int elem_bytes, const SplitChoice& sp, uint32_t M, 
 
 // Fills the split fields of g when the plan says so, the workspace is large enough and the tiles have counters; returns
 // the number of splits and, with more than one, the tile shape they run on.
-uint32_t arm_split(GemmArgs& g, int elem_bytes, void* workspace, size_t workspace_bytes, int& shape)
+uint32_t arm_split(GemmArgs& g, int elem_bytes, void* workspace, size_t workspace_bytes, int& shape, hipStream_t stream,
+                   uint64_t& ticket)
 {
+    ticket = 0;
     if (!workspace || !aligned16(workspace)) return 1;
     const SplitChoice sp = split_plan(elem_bytes, g.M, g.N, g.K);
     if (sp.splits <= 1 || workspace_bytes < split_workspace_bytes(elem_bytes, sp, g.M, g.N)) return 1;
     const TileInfo ti = dma_tile_info(elem_bytes, sp.shape, g.N);
     const uint64_t tiles = (uint64_t)((g.M + ti.bm - 1) / ti.bm) * ((g.N + ti.bn - 1) / ti.bn);
     const uint64_t n_counters = (tiles - sp.first) * split_counters_per_tile(sp.splits);
-    uint32_t* const counters = n_counters <= kSplitCounters ? take_split_counters((uint32_t)n_counters) : nullptr;
+    uint32_t* const counters = n_counters <= kSplitCounters ? take_split_counters((uint32_t)n_counters, stream, ticket) : nullptr;
     if (!counters) return 1;
     g.split_counters = counters;
     g.split_len = sp.len; g.split_count = sp.splits; g.split_first = sp.first; g.split_ws = workspace;
@@ -304,10 +358,14 @@ int gevm_maybe_split(bool f16, bool out_f32, const void* x, const void* B, const
     const uint32_t ldw = (N + 3) / 4 * 4;
     if (sp.splits > 1 && workspace && aligned16(workspace) && workspace_bytes >= (size_t)sp.splits * ldw * 4) {
         const uint32_t groups = (N + (f16 ? 64u : 32u) - 1) / (f16 ? 64u : 32u);
-        uint32_t* const counters = take_split_counters(groups);         // the last workgroup of a column group adds its ranges
-        if (counters)
-            return launch_gevm(f16, out_f32, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream, sp.len, (float*)workspace, ldw,
-                               counters);
+        uint64_t ticket;
+        uint32_t* const counters = take_split_counters(groups, stream, ticket);     // the last workgroup of a column group adds its ranges
+        if (counters) {
+            const int rc = launch_gevm(f16, out_f32, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream, sp.len, (float*)workspace, ldw,
+                                       counters);
+            commit_split_counters(ticket);
+            return rc;
+        }
     }
     return launch_gevm(f16, out_f32, x, B, c, y, K, N, ldb, incx, incc, incy, alpha, beta, stream);
 }
@@ -347,17 +405,76 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
                 lda % per16 == 0 && ldb % per16 == 0 && ldd % per16 == 0 && (!C || ldc % per16 == 0)) ? 1u : 0u;
     int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile(F16, M, N, g.vec_ok != 0) : tile;
     const bool edge = force_edge != 0 || K == 0;
+    uint64_t ticket = 0;
     if (workspace && tile == DECX_HIP_TILE_AUTO && !edge && g.vec_ok && dma_offsets_fit(g, F16 ? 2 : 4)) {
-        arm_split(g, F16 ? 2 : 4, workspace, workspace_bytes, shape);    // with ranges, the last workgroup of a tile sums them
+        arm_split(g, F16 ? 2 : 4, workspace, workspace_bytes, shape, as_stream(stream), ticket);    // with ranges, the last workgroup of a tile sums them
     }
-    return F16 ? launch_gemm_f16(shape, edge, g, as_stream(stream))
-               : launch_gemm_f32(shape, edge, g, as_stream(stream));
+    const int launched = F16 ? launch_gemm_f16(shape, edge, g, as_stream(stream))
+                             : launch_gemm_f32(shape, edge, g, as_stream(stream));
+    commit_split_counters(ticket);
+    return launched;
 }
 
 __global__ void __launch_bounds__(256) calibration_copy_kernel(uintx4* __restrict__ dst,
                                                               const uintx4* __restrict__ src, size_t n16)
 {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+}
+
+// Register-only matrix-core loops: what the matrix pipe sustains on this board with nothing else to do -- no loads,
+// no LDS, no barriers -- on operands of the caller's choosing (their values set the power drawn, and with it the
+// clock the board's power management allows).  8 wavefronts per CU, two per SIMD, the accumulator layouts of the
+// largest GEMM tiles: F16 sixteen 16x16x32 tiles (a 64 x 64 wave tile, 4 x 4 operand fragments), fp32 eight 32x32x2
+// tiles (128 x 64, 4 x 2 fragments that change every step as in a k loop).
+template <bool F16>
+__global__ void __launch_bounds__(512) calibration_mfma_kernel(const uintx4* __restrict__ operands, size_t n16, float* __restrict__ sink,
+                                                              uint32_t iters)
+{
+    const size_t at = ((size_t)blockIdx.x * 512 + threadIdx.x) * 8;
+    uintx4 raw[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) raw[i] = operands[(at + i) % n16];
+    float s = 0.f;
+    if constexpr (F16) {
+        halfx8 a[4], b[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { a[i] = __builtin_bit_cast(halfx8, raw[i]); b[i] = __builtin_bit_cast(halfx8, raw[4 + i]); }
+        floatx4 acc[4][4] = {};
+        for (uint32_t it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[j], a[i], acc[j][i], 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s += acc[j][i][0] + acc[j][i][1] + acc[j][i][2] + acc[j][i][3];
+    } else {
+        float v[32];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const floatx4 f = __builtin_bit_cast(floatx4, raw[i]);
+            v[4 * i] = f[0]; v[4 * i + 1] = f[1]; v[4 * i + 2] = f[2]; v[4 * i + 3] = f[3];
+        }
+        floatx16 acc[4][2] = {};
+        for (uint32_t it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(v[8 * k + i], v[8 * k + 4 + j], acc[i][j], 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s += acc[i][j][r];
+    }
+    sink[(size_t)blockIdx.x * 512 + threadIdx.x] = s;
 }
 
 // kmat[(kh * k_w + kw) * img_dpitch + ic][oc] = kernel oc at (kh, kw, ic); zero where ic >= depth or oc >= out_c
@@ -394,6 +511,26 @@ int decx_hip_calibration_copy(void* dst, const void* src, size_t bytes, void* st
     return (int)hipGetLastError();
 }
 
+int decx_hip_calibration_mfma(int elem_bytes, const void* operands, size_t operand_bytes, float* sink, size_t sink_floats,
+                              uint32_t iters, double* flops, void* stream)
+{
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    const uint32_t blocks = (uint32_t)g_dev.compute_units;
+    if ((elem_bytes != 2 && elem_bytes != 4) || !operands || operand_bytes < 16 || !aligned16(operands) || !sink ||
+        sink_floats < (size_t)blocks * 512)
+        return DECX_HIP_E_INVALID_ARG;
+    // per wavefront and iteration: 16 tiles of 16 x 16 x 32, or 4 steps of 8 tiles of 32 x 32 x 2
+    const double per_wave = elem_bytes == 2 ? 16.0 * 2 * 16 * 16 * 32 : 32.0 * 2 * 32 * 32 * 2;
+    if (flops) *flops = (double)blocks * 8.0 * (double)iters * per_wave;
+    if (elem_bytes == 2)
+        hipLaunchKernelGGL(calibration_mfma_kernel<true>, dim3(blocks), dim3(512), 0, as_stream(stream), (const uintx4*)operands,
+                           operand_bytes / 16, sink, iters);
+    else
+        hipLaunchKernelGGL(calibration_mfma_kernel<false>, dim3(blocks), dim3(512), 0, as_stream(stream), (const uintx4*)operands,
+                           operand_bytes / 16, sink, iters);
+    return (int)hipGetLastError();
+}
+
 int decx_hip_init(int device)
 {
     int count = 0;
@@ -411,6 +548,8 @@ int decx_hip_init(int device)
         void* p = nullptr;
         if ((e = hipGetSymbolAddress(&p, HIP_SYMBOL(split_counters))) != hipSuccess) return hip_rc(e);
         g_split_counters[device] = (uint32_t*)p;
+        std::lock_guard<std::mutex> lock(g_counter_mutex);
+        if (!g_rings[device]) g_rings[device] = new CounterRing(kSplitCounters);
     }
     g_dev.device = device;
     g_dev.compute_units = g_dev.prop.multiProcessorCount > 0 ? g_dev.prop.multiProcessorCount : 256;
@@ -468,6 +607,13 @@ int decx_hip_memset_async(void* ptr, int value, size_t bytes, void* stream)
     if (!ptr && bytes) return DECX_HIP_E_INVALID_ARG;
     if (!bytes) return DECX_HIP_OK;
     return hip_rc(hipMemsetAsync(ptr, value, bytes, as_stream(stream)));
+}
+
+int decx_hip_mem_info(size_t* free_bytes, size_t* total_bytes)
+{
+    if (!free_bytes || !total_bytes) return DECX_HIP_E_INVALID_ARG;
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    return hip_rc(hipMemGetInfo(free_bytes, total_bytes));
 }
 
 int decx_hip_memcpy2d_async(void* dst, size_t dst_pitch, const void* src, size_t src_pitch,
@@ -563,10 +709,45 @@ int decx_hip_gemm_f32_static(const float* A, const float* B, const float* C, flo
                              uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, float alpha, float beta, void* stream)
 {
     if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
-    void* const ws = g_dev.device < kMaxDevices ? g_scratch[g_dev.device] : nullptr;
+    void* ws = g_dev.device < kMaxDevices ? g_scratch[g_dev.device] : nullptr;
     if (!ws) return DECX_HIP_E_NOT_INIT;
-    if (decx_hip_gemm_workspace(4, M, N, K) > kScratchBytes) return DECX_HIP_E_TOO_LARGE;
-    return run_gemm<false>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0, ws, kScratchBytes);
+    // What the workspace form would use for THESE operands.  A column operand that does not fit is read in place (the
+    // dense copy changes no sum); a split that does not fit is refused (unsplit, the sums would come in another order).
+    if (decx_hip_gemm_workspace(4, M, N, K) > kScratchBytes) {
+        GemmArgs g;
+        std::memset(&g, 0, sizeof g);
+        g.C = C; g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldd = ldd;
+        const bool can_split = K > 0 && aligned16(A) && aligned16(B) && aligned16(D) && (!C || aligned16(C)) && lda % 4 == 0 &&
+                               ldb % 4 == 0 && ldd % 4 == 0 && (!C || ldc % 4 == 0) && dma_offsets_fit(g, 4);
+        if (N != 1 && (M == 1 || can_split)) return DECX_HIP_E_TOO_LARGE;
+        ws = nullptr;
+    }
+    return run_gemm<false>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0, ws, ws ? kScratchBytes : 0);
+}
+
+int decx_hip_reset_split_counters(void)
+{
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    const int d = g_dev.device;
+    if (d < 0 || d >= kMaxDevices || !g_split_counters[d]) return DECX_HIP_E_NOT_INIT;
+    hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess) return hip_rc(e);
+    if ((e = hipMemset(g_split_counters[d], 0, sizeof(uint32_t) * kSplitCounters)) != hipSuccess) return hip_rc(e);
+    std::lock_guard<std::mutex> lock(g_counter_mutex);
+    if (g_rings[d]) g_rings[d]->reset(g_ring_runtime);
+    return DECX_HIP_OK;
+}
+
+int decx_hip_split_counter_stats(uint64_t out[6])
+{
+    if (!out) return DECX_HIP_E_INVALID_ARG;
+    const int d = g_dev.device;
+    std::lock_guard<std::mutex> lock(g_counter_mutex);
+    if (!g_dev.ready || d < 0 || d >= kMaxDevices || !g_rings[d]) return DECX_HIP_E_NOT_INIT;
+    const CounterRing::Stats& st = g_rings[d]->stats();
+    out[0] = st.taken; out[1] = st.wraps; out[2] = st.refused; out[3] = st.events; out[4] = st.reserved;
+    out[5] = g_rings[d]->ring_size();
+    return DECX_HIP_OK;
 }
 
 int decx_hip_gemm_f16_ws(const uint16_t* A, const uint16_t* B, const uint16_t* C, uint16_t* D, uint32_t M, uint32_t N,
@@ -605,10 +786,14 @@ static int run_gemm_f64(const double* A, const double* B, const double* C, doubl
         const SplitPlan sp = plan_gevm_split(8, N, K, g_dev.compute_units);
         const uint32_t ldw = (N + 3) / 4 * 4;
         if (sp.splits > 1 && workspace && aligned16(workspace) && workspace_bytes >= (size_t)sp.splits * ldw * 8) {
-            uint32_t* const counters = take_split_counters((N + 15) / 16);
-            if (counters)
-                return launch_gevm_f64(A, B, C, D, K, N, ldb, 1, 1, 1, alpha, beta, as_stream(stream), sp.len, (double*)workspace, ldw,
-                                       counters);
+            uint64_t ticket;
+            uint32_t* const counters = take_split_counters((N + 15) / 16, as_stream(stream), ticket);
+            if (counters) {
+                const int rc = launch_gevm_f64(A, B, C, D, K, N, ldb, 1, 1, 1, alpha, beta, as_stream(stream), sp.len, (double*)workspace, ldw,
+                                               counters);
+                commit_split_counters(ticket);
+                return rc;
+            }
         }
         return launch_gevm_f64(A, B, C, D, K, N, ldb, 1, 1, 1, alpha, beta, as_stream(stream));
     }
@@ -624,10 +809,13 @@ static int run_gemm_f64(const double* A, const double* B, const double* C, doubl
     g.vec_ok = (aligned16(A) && aligned16(B) && aligned16(D) && (!C || aligned16(C)) &&
                 lda % 2 == 0 && ldb % 2 == 0 && ldd % 2 == 0 && (!C || ldc % 2 == 0)) ? 1u : 0u;
     int shape = (tile == DECX_HIP_TILE_AUTO) ? choose_tile_f64(M, N) : tile;
+    uint64_t ticket = 0;
     if (workspace && tile == DECX_HIP_TILE_AUTO && !force_plain && K > 0 && g.vec_ok && dma_offsets_fit(g, 8)) {
-        arm_split(g, 8, workspace, workspace_bytes, shape);
+        arm_split(g, 8, workspace, workspace_bytes, shape, as_stream(stream), ticket);
     }
-    return launch_gemm_f64(shape, force_plain != 0, g, as_stream(stream));
+    const int launched = launch_gemm_f64(shape, force_plain != 0, g, as_stream(stream));
+    commit_split_counters(ticket);
+    return launched;
 }
 
 int decx_hip_gemm_f64(const double* A, const double* B, const double* C, double* D, uint32_t M, uint32_t N, uint32_t K,

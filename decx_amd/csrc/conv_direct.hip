@@ -72,8 +72,8 @@ conv2d_direct_kernel(const float* __restrict__ image, const float* __restrict__ 
     }
     // The output is written once and is larger than L2: nontemporal stores, and whole cache lines per store instruction.
     // A lane's CHUNKS 16-byte pieces lie CHUNKS x 16 bytes from its neighbour's, so with two or more of them the wavefront
-    // first lays its 64 pixels out in LDS as they lie in memory (no barrier: the region is the wavefront's own, and a
-    // wavefront's LDS operations complete in order) and lane l then stores piece 64 i + l of the wavefront in its i-th
+    // first lays its 64 pixels out in LDS as they lie in memory (no workgroup barrier: the region is the wavefront's own, a
+    // wavefront's LDS operations complete in order, and a wavefront-scope fence keeps the compiler from reordering them) and lane l then stores piece 64 i + l of the wavefront in its i-th
     // store, at the offset that piece's pixel left in LDS.  1920 x 1080 x 3, 8 kernels of 3 x 3: 24.3 -> 22.9 us,
     // 3840 x 2160: 124.5 -> 84.2, 640 x 480: 7.0 -> 5.7; 16 kernels: 47.6 -> 37.3; 1000 x 700, 32 kernels: 39.1 -> 24.7.
     // (Nontemporal stores of the lanes' own pieces, half a line per instruction: 28.8 us for 8 kernels, 160 for 16.)
@@ -88,6 +88,10 @@ conv2d_direct_kernel(const float* __restrict__ image, const float* __restrict__ 
 #pragma unroll
             for (int c = 0; c < CHUNKS; ++c) *(floatx4*)(mine + 4 * c) = floatx4{acc[4 * c], acc[4 * c + 1], acc[4 * c + 2], acc[4 * c + 3]};
             offs[threadIdx.x] = live ? my_off : ~0ull;
+            // the other lanes of the wavefront read these back: writes first, for the compiler as well
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
             for (int i = 0; i < CHUNKS; ++i) {
                 const uint32_t j = (uint32_t)i * 64u + lane, px = j / (uint32_t)CHUNKS, c = j % (uint32_t)CHUNKS;

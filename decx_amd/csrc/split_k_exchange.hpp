@@ -83,7 +83,12 @@ __device__ __forceinline__ bool split_k_exchange(const GemmArgs& g, const SplitB
         __syncthreads();                                   // the flag may be written again
         return last;
     };
-    // accumulators = slot first + slot (first + step) + ... (count of them), in that order
+    // accumulators = slot first + slot (first + step) + ... (count of them), in that order.  The loads are buffer loads
+    // the compiler knows as loads (it places the waits, and no copy of a destination register can slip in between a
+    // load and its wait, as it could with loads written as inline assembly): the tile's slots are the buffer, a lane's
+    // offset is its own 16 bytes and the slot and piece go into the scalar offset.
+    const __amdgpu_buffer_rsrc_t slot_buffer = __builtin_amdgcn_make_buffer_rsrc((void*)slots, 0, 0x7fffffff, 0x00020000);
+    constexpr int kDeviceScope = 16;                       // the sc1 bit of a gfx950 load
     const auto sum_slots = [&](uint32_t first, uint32_t count, uint32_t step) {
         static_for<0, PIECES / GROUP>([&](auto gc) {
             constexpr int c0 = decltype(gc)::value * GROUP;
@@ -92,20 +97,16 @@ __device__ __forceinline__ bool split_k_exchange(const GemmArgs& g, const SplitB
 #pragma unroll
                 for (int ib = 0; ib < BATCH; ++ib) {
                     if (ib == 0 || i0 + ib < count) {      // slots beyond the last are neither loaded nor added
-                        const V* const p = slots + (size_t)(first + (i0 + ib) * step) * SLOT;
+                        const uint32_t slot_bytes = (first + (i0 + ib) * step) * (uint32_t)(SLOT * 16);
 #pragma unroll
-                        for (int c = 0; c < GROUP; ++c) {
-                            const V* const src = p + (size_t)(c0 + c) * NT + t;
-                            asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[ib][c]) : "v"(src) : "memory");
-                        }
+                        for (int c = 0; c < GROUP; ++c)
+                            v[ib][c] = __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b128(
+                                slot_buffer, (uint32_t)t * 16u, slot_bytes + (uint32_t)((c0 + c) * NT * 16), kDeviceScope));
                     }
                 }
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
                 for (int ib = 0; ib < BATCH; ++ib) {
                     if (ib == 0 || i0 + ib < count) {
-#pragma unroll
-                        for (int c = 0; c < GROUP; ++c) asm volatile("" : "+v"(v[ib][c]));     // not before the wait above
                         static_for<0, GROUP>([&](auto cc) {
                             constexpr int c = decltype(cc)::value;
                             put(std::integral_constant<int, c0 + c>{}, v[ib][c], i0 + ib == 0);

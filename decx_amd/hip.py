@@ -40,6 +40,9 @@ SYMBOLS = {
     "decx_hip_host_malloc": (_int, [ctypes.POINTER(_vp), _sz]),
     "decx_hip_host_free": (_int, [_vp]),
     "decx_hip_memset_async": (_int, [_vp, _int, _sz, _vp]),
+    "decx_hip_mem_info": (_int, [ctypes.POINTER(_sz), ctypes.POINTER(_sz)]),
+    "decx_hip_reset_split_counters": (_int, []),
+    "decx_hip_split_counter_stats": (_int, [ctypes.POINTER(ctypes.c_uint64)]),
     "decx_hip_memcpy2d_async": (_int, [_vp, _sz, _vp, _sz, _sz, _sz, _int, _vp]),
     "decx_hip_stream_create": (_int, [ctypes.POINTER(_vp)]),
     "decx_hip_stream_destroy": (_int, [_vp]),
@@ -76,6 +79,7 @@ SYMBOLS = {
     "decx_hip_gemm_f16_tile": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, _int, _int]),
     "decx_hip_gemm_plan": (_int, [_int, _u32, _u32, _u32, _int, ctypes.POINTER(Plan)]),
     "decx_hip_calibration_copy": (_int, [_vp, _vp, _sz, _vp]),
+    "decx_hip_calibration_mfma": (_int, [_int, _vp, _sz, _vp, _sz, _u32, ctypes.POINTER(ctypes.c_double), _vp]),
     "decx_hip_float_to_half": (ctypes.c_uint16, [_f]),
     "decx_hip_half_to_float": (_f, [ctypes.c_uint16]),
 }
@@ -317,6 +321,35 @@ def conv2d(image, kernels, stride_x=1, stride_y=1, extend=False, stream=None, pa
     for d in (d_img, d_ker, d_kmat, d_out):
         d.free()
     return out_raw[:oh, :ow, :OC].copy(), out_raw
+
+
+def mem_free_bytes():
+    """Free device memory as the runtime reports it."""
+    free, total = _sz(), _sz()
+    check(lib().decx_hip_mem_info(ctypes.byref(free), ctypes.byref(total)), "mem info")
+    return free.value
+
+
+def split_counter_stats():
+    """{"taken", "wraps", "refused", "events", "reserved", "ring"}: what the split-K counter windows have seen so far."""
+    out = (ctypes.c_uint64 * 6)()
+    check(lib().decx_hip_split_counter_stats(out), "split counter stats")
+    return dict(zip(("taken", "wraps", "refused", "events", "reserved", "ring"), (int(v) for v in out)))
+
+
+class Stream:
+    def __init__(self):
+        init()
+        self.handle = _vp()
+        check(lib().decx_hip_stream_create(ctypes.byref(self.handle)), "stream create")
+
+    def sync(self):
+        check(lib().decx_hip_stream_sync(self.handle), "stream sync")
+
+    def destroy(self):
+        if self.handle is not None:
+            check(lib().decx_hip_stream_destroy(self.handle), "stream destroy")
+            self.handle = None
 
 
 def sync(stream=None):

@@ -89,6 +89,8 @@ DECX_HIP_API int decx_hip_free(void* ptr);
 DECX_HIP_API int decx_hip_host_malloc(void** ptr, size_t bytes);     /* pinned host memory */
 DECX_HIP_API int decx_hip_host_free(void* ptr);
 DECX_HIP_API int decx_hip_memset_async(void* ptr, int value, size_t bytes, void* stream);
+/* free and total device memory in bytes (hipMemGetInfo) */
+DECX_HIP_API int decx_hip_mem_info(size_t* free_bytes, size_t* total_bytes);
 
 /* kind: 0 host->device, 1 device->host, 2 device->device.  Pitches and width in BYTES.
  * Replaces the cudaMemcpy2DAsync calls of de::Memcpy
@@ -133,8 +135,17 @@ DECX_HIP_API int decx_hip_gemm_f32(const float* A, const float* B, const float* 
  * size where the copy pays.  For M == 1 with few columns and a long K (1 x 512 x 32768) ranges of K go to workgroups
  * of their own, their partial sums to the workspace, and the last of a column group adds them in range order (69 -> 23 us).
  * Plays the part of the scratch the reference's planner keeps for itself (cuda_GEMM_LS_planner: the transposed
- * A, srcs/modules/BLAS/GEMM/CUDA/large_squares/common/cuda_GEMM_LS_planner.cu:95-160). */
+ * A, srcs/modules/BLAS/GEMM/CUDA/large_squares/common/cuda_GEMM_LS_planner.cu:95-160).
+ * Besides the workspace, a split launch uses a window of the library's own counter array (65 536 words per GPU, all
+ * zero between launches).  The library hands a window to a new launch only when the launches that had it before are
+ * known to be over -- they went to the same stream, an event recorded behind them has completed, or their stream is
+ * idle -- and otherwise runs the product unsplit, which is never an error.  A split launch that is recorded into a
+ * HIP graph keeps its window for the life of the process (the graph may be replayed at any time): at most half of
+ * the array can go that way, later recordings run unsplit.  Callers must not destroy a stream while split launches
+ * are in flight on it.  If a launch was cut short (a device fault, a reset), decx_hip_reset_split_counters() waits
+ * for the device, puts every counter back to zero and forgets who owned what. */
 DECX_HIP_API size_t decx_hip_gemm_f32_workspace(uint32_t M, uint32_t N, uint32_t K);
+DECX_HIP_API int decx_hip_reset_split_counters(void);
 DECX_HIP_API int decx_hip_gemm_f32_ws(const float* A, const float* B, const float* C, float* D,
                                       uint32_t M, uint32_t N, uint32_t K,
                                       uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd,
@@ -145,8 +156,12 @@ DECX_HIP_API int decx_hip_gemm_f32_ws(const float* A, const float* B, const floa
  * looked up by decx_hip_init for that device).  It has no counterpart in the reference: it is for callers that
  * cannot allocate -- code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same
  * results as decx_hip_gemm_f32_ws with a workspace of decx_hip_gemm_f32_workspace(M, N, K) bytes, bit for bit.
- * Shapes whose workspace query exceeds DECX_HIP_STATIC_WORKSPACE_BYTES return DECX_HIP_E_TOO_LARGE and launch
- * nothing (decx_hip_gemm_f32 still takes them, unsplit).  All calls on one GPU share the one array, which keeps
+ * A product that decx_hip_gemm_f32_ws would split over more than DECX_HIP_STATIC_WORKSPACE_BYTES of partial
+ * products returns DECX_HIP_E_TOO_LARGE and launches nothing (decx_hip_gemm_f32 still takes it, unsplit).  Operands
+ * that the workspace form would not split anyway (not 16-byte aligned, K == 0) are not refused, and a column
+ * operand too long for the array (N == 1, K x 4 bytes beyond it) is read in place, which changes no sum.  A split
+ * launch also takes a window of the counter array described above: recorded into a graph, it keeps that window.
+ * All calls on one GPU share the one array, which keeps
  * the last call's contents (every call writes what it reads, nothing needs clearing): calls that overlap on one
  * GPU -- two streams, two threads -- race; serialise them. */
 #define DECX_HIP_STATIC_WORKSPACE_BYTES (16u << 20)

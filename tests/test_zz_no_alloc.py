@@ -28,12 +28,13 @@ def pitch32(cols):
     return (cols + 31) // 32 * 32
 
 
-def both(hip, M, N, K, seed, with_c, alpha=1.0, beta=1.0):
-    """(result of _static, result of _ws, host A, B, C) on NaN-padded device matrices of the reference's pitches."""
+def both(hip, M, N, K, seed, with_c, alpha=1.0, beta=1.0, offset_a=0):
+    """(result of _static, result of _ws, host A, B, C) on NaN-padded device matrices of the reference's pitches.
+    Device memory the runtime reports free must be the same before and after the _static call."""
     L = hip.lib()
     A = synth.uniform_f32(M, K, seed); B = synth.uniform_f32(K, N, seed + 1)
     C = synth.uniform_f32(M, N, seed + 2) if with_c else None
-    dA = hip.DeviceMatrix(M, K, np.float32, pitch32(K), A, pad_value=np.nan)
+    dA = hip.DeviceMatrix(M, K, np.float32, pitch32(K), A, pad_value=np.nan, offset_elems=offset_a)
     dB = hip.DeviceMatrix(K, N, np.float32, pitch32(N), B, pad_value=np.nan)
     dC = hip.DeviceMatrix(M, N, np.float32, pitch32(N), C, pad_value=np.nan) if with_c else None
     need = L.decx_hip_gemm_f32_workspace(M, N, K)
@@ -46,7 +47,11 @@ def both(hip, M, N, K, seed, with_c, alpha=1.0, beta=1.0):
                 dC.pitch if with_c else 0, dD.pitch, alpha, beta]
         print("no-alloc case", (M, N, K), "C" if with_c else "-", "static" if static else "ws", "need", need, flush=True)
         if static:
+            hip.sync()
+            free_before = hip.mem_free_bytes()
             rc = L.decx_hip_gemm_f32_static(*args, None)
+            hip.sync()
+            assert hip.mem_free_bytes() == free_before, "the call changed the amount of free device memory"
         else:
             rc = L.decx_hip_gemm_f32_ws(*args, ws.ptr, need, None)
         hip.check(rc, "gemm")
@@ -97,3 +102,26 @@ def test_static_workspace_rejects_what_does_not_fit(hip):
     assert np.all(dD.download_raw() == np.float32(3.5)), "a rejected call must launch nothing"
     for d in (dA, dB, dD):
         d.free()
+
+
+def test_static_workspace_takes_what_the_workspace_form_would_not_split(hip, oracle):
+    """Operands the workspace form would not split (a base that is not 16-byte aligned: the register-staged kernel
+    runs) are no business of the static array, however much the shape's query says: not refused, same bits."""
+    M, N, K = 480, 864, 4096
+    assert hip.lib().decx_hip_gemm_f32_workspace(M, N, K) > STATIC_BYTES
+    got, want, A, B, _, _ = both(hip, M, N, K, 0x5800, False, offset_a=1)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    ref = oracle.gemm_f32(A, B, rows=np.arange(0, M, 37, dtype=np.uint32))
+    err = float(np.max(np.abs(got[::37].astype(np.float64) - ref))) / (float(np.max(np.abs(ref))) * np.sqrt(K))
+    assert err <= 1e-5, err
+
+
+def test_static_workspace_reads_a_long_column_in_place(hip):
+    """N == 1 with a column longer than the static array holds: the workspace form copies it into a dense vector
+    first, the static one reads it where it lies; the sums are the same."""
+    M, K = 64, (STATIC_BYTES // 4) + 4096
+    assert hip.lib().decx_hip_gemm_f32_workspace(M, 1, K) > STATIC_BYTES
+    got, want, A, B, _, _ = both(hip, M, 1, K, 0x5820, False)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    assert float(np.max(np.abs(got - ref))) / (float(np.max(np.abs(ref))) * np.sqrt(K)) <= 1e-5
