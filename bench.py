@@ -176,6 +176,9 @@ def make_inputs(name):
 
 
 def device_pitch(cols, itemsize):
+    """Row pitch in elements as de::GPU_Matrix lays a matrix out: rows padded to 128 bytes, a single column dense."""
+    if cols == 1:
+        return 1
     per = 128 // itemsize
     return (cols + per - 1) // per * per
 
@@ -547,6 +550,8 @@ def api_wall_time(name, repeats=10):
     dtype, M, N, K = WORKLOADS[name][:4]
     if not os.path.exists(exe) or dtype not in ("f32", "f16"):
         return None
+    if M * N * K < 2 ** 34:
+        repeats = 200
     out = subprocess.run([exe, "gemmtime", dtype, str(M), str(N), str(K), str(repeats)], capture_output=True, text=True, timeout=300)
     for l in out.stdout.splitlines():
         if l.startswith("gemmtime"):
@@ -572,6 +577,7 @@ def main():
     # the de:: API's own wall time, before this process takes the GPU
     api = api_wall_time(args.workload) if (args.workload in WORKLOADS and not args.no_extra) else None
     api16 = api_wall_time("fp16_4096") if (args.workload == "fp32_8192" and not args.no_extra) else None
+    api_gemv = api_wall_time("fp32_gemv") if (args.workload == "fp32_8192" and not args.no_extra) else None
 
     from decx_amd import hip
     hip.init(0)
@@ -648,6 +654,8 @@ def main():
                                 "*_on_zero_operands: the same launches on zeros, where the board's power management does not hold the clock down",
                         "gpu_parity_rel_err": (o.get("gpu_parity") or {}).get("rel_err"), "parity_bar": 2e-3,
                         "plan": o["plan"], "api_wall_median_ms": (api16 or {}).get("median_ms")}
+                if name == "fp32_gemv" and api_gemv is not None:
+                    o["api_wall"] = api_gemv
                 others.append(o)
                 del inp
         others.append(run_conv(200, args.warmup, parity=not args.no_cpu))

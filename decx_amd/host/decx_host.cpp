@@ -239,6 +239,12 @@ void decx::_GPU_Matrix::assign(de::_DATA_TYPES_FLAGS_ type, uint32_t width, uint
     _layout.height = height;
     const uint32_t per128 = _layout._single_element_size ? 128u / (uint32_t)_layout._single_element_size : 1u;
     _layout.pitch = round_up(width, per128 ? per128 : 1u);
+    // A single column is stored dense.  Under the 128-byte rule every element of it would sit in a cache line of its
+    // own, and a product with it (N = 1: the column is the vector of a matrix-vector product, and so is the result)
+    // would move a line per element, or copy the column together first on every call.  Neither the pitch nor the
+    // device pointer is visible through de::GPU_Matrix, so no caller can tell; de::Memcpy converts between this
+    // and the host's 32-byte rows.
+    if (width == 1) _layout.pitch = 1;
 }
 
 bool decx::_GPU_Matrix::allocate()

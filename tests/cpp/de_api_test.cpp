@@ -276,6 +276,102 @@ static int gpu_checks()
     for (int i = 0; i < 64; ++i) for (int j = 0; j < 32; ++j) ok &= (de::Half2Float(*hD.ptr<de::Half>(i, j)) == 240.f);
     CHECK(ok);
 
+    // single columns (stored dense on the device): y = M x with exact small integers, a copy into the column between
+    // two products is what the next product multiplies, the result column feeds the next product, sub-region copies
+    // of a column, a column as the LEFT operand (outer product) and as C
+    {
+        const uint32_t R = 300, Kc = 5000;
+        de::Matrix& Mh = de::CreateMatrixRef(de::_FP32_, Kc, R);
+        de::Matrix& xh = de::CreateMatrixRef(de::_FP32_, 1, Kc);
+        de::Matrix& yh = de::CreateMatrixRef(de::_FP32_, 1, R);
+        fill<float>(Mh, [](int i, int j) { return (float)((i + 2 * j) % 5 - 2); });
+        fill<float>(xh, [](int i, int) { return (float)(i % 3 - 1); });
+        de::GPU_Matrix& dM = de::CreateGPUMatrixRef(de::_FP32_, Kc, R);
+        de::GPU_Matrix& dx = de::CreateGPUMatrixRef(de::_FP32_, 1, Kc);
+        de::GPU_Matrix& dy = de::CreateGPUMatrixRef();
+        CHECK(de::Memcpy(Mh, dM, O, O, de::Point2D(Kc, R), de::DECX_MEMCPY_H2D).error_type == 0);
+        CHECK(de::Memcpy(xh, dx, O, O, de::Point2D(1u, Kc), de::DECX_MEMCPY_H2D).error_type == 0);
+        auto expect = [&](const de::Matrix& x, uint32_t row) {
+            double s = 0;
+            for (uint32_t k = 0; k < Kc; ++k) s += (double)*Mh.ptr<float>(row, k) * (double)*const_cast<de::Matrix&>(x).ptr<float>(k, 0);
+            return (float)s;
+        };
+        de::blas::cuda::GEMM(dM, dx, dy);
+        CHECK(de::GetLastError()->error_type == 0 && dy.Width() == 1 && dy.Height() == R);
+        CHECK(de::Memcpy(yh, dy, O, O, de::Point2D(1u, R), de::DECX_MEMCPY_D2H).error_type == 0);
+        bool okc = true;
+        for (uint32_t i = 0; i < R; ++i) okc &= (*yh.ptr<float>(i, 0) == expect(xh, i));
+        CHECK(okc);
+        // rows 100 .. 2099 of the column change on the device: the next product sees them
+        de::Matrix& patch = de::CreateMatrixRef(de::_FP32_, 1, 2000);
+        fill<float>(patch, [](int i, int) { return (float)(i % 7 - 3); });
+        CHECK(de::Memcpy(patch, dx, O, de::Point2D(0, 100), de::Point2D(1, 2000), de::DECX_MEMCPY_H2D).error_type == 0);
+        for (uint32_t k = 0; k < 2000; ++k) *xh.ptr<float>(100 + k, 0) = *patch.ptr<float>(k, 0);
+        de::blas::cuda::GEMM(dM, dx, dy);
+        CHECK(de::Memcpy(yh, dy, O, O, de::Point2D(1u, R), de::DECX_MEMCPY_D2H).error_type == 0);
+        okc = true;
+        for (uint32_t i = 0; i < R; ++i) okc &= (*yh.ptr<float>(i, 0) == expect(xh, i));
+        CHECK(okc);
+        // ... and reads back what was written, from an offset
+        de::Matrix& xback = de::CreateMatrixRef(de::_FP32_, 1, Kc);
+        CHECK(de::Memcpy(xback, dx, de::Point2D(0, 50), de::Point2D(0, 50), de::Point2D(1u, Kc - 50), de::DECX_MEMCPY_D2H).error_type == 0);
+        okc = *xback.ptr<float>(49, 0) == 0.f;
+        for (uint32_t k = 50; k < Kc; ++k) okc &= (*xback.ptr<float>(k, 0) == *xh.ptr<float>(k, 0));
+        CHECK(okc);
+        // the result column as the next product's vector: z = T y, T 40 x 300 of ones and minus ones; y as C: T y + 2 z0
+        de::Matrix& Th = de::CreateMatrixRef(de::_FP32_, R, 40);
+        fill<float>(Th, [](int i, int j) { return (i + j) % 2 ? 1.f : -1.f; });
+        de::GPU_Matrix& dT = de::CreateGPUMatrixRef(de::_FP32_, R, 40);
+        de::GPU_Matrix& dz = de::CreateGPUMatrixRef();
+        CHECK(de::Memcpy(Th, dT, O, O, de::Point2D(R, 40u), de::DECX_MEMCPY_H2D).error_type == 0);
+        de::blas::cuda::GEMM(dT, dy, dz);
+        CHECK(de::GetLastError()->error_type == 0 && dz.Width() == 1 && dz.Height() == 40);
+        de::Matrix& zh = de::CreateMatrixRef(de::_FP32_, 1, 40);
+        CHECK(de::Memcpy(zh, dz, O, O, de::Point2D(1, 40), de::DECX_MEMCPY_D2H).error_type == 0);
+        okc = true;
+        for (uint32_t i = 0; i < 40; ++i) {
+            double s = 0;
+            for (uint32_t k = 0; k < R; ++k) s += (double)*Th.ptr<float>(i, k) * (double)*yh.ptr<float>(k, 0);
+            okc &= (*zh.ptr<float>(i, 0) == (float)s);
+        }
+        CHECK(okc);
+        de::blas::cuda::GEMM(dT, dy, dz, dz, de::Number(1.f), de::Number(2.f));            // C = dst = the column z
+        de::Matrix& z2 = de::CreateMatrixRef(de::_FP32_, 1, 40);
+        CHECK(de::Memcpy(z2, dz, O, O, de::Point2D(1, 40), de::DECX_MEMCPY_D2H).error_type == 0);
+        okc = true;
+        for (uint32_t i = 0; i < 40; ++i) okc &= (*z2.ptr<float>(i, 0) == 3.f * *zh.ptr<float>(i, 0));
+        CHECK(okc);
+        // outer product: the column z (40 x 1) times a row (1 x 33)
+        de::Matrix& rowh = de::CreateMatrixRef(de::_FP32_, 33, 1);
+        fill<float>(rowh, [](int, int j) { return (float)(j - 16); });
+        de::GPU_Matrix& drow = de::CreateGPUMatrixRef(de::_FP32_, 33, 1);
+        de::GPU_Matrix& douter = de::CreateGPUMatrixRef();
+        CHECK(de::Memcpy(rowh, drow, O, O, de::Point2D(33, 1), de::DECX_MEMCPY_H2D).error_type == 0);
+        de::blas::cuda::GEMM(dz, drow, douter);
+        CHECK(de::GetLastError()->error_type == 0 && douter.Width() == 33 && douter.Height() == 40);
+        de::Matrix& outerh = de::CreateMatrixRef(de::_FP32_, 33, 40);
+        CHECK(de::Memcpy(outerh, douter, O, O, de::Point2D(33, 40), de::DECX_MEMCPY_D2H).error_type == 0);
+        okc = true;
+        for (uint32_t i = 0; i < 40; ++i) for (uint32_t j = 0; j < 33; ++j) okc &= (*outerh.ptr<float>(i, j) == *z2.ptr<float>(i, 0) * (float)((int)j - 16));
+        CHECK(okc);
+        // fp16 column: ones(64 x 4096) . halves of 0.5 = 2048
+        de::Matrix& hM = de::CreateMatrixRef(de::_FP16_, 4096, 64);
+        de::Matrix& hx = de::CreateMatrixRef(de::_FP16_, 1, 4096);
+        fill<de::Half>(hM, [](int, int) { de::Half h; h.val = 0x3c00; return h; });
+        fill<de::Half>(hx, [](int, int) { de::Half h; h.val = 0x3800; return h; });
+        de::GPU_Matrix& ghM = de::CreateGPUMatrixRef(de::_FP16_, 4096, 64);
+        de::GPU_Matrix& ghx = de::CreateGPUMatrixRef(de::_FP16_, 1, 4096);
+        de::GPU_Matrix& ghy = de::CreateGPUMatrixRef();
+        de::Memcpy(hM, ghM, O, O, de::Point2D(4096, 64), de::DECX_MEMCPY_H2D);
+        de::Memcpy(hx, ghx, O, O, de::Point2D(1, 4096), de::DECX_MEMCPY_H2D);
+        de::blas::cuda::GEMM(ghM, ghx, ghy);
+        de::Matrix& hy = de::CreateMatrixRef(de::_FP16_, 1, 64);
+        CHECK(de::Memcpy(hy, ghy, O, O, de::Point2D(1, 64), de::DECX_MEMCPY_D2H).error_type == 0);
+        okc = true;
+        for (int i = 0; i < 64; ++i) okc &= (de::Half2Float(*hy.ptr<de::Half>(i, 0)) == 2048.f);
+        CHECK(okc);
+    }
+
     // host-matrix overload and pinned staging
     de::Matrix& I = de::CreateMatrixRef(de::_FP32_, 50, 50);
     fill<float>(I, [](int i, int j) { return i == j ? 1.f : 0.f; });

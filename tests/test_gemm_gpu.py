@@ -167,6 +167,10 @@ def test_config5b_f32_gemv(hip, oracle):
     assert hip.plan(4, M, N, K).path == hip.PATH_GEMV
     assert rel_err(run(hip, A, B), oracle.gemm_f32(A, B), K) <= TOL_F32
     assert rel_err(run(hip, A, B, C, 0.5, -2.0), oracle.gemm_f32(A, B, C, 0.5, -2.0), K) <= TOL_F32
+    # the columns stored dense, as de::GPU_Matrix keeps a single column: the same sums
+    dense = (device_pitch(K, np.float32), 1, 1, 1)
+    assert np.array_equal(run(hip, A, B, pitches=dense), run(hip, A, B))
+    assert np.array_equal(run(hip, A, B, C, 0.5, -2.0, pitches=dense), run(hip, A, B, C, 0.5, -2.0))
     # and the same column through the tiled kernel
     assert rel_err(run(hip, A, B, tile=2), oracle.gemm_f32(A, B), K) <= TOL_F32
 
