@@ -126,9 +126,15 @@ int choose_tile_f64(uint32_t M, uint32_t N)
 
 int choose_tile(bool f16, uint32_t M, uint32_t N, bool aligned)
 {
+    // candidates from the smallest to the largest tile: ties go to the larger one
+    static const int kBasic[] = {TILE_SMALL, TILE_MEDIUM, TILE_LARGE};
+    static const int kF16Aligned[] = {TILE_SMALL, TILE_MEDIUM, TILE_F16_192x192, TILE_F16_192x256, TILE_F16_256x192, TILE_LARGE};
+    const int* const shapes = f16 && aligned ? kF16Aligned : kBasic;
+    const int count = f16 && aligned ? 6 : 3;
     int best = TILE_SMALL;
     double best_cost = 1e300;
-    for (int s = TILE_COUNT - 1; s >= 0; --s) {
+    for (int c = 0; c < count; ++c) {
+        const int s = shapes[c];
         const TileInfo ti = f16 ? tile_info_f16(s, aligned) : tile_info_f32(s, aligned, N);
         const uint64_t tiles = (uint64_t)((M + ti.bm - 1) / ti.bm) * ((N + ti.bn - 1) / ti.bn);
         const double cost = tile_cost(ti, tiles, g_dev.compute_units);
@@ -378,7 +384,7 @@ int run_gemm(const void* A, const void* B, const void* C, void* D, uint32_t M, u
     if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
     const int rc = check_gemm(A, B, C, D, M, N, K, lda, ldb, ldc, ldd);
     if (rc != DECX_HIP_OK || M == 0 || N == 0) return rc;
-    if (tile != DECX_HIP_TILE_AUTO && (tile < 0 || tile >= TILE_COUNT)) return DECX_HIP_E_INVALID_ARG;
+    if (tile != DECX_HIP_TILE_AUTO && (tile < 0 || tile >= (F16 ? TILE_F16_COUNT : TILE_COUNT))) return DECX_HIP_E_INVALID_ARG;
 
     // the two vector corners are bandwidth-bound and have kernels of their own
     if (N == 1 && tile == DECX_HIP_TILE_AUTO && K > 0) {

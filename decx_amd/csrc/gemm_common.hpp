@@ -112,7 +112,12 @@ enum TileShape : int {
     TILE_LARGE  = 0,
     TILE_MEDIUM = 1,
     TILE_SMALL  = 2,
-    TILE_COUNT  = 3,
+    TILE_COUNT  = 3,                // the classes every element type has
+    // fp16 on 16-byte aligned operands only: tiles between the two largest classes
+    TILE_F16_192x192 = 3,
+    TILE_F16_192x256 = 4,
+    TILE_F16_256x192 = 5,
+    TILE_F16_COUNT = 6,
 };
 
 // per_cu: workgroups of the shape that fit a CU together.  full: throughput of a CU filled with them, alone: of
@@ -160,11 +165,19 @@ __host__ inline TileInfo tile_info_f32(int shape, bool aligned = true, uint32_t 
         return { 64,  64, 256, aligned ? 4 : 2, aligned ? 0.90f : 0.70f, aligned ? 0.865f : 0.49f};
     }
 }
-// fp16 (TFLOP/s per CU): 256 x 256 4.64 on a full chip, 6.4 with at most half the CUs busy; 128 x 128 3.1 alone,
+// fp16 (TFLOP/s per CU; TILE_F16_*: tiles between the two largest classes, one workgroup per CU, chosen where they cut
+// the output into a number of pieces that suits the CUs better -- 3000^3: 256 tiles of 192 x 192, 52.7 us, against 144 of
+// 256 x 256, 56.5 us; 4608^3: 432 of 256 x 192, 174 us, against 324, 186 us): 256 x 256 4.64 on a full chip, 6.4 with at most half the CUs busy; 128 x 128 3.1 alone,
 // 3.9 two per CU; 64 x 64 1.27 alone, 2.4 four per CU.  Predicated register-staged kernels about 1 : 0.6 : 0.25.
 __host__ inline TileInfo tile_info_f16(int shape, bool aligned = true)
 {
     switch (shape) {
+    // per flop these read a third more from LDS than 256 x 256 (wave tiles of 48 x 96 and 96 x 64): measured 0.80 /
+    // 0.89 / 0.88 of its rate on a full chip (6144^3: 1132 / 1242 / 1227 TFLOP/s against 1400) and 0.65 / 0.74 / 0.74
+    // of it on a chip at most half busy, where the largest tile runs 1.38 times its full-chip rate
+    case TILE_F16_192x192: return {192, 192, 512, 1, 0.80f, 0.90f};
+    case TILE_F16_192x256: return {192, 256, 512, 1, 0.89f, 1.02f};
+    case TILE_F16_256x192: return {256, 192, 512, 1, 0.88f, 1.02f};
     case TILE_LARGE: return {256, 256, aligned ? 512 : 256, 1, 1.00f, aligned ? 1.38f : 1.00f};
     case TILE_MEDIUM: return {128, 128, aligned ? 512 : 128, 2, aligned ? 0.84f : 0.60f, aligned ? 0.70f : 0.50f};
     default:           return { 64,  64, aligned ? 256 :  64, aligned ? 4 : 2, aligned ? 0.55f : 0.25f, aligned ? 0.27f : 0.12f};

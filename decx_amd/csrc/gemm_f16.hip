@@ -230,6 +230,7 @@ int launch_gemm_f16(int shape, bool edge, const GemmArgs& args, hipStream_t stre
 {
     if (!edge && args.vec_ok && args.K > 0 && dma_offsets_fit(args, 2)) return launch_gemm_f16_dma(shape, args, stream);
     switch (shape) {
+    case TILE_F16_192x192: case TILE_F16_192x256: case TILE_F16_256x192:        // (classes of the direct-to-LDS family only)
     case TILE_LARGE: return launch_shape<256, 256, 64, 2, 2>(args, stream);
     case TILE_MEDIUM: return launch_shape<128, 128, 64, 2, 1>(args, stream);
     case TILE_SMALL:   return launch_shape< 64,  64, 64, 1, 1>(args, stream);

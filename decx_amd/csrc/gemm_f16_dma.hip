@@ -82,7 +82,7 @@ template <int MFMAS, int READS> __device__ __forceinline__ void interleave()
 // partial products and rounds once (split_k_exchange).
 template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool SPLIT = false>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
-__attribute__((amdgpu_waves_per_eu((BM * BN >= 256 * 256 || STAGES > 2) ? 2 : 4)))     // as scheduled: one 256 x 256 workgroup per CU, two of 128 x 128, four of 64 x 64 (rings of 2 stages)
+__attribute__((amdgpu_waves_per_eu((BM * BN >= 192 * 192 || STAGES > 2) ? 2 : 4)))     // as scheduled: one workgroup of 192 x 192 and up per CU, two of 128 x 128, four of 64 x 64 (rings of 2 stages)
 gemm_f16_dma_kernel(const GemmArgs g_in)
 {
     struct Nothing {};
@@ -107,13 +107,13 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 16, TN = WN / 16;
     constexpr int HALVES = TM >= 8 ? 2 : 1, TMH = TM / HALVES;        // the A fragments of a k step come in this many parts
     constexpr int RB = BK * 2, CPR = RB / 16, RPB = 16 / CPR;         // A row bytes, chunks per row, rows per 256 bytes
-    constexpr int BRB = BN * 2, CBR = BRB / 16, BROWS = 1024 / BRB;   // B row bytes, chunks per row, k rows per direct load
+    constexpr int BRB = BN * 2, CBR = BRB / 16;                       // B row bytes, chunks per row
     constexpr int A_STAGE_BYTES = BM * RB, B_STAGE_BYTES = BK * BRB, STAGE_BYTES = A_STAGE_BYTES + B_STAGE_BYTES;
     constexpr int A_LOADS = A_STAGE_BYTES / 1024 / WAVES, B_LOADS = B_STAGE_BYTES / 1024 / WAVES, LOADS = A_LOADS + B_LOADS;
     constexpr int KS = BK / 32;                                       // MFMA k steps per slab
     constexpr int UNITS = KS * HALVES;
     static_assert(TM >= 1 && TN >= 1 && BK == 64 && UNITS % 2 == 0, "shape");
-    static_assert(BN == 64 || BN == 128 || BN == 256, "B row must be 128, 256 or 512 bytes");
+    static_assert(BN == 64 || BN == 128 || BN == 192 || BN == 256, "B row must be 128, 256, 384 or 512 bytes");
     static_assert(A_LOADS >= 1 && B_LOADS >= 1 && A_LOADS * WAVES * 1024 == A_STAGE_BYTES &&
                   B_LOADS * WAVES * 1024 == B_STAGE_BYTES, "copy plan must divide evenly");
     constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
@@ -134,15 +134,20 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     const size_t lda_b = (size_t)g.lda * 2, ldb_b = (size_t)g.ldb * 2;
 
     // chunk permutation of B row k: the transposing read of a half-wave takes 4 k rows from each of two groups of
-    // 8 k (rows 8 apart), 32 bytes each: all 16 pieces must fall into different 16-byte bank groups
-    auto b_key = [](int k) { return (BN >= 128 ? 4 * (k & 3) : 4 * ((k >> 1) & 1)) ^ (2 * ((k >> 3) & 1)); };
+    // 8 k (rows 8 apart), 32 bytes each: all 16 pieces must fall into different 16-byte bank groups.  (384-byte rows:
+    // consecutive rows already lie half the banks apart, so the key tells apart the rows two apart and eight apart.)
+    auto b_key = [](int k) {
+        if constexpr (BN == 192) return (4 * ((k >> 3) & 1)) ^ (2 * ((k >> 1) & 1));
+        else return (BN >= 128 ? 4 * (k & 3) : 4 * ((k >> 1) & 1)) ^ (2 * ((k >> 3) & 1));
+    };
 
     const unsigned char* a_src[A_LOADS];
     const unsigned char* b_src[B_LOADS];
     // chunk of its row that copy lane i of A fetches / k row of copy lane i of B (functions, not arrays: the partial last
     // slab is the only other place that wants them, and registers that live across the K loop are scarce)
     auto a_chunk_of = [&](int i) { const int row = (64 / CPR) * (wave * A_LOADS + i) + lane / CPR; return (lane % CPR) ^ ((row / RPB) % CPR); };
-    auto b_krow_of = [&](int i) { return BROWS * (wave * B_LOADS + i) + lane / CBR; };
+    // (a direct load fills 1024 contiguous bytes of the stage: 16-byte piece 64 I + lane of the B slab, whatever the row length)
+    auto b_krow_of = [&](int i) { return (64 * (wave * B_LOADS + i) + lane) / CBR; };
     const uint32_t last_row = g.M - 1, last_col_chunk = (g.N - 1) / 8;
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
@@ -153,9 +158,8 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     }
 #pragma unroll
     for (int i = 0; i < B_LOADS; ++i) {
-        const int I = wave * B_LOADS + i;
         const int krow = b_krow_of(i);
-        const int chunk = (lane % CBR) ^ b_key(krow);
+        const int chunk = ((64 * (wave * B_LOADS + i) + lane) % CBR) ^ b_key(krow);
         const uint32_t gchunk = (n0 / 8 + chunk) < last_col_chunk ? (n0 / 8 + chunk) : last_col_chunk;
         b_src[i] = B + (size_t)krow * ldb_b + (size_t)gchunk * 16;
     }
@@ -364,9 +368,13 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
     // buffer (two of them, taking turns) and stores whole rows: WN * 2 contiguous bytes per row.  Tiles on a ragged
     // edge take the same way and leave out rows beyond M and 16-byte pieces beyond N; only a piece that straddles N is
     // stored element by element (stored that way as a whole, a 256 x 256 edge tile took a third longer than an interior one).
-    constexpr int ROW_BYTES = WN * 2, PPR = WN / 8, RPG = 256 / ROW_BYTES, ROWS_PER_STORE = 64 / PPR, STORES = 16 / ROWS_PER_STORE;
-    static_assert(PPR == 4 || PPR == 8 || PPR == 16, "staging rows of 64, 128 or 256 bytes");
-    static_assert(WAVES * 2 * 16 * ROW_BYTES <= LDS_BYTES, "staging rows must fit in the ring");
+    // (Rows of 192 bytes -- a wave tile 96 columns wide -- are not permuted but laid 16 bytes further apart.)
+    constexpr int ROW_BYTES = WN * 2, PPR = WN / 8, STORES = PPR / 4;
+    constexpr bool POW2 = (PPR & (PPR - 1)) == 0;
+    constexpr int ROW_PITCH = POW2 ? ROW_BYTES : ROW_BYTES + 16, RPG = POW2 ? 256 / ROW_BYTES : 1;
+    static_assert(PPR == 4 || PPR == 8 || PPR == 12 || PPR == 16, "staging rows of 64, 128, 192 or 256 bytes");
+    static_assert(WAVES * 2 * 16 * ROW_PITCH <= LDS_BYTES, "staging rows must fit in the ring");
+    auto piece_slot = [](int piece, int row) { if constexpr (POW2) return piece ^ ((row / RPG) % PPR); else return piece; };
     auto wave_sync = [] {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -375,7 +383,7 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const uint32_t row = m0 + wm0 + 16 * i + l16;
-        unsigned char* stage_rows = lds + (wave * 2 + (i & 1)) * (16 * ROW_BYTES);
+        unsigned char* stage_rows = lds + (wave * 2 + (i & 1)) * (16 * ROW_PITCH);
         // interior tiles ask for the C values of all TN blocks of the row before the first is used (one load, its wait and
         // the fmas block by block made the C term cost 6 to 12 %)
         halfx4 c_row[TN];
@@ -408,13 +416,13 @@ gemm_f16_dma_kernel(const GemmArgs g_in)
             // piece p (16 bytes) of row l16, half kg & 1 of it; pieces XOR-permuted so that the 32 lanes of a write
             // and the 16 lanes of a read-back each cover all banks once
             const int p = 2 * j + (kg >> 1);
-            *(uintx2*)(stage_rows + l16 * ROW_BYTES + ((p ^ ((l16 / RPG) % PPR)) * 16) + (kg & 1) * 8) = out;
+            *(uintx2*)(stage_rows + l16 * ROW_PITCH + piece_slot(p, l16) * 16 + (kg & 1) * 8) = out;
         }
         wave_sync();
 #pragma unroll
         for (int t2 = 0; t2 < STORES; ++t2) {
-            const int r = ROWS_PER_STORE * t2 + lane / PPR, pc = lane % PPR;
-            const uintx4 v = *(const uintx4*)(stage_rows + r * ROW_BYTES + ((pc ^ ((r / RPG) % PPR)) * 16));
+            const int r = (64 * t2 + lane) / PPR, pc = (64 * t2 + lane) % PPR;
+            const uintx4 v = *(const uintx4*)(stage_rows + r * ROW_PITCH + piece_slot(pc, r) * 16);
             const uint32_t grow = m0 + wm0 + 16 * i + r, gcol = n0 + wn0 + 8 * pc;
             _Float16* out = D + (size_t)grow * g.ldd + gcol;
             if (interior || (grow < g.M && gcol + 8 <= g.N)) {
@@ -443,7 +451,7 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
     if (g.split_len) {                                     // the planner splits K on the two smaller tiles only
-        if constexpr (BM <= 128) {
+        if constexpr (BM <= 128 && BN <= 128) {
             const uint32_t splits = g.split_count;
             hipLaunchKernelGGL((gemm_f16_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, true>), dim3(g.split_first + (nb - g.split_first) * splits),
                                dim3(WAVES_M * WAVES_N * 64), 0, stream, g);
@@ -489,6 +497,11 @@ int launch_gemm_f16_dma(int shape, const GemmArgs& args, hipStream_t stream)
         return blocks <= 512 ? launch_dma<64, 64, 2, 2, 64, 4>(args, stream)
                              : launch_dma<64, 64, 2, 2, 64, 2>(args, stream);
     }
+    // tiles between 128 x 128 and 256 x 256, one workgroup of 8 wavefronts per CU, for outputs that the largest tile
+    // cuts into an awkward number of pieces (3000^3: 144 tiles of 256 x 256 on 256 CUs, but 256 of 192 x 192)
+    case TILE_F16_192x192: return launch_dma<192, 192, 4, 2, 64, 2>(args, stream);     // wavefronts of 48 x 96
+    case TILE_F16_192x256: return launch_dma<192, 256, 2, 4, 64, 2>(args, stream);     // 96 x 64
+    case TILE_F16_256x192: return launch_dma<256, 192, 4, 2, 64, 2>(args, stream);     // 64 x 96
     default:           return (int)hipErrorInvalidValue;
     }
 }

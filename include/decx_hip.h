@@ -58,6 +58,11 @@ enum {
     DECX_HIP_TILE_LARGE  = 0,
     DECX_HIP_TILE_MEDIUM = 1,
     DECX_HIP_TILE_SMALL  = 2,
+    /* fp16 on 16-byte aligned operands only: tiles between 128 x 128 and 256 x 256, for outputs that the largest tile
+     * cuts into an awkward number of pieces (unaligned operands run these classes on the 256 x 256 register-staged kernel) */
+    DECX_HIP_TILE_F16_192x192 = 3,
+    DECX_HIP_TILE_F16_192x256 = 4,
+    DECX_HIP_TILE_F16_256x192 = 5,
     DECX_HIP_PATH_GEMV   = 16,    /* N == 1: bandwidth-bound row-dot kernel */
     DECX_HIP_PATH_GEVM   = 17     /* M == 1: bandwidth-bound column-sum kernel */
 };

@@ -224,8 +224,8 @@ def test_f32_large_ragged_sampled(hip, oracle):
     assert np.max(np.abs(got.astype(np.float64).sum(axis=0) - colsum)) / np.max(np.abs(colsum)) < 1e-5
 
 
-@pytest.mark.parametrize("M,N,K", SHAPES)
-@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("M,N,K", SHAPES + [(193, 385, 130), (500, 390, 200)])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
 def test_f16_ragged_shapes_every_tile(hip, oracle, M, N, K, tile):
     A = synth.normal_half(M, K, 111); B = synth.normal_half(K, N, 112); C = synth.normal_half(M, N, 113)
     assert rel_err(run(hip, A, B, tile=tile), oracle.gemm_f16(A, B), K) <= TOL_F16
@@ -589,8 +589,8 @@ def test_c_may_alias_d(hip, oracle):
     assert rel_err(dD.download(), oracle.gemm_f32(A, B, C, 1.0, 1.0), K) <= TOL_F32
 
 
-@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.float64])
-@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("dtype,tile", [(d, t) for d in (np.float32, np.float16, np.float64) for t in (0, 1, 2)] +
+                         [(np.float16, t) for t in (3, 4, 5)])
 def test_c_term_on_interior_and_edge_tiles_of_every_tile(hip, oracle, dtype, tile):
     """alpha A.B + beta C on an output that holds interior tiles, tiles on the right and lower edges and the corner tile of
     every tile class, with C apart from D and with C = D (the epilogues ask for the C values of several rows ahead of
@@ -748,3 +748,22 @@ def test_split_k_on_two_streams_at_once(hip, oracle, dtype, M, N, K):
         assert L.decx_hip_stream_destroy(ln["stream"]) == 0
         for k in ("A", "B", "D", "ws"):
             ln[k].free()
+
+
+@pytest.mark.parametrize("M,N,K,tile_m,tile_n", [(3000, 3000, 3000, 192, 192), (8192, 4608, 256, 256, 192), (4608, 4608, 512, 192, 256)])
+def test_f16_tiles_between_the_two_largest_are_planned_and_right(hip, oracle, M, N, K, tile_m, tile_n):
+    """Outputs that 256 x 256 tiles cut into an awkward number of pieces for the CUs take a tile of 192 rows or columns:
+    the plan says so, the result holds on sampled rows (first and last tile rows included), bit-equal to the forced
+    tile, and a column checksum covers every element."""
+    p = hip.plan(2, M, N, K)
+    assert (p.tile_m, p.tile_n) == (tile_m, tile_n) and p.k_splits == 1
+    A = synth.normal_half(M, K, 171); B = synth.normal_half(K, N, 172)
+    got = run(hip, A, B)
+    rows = np.unique(np.concatenate([[0, 1, tile_m - 1, tile_m, M - 2, M - 1], sample_rows(M, 40, 9)])).astype(np.uint32)
+    assert rel_err(got[rows], oracle.gemm_f16(A, B, rows=rows), K) <= TOL_F16
+    # ones . (A B) = (ones . A) B in float64, against the sum of the rounded outputs: rounding errors average out
+    want = (A.astype(np.float64).sum(axis=0) @ B.astype(np.float64))
+    have = got.astype(np.float64).sum(axis=0)
+    assert float(np.max(np.abs(have - want))) <= 2e-3 * float(np.max(np.abs(want))) + 0.05 * np.sqrt(M)
+    forced = {(192, 192): 3, (192, 256): 4, (256, 192): 5}[(tile_m, tile_n)]
+    assert np.array_equal(run(hip, A, B, tile=forced).view(np.uint16), got.view(np.uint16))
