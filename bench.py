@@ -468,6 +468,142 @@ CPU_LEGS = {
 }
 
 
+# ---- the planner against every other plan, on shapes it was not fitted on -------------------------------------------------
+
+SWEEP_TILES = {"f32": {0: (256, 128), 1: (128, 128), 2: (64, 64)},
+               "f16": {0: (256, 256), 1: (128, 128), 2: (64, 64), 3: (192, 192), 4: (192, 256), 5: (256, 192)},
+               "f64": {0: (256, 128), 1: (128, 128), 2: (64, 64)}}
+SWEEP_SPLIT_FIT = {"f32": {2: 4}, "f16": {2: 4, 1: 2}, "f64": {2: 2}}       # tile classes whose kernels split K: workgroups that share a CU
+
+
+def sweep_shapes(seed, per_type):
+    """Seeded shapes with log-uniform sides, none of them round: M, N in 40 .. 6500, K in 300 .. 14000, between 0.2 and
+    150 GFLOP (fp64: 50)."""
+    rng = np.random.default_rng(seed)
+    shapes = []
+    for dt in ("f32", "f16", "f64"):
+        got = 0
+        while got < per_type:
+            M, N = (int(math.exp(rng.uniform(math.log(40), math.log(6500)))) for _ in range(2))
+            K = int(math.exp(rng.uniform(math.log(300), math.log(14000))))
+            flops = 2.0 * M * N * K
+            if flops < 2e8 or flops > (5e10 if dt == "f64" else 1.5e11) or M % 64 == 0 or N % 64 == 0:
+                continue
+            shapes.append((dt, M, N, K)); got += 1
+    return shapes
+
+
+def planner_sweep(seed=20261125, per_type=16, batches=3, launches=10):
+    """Every shape runs on the planner's pick (the *_ws entry point with the workspace it asks for) and on every other
+    plan there is a kernel for: each tile class whole, and K on 2 .. 32 ranges on the classes that split, for all
+    tiles, for the tiles of a ragged last round, and for the tiles beyond one to three whole ones per CU.  A plan's
+    time is the best of `batches` batches of `launches` launches (HIP events); the pick and the best other plan are
+    then timed again in turns, and the ratio of those two is what the summary counts."""
+    from decx_amd import hip, synth
+    L = hip.lib()
+    cus = int(hip.device_props().compute_units)
+    npdt = {"f32": np.float32, "f16": np.float16, "f64": np.float64}
+    draw = {"f32": synth.uniform_f32, "f16": synth.normal_half, "f64": synth.uniform_f64}
+    peak = {"f32": PEAK_F32_TFLOPS, "f16": PEAK_F16_TFLOPS, "f64": PEAK_F64_TFLOPS}
+    ws_cap = 1 << 30
+    ws = hip.DeviceMatrix(1, ws_cap // 4, np.float32)
+
+    def time_call(call):
+        best = 1e30
+        for _ in range(batches):
+            call(); call()
+            timer = hip.Timer(); timer.start()
+            for _ in range(launches):
+                call()
+            best = min(best, timer.stop() / launches)
+        return best * 1e3                                   # microseconds
+
+    rows = []
+    for dt, M, N, K in sweep_shapes(seed, per_type):
+        isz = np.dtype(npdt[dt]).itemsize
+        dA = hip.DeviceMatrix(M, K, npdt[dt], device_pitch(K, isz), draw[dt](M, K, 0xA500 + M))
+        dB = hip.DeviceMatrix(K, N, npdt[dt], device_pitch(N, isz), draw[dt](K, N, 0xB500 + N))
+        dD = hip.DeviceMatrix(M, N, npdt[dt], device_pitch(N, isz))
+        p = hip.plan(isz, M, N, K)
+        pick_plan = {"tile": [int(p.tile_m), int(p.tile_n)], "k_splits": int(p.k_splits), "whole_tiles": int(p.whole_tiles)}
+        ws_entry = {"f32": L.decx_hip_gemm_f32_ws, "f16": L.decx_hip_gemm_f16_ws, "f64": L.decx_hip_gemm_f64_ws}[dt]
+        pick = lambda: hip.check(ws_entry(dA.ptr, dB.ptr, None, dD.ptr, M, N, K, dA.pitch, dB.pitch, 0, dD.pitch, 1.0, 1.0, ws.ptr, ws_cap, None))
+
+        def forced(tile, splits, whole):
+            return lambda: hip.check(L.decx_hip_gemm_forced_plan(isz, dA.ptr, dB.ptr, None, dD.ptr, M, N, K, dA.pitch, dB.pitch, 0, dD.pitch,
+                                                                 1.0, 1.0, tile, splits, whole, ws.ptr, ws_cap, None))
+        cands = [({"tile": list(t), "k_splits": 1, "whole_tiles": 0}, forced(c, 1, 0)) for c, t in SWEEP_TILES[dt].items()]
+        for c, fit in SWEEP_SPLIT_FIT[dt].items():
+            bm, bn = SWEEP_TILES[dt][c]
+            if dt == "f32" and c == 2 and N <= 32:
+                bm, bn = 128, 32
+            t = -(-M // bm) * -(-N // bn)
+            if t > 16 * cus:
+                continue
+            slots = fit * cus
+            wholes = {0}
+            if t > slots and t % slots:
+                wholes.add(t // slots * slots)
+            wholes.update(j * cus for j in range(1, fit) if j * cus < t)
+            for ranges in (2, 3, 4, 5, 6, 8, 10, 12, 16, 24, 32):
+                if K // ranges < 256 or (c != 2 and ranges > 8):
+                    continue
+                for whole in sorted(wholes):
+                    if (t - whole) * ranges > 4096 or (t - whole) * ranges * bm * bn * (8 if dt == "f64" else 4) > ws_cap:
+                        continue
+                    call = forced(c, ranges, whole)
+                    if L.decx_hip_gemm_forced_plan(isz, dA.ptr, dB.ptr, None, dD.ptr, M, N, K, dA.pitch, dB.pitch, 0, dD.pitch, 1.0, 1.0,
+                                                   c, ranges, whole, ws.ptr, ws_cap, None) != 0:
+                        continue                            # no kernel for this plan (ranges that do not come out even)
+                    cands.append(({"tile": [bm, bn], "k_splits": ranges, "whole_tiles": whole}, call))
+        hip.sync()
+        t_pick = time_call(pick)
+        timed = [(time_call(call), plan) for plan, call in cands]
+        t_best, best_plan = min(timed, key=lambda x: x[0])
+        best_call = [call for plan, call in cands if plan == best_plan][0]
+        # the two in turns: what the summary counts
+        again_pick, again_best = [], []
+        for _ in range(3):
+            again_pick.append(time_call(pick)); again_best.append(time_call(best_call))
+        t_pick, t_best = min(again_pick + [t_pick]), min(again_best + [t_best])
+        flops = 2.0 * M * N * K
+        rows.append({"dtype": dt, "M": M, "N": N, "K": K, "pick": pick_plan, "pick_us": round(t_pick, 2),
+                     "pick_tflops": round(flops / t_pick / 1e6, 1), "frac_of_peak": round(flops / t_pick / 1e6 / peak[dt], 3),
+                     "best_other": best_plan, "best_other_us": round(t_best, 2), "plans_timed": len(cands),
+                     "pick_over_best": round(t_pick / t_best, 4), "pick_is_best_plan": best_plan == pick_plan})
+        print("sweep %s %5d x %5d x %5d  pick %s %.1f us  best other %s %.1f us  ratio %.3f  (%d plans)" % (
+            dt, M, N, K, pick_plan, t_pick, best_plan, t_best, t_pick / t_best, len(cands)), file=sys.stderr, flush=True)
+        for d in (dA, dB, dD):
+            d.free()
+    ws.free()
+    ratios = sorted(r["pick_over_best"] for r in rows)
+    summary = {"shapes": len(rows), "median_pick_over_best": ratios[len(ratios) // 2], "worst_pick_over_best": ratios[-1],
+               "within_3_percent": sum(r <= 1.03 for r in ratios), "within_10_percent": sum(r <= 1.10 for r in ratios)}
+    for dt in ("f32", "f16", "f64"):
+        rr = sorted(r["pick_over_best"] for r in rows if r["dtype"] == dt)
+        summary[dt] = {"shapes": len(rr), "median": rr[len(rr) // 2], "worst": rr[-1]}
+    return {"workload": "planner sweep: the planner's pick against every other plan on seeded shapes it was not fitted on",
+            "seed": seed, "summary": summary, "shapes": rows}
+
+
+def sweep_markdown(result):
+    """The sweep as a table (what profiles/planner_sweep.md holds below its header)."""
+    s = result["summary"]
+    out = ["| dtype | M | N | K | planner's pick (tile, ranges, whole tiles) | us | TFLOP/s | of peak | best other plan | us | pick / best | plans timed |",
+           "|---|---|---|---|---|---|---|---|---|---|---|---|"]
+    fmt = lambda p: "%d x %d, %d, %d" % (p["tile"][0], p["tile"][1], p["k_splits"], p["whole_tiles"])
+    for r in result["shapes"]:
+        out.append("| %s | %d | %d | %d | %s | %.1f | %.1f | %.3f | %s | %.1f | %.3f | %d |" % (
+            r["dtype"], r["M"], r["N"], r["K"], fmt(r["pick"]), r["pick_us"], r["pick_tflops"], r["frac_of_peak"], fmt(r["best_other"]),
+            r["best_other_us"], r["pick_over_best"], r["plans_timed"]))
+    out.append("")
+    out.append("Pick over best: median %.3f, worst %.3f over %d shapes (%d within 3 %%, %d within 10 %%); fp32 median %.3f worst %.3f, "
+               "fp16 %.3f / %.3f, fp64 %.3f / %.3f." % (s["median_pick_over_best"], s["worst_pick_over_best"], s["shapes"], s["within_3_percent"],
+                                                       s["within_10_percent"], s["f32"]["median"], s["f32"]["worst"], s["f16"]["median"],
+                                                       s["f16"]["worst"], s["f64"]["median"], s["f64"]["worst"]))
+    return "\n".join(out)
+
+
 def cpu_baseline(name, A, B, C, D_gpu):
     """Times the AVX2 restatement of the reference CPU GEMM on this host (best of a few calls for the short
     workloads), checks it bit-for-bit against the scalar fma chain on sampled rows, and compares the GPU's
@@ -567,9 +703,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="fp32_8192", choices=sorted(WORKLOADS) + ["copy_1GiB", "mfma_f16", "conv2d", "conv2d_rgb", "c64_4096", "c128_2048"])
+    ap.add_argument("--workload", default="fp32_8192", choices=sorted(WORKLOADS) + ["copy_1GiB", "mfma_f16", "planner_sweep", "conv2d", "conv2d_rgb", "c64_4096", "c128_2048"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
+    ap.add_argument("--sweep-seed", type=int, default=20261125, help="planner_sweep: seed of the shapes")
+    ap.add_argument("--sweep-shapes", type=int, default=16, help="planner_sweep: shapes per element type")
+    ap.add_argument("--sweep-markdown", default=None, help="planner_sweep: also write the table to this file")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this GEMM path runs on one GPU; --gpus %d is not supported (use --gpus 1)" % args.gpus)
@@ -596,6 +735,13 @@ def main():
             hip.check(hip.lib().decx_hip_calibration_copy(dst.ptr, src.ptr, n, None))
         ms = timer.stop() / args.steps
         print(json.dumps({"workload": "calibration copy 1 GiB", "kernel_ms": ms, "GB/s_read_plus_write": 2 * n / ms / 1e6}))
+        return
+    if args.workload == "planner_sweep":
+        result = planner_sweep(seed=args.sweep_seed, per_type=args.sweep_shapes)
+        if args.sweep_markdown:
+            with open(args.sweep_markdown, "w") as f:
+                f.write(sweep_markdown(result) + "\n")
+        print(json.dumps(result))
         return
     if args.workload == "mfma_f16":
         print(json.dumps(dict(sustained_mfma(launches=args.steps), workload="register-only matrix-core loop")))

@@ -354,6 +354,32 @@ uint32_t arm_split(GemmArgs& g, int elem_bytes, void* workspace, size_t workspac
     return sp.splits;
 }
 
+// The same with the plan given by the caller (a measurement aid: the planner's pick is held against every other plan):
+// `splits` ranges on tile class `shape`, the first `first` tiles whole.  Returns false when that plan cannot run.
+bool arm_split_forced(GemmArgs& g, int elem_bytes, void* workspace, size_t workspace_bytes, int shape, uint32_t splits, uint32_t first,
+                      hipStream_t stream, uint64_t& ticket)
+{
+    ticket = 0;
+    const SplitModel& md = elem_bytes == 8 ? kSplitF64 : elem_bytes == 2 ? kSplitF16 : kSplitF32;
+    bool has_kernel = false;
+    for (int i = 0; i < md.n_tiles; ++i) has_kernel |= md.tiles[i].shape == shape;
+    if (!has_kernel || splits < 2 || splits > 64 || !workspace || !aligned16(workspace)) return false;
+    const RangeLen rl = range_len(g.K, splits, md.len_align);
+    if (rl.ranges != splits || (shape != TILE_SMALL && splits > kSplitFlat)) return false;
+    const TileInfo ti = dma_tile_info(elem_bytes, shape, g.N);
+    const uint64_t tiles = (uint64_t)((g.M + ti.bm - 1) / ti.bm) * ((g.N + ti.bn - 1) / ti.bn);
+    if (first >= tiles) return false;
+    const SplitChoice sp = {shape, splits, rl.len, first, 0};
+    if (workspace_bytes < split_workspace_bytes(elem_bytes, sp, g.M, g.N)) return false;
+    const uint64_t n_counters = (tiles - first) * split_counters_per_tile(splits);
+    uint32_t* const counters = n_counters <= kSplitCounters ? take_split_counters((uint32_t)n_counters, stream, ticket) : nullptr;
+    if (!counters) return false;
+    g.split_counters = counters;
+    g.split_len = sp.len; g.split_count = splits; g.split_first = first; g.split_ws = workspace;
+    g.split_urgent = 0;
+    return true;
+}
+
 // y = alpha * x.B (+ beta * c).  Few columns and a long K: with a workspace, ranges of K go to workgroups of their
 // own, and the last of a column group to finish adds their partial sums in range order.
 int gevm_maybe_split(bool f16, bool out_f32, const void* x, const void* B, const void* c, void* y, uint32_t K, uint32_t N,
@@ -729,6 +755,37 @@ int decx_hip_gemm_f32_static(const float* A, const float* B, const float* C, flo
         ws = nullptr;
     }
     return run_gemm<false>(A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, stream, DECX_HIP_TILE_AUTO, 0, ws, ws ? kScratchBytes : 0);
+}
+
+int decx_hip_gemm_forced_plan(int elem_bytes, const void* A, const void* B, const void* C, void* D, uint32_t M, uint32_t N, uint32_t K,
+                              uint32_t lda, uint32_t ldb, uint32_t ldc, uint32_t ldd, double alpha, double beta, int tile,
+                              uint32_t k_splits, uint32_t whole_tiles, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    if (elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8) return DECX_HIP_E_INVALID_ARG;
+    const int rc = check_gemm(A, B, C, D, M, N, K, lda, ldb, ldc, ldd);
+    if (rc != DECX_HIP_OK) return rc;
+    if (M == 0 || N == 0 || K == 0) return DECX_HIP_E_INVALID_ARG;
+    if (tile < 0 || tile >= (elem_bytes == 2 ? TILE_F16_COUNT : TILE_COUNT)) return DECX_HIP_E_INVALID_ARG;
+    const uint32_t per16 = 16u / (uint32_t)elem_bytes;
+    GemmArgs g;
+    std::memset(&g, 0, sizeof g);
+    g.cus = (uint32_t)g_dev.compute_units;
+    g.A = A; g.B = B; g.C = C; g.D = D;
+    g.M = M; g.N = N; g.K = K;
+    g.lda = lda; g.ldb = ldb; g.ldc = ldc; g.ldd = ldd;
+    g.alpha = (float)alpha; g.beta = (float)beta; g.alpha64 = alpha; g.beta64 = beta;
+    g.vec_ok = (aligned16(A) && aligned16(B) && aligned16(D) && (!C || aligned16(C)) && lda % per16 == 0 && ldb % per16 == 0 &&
+                ldd % per16 == 0 && (!C || ldc % per16 == 0)) ? 1u : 0u;
+    if (!g.vec_ok || !dma_offsets_fit(g, (uint32_t)elem_bytes)) return DECX_HIP_E_INVALID_ARG;      // the direct-to-LDS kernels only
+    uint64_t ticket = 0;
+    if (k_splits > 1 && !arm_split_forced(g, elem_bytes, workspace, workspace_bytes, tile, k_splits, whole_tiles, as_stream(stream), ticket))
+        return DECX_HIP_E_INVALID_ARG;
+    const int launched = elem_bytes == 8 ? launch_gemm_f64(tile, false, g, as_stream(stream))
+                       : elem_bytes == 2 ? launch_gemm_f16(tile, false, g, as_stream(stream))
+                                         : launch_gemm_f32(tile, false, g, as_stream(stream));
+    commit_split_counters(ticket);
+    return launched;
 }
 
 int decx_hip_reset_split_counters(void)

@@ -27,6 +27,18 @@ DECX_HIP_API int decx_hip_calibration_copy(void* dst, const void* src, size_t by
 DECX_HIP_API int decx_hip_calibration_mfma(int elem_bytes, const void* operands, size_t operand_bytes, float* sink,
                                            size_t sink_floats, uint32_t iters, double* flops, void* stream);
 
+/* A GEMM on a plan of the caller's choosing instead of the planner's: tile class `tile` (DECX_HIP_TILE_*), and with
+ * k_splits > 1 that many ranges of K for all tiles but the first `whole_tiles` (workspace: k_splits slots of
+ * tile_m x tile_n accumulators, 4 bytes each, 8 for fp64, per split tile).  16-byte aligned operands only (the
+ * direct-to-LDS kernels); plans that have no kernel -- a split on a tile class whose kernels do not split, ranges
+ * shorter than a slab -- return DECX_HIP_E_INVALID_ARG.  alpha and beta as doubles for every type.  It exists so that
+ * the planner's pick can be timed against every other plan on shapes it was not fitted on (bench.py --workload
+ * planner_sweep); the product path never calls it. */
+DECX_HIP_API int decx_hip_gemm_forced_plan(int elem_bytes, const void* A, const void* B, const void* C, void* D,
+                                           uint32_t M, uint32_t N, uint32_t K, uint32_t lda, uint32_t ldb, uint32_t ldc,
+                                           uint32_t ldd, double alpha, double beta, int tile, uint32_t k_splits,
+                                           uint32_t whole_tiles, void* workspace, size_t workspace_bytes, void* stream);
+
 /* What the split-K counter windows of the current device have seen so far: out[0] windows handed out, out[1] times
  * the ring wrapped round, out[2] requests refused (the product then ran unsplit), out[3] events recorded (only once
  * launches have come from more than one stream), out[4] counters given to launches recorded into graphs, out[5] the
