@@ -473,27 +473,30 @@ CPU_LEGS = {
 SWEEP_TILES = {"f32": {0: (256, 128), 1: (128, 128), 2: (64, 64)},
                "f16": {0: (256, 256), 1: (128, 128), 2: (64, 64), 3: (192, 192), 4: (192, 256), 5: (256, 192)},
                "f64": {0: (256, 128), 1: (128, 128), 2: (64, 64)}}
-SWEEP_SPLIT_FIT = {"f32": {2: 4}, "f16": {2: 4, 1: 2}, "f64": {2: 2}}       # tile classes whose kernels split K: workgroups that share a CU
+SWEEP_SPLIT_FIT = {"f32": {2: 4}, "f16": {2: 4, 1: 2, 0: 1}, "f64": {2: 2}}       # tile classes whose kernels split K: workgroups that share a CU
 
 
-def sweep_shapes(seed, per_type):
+def sweep_shapes(seed, per_type, large=False):
     """Seeded shapes with log-uniform sides, none of them round: M, N in 40 .. 6500, K in 300 .. 14000, between 0.2 and
-    150 GFLOP (fp64: 50)."""
-    rng = np.random.default_rng(seed)
+    150 GFLOP (fp64: 50); large: M, N in 1200 .. 9000, K in 500 .. 9000, up to 1200 GFLOP (fp64: 400)."""
+    rng = np.random.default_rng(seed + (1 if large else 0))
+    side = (1200, 9000) if large else (40, 6500)
+    depth = (500, 9000) if large else (300, 14000)
     shapes = []
     for dt in ("f32", "f16", "f64"):
         got = 0
+        cap = (4e11 if dt == "f64" else 1.2e12) if large else (5e10 if dt == "f64" else 1.5e11)
         while got < per_type:
-            M, N = (int(math.exp(rng.uniform(math.log(40), math.log(6500)))) for _ in range(2))
-            K = int(math.exp(rng.uniform(math.log(300), math.log(14000))))
+            M, N = (int(math.exp(rng.uniform(math.log(side[0]), math.log(side[1])))) for _ in range(2))
+            K = int(math.exp(rng.uniform(math.log(depth[0]), math.log(depth[1]))))
             flops = 2.0 * M * N * K
-            if flops < 2e8 or flops > (5e10 if dt == "f64" else 1.5e11) or M % 64 == 0 or N % 64 == 0:
+            if flops < 2e8 or flops > cap or M % 64 == 0 or N % 64 == 0:
                 continue
             shapes.append((dt, M, N, K)); got += 1
     return shapes
 
 
-def planner_sweep(seed=20261125, per_type=16, batches=3, launches=10):
+def planner_sweep(seed=20261125, per_type=16, batches=3, launches=10, large=False, only=None):
     """Every shape runs on the planner's pick (the *_ws entry point with the workspace it asks for) and on every other
     plan there is a kernel for: each tile class whole, and K on 2 .. 32 ranges on the classes that split, for all
     tiles, for the tiles of a ragged last round, and for the tiles beyond one to three whole ones per CU.  A plan's
@@ -519,7 +522,9 @@ def planner_sweep(seed=20261125, per_type=16, batches=3, launches=10):
         return best * 1e3                                   # microseconds
 
     rows = []
-    for dt, M, N, K in sweep_shapes(seed, per_type):
+    for dt, M, N, K in sweep_shapes(seed, per_type, large):
+        if only and dt not in only:
+            continue
         isz = np.dtype(npdt[dt]).itemsize
         dA = hip.DeviceMatrix(M, K, npdt[dt], device_pitch(K, isz), draw[dt](M, K, 0xA500 + M))
         dB = hip.DeviceMatrix(K, N, npdt[dt], device_pitch(N, isz), draw[dt](K, N, 0xB500 + N))
@@ -580,10 +585,10 @@ def planner_sweep(seed=20261125, per_type=16, batches=3, launches=10):
     summary = {"shapes": len(rows), "median_pick_over_best": ratios[len(ratios) // 2], "worst_pick_over_best": ratios[-1],
                "within_3_percent": sum(r <= 1.03 for r in ratios), "within_10_percent": sum(r <= 1.10 for r in ratios)}
     for dt in ("f32", "f16", "f64"):
-        rr = sorted(r["pick_over_best"] for r in rows if r["dtype"] == dt)
+        rr = sorted(r["pick_over_best"] for r in rows if r["dtype"] == dt) or [float("nan")]
         summary[dt] = {"shapes": len(rr), "median": rr[len(rr) // 2], "worst": rr[-1]}
     return {"workload": "planner sweep: the planner's pick against every other plan on seeded shapes it was not fitted on",
-            "seed": seed, "summary": summary, "shapes": rows}
+            "seed": seed, "large": large, "summary": summary, "shapes": rows}
 
 
 def sweep_markdown(result):
@@ -708,6 +713,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     ap.add_argument("--sweep-seed", type=int, default=20261125, help="planner_sweep: seed of the shapes")
     ap.add_argument("--sweep-shapes", type=int, default=16, help="planner_sweep: shapes per element type")
+    ap.add_argument("--sweep-large", action="store_true", help="planner_sweep: sides of 1200 .. 9000 instead of 40 .. 6500")
+    ap.add_argument("--sweep-dtypes", default=None, help="planner_sweep: only these element types, e.g. f16 or f32,f64")
     ap.add_argument("--sweep-markdown", default=None, help="planner_sweep: also write the table to this file")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -737,7 +744,8 @@ def main():
         print(json.dumps({"workload": "calibration copy 1 GiB", "kernel_ms": ms, "GB/s_read_plus_write": 2 * n / ms / 1e6}))
         return
     if args.workload == "planner_sweep":
-        result = planner_sweep(seed=args.sweep_seed, per_type=args.sweep_shapes)
+        result = planner_sweep(seed=args.sweep_seed, per_type=args.sweep_shapes, large=args.sweep_large, launches=4 if args.sweep_large else 10,
+                               only=args.sweep_dtypes.split(",") if args.sweep_dtypes else None)
         if args.sweep_markdown:
             with open(args.sweep_markdown, "w") as f:
                 f.write(sweep_markdown(result) + "\n")

@@ -174,7 +174,7 @@ struct SplitTile {
     double ns_per_k_one_round[5];    // the same in a launch of at most fit x CUs workgroups, where the kernel has a tighter loop (0: none)
 };
 struct SplitModel {
-    SplitTile tiles[2]; int n_tiles;
+    SplitTile tiles[3]; int n_tiles;
     uint32_t len_align, acc_bytes;   // ranges are multiples of the deepest slab; bytes of an accumulator
     double us_fixed, us_per_trip, us_per_mb, whole_flop_per_us;      // the last: the largest tile, per CU of a full chip
     bool uneven_second_round;
@@ -187,11 +187,11 @@ struct SplitModel {
     uint32_t urgent_max_k;
 };
 // 64 x 64 tiles of 32 KB LDS: four fit a CU (160 KB would hold five, but time against the number of tiles steps as for four)
-static const SplitModel kSplitF32 = {{{TILE_SMALL, 4, 4, {0, 17.72, 15.51, 15.07, 14.77}, {0, 15.8, 15.1, 15.0, 14.96}}, {}}, 1, 32, 4, 1.0, 0.4, 0.15, 0.600e6, true,
+static const SplitModel kSplitF32 = {{{TILE_SMALL, 4, 4, {0, 17.72, 15.51, 15.07, 14.77}, {0, 15.8, 15.1, 15.0, 14.96}}, {}, {}}, 1, 32, 4, 1.0, 0.4, 0.15, 0.600e6, true,
                                      0, 6.2, 14.0, 0, 2048};
-static const SplitModel kSplitF16 = {{{TILE_SMALL, 4, 4, {0, 3.4, 3.3, 3.15, 3.1}}, {TILE_MEDIUM, 2, 8, {0, 7.4, 7.0}}}, 2,
+static const SplitModel kSplitF16 = {{{TILE_SMALL, 4, 4, {0, 3.4, 3.3, 3.15, 3.1}}, {TILE_MEDIUM, 2, 8, {0, 7.4, 7.0}}, {TILE_LARGE, 1, 32, {0, 22.7}}}, 3,
                                      64, 4, 2.0, 2.0, 0.15, 5.4e6, false, 1, 4.3, 6.5, 1.6, 0};     // (fixed: 2.0 us; with 0.5, 4096 x 512 x 2048 went on two ranges, 15.8 us, where whole takes 14.0)
-static const SplitModel kSplitF64 = {{{TILE_SMALL, 2, 4, {0, 28.2, 28.8}}, {}}, 1, 32, 8, 0.5, 2.0, 0.30, 0.300e6, false,
+static const SplitModel kSplitF64 = {{{TILE_SMALL, 2, 4, {0, 28.2, 28.8}}, {}, {}}, 1, 32, 8, 0.5, 2.0, 0.30, 0.300e6, false,
                                      0, 5.7, 27.8, 0, 1u << 30};
 
 TileInfo dma_tile_info(int elem_bytes, int shape, uint32_t N);
@@ -251,8 +251,9 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
     };
     const uint64_t whole_tiles = (uint64_t)((M + whole.bm - 1) / whole.bm) * ((N + whole.bn - 1) / whole.bn);
     double whole_us = tile_cost(whole, whole_tiles, cus) * 2.0 * K / md.whole_flop_per_us + kLaunch;
+    const double whole_us_by_cost = whole_us;
     for (int i = 0; i < md.n_tiles; ++i)                        // the model's own figure where the whole product runs on one of its tiles
-        if (md.tiles[i].shape == whole_shape)
+        if (md.tiles[i].shape == whole_shape && whole_shape != TILE_LARGE)
             whole_us = estimate(md.tiles[i], tiles_of(whole_shape), (K + md.len_align - 1) / md.len_align * md.len_align, 1);
     SplitChoice best = {whole_shape, 1, 0, 0};
     double best_us = whole_us / 1.04;
@@ -260,6 +261,7 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
     for (int i = 0; i < md.n_tiles; ++i) {
         const SplitTile& st = md.tiles[i];
         const uint64_t t = tiles_of(st.shape), slots = (uint64_t)st.fit * cus;
+        if (st.shape == TILE_LARGE) continue;                  // (planned below)
         if (t > 16ull * cus) continue;
         const uint32_t tile_max_p = st.shape == TILE_SMALL ? max_p : (max_p < kSplitFlat ? max_p : kSplitFlat);     // only the smallest tiles sum on two levels
         // all tiles split, or only those of the ragged last round (the full rounds in front stay whole)
@@ -303,6 +305,29 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
                     if (us < best_us) { best_us = us; best = {st.shape, ranges, rl.len, (uint32_t)(j * cus), K <= md.urgent_max_k ? 1u : 0u}; }
                 }
             }
+        }
+    }
+    // fp16, more 256 x 256 tiles than CUs: the full rounds stay whole and the few tiles of the last round go on 2 to 8 ranges
+    // each (one workgroup per CU, so a last round of R tiles otherwise leaves all but R CUs idle for a whole tile's time).
+    // 22.7 ns per k step of a round on a full chip, 17.4 where at most half the CUs are busy (the power cap); the last
+    // workgroup of a tile reads its 32 pieces per lane and slot in two trips of about 2 us.  Measured: 7000^3 (784 tiles:
+    // 768 + 16 on 7 ranges) 602 -> 533 us, 4352 x 4352 x 8192 (256 + 33 on 4) 313 -> 249, 6948 x 4688 x 5282 (512 + 20 on 5)
+    // 315 -> 291, 4098 x 7824 x 5104 302 -> 281, 2023 x 8829 x 4246 153 -> 142.  Held against the whole product as the
+    // tile cost model prices it (for full rounds of 128 x 128 tiles the rates above are too kind).
+    if (elem_bytes == 2 && md.n_tiles > 2 && md.tiles[2].shape == TILE_LARGE) {
+        const SplitTile& st = md.tiles[2];
+        const uint64_t t = tiles_of(TILE_LARGE), rounds = t / cus, rest = t % cus;
+        const uint32_t k_whole = (K + md.len_align - 1) / md.len_align * md.len_align;
+        double bar = best.splits > 1 ? best_us : whole_us_by_cost / 1.03;
+        if (whole_us / 1.04 < bar && whole_shape == TILE_LARGE) bar = whole_us / 1.04;
+        for (uint32_t p = 2; rounds >= 1 && rest > 0 && p <= kSplitFlat && p <= max_p && rest * p <= cus; ++p) {
+            const RangeLen rl = range_len(K, p, md.len_align);
+            if (rl.ranges < 2) continue;
+            const uint64_t wgs = rest * rl.ranges;
+            const double lone = wgs <= cus / 2 ? 17.4 : 17.4 + (st.ns_per_k[1] - 17.4) * (double)(wgs - cus / 2) / (double)(cus - cus / 2);
+            const double us = kLaunch + ((double)rounds * k_whole * st.ns_per_k[1] + (double)rl.longest * lone) * 1e-3 + md.us_fixed +
+                              md.us_per_trip * rl.ranges * (st.pieces / 16) + md.us_per_mb * rl.ranges * out_mb * (double)rest / (double)t;
+            if (us < bar) { bar = us; best_us = us; best = {TILE_LARGE, rl.ranges, rl.len, (uint32_t)(rounds * cus), 0}; }
         }
     }
     return best;

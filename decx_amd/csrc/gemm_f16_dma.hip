@@ -450,8 +450,8 @@ int launch_dma(const GemmArgs& args, hipStream_t stream)
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     const uint32_t nb = g.tiles_m * g.tiles_n;
-    if (g.split_len) {                                     // the planner splits K on the two smaller tiles only
-        if constexpr (BM <= 128 && BN <= 128) {
+    if (g.split_len) {                                     // (the tiles of 192 rows or columns have no split form)
+        if constexpr ((BM <= 128 && BN <= 128) || (BM == 256 && BN == 256)) {
             const uint32_t splits = g.split_count;
             hipLaunchKernelGGL((gemm_f16_dma_kernel<BM, BN, WAVES_M, WAVES_N, BK, STAGES, true>), dim3(g.split_first + (nb - g.split_first) * splits),
                                dim3(WAVES_M * WAVES_N * 64), 0, stream, g);

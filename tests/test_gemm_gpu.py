@@ -767,3 +767,46 @@ def test_f16_tiles_between_the_two_largest_are_planned_and_right(hip, oracle, M,
     assert float(np.max(np.abs(have - want))) <= 2e-3 * float(np.max(np.abs(want))) + 0.05 * np.sqrt(M)
     forced = {(192, 192): 3, (192, 256): 4, (256, 192): 5}[(tile_m, tile_n)]
     assert np.array_equal(run(hip, A, B, tile=forced).view(np.uint16), got.view(np.uint16))
+
+
+@pytest.mark.parametrize("M,N,K,with_c", [(4300, 4352, 3000, False), (4352, 4352, 4096, True)])
+def test_f16_last_round_of_the_largest_tiles_split_along_k(hip, oracle, M, N, K, with_c):
+    """More 256 x 256 tiles than CUs: the full rounds stay whole, the few tiles of the last round are cut along K and
+    summed in range order inside the launch.  The plan says so; sampled rows (from whole and from split tiles) hold
+    against the oracle, a column checksum covers every element, two runs agree bit for bit, D's padding stays."""
+    p = hip.plan(2, M, N, K)
+    tiles = -(-M // 256) * -(-N // 256)
+    assert (p.tile_m, p.tile_n) == (256, 256) and p.k_splits > 1 and p.whole_tiles == tiles // 256 * 256
+    assert p.grid == p.whole_tiles + (tiles - p.whole_tiles) * p.k_splits
+    need = hip.lib().decx_hip_gemm_workspace(2, M, N, K)
+    assert need == (tiles - p.whole_tiles) * p.k_splits * 256 * 256 * 4
+    A = synth.normal_half(M, K, 181); B = synth.normal_half(K, N, 182)
+    C = synth.normal_half(M, N, 183) if with_c else None
+    pk, pn = device_pitch(K, np.float16), device_pitch(N, np.float16)
+    dA = hip.DeviceMatrix(M, K, np.float16, pk, A, pad_value=np.nan); dB = hip.DeviceMatrix(K, N, np.float16, pn, B, pad_value=np.nan)
+    dC = hip.DeviceMatrix(M, N, np.float16, pn, C, pad_value=np.nan) if with_c else None
+    ws = hip.DeviceMatrix(1, need // 4, np.float32)
+    ws.upload_raw(np.full((1, ws.pitch), np.nan, np.float32))
+    outs = []
+    for _ in range(2):
+        dD = hip.DeviceMatrix(M, N, np.float16, pn)
+        dD.upload_raw(np.full((M, pn), -12345.0, np.float16))
+        hip.gemm(dA, dB, dD, dC, 0.5 if with_c else 1.0, -2.0 if with_c else 1.0, workspace=ws)
+        hip.sync()
+        raw = dD.download_raw()
+        assert np.all(raw[:, N:] == np.float16(-12345.0))
+        outs.append(raw[:, :N].copy())
+        dD.free()
+    assert np.array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
+    got = outs[0]
+    rows = np.unique(np.concatenate([[0, 255, 256, M - 257, M - 256, M - 2, M - 1], sample_rows(M, 40, 19)])).astype(np.uint32)
+    ref = oracle.gemm_f16(A, B, C, 0.5, -2.0, rows=rows) if with_c else oracle.gemm_f16(A, B, rows=rows)
+    assert rel_err(got[rows], ref, K) <= TOL_F16
+    want = A.astype(np.float64).sum(axis=0) @ B.astype(np.float64)
+    if with_c:
+        want = 0.5 * want - 2.0 * C.astype(np.float64).sum(axis=0)
+    have = got.astype(np.float64).sum(axis=0)
+    assert float(np.max(np.abs(have - want))) <= 2e-3 * float(np.max(np.abs(want))) + 0.05 * np.sqrt(M)
+    for d in (dA, dB, dC, ws):
+        if d is not None:
+            d.free()
