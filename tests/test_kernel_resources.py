@@ -62,8 +62,12 @@ def test_fp16_and_fp64_kernels_keep_their_workgroups_per_cu(tmp_path):
     r = resource_report("gemm_f16_dma.hip", tmp_path)
     for k, (waves, scratch) in r.items():
         assert scratch == 0, (k, "spills")
-    waves, _ = find(r, "gemm_f16_dma_kernelILi256ELi256ELi2ELi4ELi64ELi2ELb0E")          # 8 wavefronts, one workgroup per CU
-    assert waves >= 2
+    for split in (0, 1):                                                                # 8 wavefronts, one workgroup per CU; whole and
+        waves, _ = find(r, "gemm_f16_dma_kernelILi256ELi256ELi2ELi4ELi64ELi2ELb%dE" % split)   # on ranges of K (the last round's tiles)
+        assert waves >= 2, split
+    for shape in ("Li192ELi192ELi4ELi2E", "Li192ELi256ELi2ELi4E", "Li256ELi192ELi4ELi2E"):    # the tiles of 192 rows or columns: the same
+        waves, _ = find(r, "gemm_f16_dma_kernelI" + shape + "Li64ELi2ELb0E")
+        assert waves >= 2, shape
     # (the compiler's figure counts LDS in: the rings of 4 stages are those of workgroups that have a CU to themselves)
     for stages, want in ((2, 4), (4, 2)):                                               # 128 x 128, 8 wavefronts: two per CU / one
         for split in (0, 1):
