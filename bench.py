@@ -40,59 +40,67 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
 # ("plan": what decx_hip_gemm_plan reported then).
 MEASURED_TRAFFIC = {
     "fp32_8192": {"plan": {"tile": [256, 128], "grid": 2048, "k_splits": 1, "whole_tiles": 0},
-             "bytes": 5.67e9, "counters": "FETCH_SIZE 2.6361e6 x 2.0 KiB + WRITE_SIZE 2.621e5 KiB (FETCH_SIZE 2.64e6 ... 3.40e6 from run to run)",
+             "bytes": 5.67e9, "counters": "FETCH_SIZE 2.6357e6 x 2.0 KiB + WRITE_SIZE 2.621e5 KiB (FETCH_SIZE 2.64e6 ... 3.40e6 from run to run)",
                   "kernel": "gemm_f32_dma_kernel<256, 128, 2, 2, 16, 2, false, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                  "source_sha256": "76fb449e905c676f571eeadb730abe3ca3c578d0851a8ba3d400b84d9dac7646", "profile": "profiles/gemm_f32_dma_fp32_8192cubed.md"},
+                  "source_sha256": "05e995711ad2ff03fbcdb66fe8e73d86fadc8c04529cec00e667e61192f79bc9", "profile": "profiles/gemm_f32_dma_fp32_8192cubed.md"},
     "fp16_4096": {"plan": {"tile": [256, 256], "grid": 256, "k_splits": 1, "whole_tiles": 0},
              "bytes": 2.35e8, "counters": "FETCH_SIZE 98 543 x 2.0 KiB + WRITE_SIZE 32 772 KiB",
                   "kernel": "gemm_f16_dma_kernel<256, 256, 2, 4, 64, 2, false>", "source": "decx_amd/csrc/gemm_f16_dma.hip",
-                  "source_sha256": "01ecb755392386c03aae0f5c0f2b46e2726495319ab46b6fdf98e9d4d8ca4dbe", "profile": "profiles/gemm_f16_dma_fp16_4096cubed.md"},
+                  "source_sha256": "2b04e868882c6407c3754860b2f2ac9b2e3ee34ede28e59ee9a4296e973c1d22", "profile": "profiles/gemm_f16_dma_fp16_4096cubed.md"},
+    "fp16_3000": {"plan": {"tile": [192, 192], "grid": 256, "k_splits": 1, "whole_tiles": 0},
+        "bytes": 1.29e8, "counters": "FETCH_SIZE 53 033 x 2.0 KiB + WRITE_SIZE 19 829 KiB",
+                  "kernel": "gemm_f16_dma_kernel<192, 192, 4, 2, 64, 2, false>", "source": "decx_amd/csrc/gemm_f16_dma.hip",
+                  "source_sha256": "2b04e868882c6407c3754860b2f2ac9b2e3ee34ede28e59ee9a4296e973c1d22", "profile": "profiles/gemm_f16_dma_tiles_of_192_and_last_round_split.md"},
+    "fp16_7000": {"plan": {"tile": [256, 256], "grid": 848, "k_splits": 5, "whole_tiles": 768},
+        "bytes": 1.27e9, "counters": "FETCH_SIZE 563 674 x 2.0 KiB + WRITE_SIZE 116 314 KiB (operands, the output, and the slots of the 16 tiles that are split in five)",
+                  "kernel": "gemm_f16_dma_kernel<256, 256, 2, 4, 64, 2, true>", "source": "decx_amd/csrc/gemm_f16_dma.hip",
+                  "source_sha256": "2b04e868882c6407c3754860b2f2ac9b2e3ee34ede28e59ee9a4296e973c1d22", "profile": "profiles/gemm_f16_dma_tiles_of_192_and_last_round_split.md"},
     "fp64_4096": {"plan": {"tile": [256, 128], "grid": 512, "k_splits": 1, "whole_tiles": 0},
              "bytes": 1.21e9, "counters": "FETCH_SIZE 524 460 x 2.0 KiB + WRITE_SIZE 131 099 KiB",
                   "kernel": "gemm_f64_dma_kernel<256, 128, 4, 2, 16, 3, false>", "source": "decx_amd/csrc/gemm_f64.hip",
-                  "source_sha256": "a35256187572bedc339c2dec0b155b1a87bc39fb226006a00774161acea7cdf0", "profile": "profiles/gemm_f64_dma_fp64_4096cubed.md"},
+                  "source_sha256": "9b5e3fa596b998df4fc2b5621237519022c52fca841bb3593d9a27a39c34f335", "profile": "profiles/gemm_f64_dma_fp64_4096cubed.md"},
     "fp32_1024": {"plan": {"tile": [64, 64], "grid": 256, "k_splits": 1, "whole_tiles": 0},
-             "bytes": 2.95e7, "counters": "FETCH_SIZE 12 335 x 2.0 KiB + WRITE_SIZE 4 096 KiB",
+             "bytes": 2.95e7, "counters": "FETCH_SIZE 12 345 x 2.0 KiB + WRITE_SIZE 4 096 KiB",
                   "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                  "source_sha256": "76fb449e905c676f571eeadb730abe3ca3c578d0851a8ba3d400b84d9dac7646", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+                  "source_sha256": "05e995711ad2ff03fbcdb66fe8e73d86fadc8c04529cec00e667e61192f79bc9", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
     "fp32_ragged": {"plan": {"tile": [64, 64], "grid": 512, "k_splits": 2, "whole_tiles": 256},
-               "bytes": 4.44e7, "counters": "FETCH_SIZE 16 659 x 2.0 KiB + WRITE_SIZE 9 983 KiB (operands, and the slots of the 128 tiles that are split in two; 256 tiles are whole)",
+               "bytes": 4.43e7, "counters": "FETCH_SIZE 16 662 x 2.0 KiB + WRITE_SIZE 9 983 KiB (operands, and the slots of the 128 tiles that are split in two; 256 tiles are whole)",
                     "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                    "source_sha256": "76fb449e905c676f571eeadb730abe3ca3c578d0851a8ba3d400b84d9dac7646", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+                    "source_sha256": "05e995711ad2ff03fbcdb66fe8e73d86fadc8c04529cec00e667e61192f79bc9", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
     "fp32_ragged_abc": {"plan": {"tile": [64, 64], "grid": 512, "k_splits": 2, "whole_tiles": 256},
-                   "bytes": 5.04e7, "counters": "FETCH_SIZE 19 601 x 2.0 KiB + WRITE_SIZE 9 983 KiB",
+                   "bytes": 5.04e7, "counters": "FETCH_SIZE 19 595 x 2.0 KiB + WRITE_SIZE 9 983 KiB",
                         "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, true>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                        "source_sha256": "76fb449e905c676f571eeadb730abe3ca3c578d0851a8ba3d400b84d9dac7646", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+                        "source_sha256": "05e995711ad2ff03fbcdb66fe8e73d86fadc8c04529cec00e667e61192f79bc9", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
     "fp32_tall_skinny": {"plan": {"tile": [256, 128], "grid": 512, "k_splits": 1, "whole_tiles": 0},
-                    "bytes": 3.58e8, "counters": "FETCH_SIZE 141 987 x 2.0 KiB + WRITE_SIZE 65 536 KiB",
+                    "bytes": 3.58e8, "counters": "FETCH_SIZE 142 002 x 2.0 KiB + WRITE_SIZE 65 541 KiB",
                          "kernel": "gemm_f32_dma_kernel<256, 128, 2, 2, 16, 2, false, 0, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                         "source_sha256": "76fb449e905c676f571eeadb730abe3ca3c578d0851a8ba3d400b84d9dac7646", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
+                         "source_sha256": "05e995711ad2ff03fbcdb66fe8e73d86fadc8c04529cec00e667e61192f79bc9", "profile": "profiles/gemm_f32_dma_small_and_ragged.md"},
     "fp32_mid_long_k": {"plan": {"tile": [64, 64], "grid": 512, "k_splits": 4, "whole_tiles": 256},
-                   "bytes": 3.12e8, "counters": "FETCH_SIZE 147 752 x 2.0 KiB + WRITE_SIZE 9 226 KiB (operands, and the slots of the 64 tiles that are split in four; 256 tiles are whole)",
+                   "bytes": 3.12e8, "counters": "FETCH_SIZE 147 815 x 2.0 KiB + WRITE_SIZE 9 226 KiB (operands, and the slots of the 64 tiles that are split in four; 256 tiles are whole)",
                         "kernel": "gemm_f32_dma_kernel<64, 64, 2, 2, 32, 2, true, 0, true, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-                        "source_sha256": "76fb449e905c676f571eeadb730abe3ca3c578d0851a8ba3d400b84d9dac7646", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
+                        "source_sha256": "05e995711ad2ff03fbcdb66fe8e73d86fadc8c04529cec00e667e61192f79bc9", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
     "fp32_gemv": {"plan": {"tile": [32, 1], "grid": 256, "k_splits": 1, "whole_tiles": 0},
-             "bytes": 2.70e8, "counters": "FETCH_SIZE (131 258 + 522) x 2.0 KiB + WRITE_SIZE (256 + 32) KiB: matrix-vector kernel + the copy of x",
+             "bytes": 2.69e8, "counters": "FETCH_SIZE 131 258 x 2.0 KiB + WRITE_SIZE 32 KiB (x and y are dense columns)",
                   "kernel": "gemv_kernel<float, float, 2, 1>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "f9881524ceb3a6641140288364cd04af404cc4af5f2621b325a961744ac47258", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "a71aab952629f211b96873f786e22f30f3fd404ebf5bdd1262aadd103806703e", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp32_gevm": {"plan": {"tile": [1, 32], "grid": 256, "k_splits": 1, "whole_tiles": 0},
              "bytes": 2.69e8, "counters": "FETCH_SIZE 131 233 x 2.0 KiB + WRITE_SIZE 32 KiB",
                   "kernel": "gevm_kernel<float, float, 8>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "f9881524ceb3a6641140288364cd04af404cc4af5f2621b325a961744ac47258", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "a71aab952629f211b96873f786e22f30f3fd404ebf5bdd1262aadd103806703e", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp16_gemv": {"plan": {"tile": [32, 1], "grid": 256, "k_splits": 1, "whole_tiles": 0},
-             "bytes": 1.36e8, "counters": "FETCH_SIZE (65 647 + 522) x 2.0 KiB + WRITE_SIZE (256 + 16) KiB: matrix-vector kernel + the copy of x",
+             "bytes": 1.34e8, "counters": "FETCH_SIZE 65 647 x 2.0 KiB + WRITE_SIZE 16 KiB (x and y are dense columns)",
                   "kernel": "gemv_kernel<_Float16, _Float16, 2, 1>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "f9881524ceb3a6641140288364cd04af404cc4af5f2621b325a961744ac47258", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "a71aab952629f211b96873f786e22f30f3fd404ebf5bdd1262aadd103806703e", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp16_gevm": {"plan": {"tile": [1, 64], "grid": 256, "k_splits": 2, "whole_tiles": 0},
              "bytes": 1.35e8, "counters": "FETCH_SIZE 65 685 x 2.0 KiB + WRITE_SIZE 92 KiB",
                   "kernel": "gevm_kernel<_Float16, _Float16, 8>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "f9881524ceb3a6641140288364cd04af404cc4af5f2621b325a961744ac47258", "profile": "profiles/gemv_gevm_8192x8192.md"},
-    "conv2d": {"bytes": 1.08e8, "counters": "FETCH_SIZE 20 512 x 2.0 KiB + WRITE_SIZE 64 559 KiB",
+                  "source_sha256": "a71aab952629f211b96873f786e22f30f3fd404ebf5bdd1262aadd103806703e", "profile": "profiles/gemv_gevm_8192x8192.md"},
+    "conv2d": {"bytes": 1.08e8, "counters": "FETCH_SIZE 20 527 x 2.0 KiB + WRITE_SIZE 64 546 KiB",
                "kernel": "gemm_f32_dma_kernel<256, 256, 2, 4, 16, 4, false, 2, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
-               "source_sha256": "76fb449e905c676f571eeadb730abe3ca3c578d0851a8ba3d400b84d9dac7646", "profile": "profiles/conv2d_implicit_gemm_256x256x112_3x3x256.md"},
-    "conv2d_rgb": {"bytes": 1.01e8, "counters": "FETCH_SIZE 16 457 x 2.0 KiB + WRITE_SIZE 66 130 KiB",
+               "source_sha256": "05e995711ad2ff03fbcdb66fe8e73d86fadc8c04529cec00e667e61192f79bc9", "profile": "profiles/conv2d_implicit_gemm_256x256x112_3x3x256.md"},
+    "conv2d_rgb": {"bytes": 1.01e8, "counters": "FETCH_SIZE 16 457 x 2.0 KiB + WRITE_SIZE 66 138 KiB",
                    "kernel": "conv2d_direct_kernel<8, 3>", "source": "decx_amd/csrc/conv_direct.hip",
-                   "source_sha256": "84ef56bdb16515a688bf81f1e7616863ba4917ab9f569a9353d866eeee6872e4", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
+                   "source_sha256": "c7eb7cf36f24f0ea5cbad9b81e882fd40584839840d91afe1e302abf4bd8fcc0", "profile": "profiles/split_k_mid_size_and_direct_conv.md"},
 }
 
 
@@ -151,6 +159,8 @@ WORKLOADS = {
     # name: (dtype, M, N, K, bound, config number for seeds, description)
     "fp32_8192": ("f32", 8192, 8192, 8192, "mfma", 4, "fp32 GEMM C=A.B M=N=K=8192, uniform[-1,1]"),
     "fp16_4096": ("f16", 4096, 4096, 4096, "mfma", 3, "fp16 GEMM (fp32 accumulate, fp16 out) M=N=K=4096, normal(0,0.5) clipped to [-4,4]"),
+    "fp16_3000": ("f16", 3000, 3000, 3000, "mfma", 9, "fp16 GEMM M=N=K=3000 (256 tiles of 192 x 192 where 256 x 256 gives 144 for 256 CUs), normal(0,0.5)"),
+    "fp16_7000": ("f16", 7000, 7000, 7000, "mfma", 10, "fp16 GEMM M=N=K=7000 (784 tiles of 256 x 256: three rounds whole, the 16 of the last round split along K), normal(0,0.5)"),
     "fp64_4096": ("f64", 4096, 4096, 4096, "mfma", 7, "fp64 GEMM M=N=K=4096, uniform[-1,1]"),
     "fp32_1024": ("f32", 1024, 1024, 1024, "mfma", 1, "fp32 GEMM M=N=K=1024, uniform[-1,1]"),
     "fp32_ragged": ("f32", 1000, 1500, 777, "mfma", 2, "fp32 GEMM M=1000 N=1500 K=777, uniform[-1,1]"),
@@ -320,10 +330,18 @@ def copy_rate(steps=10, warmup=3):
     for _ in range(steps):
         hip.check(hip.lib().decx_hip_calibration_copy(dst.ptr, src.ptr, n, None))
     ms = timer.stop() / steps
+    # and a write-only pass over the same gigabyte (the runtime's fill kernel behind decx_hip_memset_async)
+    for _ in range(warmup):
+        hip.check(hip.lib().decx_hip_memset_async(dst.ptr, 0, n, None))
+    hip.sync()
+    timer.start()
+    for _ in range(steps):
+        hip.check(hip.lib().decx_hip_memset_async(dst.ptr, 0, n, None))
+    fill_ms = timer.stop() / steps
     for d in (src, dst):
         d.free()
     return {"value": round(2 * n / ms / 1e6, 1), "unit": "GB/s", "what": "calibration copy kernel, 1 GiB read + 1 GiB written per launch",
-            "kernel_ms": round(ms, 4)}
+            "kernel_ms": round(ms, 4), "write_only_gbs": round(n / fill_ms / 1e6, 1), "write_only_what": "fill of 1 GiB (hipMemsetAsync)"}
 
 
 def add_sustained(out, sustained):
@@ -764,7 +782,7 @@ def main():
 
     main_out, inputs = run_workload(args.workload, args.steps, args.warmup, keep_inputs=not args.no_cpu,
                                     settle_s=0.25 if args.workload != "fp32_8192" else 0.0)
-    if args.workload == "fp16_4096":
+    if args.workload == "fp16_4096" and not args.no_extra:
         add_sustained(main_out, sustained_mfma())
         main_out["roofline"]["on_zero_operands"] = zero_operand_rate("fp16_4096")
     line = {
@@ -816,6 +834,7 @@ def main():
         rgb = run_conv(200, args.warmup, c=CONV_RGB, parity=not args.no_cpu)
         rgb["roofline"]["copy_rate_gbs"] = copy["value"]           # what this board moves when half the traffic is writes
         rgb["roofline"]["frac_of_copy_rate"] = round(rgb["roofline"]["achieved"] / copy["value"], 4)
+        rgb["roofline"]["write_only_gbs"] = copy["write_only_gbs"]  # ... and when all of it is (73 % of this workload's bytes are)
         others.append(rgb)
         others.append(run_complex(False, 4096, args.steps, args.warmup, parity=not args.no_cpu))
         others.append(run_complex(True, 2048, 50, args.warmup, parity=not args.no_cpu))
