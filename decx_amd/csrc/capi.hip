@@ -166,7 +166,7 @@ int check_gemm(const void* A, const void* B, const void* C, const void* D, uint3
 //   memory per 16 pieces a lane loads (us_per_trip: where several workgroups share a CU the others hide most of it).
 // fp32 fitted to 20 output shapes x K = 777 ... 16384 x 1 ... 8 ranges, fp16 and fp64 to 12 and 9 shapes x 2 ... 32
 // ranges: the estimate is within 4 % of the measurement on most, the pick within 1 % (fp16: 2.5 %) of the best on
-// average.  The whole product is kept unless the split promises 4 %.
+// average.  The whole product is kept unless the split promises 3 % (4 % left a launch-bound fp16 shape of the held-out sweep 10 % off its best plan).
 struct SplitChoice { int shape; uint32_t splits, len, first, urgent; };     // first: tiles in front that stay whole; urgent: GemmArgs::split_urgent
 struct SplitTile {
     int shape, fit, pieces;          // size class, workgroups per CU, 16-byte pieces of accumulators per lane
@@ -256,7 +256,7 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
         if (md.tiles[i].shape == whole_shape && whole_shape != TILE_LARGE)
             whole_us = estimate(md.tiles[i], tiles_of(whole_shape), (K + md.len_align - 1) / md.len_align * md.len_align, 1);
     SplitChoice best = {whole_shape, 1, 0, 0};
-    double best_us = whole_us / 1.04;
+    double best_us = whole_us / 1.03;
     const uint32_t max_p = K / 256 < 64u ? K / 256 : 64u;
     for (int i = 0; i < md.n_tiles; ++i) {
         const SplitTile& st = md.tiles[i];
