@@ -318,6 +318,8 @@ SplitChoice split_plan_model(int elem_bytes, uint32_t M, uint32_t N, uint32_t K,
         const SplitTile& st = md.tiles[2];
         const uint64_t t = tiles_of(TILE_LARGE), rounds = t / cus, rest = t % cus;
         const uint32_t k_whole = (K + md.len_align - 1) / md.len_align * md.len_align;
+        // What it must beat: the best plan so far, and by 4 % (not 3) a whole product on these same tiles -- both estimates
+        // then rest on the same rate for the full rounds, and a promise smaller than that did not show in the measurements.
         double bar = best.splits > 1 ? best_us : whole_us_by_cost / 1.03;
         if (whole_us / 1.04 < bar && whole_shape == TILE_LARGE) bar = whole_us / 1.04;
         for (uint32_t p = 2; rounds >= 1 && rest > 0 && p <= kSplitFlat && p <= max_p && rest * p <= cus; ++p) {
