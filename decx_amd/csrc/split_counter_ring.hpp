@@ -9,9 +9,10 @@
 // A window whose earlier owners cannot be shown to be over is NOT handed out: take() returns kNone and the caller runs
 // the product unsplit.  Events are only recorded once launches have been seen on more than one stream; a caller with
 // one stream pays nothing.
-// Launches recorded into a graph are replayed at times the host does not see: they get windows of their own from
-// the top of the array, which are never handed out again (the ring below them shrinks), and only while no other split
-// launch is in flight.
+// Launches recorded into a graph are replayed at times the host does not see: they get windows of their own from the
+// upper half of the array, which the ring never enters and which are never handed out twice.  Nothing has to be proved
+// over for them, so recording a graph asks the runtime nothing (a query made while a stream records can end the
+// recording with an error).
 #pragma once
 #include <cstddef>
 #include <cstdint>
@@ -34,7 +35,7 @@ public:
     static constexpr uint32_t kNone = 0xffffffffu;
     struct Stats { uint64_t taken, wraps, refused, events, reserved; };
 
-    explicit CounterRing(uint32_t capacity) : capacity_(capacity), top_(capacity) {}
+    explicit CounterRing(uint32_t capacity) : capacity_(capacity), top_(capacity / 2), graph_top_(capacity) {}
 
     // A window of `n` counters for a launch on `stream` (`key`: the stream's identity -- the handle, made unique per
     // thread where one handle names a stream per thread).  Returns its first index, or kNone.  `capturing`: the launch
@@ -43,8 +44,8 @@ public:
     uint32_t take(CounterRingRuntime& rt, void* stream, uint64_t key, uint32_t n, bool capturing, uint64_t* ticket = nullptr)
     {
         if (ticket) *ticket = 0;
+        if (capturing) return reserve(n);
         if (n == 0 || n > top_) { ++stats_.refused; return kNone; }
-        if (capturing) return reserve(rt, n);
         if (have_last_ && key != last_key_) multi_stream_ = true;
         last_key_ = key; have_last_ = true;
         uint32_t begin = cursor_;
@@ -82,7 +83,8 @@ public:
         }
     }
 
-    // Forgets every owner (the caller has waited for the device, or has put the counters back to zero itself).
+    // Forgets every owner (the caller has waited for the device, or has put the counters back to zero itself).  Windows
+    // of graph launches stay theirs: the graphs still exist.
     void reset(CounterRingRuntime& rt)
     {
         for (Owner& o : owners_) if (o.event) rt.release_event(o.event);
@@ -90,34 +92,28 @@ public:
         cursor_ = 0;
     }
 
-    uint32_t ring_size() const { return top_; }           // what the graph launches have left of it
+    uint32_t ring_size() const { return top_; }           // the lower half: what launches outside graphs go round in
+    uint32_t graph_left() const { return graph_top_ - top_; }
     uint32_t capacity() const { return capacity_; }
     const Stats& stats() const { return stats_; }
 
 private:
     struct Owner { uint32_t begin, end; void* stream; uint64_t key; void* event; uint64_t seq; };
 
-    // Windows for graph launches come off the top, at a moment when every launch the ring knows of is over: an owner
-    // that a later launch on its own stream has replaced is no longer listed although it may still run, and only
-    // the sequential walk of the cursor is safe against those, not a cut at an arbitrary place.
-    uint32_t reserve(CounterRingRuntime& rt, uint32_t n)
+    // Windows for graph launches come off the top of the upper half, each once.
+    uint32_t reserve(uint32_t n)
     {
-        if (n > top_ / 2) { ++stats_.refused; return kNone; }        // the ring keeps at least half of the array
-        for (size_t i = 0; i < owners_.size(); ++i)
-            if (!over(rt, i, kNoKey)) { ++stats_.refused; return kNone; }
-        for (Owner& o : owners_) if (o.event) rt.release_event(o.event);
-        owners_.clear();
-        top_ -= n;
-        if (cursor_ > top_) cursor_ = top_;
+        if (n == 0 || n > graph_top_ - top_) { ++stats_.refused; return kNone; }
+        graph_top_ -= n;
         stats_.reserved += n;
-        return top_;
+        return graph_top_;
     }
 
     // Is the launch of owner i over, as far as a new launch on the stream `key` is concerned?
     bool over(CounterRingRuntime& rt, size_t i, uint64_t key)
     {
         const Owner& o = owners_[i];
-        if (key != kNoKey && o.key == key) return true;              // same stream: in order
+        if (o.key == key) return true;                               // same stream: in order
         if (o.event && rt.event_done(o.event)) return true;
         for (size_t j = i + 1; j < owners_.size(); ++j)              // a later launch on its stream whose event is done covers it
             if (owners_[j].key == o.key && owners_[j].event && rt.event_done(owners_[j].event)) return true;
@@ -143,8 +139,7 @@ private:
         return true;
     }
 
-    static constexpr uint64_t kNoKey = ~0ull;
-    uint32_t capacity_, top_;
+    uint32_t capacity_, top_, graph_top_;
     uint32_t cursor_ = 0;
     std::deque<Owner> owners_;          // in the order taken = ring order starting at the oldest
     bool multi_stream_ = false, have_last_ = false;

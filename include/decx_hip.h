@@ -142,12 +142,13 @@ DECX_HIP_API int decx_hip_gemm_f32(const float* A, const float* B, const float* 
  * Plays the part of the scratch the reference's planner keeps for itself (cuda_GEMM_LS_planner: the transposed
  * A, srcs/modules/BLAS/GEMM/CUDA/large_squares/common/cuda_GEMM_LS_planner.cu:95-160).
  * Besides the workspace, a split launch uses a window of the library's own counter array (65 536 words per GPU, all
- * zero between launches).  The library hands a window to a new launch only when the launches that had it before are
- * known to be over -- they went to the same stream, an event recorded behind them has completed, or their stream is
- * idle -- and otherwise runs the product unsplit, which is never an error.  A split launch that is recorded into a
- * HIP graph keeps its window for the life of the process (the graph may be replayed at any time): at most half of
- * the array can go that way, later recordings run unsplit.  Callers must not destroy a stream while split launches
- * are in flight on it.  If a launch was cut short (a device fault, a reset), decx_hip_reset_split_counters() waits
+ * zero between launches).  Launches outside graphs go round the lower half: the library hands a window to a new launch
+ * only when the launches that had it before are known to be over -- they went to the same stream, an event recorded
+ * behind them has completed, or their stream is idle -- and otherwise runs the product unsplit, which is never an
+ * error.  A split launch that is recorded into a HIP graph gets a window of the upper half and keeps it for the life
+ * of the process (the graph may be replayed at any time; recording asks the runtime nothing but whether the stream is
+ * recording); when that half is used up, later recordings run unsplit.  A graph's replays must not overlap each other.
+ * Callers must not destroy a stream while split launches are in flight on it.  If a launch was cut short (a device fault, a reset), decx_hip_reset_split_counters() waits
  * for the device, puts every counter back to zero and forgets who owned what. */
 DECX_HIP_API size_t decx_hip_gemm_f32_workspace(uint32_t M, uint32_t N, uint32_t K);
 DECX_HIP_API int decx_hip_reset_split_counters(void);

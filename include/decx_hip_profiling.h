@@ -42,7 +42,7 @@ DECX_HIP_API int decx_hip_gemm_forced_plan(int elem_bytes, const void* A, const 
 /* What the split-K counter windows of the current device have seen so far: out[0] windows handed out, out[1] times
  * the ring wrapped round, out[2] requests refused (the product then ran unsplit), out[3] events recorded (only once
  * launches have come from more than one stream), out[4] counters given to launches recorded into graphs, out[5] the
- * counters left to the ring.  For tests. */
+ * counters the ring goes round in (the lower half of the array; graphs draw on the upper half).  For tests. */
 DECX_HIP_API int decx_hip_split_counter_stats(uint64_t out[6]);
 
 #ifdef __cplusplus

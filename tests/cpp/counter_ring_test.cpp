@@ -1,7 +1,7 @@
 // CPU test of the split-K counter windows (decx_amd/csrc/split_counter_ring.hpp) against a simulated runtime:
 // streams are FIFO queues of launches and event markers that the test advances by hand.  The property that matters:
 // a window handed to a launch never overlaps the window of a launch still queued on ANOTHER stream, nor a window that
-// was given to a graph launch.  Prints "ok <name>" per scenario; any failure aborts with a message.
+// was given to a graph launch (those come from the upper half of the array, which the ring never enters).  Prints "ok <name>" per scenario; any failure aborts with a message.
 #include "../../decx_amd/csrc/split_counter_ring.hpp"
 
 #include <cstdio>
@@ -68,7 +68,7 @@ static uint32_t submit(CounterRing& ring, SimRuntime& rt, int stream, uint32_t n
 
 static void one_stream_wraps_freely()
 {
-    CounterRing ring(1024); SimRuntime rt;
+    CounterRing ring(2 * 1024); SimRuntime rt;
     for (int i = 0; i < 100; ++i) REQUIRE(submit(ring, rt, 0, 100) != CounterRing::kNone);   // never advanced: all queued
     REQUIRE(ring.stats().wraps >= 9 && ring.stats().refused == 0 && ring.stats().events == 0);
     std::puts("ok one_stream_wraps_freely");
@@ -76,7 +76,7 @@ static void one_stream_wraps_freely()
 
 static void second_stream_waits_for_the_first()
 {
-    CounterRing ring(1024); SimRuntime rt;
+    CounterRing ring(2 * 1024); SimRuntime rt;
     for (int i = 0; i < 8; ++i) REQUIRE(submit(ring, rt, 0, 128) == (uint32_t)(128 * i));   // the ring is full of stream 0
     REQUIRE(submit(ring, rt, 1, 128) == CounterRing::kNone);       // stream 0 is busy, its launches carry no events
     REQUIRE(ring.stats().refused == 1);
@@ -95,7 +95,7 @@ static void second_stream_waits_for_the_first()
 
 static void a_later_event_covers_earlier_launches()
 {
-    CounterRing ring(1000); SimRuntime rt;
+    CounterRing ring(2 * 1000); SimRuntime rt;
     REQUIRE(submit(ring, rt, 0, 100) == 0);                        // no event: one stream so far
     REQUIRE(submit(ring, rt, 1, 100) == 100);                      // event
     REQUIRE(submit(ring, rt, 0, 100) == 200);                      // event, behind the first launch of stream 0
@@ -110,26 +110,31 @@ static void a_later_event_covers_earlier_launches()
 
 static void graph_launches_keep_their_windows()
 {
-    CounterRing ring(1024); SimRuntime rt;
-    REQUIRE(submit(ring, rt, 0, 1000) == 0);
+    CounterRing ring(2048); SimRuntime rt;                         // launches outside graphs go round in [0, 1024)
+    REQUIRE(ring.ring_size() == 1024 && ring.graph_left() == 1024);
+    REQUIRE(submit(ring, rt, 0, 1000) == 0);                       // queued, never advanced
     uint64_t ticket = 77;
-    REQUIRE(ring.take(rt, S(1), 1, 100, true, &ticket) == CounterRing::kNone);   // the top is owned by a queued launch of stream 0
-    rt.advance(S(0), 10);
-    REQUIRE(ring.take(rt, S(1), 1, 100, true, &ticket) == 924);
-    REQUIRE(ticket == 0 && ring.ring_size() == 924);
-    REQUIRE(ring.take(rt, S(1), 1, 500, true) == CounterRing::kNone);            // more than half of what is left
-    REQUIRE(ring.take(rt, S(1), 1, 24, true) == 900);
+    // a graph launch asks nothing of the queued one: its windows lie where the ring never goes
+    REQUIRE(ring.take(rt, S(1), 1, 100, true, &ticket) == 1948);
+    REQUIRE(ticket == 0 && ring.ring_size() == 1024 && ring.graph_left() == 924);
+    REQUIRE(ring.take(rt, S(1), 1, 24, true) == 1924);
+    REQUIRE(ring.take(rt, S(1), 1, 901, true) == CounterRing::kNone);            // more than is left up there
+    REQUIRE(ring.take(rt, S(1), 1, 900, true) == 1024);
+    REQUIRE(ring.take(rt, S(1), 1, 1, true) == CounterRing::kNone);
+    REQUIRE(ring.stats().reserved == 1024 && ring.stats().refused == 2);
     for (int i = 0; i < 50; ++i) {
         const uint32_t at = submit(ring, rt, 0, 300);
-        REQUIRE(at != CounterRing::kNone && at + 300 <= 900);
+        REQUIRE(at != CounterRing::kNone && at + 300 <= 1024);
     }
-    REQUIRE(submit(ring, rt, 0, 901) == CounterRing::kNone);
+    REQUIRE(submit(ring, rt, 0, 1025) == CounterRing::kNone);
+    ring.reset(rt);                                                // the graphs still exist: nothing comes back
+    REQUIRE(ring.graph_left() == 0);
     std::puts("ok graph_launches_keep_their_windows");
 }
 
 static void reset_forgets()
 {
-    CounterRing ring(256); SimRuntime rt;
+    CounterRing ring(2 * 256); SimRuntime rt;
     REQUIRE(submit(ring, rt, 0, 256) == 0);
     REQUIRE(submit(ring, rt, 1, 256) == CounterRing::kNone);
     rt.queues.clear();                                             // "the caller has waited for the device"
@@ -140,7 +145,7 @@ static void reset_forgets()
 
 static void random_traffic(unsigned seed, int streams, uint32_t capacity, uint32_t max_n)
 {
-    CounterRing ring(capacity); SimRuntime rt;
+    CounterRing ring(2 * capacity); SimRuntime rt;                  // `capacity` counters to go round in, as many for graphs
     std::mt19937 rng(seed);
     uint64_t handed = 0, refused = 0;
     std::vector<std::pair<uint32_t, uint32_t>> reserved;

@@ -10,7 +10,6 @@ from decx_amd import synth
 pytestmark = pytest.mark.gpu
 
 TOL_F32 = 1e-5
-COUNTERS = 1 << 16
 
 
 @pytest.fixture(scope="module")
@@ -67,7 +66,7 @@ def test_one_stream_walks_the_array_round(hip, oracle):
     assert float(np.max(np.abs(want.astype(np.float64) - ref))) / (float(np.max(np.abs(ref))) * np.sqrt(K)) <= TOL_F32
     per = counters_per_launch(hip, M, N, K)
     before = hip.split_counter_stats()
-    launches = 2 * (COUNTERS // per) + 50
+    launches = 2 * (before["ring"] // per) + 50
     print("one stream:", launches, "launches of", per, "counters", flush=True)
     for i in range(launches):
         prod.launch()
@@ -89,8 +88,8 @@ def test_two_streams_walk_the_array_round(hip):
     plain = [p.alone(split=False) for p in prods]
     streams = [hip.Stream(), hip.Stream()]
     per = sum(counters_per_launch(hip, *s) for s in shapes)
-    rounds = 2 * (COUNTERS // per) + 20
     before = hip.split_counter_stats()
+    rounds = 2 * (before["ring"] // per) + 20
     print("two streams:", rounds, "rounds of", per, "counters", flush=True)
     for i in range(rounds):
         for p, s in zip(prods, streams):
@@ -127,8 +126,8 @@ def test_a_window_of_a_busy_stream_is_not_handed_out(hip, oracle):
     assert not np.array_equal(want_b, plain_b)                  # (the two orders of summation differ in some bit)
     sa, sb = hip.Stream(), hip.Stream()
     per_b = counters_per_launch(hip, 1000, 1500, 777)
-    launches = COUNTERS // per_b + 8
     before = hip.split_counter_stats()
+    launches = before["ring"] // per_b + 8
     print("busy stream: 24 products of", big, "cubed on A, then", launches, "split launches on B", flush=True)
     for _ in range(24):                                         # about 70 ms of work in front of A's split launch
         hip.gemm(dX, dX, dY, stream=sa.handle)
