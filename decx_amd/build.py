@@ -70,7 +70,7 @@ def build_api_test(verbose=False):
     """The C++ program the tests drive the public de:: API with (tests/cpp/de_api_test)."""
     src = os.path.join(ROOT, "tests", "cpp", "de_api_test.cpp")
     out = os.path.join(ROOT, "tests", "cpp", "de_api_test")
-    _run(["g++", "-O1", "-std=c++17", "-Wall", "-I" + os.path.join(ROOT, "include"), src, "-o", out,
+    _run(["g++", "-O1", "-std=c++17", "-Wall", "-pthread", "-I" + os.path.join(ROOT, "include"), src, "-o", out,
           "-L" + LIB, "-lDECX_BLAS_HIP", "-ldecx_hip", "-Wl,-rpath," + LIB, "-Wl,-rpath,$ORIGIN/../../decx_amd/lib"])
     if verbose:
         print("built", out)

@@ -9,6 +9,7 @@
 //   de_api_test hostgemm <dir> <f32|f16> M N K <withC 0|1|2> <pinned 0|1> <repeats>
 //                                         the same through the host-matrix overloads (withC = 2: C is dst);
 //                                         prints the wall time of each repeat
+//   de_api_test threads                   several host threads through GEMM and Memcpy at once, each on matrices of its own
 //   de_api_test tensor_host               tensor / tensor-array layouts and views, no GPU
 //   de_api_test conv <dir> W H C OC KW KH sx sy <extend 0|2>
 //                                         reads image.bin [H][W][C] and kernels.bin [OC][KH][KW][C] (dense fp32),
@@ -26,7 +27,9 @@
 #include <cstring>
 #include <fstream>
 #include <iostream>
+#include <atomic>
 #include <string>
+#include <thread>
 #include <vector>
 
 static int g_failures = 0;
@@ -591,6 +594,103 @@ template <typename T> static int gemm_files(const std::string& dir, de::_DATA_TY
     return out ? 0 : 2;
 }
 
+// Several host threads call GEMM and Memcpy at the same time, each on matrices of its own.  The original allows one
+// caller at a time; this module serialises them, so every thread must get its own product, bit for bit what the same
+// call gave before the threads started.  (The last-error handle is one per process, as in the original: with several
+// callers it says what the latest of them did, so the threads look at their results, not at it.)
+struct ThreadJob {
+    de::_DATA_TYPES_FLAGS_ type; uint32_t M, N, K; bool with_c;
+    de::Matrix *A, *B, *C, *D; de::GPU_Matrix *dA, *dB, *dC, *dD;
+    std::vector<char> want;
+};
+static size_t elem_size(de::_DATA_TYPES_FLAGS_ t) { return t == de::_FP64_ ? 8 : t == de::_FP16_ ? 2 : 4; }
+static void put(de::Matrix& m, de::_DATA_TYPES_FLAGS_ t, uint32_t i, uint32_t j, float v)
+{
+    if (t == de::_FP32_) *m.ptr<float>(i, j) = v;
+    else if (t == de::_FP64_) *m.ptr<double>(i, j) = v;
+    else *m.ptr<de::Half>(i, j) = de::Float2Half(v);
+}
+static void run_job(ThreadJob& jb)
+{
+    if (!jb.with_c) { de::blas::cuda::GEMM(*jb.dA, *jb.dB, *jb.dD); return; }
+    if (jb.type == de::_FP32_) de::blas::cuda::GEMM(*jb.dA, *jb.dB, *jb.dC, *jb.dD, de::Number(0.75f), de::Number(-1.25f));
+    else if (jb.type == de::_FP64_) de::blas::cuda::GEMM(*jb.dA, *jb.dB, *jb.dC, *jb.dD, de::Number(0.75), de::Number(-1.25));
+    else de::blas::cuda::GEMM(*jb.dA, *jb.dB, *jb.dC, *jb.dD, de::Number(de::Float2Half(0.75f)), de::Number(de::Float2Half(-1.25f)));
+}
+static std::vector<char> fetch(ThreadJob& jb)
+{
+    const de::Point2D O(0, 0);
+    de::Memcpy(*jb.D, *jb.dD, O, O, de::Point2D(jb.N, jb.M), de::DECX_MEMCPY_D2H);
+    const size_t row = (size_t)jb.N * elem_size(jb.type);
+    std::vector<char> out((size_t)jb.M * row);
+    for (uint32_t i = 0; i < jb.M; ++i) {
+        const void* src = jb.type == de::_FP32_ ? (const void*)jb.D->ptr<float>(i, 0)
+                        : jb.type == de::_FP64_ ? (const void*)jb.D->ptr<double>(i, 0) : (const void*)jb.D->ptr<de::Half>(i, 0);
+        std::memcpy(out.data() + i * row, src, row);
+    }
+    return out;
+}
+static int threads_checks()
+{
+    de::InitCPUInfo();
+    de::InitCuda();
+    de::ResetLastError();
+    const de::Point2D O(0, 0);
+    // a product split along K, a ragged one with a C term, fp16, fp64, and the two vector corners with their workspaces
+    ThreadJob jobs[] = {{de::_FP32_, 300, 300, 8192, false}, {de::_FP32_, 1000, 1500, 777, true}, {de::_FP16_, 257, 130, 515, true},
+                        {de::_FP64_, 500, 300, 333, true}, {de::_FP32_, 1100, 1, 8200, false}, {de::_FP16_, 1, 513, 33000, false}};
+    const int n_jobs = (int)(sizeof jobs / sizeof jobs[0]);
+    for (int t = 0; t < n_jobs; ++t) {
+        ThreadJob& jb = jobs[t];
+        jb.A = &de::CreateMatrixRef(jb.type, jb.K, jb.M); jb.B = &de::CreateMatrixRef(jb.type, jb.N, jb.K);
+        jb.C = &de::CreateMatrixRef(jb.type, jb.N, jb.M); jb.D = &de::CreateMatrixRef(jb.type, jb.N, jb.M);
+        // small multiples of 1/8: exact in half, different from job to job
+        for (uint32_t i = 0; i < jb.M; ++i) for (uint32_t k = 0; k < jb.K; ++k) put(*jb.A, jb.type, i, k, (float)((int)((i * 7u + k * 13u + t) % 17u) - 8) / 8.f);
+        for (uint32_t k = 0; k < jb.K; ++k) for (uint32_t j = 0; j < jb.N; ++j) put(*jb.B, jb.type, k, j, (float)((int)((k * 5u + j * 11u + 3u * t) % 19u) - 9) / 8.f);
+        for (uint32_t i = 0; i < jb.M; ++i) for (uint32_t j = 0; j < jb.N; ++j) put(*jb.C, jb.type, i, j, (float)((int)((i + 3u * j + t) % 23u) - 11) / 4.f);
+        jb.dA = &de::CreateGPUMatrixRef(jb.type, jb.K, jb.M); jb.dB = &de::CreateGPUMatrixRef(jb.type, jb.N, jb.K);
+        jb.dC = &de::CreateGPUMatrixRef(jb.type, jb.N, jb.M); jb.dD = &de::CreateGPUMatrixRef();
+        CHECK(de::Memcpy(*jb.A, *jb.dA, O, O, de::Point2D(jb.K, jb.M), de::DECX_MEMCPY_H2D).error_type == 0);
+        CHECK(de::Memcpy(*jb.B, *jb.dB, O, O, de::Point2D(jb.N, jb.K), de::DECX_MEMCPY_H2D).error_type == 0);
+        CHECK(de::Memcpy(*jb.C, *jb.dC, O, O, de::Point2D(jb.N, jb.M), de::DECX_MEMCPY_H2D).error_type == 0);
+        run_job(jb);
+        CHECK(de::GetLastError()->error_type == 0);
+        jb.want = fetch(jb);
+        // the product is not all zeros, and job 0 is what its closed form says: small integers over 64, summed exactly
+        bool any = false;
+        for (char c : jb.want) any |= c != 0;
+        CHECK(any);
+    }
+    {
+        const ThreadJob& jb = jobs[0];
+        double worst = 0;
+        for (uint32_t i = 0; i < jb.M; i += 37) for (uint32_t j = 0; j < jb.N; j += 41) {
+            double sum = 0;
+            for (uint32_t k = 0; k < jb.K; ++k)
+                sum += (double)((int)((i * 7u + k * 13u) % 17u) - 8) / 8.0 * ((double)((int)((k * 5u + j * 11u) % 19u) - 9) / 8.0);
+            worst = std::fmax(worst, std::fabs(sum - (double)((const float*)jb.want.data())[(size_t)i * jb.N + j]));
+        }
+        if (worst != 0) std::cerr << "closed form: worst difference " << worst << "\n";
+        CHECK(worst == 0);                                  // every partial sum is a multiple of 1/64 below 2^24 / 64
+    }
+    std::atomic<int> wrong(0), calls(0);
+    std::vector<std::thread> threads;
+    for (int t = 0; t < n_jobs; ++t)
+        threads.emplace_back([&jobs, &wrong, &calls, t]() {
+            ThreadJob& jb = jobs[t];
+            for (int rep = 0; rep < 40; ++rep) {
+                run_job(jb);
+                if (fetch(jb) != jb.want) ++wrong;
+                ++calls;
+            }
+        });
+    for (std::thread& th : threads) th.join();
+    CHECK(wrong.load() == 0);
+    CHECK(calls.load() == 40 * n_jobs);
+    std::cout << "threads: " << n_jobs << " threads x 40 products, " << wrong.load() << " wrong\n";
+    return g_failures == 0 ? 0 : 1;
+}
+
 static int tensor_host_checks()
 {
     // host tensors: width padded to 4 columns, depth to 16 bytes of elements; element (row, column, channel)
@@ -800,6 +900,7 @@ int main(int argc, char** argv)
         rc = std::string(argv[2]) == "f16" ? hostgemm_wall_time<de::Half>(de::_FP16_, M, N, K, repeats, pinned)
                                            : hostgemm_wall_time<float>(de::_FP32_, M, N, K, repeats, pinned);
     }
+    else if (mode == "threads") rc = threads_checks();
     else if (mode == "tensor_host") rc = tensor_host_checks();
     else if (mode == "conv" && argc == 12)
         rc = conv_files(argv[2], std::atoi(argv[3]), std::atoi(argv[4]), std::atoi(argv[5]), std::atoi(argv[6]), std::atoi(argv[7]),
@@ -821,7 +922,7 @@ int main(int argc, char** argv)
                  : std::string(argv[3]) == "f64" ? gemm_files<double>(argv[2], de::_FP64_, M, N, K, with_c, alpha, beta)
                  : gemm_files<float>(argv[2], de::_FP32_, M, N, K, with_c, alpha, beta);
     } else {
-        std::cerr << "usage: de_api_test host | gpu | vector_host | vector_gpu | gemm <dir> <f32|f16> M N K withC alpha beta"
+        std::cerr << "usage: de_api_test host | gpu | threads | vector_host | vector_gpu | gemm <dir> <f32|f16> M N K withC alpha beta"
                      " | vmm <dir> <f32|f16> <mv|vm> W H level | gemmtime <f32|f16> M N K repeats | hostgemmtime <f32|f16> M N K repeats pinned\n";
         return 64;
     }

@@ -64,6 +64,15 @@ def test_gpu_side_closed_forms_and_error_paths():
 
 
 @pytest.mark.gpu
+def test_several_host_threads_each_get_their_own_product():
+    """Six host threads in GEMM and Memcpy at once, each on its own matrices (a product split along K, a ragged one with
+    C, fp16, fp64, the two vector corners): the module serialises them, every result bit-equal to the same call alone."""
+    rc, out = run_exe("threads")
+    assert rc == 0, out
+    assert "0 wrong" in out
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dt,M,N,K,with_c,alpha,beta", [
     ("f32", 1000, 1500, 777, False, 1.0, 1.0),
     ("f32", 1000, 1500, 777, True, 1.0, 1.0),

@@ -157,6 +157,52 @@ def test_a_window_of_a_busy_stream_is_not_handed_out(hip, oracle):
     a.free(); b.free()
 
 
+def test_host_threads_with_streams_of_their_own(hip):
+    """Four host threads launch split products at the same time, each on its own stream, workspace and output: the
+    windows are handed out under the library's lock, and whatever a thread gets (a window, or a refusal while another
+    stream's launch still holds it) its product has the bits of the split or of the unsplit form."""
+    import threading
+    shapes = [(1000, 1500, 777), (300, 300, 8192), (640, 640, 4096), (100, 120, 4096)]
+    prods = [Product(hip, *s, 0x6500 + 16 * i) for i, s in enumerate(shapes)]
+    want = [p.alone() for p in prods]
+    plain = [p.alone(split=False) for p in prods]
+    streams = [hip.Stream() for _ in prods]
+    before = hip.split_counter_stats()
+    wrong = []
+
+    def work(i):
+        p, s = prods[i], streams[i]
+        try:
+            for n in range(400):
+                p.launch(s.handle)
+                if n % 80 == 79:
+                    s.sync()
+                    got = p.dD.download().view(np.uint32)
+                    if not (np.array_equal(got, want[i].view(np.uint32)) or np.array_equal(got, plain[i].view(np.uint32))):
+                        wrong.append((i, n))
+        except Exception as e:                                   # noqa: BLE001 -- reported by the main thread
+            wrong.append((i, repr(e)))
+
+    print("four host threads, 400 split launches each", flush=True)
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(prods))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for s in streams:
+        s.sync()
+    assert not wrong, wrong
+    after = hip.split_counter_stats()
+    assert after["taken"] + after["refused"] - before["taken"] - before["refused"] == 400 * len(prods)
+    assert after["taken"] - before["taken"] >= 400              # most launches do get their window
+    for p, w in zip(prods, want):                               # all counters are back at zero
+        assert np.array_equal(p.alone().view(np.uint32), w.view(np.uint32))
+    for s in streams:
+        s.destroy()
+    for p in prods:
+        p.free()
+
+
 def test_reset_puts_the_counters_back(hip):
     p = Product(hip, 300, 300, 8192, 0x6400)
     want = p.alone()
