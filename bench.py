@@ -82,19 +82,19 @@ MEASURED_TRAFFIC = {
     "fp32_gemv": {"plan": {"tile": [32, 1], "grid": 256, "k_splits": 1, "whole_tiles": 0},
              "bytes": 2.69e8, "counters": "FETCH_SIZE 131 258 x 2.0 KiB + WRITE_SIZE 32 KiB (x and y are dense columns)",
                   "kernel": "gemv_kernel<float, float, 2, 1>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "a71aab952629f211b96873f786e22f30f3fd404ebf5bdd1262aadd103806703e", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "bd1e8a2fd885c5a4483c53bea615087b75da480171828cff8a68b201a3d6b229", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp32_gevm": {"plan": {"tile": [1, 32], "grid": 256, "k_splits": 1, "whole_tiles": 0},
-             "bytes": 2.69e8, "counters": "FETCH_SIZE 131 233 x 2.0 KiB + WRITE_SIZE 32 KiB",
+             "bytes": 2.69e8, "counters": "FETCH_SIZE 131 241 x 2.0 KiB + WRITE_SIZE 32 KiB",
                   "kernel": "gevm_kernel<float, float, 8>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "a71aab952629f211b96873f786e22f30f3fd404ebf5bdd1262aadd103806703e", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "bd1e8a2fd885c5a4483c53bea615087b75da480171828cff8a68b201a3d6b229", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp16_gemv": {"plan": {"tile": [32, 1], "grid": 256, "k_splits": 1, "whole_tiles": 0},
-             "bytes": 1.34e8, "counters": "FETCH_SIZE 65 647 x 2.0 KiB + WRITE_SIZE 16 KiB (x and y are dense columns)",
+             "bytes": 1.34e8, "counters": "FETCH_SIZE 65 659 x 2.0 KiB + WRITE_SIZE 16 KiB (x and y are dense columns)",
                   "kernel": "gemv_kernel<_Float16, _Float16, 2, 1>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "a71aab952629f211b96873f786e22f30f3fd404ebf5bdd1262aadd103806703e", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "bd1e8a2fd885c5a4483c53bea615087b75da480171828cff8a68b201a3d6b229", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "fp16_gevm": {"plan": {"tile": [1, 64], "grid": 256, "k_splits": 2, "whole_tiles": 0},
-             "bytes": 1.35e8, "counters": "FETCH_SIZE 65 685 x 2.0 KiB + WRITE_SIZE 92 KiB",
+             "bytes": 1.35e8, "counters": "FETCH_SIZE 65 683 x 2.0 KiB + WRITE_SIZE 92 KiB",
                   "kernel": "gevm_kernel<_Float16, _Float16, 8>", "source": "decx_amd/csrc/gemv.hip",
-                  "source_sha256": "a71aab952629f211b96873f786e22f30f3fd404ebf5bdd1262aadd103806703e", "profile": "profiles/gemv_gevm_8192x8192.md"},
+                  "source_sha256": "bd1e8a2fd885c5a4483c53bea615087b75da480171828cff8a68b201a3d6b229", "profile": "profiles/gemv_gevm_8192x8192.md"},
     "conv2d": {"bytes": 1.08e8, "counters": "FETCH_SIZE 20 527 x 2.0 KiB + WRITE_SIZE 64 546 KiB",
                "kernel": "gemm_f32_dma_kernel<256, 256, 2, 4, 16, 4, false, 2, false, false>", "source": "decx_amd/csrc/gemm_f32_dma.hip",
                "source_sha256": "05e995711ad2ff03fbcdb66fe8e73d86fadc8c04529cec00e667e61192f79bc9", "profile": "profiles/conv2d_implicit_gemm_256x256x112_3x3x256.md"},
@@ -342,6 +342,37 @@ def copy_rate(steps=10, warmup=3):
         d.free()
     return {"value": round(2 * n / ms / 1e6, 1), "unit": "GB/s", "what": "calibration copy kernel, 1 GiB read + 1 GiB written per launch",
             "kernel_ms": round(ms, 4), "write_only_gbs": round(n / fill_ms / 1e6, 1), "write_only_what": "fill of 1 GiB (hipMemsetAsync)"}
+
+
+def gemv_sizes(launches=50, batches=5):
+    """y = A.x through decx_hip_gemm_* on matrices of 2 MB to 2 GB (fp32 and fp16, dense x): time against size separates
+    what a launch costs whatever it moves from the rate at which the rows stream once they do.  Matrices beyond the
+    256 MB of the memory-side cache show the rate of HBM itself; the smaller ones are partly served by that cache from
+    launch to launch."""
+    from decx_amd import hip
+    rows = []
+    for dt, name in ((np.float32, "f32"), (np.float16, "f16")):
+        for M, K in ((8192, 64), (8192, 512), (8192, 2048), (8192, 4096), (8192, 8192), (8192, 16384), (16384, 8192), (32768, 8192),
+                     (65536, 8192)):
+            A = hip.DeviceMatrix(M, K, dt, K); X = hip.DeviceMatrix(K, 1, dt, 1); Y = hip.DeviceMatrix(M, 1, dt, 1)
+            hip.check(hip.lib().decx_hip_memset_async(A.ptr, 0, M * K * np.dtype(dt).itemsize, None))
+            for _ in range(10):
+                hip.gemm(A, X, Y)
+            hip.sync()
+            timer = hip.Timer(); best = 1e30
+            for _ in range(batches):
+                timer.start()
+                for _ in range(launches):
+                    hip.gemm(A, X, Y)
+                best = min(best, timer.stop() / launches)
+            mb = M * K * np.dtype(dt).itemsize / 1e6
+            rows.append({"dtype": name, "M": M, "K": K, "matrix_MB": round(mb, 1), "kernel_us": round(best * 1e3, 2),
+                         "GB/s": round(mb / best, 1)})
+            for d in (A, X, Y):
+                d.free()
+    big = [r for r in rows if r["matrix_MB"] > 1000]
+    return {"workload": "gemv over matrix sizes", "launches": launches, "batches": batches, "rows": rows,
+            "floor_us": min(r["kernel_us"] for r in rows), "streaming_GB/s": max(r["GB/s"] for r in big)}
 
 
 def add_sustained(out, sustained):
@@ -726,7 +757,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="fp32_8192", choices=sorted(WORKLOADS) + ["copy_1GiB", "mfma_f16", "planner_sweep", "conv2d", "conv2d_rgb", "c64_4096", "c128_2048"])
+    ap.add_argument("--workload", default="fp32_8192", choices=sorted(WORKLOADS) + ["copy_1GiB", "mfma_f16", "gemv_sizes", "planner_sweep", "conv2d", "conv2d_rgb", "c64_4096", "c128_2048"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     ap.add_argument("--sweep-seed", type=int, default=20261125, help="planner_sweep: seed of the shapes")
@@ -771,6 +802,9 @@ def main():
         return
     if args.workload == "mfma_f16":
         print(json.dumps(dict(sustained_mfma(launches=args.steps), workload="register-only matrix-core loop")))
+        return
+    if args.workload == "gemv_sizes":
+        print(json.dumps(gemv_sizes()))
         return
 
     if args.workload in ("conv2d", "conv2d_rgb"):

@@ -17,7 +17,7 @@
 //   matrices of fewer than 8192 rows, and below 4096 rows 2, 4, 8 or all 16 wavefronts share a row
 //   (they deal the steps of K among themselves), always the fewest that still give every CU a
 //   workgroup (2048 x 8192: 24.3 -> 16.1 us with a dense x, 512 x 32768: 60.9 -> 23.8); x is staged in LDS once per
-//   workgroup, as fp32, in chunks of 4096 -- x may be strided (the single column of a
+//   workgroup, as fp32, in chunks of 4096 (fp16: 8192) -- x may be strided (the single column of a
 //   pitched K x 1 matrix puts every element in its own cache line), so staging it once per
 //   32 rows keeps that gather small -- and a chunk of x is loaded into registers while the chunk
 //   before is being multiplied, so that its latency hides behind the rows (8192 x 8192: fp32 43.1 -> 42.0 us,
@@ -38,7 +38,7 @@ namespace {
 constexpr int GEMV_THREADS = 1024;
 constexpr int GEMV_WAVES = GEMV_THREADS / 64;
 constexpr int GEMV_ROWS_PER_BLOCK = 2 * GEMV_WAVES;
-constexpr int GEMV_KC = 4096;            // elements of x staged per chunk (16 KB of LDS, 32 KB for fp64)
+constexpr int GEMV_KC = 4096;            // elements of x staged per chunk (16 KB of LDS, 32 KB for fp64 and for gemv's fp16 chunks of twice as many)
 constexpr int GEMV_XPT = GEMV_KC / GEMV_THREADS;   // of which a thread carries this many
 
 typedef double doublex2 __attribute__((ext_vector_type(2)));
@@ -100,7 +100,12 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
 {
     typedef typename Acc<T>::type A_t;
     constexpr int N16 = Per16<T>::n;
-    __shared__ __attribute__((aligned(16))) A_t xs[GEMV_KC];
+    // fp16 rows are half as long in bytes: chunks of twice as many elements give a wavefront the same 16 KB of a row per
+    // chunk as fp32 and, with 16 steps per chunk, every wavefront of the workgroup a start of its own (with 8 they
+    // collided in pairs: 65536 x 8192 189 -> 177 us, 8192 x 16384 41.7 -> 40.8; fp32 gained nothing from the same, and
+    // four times as many take the kernel beyond 64 VGPRs)
+    constexpr int KC = sizeof(T) == 2 ? 2 * GEMV_KC : GEMV_KC, XPT = KC / GEMV_THREADS;
+    __shared__ __attribute__((aligned(16))) A_t xs[KC];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     static_assert(WPR == 1 || RPW == 1, "rows are split over wavefronts only one at a time");
     __shared__ A_t wave_sums[GEMV_WAVES];
@@ -114,7 +119,7 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
     // Every workgroup walks the same K range of rows that lie a whole number of pitches apart; started
     // together at k = 0 they would all pull on the same memory channels at the same time.  So each
     // workgroup starts at another chunk and each wavefront at another step inside it (sums commute).
-    const uint32_t chunks = (K + GEMV_KC - 1) / GEMV_KC;
+    const uint32_t chunks = (K + KC - 1) / KC;
     const uint32_t chunk0 = chunks ? (blockIdx.x * 3u) % chunks : 0u;
     // x travels one chunk ahead in registers, its loads dealt out among the steps of the chunk before: a strided x
     // (the column of a pitched K x 1 matrix) touches a cache line per element, and with one workgroup per CU the loads
@@ -122,28 +127,28 @@ gemv_kernel(const T* __restrict__ A, const T* __restrict__ x, const T* __restric
     // gevm_kernel does for B, takes this kernel beyond 64 VGPRs and with that from two workgroups per CU to one:
     // 16384 x 1024 13.2 -> 15.3 us, fp16 6.5 -> 9.9.)
     constexpr uint32_t STEP = 64 * N16;
-    constexpr int PER = GEMV_KC / (int)STEP / GEMV_XPT;    // steps per load of x: fp32 4, fp16 2, fp64 8
+    constexpr int PER = KC / (int)STEP / XPT;    // steps per load of x: fp32 4, fp16 2, fp64 8
     constexpr int XG = PER >= 4 ? 1 : 4 / PER;             // loads of x per group of at least 4 steps
-    constexpr int GROUPS = GEMV_XPT / XG;
-    T xr[GEMV_XPT];
+    constexpr int GROUPS = XPT / XG;
+    T xr[XPT];
     const auto fetch_x = [&](uint32_t kc, int j) {
         const uint32_t i = t + j * GEMV_THREADS;
         xr[j] = kc + i < K ? x[(size_t)(kc + i) * incx] : T(0);
     };
     if (chunks) {
 #pragma unroll
-        for (int j = 0; j < GEMV_XPT; ++j) fetch_x(chunk0 * GEMV_KC, j);
+        for (int j = 0; j < XPT; ++j) fetch_x(chunk0 * KC, j);
     }
     for (uint32_t ci = 0; ci < chunks; ++ci) {
         const uint32_t chunk = chunk0 + ci < chunks ? chunk0 + ci : chunk0 + ci - chunks;
-        const uint32_t kc = chunk * GEMV_KC;
-        const uint32_t len = (K - kc) < (uint32_t)GEMV_KC ? (K - kc) : (uint32_t)GEMV_KC;
+        const uint32_t kc = chunk * KC;
+        const uint32_t len = (K - kc) < (uint32_t)KC ? (K - kc) : (uint32_t)KC;
         __syncthreads();                                   // previous chunk fully consumed
 #pragma unroll
-        for (int j = 0; j < GEMV_XPT; ++j) xs[t + j * GEMV_THREADS] = to_acc(xr[j]);
+        for (int j = 0; j < XPT; ++j) xs[t + j * GEMV_THREADS] = to_acc(xr[j]);
         __syncthreads();
         const bool more = ci + 1 < chunks;
-        const uint32_t kc_next = (chunk + 1 < chunks ? chunk + 1 : 0u) * GEMV_KC;
+        const uint32_t kc_next = (chunk + 1 < chunks ? chunk + 1 : 0u) * KC;
         const uint32_t lenv = vec_ok ? (len / N16) * N16 : 0u;   // part done with 128-bit loads
         const uint32_t steps = (lenv + STEP - 1) / STEP;
         const uint32_t mine = has0 && steps > (uint32_t)sub ? (steps - sub + WPR - 1) / WPR : 0u;   // steps of this wavefront
