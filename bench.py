@@ -353,7 +353,7 @@ def gemv_sizes(launches=50, batches=5):
     rows = []
     for dt, name in ((np.float32, "f32"), (np.float16, "f16")):
         for M, K in ((8192, 64), (8192, 512), (8192, 2048), (8192, 4096), (8192, 8192), (8192, 16384), (16384, 8192), (32768, 8192),
-                     (65536, 8192)):
+                     (65536, 8192), (32768, 16384), (65536, 4096), (262144, 1024)):
             A = hip.DeviceMatrix(M, K, dt, K); X = hip.DeviceMatrix(K, 1, dt, 1); Y = hip.DeviceMatrix(M, 1, dt, 1)
             hip.check(hip.lib().decx_hip_memset_async(A.ptr, 0, M * K * np.dtype(dt).itemsize, None))
             for _ in range(10):
