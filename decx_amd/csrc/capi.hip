@@ -46,13 +46,28 @@ uint32_t* g_split_counters[kMaxDevices] = {};
 std::mutex g_counter_mutex;
 
 struct HipRingRuntime final : CounterRingRuntime {
-    std::vector<hipEvent_t> pool;
+    // Events that are not in use, per device (an event belongs to the device it was created on).  decx_hip_init() puts
+    // kEventsAtInit of them here, so that launches from several streams do not create events in the middle of a
+    // caller's loop; more are made only when that many windows are in flight at once.
+    static constexpr int kEventsAtInit = 32;
+    std::vector<hipEvent_t> pools[kMaxDevices];
+    std::vector<hipEvent_t>& pool() { return pools[g_dev.device >= 0 && g_dev.device < kMaxDevices ? g_dev.device : 0]; }
+    void prefill()
+    {
+        std::vector<hipEvent_t>& p = pool();
+        while ((int)p.size() < kEventsAtInit) {
+            hipEvent_t ev = nullptr;
+            if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) { (void)hipGetLastError(); return; }
+            p.push_back(ev);
+        }
+    }
     void* record_event(void* stream) override
     {
+        std::vector<hipEvent_t>& p = pool();
         hipEvent_t ev = nullptr;
-        if (!pool.empty()) { ev = pool.back(); pool.pop_back(); }
+        if (!p.empty()) { ev = p.back(); p.pop_back(); }
         else if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
-        if (hipEventRecord(ev, (hipStream_t)stream) != hipSuccess) { (void)hipGetLastError(); pool.push_back(ev); return nullptr; }
+        if (hipEventRecord(ev, (hipStream_t)stream) != hipSuccess) { (void)hipGetLastError(); p.push_back(ev); return nullptr; }
         return ev;
     }
     bool event_done(void* event) override
@@ -61,7 +76,7 @@ struct HipRingRuntime final : CounterRingRuntime {
         if (e != hipSuccess) (void)hipGetLastError();              // "not ready" is no error of the caller's
         return e == hipSuccess;
     }
-    void release_event(void* event) override { pool.push_back((hipEvent_t)event); }
+    void release_event(void* event) override { pool().push_back((hipEvent_t)event); }
     bool stream_idle_or_gone(void* stream) override
     {
         const auto gone = [](hipError_t e) {
@@ -611,6 +626,10 @@ int decx_hip_init(int device)
         if (!g_rings[device]) g_rings[device] = new CounterRing(kSplitCounters);
     }
     g_dev.device = device;
+    if (device < kMaxDevices) {
+        std::lock_guard<std::mutex> lock(g_counter_mutex);
+        g_ring_runtime.prefill();
+    }
     g_dev.compute_units = g_dev.prop.multiProcessorCount > 0 ? g_dev.prop.multiProcessorCount : 256;
     g_dev.ready = true;
     return DECX_HIP_OK;

@@ -145,7 +145,8 @@ DECX_HIP_API int decx_hip_gemm_f32(const float* A, const float* B, const float* 
  * zero between launches).  Launches outside graphs go round the lower half: the library hands a window to a new launch
  * only when the launches that had it before are known to be over -- they went to the same stream, an event recorded
  * behind them has completed, or their stream is idle -- and otherwise runs the product unsplit, which is never an
- * error.  A split launch that is recorded into a HIP graph gets a window of the upper half and keeps it for the life
+ * error.  (Events are recorded only once launches have come from more than one stream; they are drawn from a pool of 32
+ * that decx_hip_init makes, and more are created only while more windows than that are in flight at once.)  A split launch that is recorded into a HIP graph gets a window of the upper half and keeps it for the life
  * of the process (the graph may be replayed at any time; recording asks the runtime nothing but whether the stream is
  * recording); when that half is used up, later recordings run unsplit.  A graph's replays must not overlap each other.
  * Callers must not destroy a stream while split launches are in flight on it.  If a launch was cut short (a device fault, a reset), decx_hip_reset_split_counters() waits

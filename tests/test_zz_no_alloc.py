@@ -130,3 +130,41 @@ def test_static_workspace_reads_a_long_column_in_place(hip):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     ref = A.astype(np.float64) @ B.astype(np.float64)
     assert float(np.max(np.abs(got - ref))) / (float(np.max(np.abs(ref))) * np.sqrt(K)) <= 1e-5
+
+
+def test_static_workspace_allocates_nothing_between_two_streams(hip):
+    """Split launches from two streams carry events (a window goes to another stream only behind a completed one): they
+    come from the pool decx_hip_init made, so the amount of free device memory does not move here either."""
+    L = hip.lib()
+    M, N, K = 300, 300, 8192
+    A = synth.uniform_f32(M, K, 0x5900); B = synth.uniform_f32(K, N, 0x5901)
+    dA = hip.DeviceMatrix(M, K, np.float32, pitch32(K), A); dB = hip.DeviceMatrix(K, N, np.float32, pitch32(N), B)
+    dD1 = hip.DeviceMatrix(M, N, np.float32, pitch32(N)); dD2 = hip.DeviceMatrix(M, N, np.float32, pitch32(N))
+    need = L.decx_hip_gemm_f32_workspace(M, N, K)
+    ws = hip.DeviceMatrix(1, need // 4, np.float32)
+    s1, s2 = hip.Stream(), hip.Stream()
+
+    def round_of_two():
+        hip.check(L.decx_hip_gemm_f32_ws(dA.ptr, dB.ptr, None, dD2.ptr, M, N, K, dA.pitch, dB.pitch, 0, dD2.pitch, 1.0, 1.0,
+                                         ws.ptr, need, s2.handle), "gemm")
+        hip.check(L.decx_hip_gemm_f32_static(dA.ptr, dB.ptr, None, dD1.ptr, M, N, K, dA.pitch, dB.pitch, 0, dD1.pitch, 1.0, 1.0,
+                                             s1.handle), "gemm")
+
+    round_of_two(); s1.sync(); s2.sync()
+    want = dD1.download()
+    assert np.array_equal(want.view(np.uint32), dD2.download().view(np.uint32))
+    before = hip.split_counter_stats()
+    free_before = hip.mem_free_bytes()
+    print("no-alloc, two streams: 60 rounds", flush=True)
+    for _ in range(60):
+        round_of_two()
+    s1.sync(); s2.sync()
+    assert hip.mem_free_bytes() == free_before, "the calls changed the amount of free device memory"
+    after = hip.split_counter_stats()
+    assert after["events"] - before["events"] >= 100            # nearly every launch recorded one
+    assert np.array_equal(dD1.download().view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(dD2.download().view(np.uint32), want.view(np.uint32))
+    for s in (s1, s2):
+        s.destroy()
+    for d in (dA, dB, dD1, dD2, ws):
+        d.free()
