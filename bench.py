@@ -370,8 +370,31 @@ def gemv_sizes(launches=50, batches=5):
                          "GB/s": round(mb / best, 1)})
             for d in (A, X, Y):
                 d.free()
+    # the transposed form, y = x.B (K x N), with the workspace its split over ranges of K wants
+    gevm_rows = []
+    for dt, name in ((np.float32, "f32"), (np.float16, "f16")):
+        esz = np.dtype(dt).itemsize
+        for K, N in ((8192, 8192), (32768, 8192), (8192, 32768), (131072, 2048)):
+            B = hip.DeviceMatrix(K, N, dt, N); X = hip.DeviceMatrix(1, K, dt, K); Y = hip.DeviceMatrix(1, N, dt, N)
+            hip.check(hip.lib().decx_hip_memset_async(B.ptr, 0, K * N * esz, None))
+            need = int(hip.lib().decx_hip_gemm_workspace(esz, 1, N, K))
+            W = hip.DeviceMatrix(1, max(need // 4, 4), np.float32)
+            for _ in range(10):
+                hip.gemm(X, B, Y, workspace=W)
+            hip.sync()
+            timer = hip.Timer(); best = 1e30
+            for _ in range(batches):
+                timer.start()
+                for _ in range(launches):
+                    hip.gemm(X, B, Y, workspace=W)
+                best = min(best, timer.stop() / launches)
+            mb = K * N * esz / 1e6
+            gevm_rows.append({"dtype": name, "K": K, "N": N, "matrix_MB": round(mb, 1), "kernel_us": round(best * 1e3, 2),
+                              "GB/s": round(mb / best, 1), "k_splits": int(hip.plan(esz, 1, N, K).k_splits)})
+            for d in (B, X, Y, W):
+                d.free()
     big = [r for r in rows if r["matrix_MB"] > 1000]
-    return {"workload": "gemv over matrix sizes", "launches": launches, "batches": batches, "rows": rows,
+    return {"workload": "gemv over matrix sizes", "launches": launches, "batches": batches, "rows": rows, "gevm_rows": gevm_rows,
             "floor_us": min(r["kernel_us"] for r in rows), "streaming_GB/s": max(r["GB/s"] for r in big)}
 
 
