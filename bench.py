@@ -338,10 +338,24 @@ def copy_rate(steps=10, warmup=3):
     for _ in range(steps):
         hip.check(hip.lib().decx_hip_memset_async(dst.ptr, 0, n, None))
     fill_ms = timer.stop() / steps
+    # and a read-only pass over both gigabytes, laid end to end: far more than the 256 MB memory-side cache holds
     for d in (src, dst):
         d.free()
+    both = hip.DeviceMatrix(1, 2 * n // 4, np.float32)
+    sink = hip.DeviceMatrix(1, 2 * n // 2048, np.uint32)
+    hip.check(hip.lib().decx_hip_memset_async(both.ptr, 1, 2 * n, None))
+    for _ in range(warmup):
+        hip.check(hip.lib().decx_hip_calibration_read(both.ptr, 2 * n, sink.ptr, 2 * n // 2048, None))
+    hip.sync()
+    timer.start()
+    for _ in range(steps):
+        hip.check(hip.lib().decx_hip_calibration_read(both.ptr, 2 * n, sink.ptr, 2 * n // 2048, None))
+    read_ms = timer.stop() / steps
+    for d in (both, sink):
+        d.free()
     return {"value": round(2 * n / ms / 1e6, 1), "unit": "GB/s", "what": "calibration copy kernel, 1 GiB read + 1 GiB written per launch",
-            "kernel_ms": round(ms, 4), "write_only_gbs": round(n / fill_ms / 1e6, 1), "write_only_what": "fill of 1 GiB (hipMemsetAsync)"}
+            "kernel_ms": round(ms, 4), "write_only_gbs": round(n / fill_ms / 1e6, 1), "write_only_what": "fill of 1 GiB (hipMemsetAsync)",
+            "read_only_gbs": round(2 * n / read_ms / 1e6, 1), "read_only_what": "calibration read kernel over 2 GiB (128-bit loads in the order the matrix x vector kernel reads rows of 64 KB, nothing stored)"}
 
 
 def gemv_sizes(launches=50, batches=5):
@@ -396,6 +410,27 @@ def gemv_sizes(launches=50, batches=5):
     big = [r for r in rows if r["matrix_MB"] > 1000]
     return {"workload": "gemv over matrix sizes", "launches": launches, "batches": batches, "rows": rows, "gevm_rows": gevm_rows,
             "floor_us": min(r["kernel_us"] for r in rows), "streaming_GB/s": max(r["GB/s"] for r in big)}
+
+
+def launch_floor(launches=200, batches=3):
+    """Microseconds from launch to launch of a kernel that has next to nothing to do (y = A.x on a 2 MB matrix, one
+    workgroup per CU): what any single launch costs on this board before its own work counts."""
+    from decx_amd import hip
+    M, K = 8192, 64
+    A = hip.DeviceMatrix(M, K, np.float32, K); X = hip.DeviceMatrix(K, 1, np.float32, 1); Y = hip.DeviceMatrix(M, 1, np.float32, 1)
+    hip.check(hip.lib().decx_hip_memset_async(A.ptr, 0, M * K * 4, None))
+    for _ in range(20):
+        hip.gemm(A, X, Y)
+    hip.sync()
+    timer = hip.Timer(); best = 1e30
+    for _ in range(batches):
+        timer.start()
+        for _ in range(launches):
+            hip.gemm(A, X, Y)
+        best = min(best, timer.stop() / launches)
+    for d in (A, X, Y):
+        d.free()
+    return round(best * 1e3, 2)
 
 
 def add_sustained(out, sustained):
@@ -861,6 +896,8 @@ def main():
     if not args.no_extra:
         copy = copy_rate()
         line["config"]["copy_rate"] = copy
+        floor_us = launch_floor()
+        line["config"]["launch_floor_us"] = floor_us
         for name in WORKLOADS:
             if name != args.workload:
                 small = WORKLOADS[name][1] * WORKLOADS[name][2] * WORKLOADS[name][3] < 2 ** 38
@@ -892,6 +929,9 @@ def main():
         rgb["roofline"]["copy_rate_gbs"] = copy["value"]           # what this board moves when half the traffic is writes
         rgb["roofline"]["frac_of_copy_rate"] = round(rgb["roofline"]["achieved"] / copy["value"], 4)
         rgb["roofline"]["write_only_gbs"] = copy["write_only_gbs"]  # ... and when all of it is (73 % of this workload's bytes are)
+        # a launch of next to nothing, plus the workload's algorithmic bytes at the copy kernel's rate
+        rgb["roofline"]["floor_us"] = round(floor_us + rgb["roofline"]["achieved"] * rgb["kernel_ms"] * 1e3 / copy["value"], 2)
+        rgb["roofline"]["frac_of_floor"] = round(rgb["roofline"]["floor_us"] / (rgb["kernel_ms"] * 1e3), 4)
         others.append(rgb)
         others.append(run_complex(False, 4096, args.steps, args.warmup, parity=not args.no_cpu))
         others.append(run_complex(True, 2048, 50, args.warmup, parity=not args.no_cpu))

@@ -495,6 +495,58 @@ __global__ void __launch_bounds__(256) calibration_copy_kernel(uintx4* __restric
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
 }
 
+// A read-only pass in the pattern the matrix x vector kernel reads its rows in, which is the one HBM answers best of those
+// tried (2 GiB: a grid-stride loop 5.5 TB/s, a contiguous region per wavefront or per workgroup 6.0-6.3, this 6.6-6.7): the
+// buffer as rows of 64 KB, a workgroup of 16 wavefronts on 32 of them, a wavefront on two, 1 KB of each a step, every
+// wavefront starting at another step.  Every 16-byte piece is loaded once and folded into a word per lane that is stored
+// only if it comes out as a value the fold cannot produce from a buffer filled with one byte value: nothing is written.
+constexpr uint32_t kReadRow16 = 65536 / 16;        // 16-byte pieces per row
+__global__ void __launch_bounds__(1024) calibration_read_kernel(const uintx4* __restrict__ src, uint32_t* __restrict__ sink, uint32_t never)
+{
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uintx4* a = src + ((size_t)blockIdx.x * 32 + wave * 2) * kReadRow16 + lane;
+    const uintx4* b = a + kReadRow16;
+    constexpr uint32_t steps = kReadRow16 / 64;
+    const uint32_t s0 = ((blockIdx.x * 16 + wave) * 5u) % steps;
+    uint32_t fold = 0;
+    for (uint32_t s = 0; s < steps; s += 4) {
+        uintx4 v[4], w[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            const uint32_t at = (s0 + s + u) % steps;
+            v[u] = a[(size_t)at * 64]; w[u] = b[(size_t)at * 64];
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) fold ^= v[u][0] ^ v[u][1] ^ v[u][2] ^ v[u][3] ^ w[u][0] ^ w[u][1] ^ w[u][2] ^ w[u][3];
+    }
+    if (fold == never) sink[(size_t)blockIdx.x * 1024 + threadIdx.x] = fold;
+}
+
+// The copy in the same order (whole blocks of 2 MiB; what is left over goes through calibration_copy_kernel), with
+// streaming stores.  1 GiB: 5.7-5.9 TB/s of reads plus writes, where the grid-stride loop above moves 4.6-4.8 and the
+// runtime's own device-to-device copy 5.0.
+__global__ void __launch_bounds__(1024) calibration_copy_rows_kernel(uintx4* __restrict__ dst, const uintx4* __restrict__ src)
+{
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const size_t a = ((size_t)blockIdx.x * 32 + wave * 2) * kReadRow16 + lane, b = a + kReadRow16;
+    constexpr uint32_t steps = kReadRow16 / 64;
+    const uint32_t s0 = ((blockIdx.x * 16 + wave) * 5u) % steps;
+    for (uint32_t s = 0; s < steps; s += 4) {
+        uintx4 v[4], w[4];
+        size_t at[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            at[u] = (size_t)((s0 + s + u) % steps) * 64;
+            v[u] = src[a + at[u]]; w[u] = src[b + at[u]];
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            __builtin_nontemporal_store(v[u], dst + a + at[u]);
+            __builtin_nontemporal_store(w[u], dst + b + at[u]);
+        }
+    }
+}
+
 // Register-only matrix-core loops: what the matrix pipe sustains on this board with nothing else to do -- no loads,
 // no LDS, no barriers -- on operands of the caller's choosing (their values set the power drawn, and with it the
 // clock the board's power management allows).  8 wavefronts per CU, two per SIMD, the accumulator layouts of the
@@ -578,10 +630,28 @@ int decx_hip_calibration_copy(void* dst, const void* src, size_t bytes, void* st
     if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
     if (!bytes) return DECX_HIP_OK;
     if (!dst || !src || (bytes & 15u) || !aligned16(dst) || !aligned16(src)) return DECX_HIP_E_INVALID_ARG;
-    const size_t n16 = bytes / 16;
-    const size_t want = (n16 + 255) / 256;
-    const dim3 grid((unsigned)(want < 16384 ? want : 16384)), block(256);
-    hipLaunchKernelGGL(calibration_copy_kernel, grid, block, 0, as_stream(stream), (uintx4*)dst, (const uintx4*)src, n16);
+    constexpr size_t kBlockBytes = (size_t)32 * kReadRow16 * 16;           // 2 MiB per workgroup of the fast form
+    const size_t blocks = bytes / kBlockBytes < 0x7fffffffu ? bytes / kBlockBytes : 0;
+    if (blocks)
+        hipLaunchKernelGGL(calibration_copy_rows_kernel, dim3((unsigned)blocks), dim3(1024), 0, as_stream(stream), (uintx4*)dst, (const uintx4*)src);
+    const size_t done16 = blocks * kBlockBytes / 16, n16 = bytes / 16 - done16;
+    if (n16) {
+        const size_t want = (n16 + 255) / 256;
+        const dim3 grid((unsigned)(want < 16384 ? want : 16384)), block(256);
+        hipLaunchKernelGGL(calibration_copy_kernel, grid, block, 0, as_stream(stream), (uintx4*)dst + done16, (const uintx4*)src + done16, n16);
+    }
+    return (int)hipGetLastError();
+}
+
+int decx_hip_calibration_read(const void* src, size_t bytes, uint32_t* sink, size_t sink_words, void* stream)
+{
+    if (!g_dev.ready) return DECX_HIP_E_NOT_INIT;
+    if (!bytes) return DECX_HIP_OK;
+    constexpr size_t kBlockBytes = (size_t)32 * kReadRow16 * 16;           // 2 MiB per workgroup
+    const size_t blocks = bytes / kBlockBytes;
+    if (!src || bytes % kBlockBytes || blocks > 0x7fffffffu || !aligned16(src) || !sink || sink_words < blocks * 1024) return DECX_HIP_E_INVALID_ARG;
+    hipLaunchKernelGGL(calibration_read_kernel, dim3((unsigned)blocks), dim3(1024), 0, as_stream(stream), (const uintx4*)src, sink,
+                       0x5a5a5a5bu);                           // (a buffer filled with one byte value folds to a word of four equal bytes)
     return (int)hipGetLastError();
 }
 

@@ -9,7 +9,8 @@
 // instruction; the vector pipe does one fma per (pixel, patch element, kernel), which is the arithmetic itself.
 //
 // What bounds it is the memory system's rate for traffic that is mostly writes (1920 x 1080 x 3, 8 kernels: 25 MB in,
-// 66 MB out in 23 us; a plain copy kernel moves 4.6 TB/s of reads plus writes on this part, i.e. 20 us for these 91 MB):
+// 66 MB out in 20.5-23 us; a copy kernel in the access order this part answers best moves 5.7-6.0 TB/s of reads plus
+// writes, i.e. 15 us for these 91 MB, and a launch of next to nothing takes 4 us):
 // the same arithmetic on the matrix cores (v_mfma_f32_4x4x1_16b_f32 with the weights of four kernels as one operand and
 // the lane's own patch element as the other leaves every lane with its pixel's four outputs, bit for bit the same chain,
 // in a sixteenth of the instructions) measured 23.2 us there and lost on smaller and larger images (640 x 480: 8.5

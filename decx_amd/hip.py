@@ -79,6 +79,7 @@ SYMBOLS = {
     "decx_hip_gemm_f16_tile": (_int, [_vp] * 4 + [_u32] * 7 + [_f, _f, _vp, _int, _int]),
     "decx_hip_gemm_plan": (_int, [_int, _u32, _u32, _u32, _int, ctypes.POINTER(Plan)]),
     "decx_hip_calibration_copy": (_int, [_vp, _vp, _sz, _vp]),
+    "decx_hip_calibration_read": (_int, [_vp, _sz, _vp, _sz, _vp]),
     "decx_hip_gemm_forced_plan": (_int, [_int] + [_vp] * 4 + [_u32] * 7 + [ctypes.c_double, ctypes.c_double, _int, _u32, _u32, _vp, _sz, _vp]),
     "decx_hip_calibration_mfma": (_int, [_int, _vp, _sz, _vp, _sz, _u32, ctypes.POINTER(ctypes.c_double), _vp]),
     "decx_hip_float_to_half": (ctypes.c_uint16, [_f]),

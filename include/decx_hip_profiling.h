@@ -17,6 +17,13 @@ extern "C" {
  * (reads = writes = `bytes`). */
 DECX_HIP_API int decx_hip_calibration_copy(void* dst, const void* src, size_t bytes, void* stream);
 
+/* A read-only pass over `bytes` (a multiple of 2 MiB, 16-byte aligned) of device memory filled with ONE byte value
+ * (decx_hip_memset_async): 128-bit loads in the order the matrix x vector kernel reads rows of 64 KB, nothing stored --
+ * `sink` (at least bytes / 2048 words) is only written if the fold of the loaded words came out as a value such a fill
+ * cannot give.  What the memory system gives a pure read stream, the yardstick for the matrix x vector kernels.  No
+ * counterpart in the reference. */
+DECX_HIP_API int decx_hip_calibration_read(const void* src, size_t bytes, uint32_t* sink, size_t sink_words, void* stream);
+
 /* A register-only loop on the matrix cores: no loads, no LDS, no barriers -- what the matrix pipe sustains on this
  * board under its power management, for the operand values given.  One workgroup of 8 wavefronts per CU, each wavefront
  * `iters` times over 16 tiles of v_mfma_f32_16x16x32_f16 (elem_bytes 2: operands are halves) or 4 steps over 8 tiles of
