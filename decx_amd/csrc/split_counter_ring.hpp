@@ -8,7 +8,8 @@
 //   * its stream is idle, or no longer exists (a stream is only destroyed once its work is done).
 // A window whose earlier owners cannot be shown to be over is NOT handed out: take() returns kNone and the caller runs
 // the product unsplit.  Events are only recorded once launches have been seen on more than one stream; a caller with
-// one stream pays nothing.
+// one stream pays nothing.  The oldest owners are let go as soon as they are over for every stream (one query per
+// take()), so that no more events are out than launches are in flight.
 // Launches recorded into a graph are replayed at times the host does not see: they get windows of their own from the
 // upper half of the array, which the ring never enters and which are never handed out twice.  Nothing has to be proved
 // over for them, so recording a graph asks the runtime nothing (a query made while a stream records can end the
@@ -48,6 +49,12 @@ public:
         if (n == 0 || n > top_) { ++stats_.refused; return kNone; }
         if (have_last_ && key != last_key_) multi_stream_ = true;
         last_key_ = key; have_last_ = true;
+        // the oldest owners whose events have completed are over for everybody: their events go back to the runtime now, so
+        // that no more of them are out than launches are in flight
+        while (multi_stream_ && !owners_.empty() && over(rt, 0, kNobody)) {
+            if (owners_.front().event) rt.release_event(owners_.front().event);
+            owners_.pop_front();
+        }
         uint32_t begin = cursor_;
         const bool wrap = begin + n > top_;
         // the stretch the cursor passes over: up to the top when the window does not fit in front of it, then the window
@@ -113,7 +120,7 @@ private:
     bool over(CounterRingRuntime& rt, size_t i, uint64_t key)
     {
         const Owner& o = owners_[i];
-        if (o.key == key) return true;                               // same stream: in order
+        if (key != kNobody && o.key == key) return true;             // same stream: in order
         if (o.event && rt.event_done(o.event)) return true;
         for (size_t j = i + 1; j < owners_.size(); ++j)              // a later launch on its stream whose event is done covers it
             if (owners_[j].key == o.key && owners_[j].event && rt.event_done(owners_[j].event)) return true;
@@ -139,6 +146,7 @@ private:
         return true;
     }
 
+    static constexpr uint64_t kNobody = ~0ull;      // over(): the launch is over for every stream, not only for its own
     uint32_t capacity_, top_, graph_top_;
     uint32_t cursor_ = 0;
     std::deque<Owner> owners_;          // in the order taken = ring order starting at the oldest

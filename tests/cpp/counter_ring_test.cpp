@@ -143,6 +143,20 @@ static void reset_forgets()
     std::puts("ok reset_forgets");
 }
 
+static void events_come_back_when_launches_finish()
+{
+    CounterRing ring(2 * 65536); SimRuntime rt;                    // far from wrapping: nothing is retired by the cursor
+    int most = 0;
+    for (int i = 0; i < 1000; ++i) {
+        REQUIRE(submit(ring, rt, i & 1, 10) != CounterRing::kNone);
+        if (i % 4 == 3) { rt.advance(S(0), 100); rt.advance(S(1), 100); }      // both streams drain every four launches
+        most = rt.live_events > most ? rt.live_events : most;
+    }
+    REQUIRE(ring.stats().events >= 998);
+    REQUIRE(most <= 8);                                            // as many events out as launches in flight, not as launches made
+    std::puts("ok events_come_back_when_launches_finish");
+}
+
 static void random_traffic(unsigned seed, int streams, uint32_t capacity, uint32_t max_n)
 {
     CounterRing ring(2 * capacity); SimRuntime rt;                  // `capacity` counters to go round in, as many for graphs
@@ -187,6 +201,7 @@ int main()
     a_later_event_covers_earlier_launches();
     graph_launches_keep_their_windows();
     reset_forgets();
+    events_come_back_when_launches_finish();
     random_traffic(1, 1, 4096, 512);
     random_traffic(2, 2, 4096, 512);
     random_traffic(3, 5, 65536, 4096);

@@ -16,6 +16,6 @@ def test_counter_windows_on_simulated_streams(tmp_path):
     assert run.returncode == 0, run.stdout + run.stderr
     assert "all ok" in run.stdout
     for name in ("one_stream_wraps_freely", "second_stream_waits_for_the_first", "a_later_event_covers_earlier_launches",
-                 "graph_launches_keep_their_windows", "reset_forgets"):
+                 "graph_launches_keep_their_windows", "reset_forgets", "events_come_back_when_launches_finish"):
         assert "ok " + name in run.stdout
     assert run.stdout.count("ok random_traffic") == 4
